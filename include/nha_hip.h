@@ -1,0 +1,175 @@
+/*
+ * nha_hip.h -- C ABI of libnha_hip.so: the MI355X (gfx950) implementation of NHA's fused
+ * hybrid-attention hot path (gated-slot memory + sliding window under ONE softmax).
+ *
+ * The reference (JusenD/NHA) has no FFI layer: its boundary is the Python op API
+ *   nha_fla/ops/nha/chunk.py:568-585            chunk_nha
+ *   nha_fla/ops/nha/chunk_fused.py:291-303      fused_chunk_nha_prefill
+ *   nha_fla/ops/nha/fused_recurrent.py:431-445  fused_recurrent_nha_decode
+ *   nha_fla/ops/nha/fused_recurrent.py:588-598  fused_recurrent_nha
+ * Each entry point below states which of those it sits behind.  The host-side mirror of that
+ * Python API (same names, argument meaning and error behaviour) is nha_amd/ops.py, which binds
+ * this library with ctypes; no torch type crosses this boundary.
+ *
+ * Conventions: every pointer is a DEVICE pointer unless marked "host"; the caller owns every
+ * buffer (the library never allocates or frees device memory); tensors are dense row-major in
+ * the stated shape; functions return NHA_OK or a negative NHA_ERR_* code and never throw;
+ * nha_last_error() gives the message of the calling thread's last failure.  Work is enqueued on
+ * `stream` (a hipStream_t, may be NULL for the default stream) and is asynchronous.
+ */
+#ifndef NHA_HIP_H
+#define NHA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NHA_ABI_VERSION 1
+
+enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
+enum {
+  NHA_OK = 0,
+  NHA_ERR_INVALID = -1,      /* bad argument (null pointer, non-positive dim, HQ % H != 0 ...) */
+  NHA_ERR_UNSUPPORTED = -2,  /* valid call the kernels cannot serve (shape outside the built set) */
+  NHA_ERR_SCRATCH = -3,      /* scratch buffer smaller than nha_prefill_scratch_bytes() */
+  NHA_ERR_LAUNCH = -4        /* HIP reported an error at launch */
+};
+enum { NHA_IMPL_AUTO = 0, NHA_IMPL_SIMPLE = 1, NHA_IMPL_MFMA = 2 };
+
+/* ------------------------------------------------------------------------------------------
+ * Chunked prefill forward.  Replaces ChunkNativeHybridAttentionFunction.forward
+ * (nha_fla/ops/nha/chunk.py:367-488: optional slot-branch shift :401-420, SWA branch :423-431,
+ * GSA branch :437-445, LSE merge :459-470) and the two kernels of fused_chunk_nha_prefill
+ * (nha_fla/ops/nha/chunk_fused.py:30-283), GQA-native.
+ *
+ * Packed token-major layout (the reference's flattened '(b t) h d', chunk.py:665-671):
+ *   q_swa, q_gsa [T_tot, HQ, K]   k_swa, k_gsa [T_tot, H, K]   v [T_tot, H, V]   s, g [T_tot, H, M]
+ *   o [T_tot, HQ, V] (input dtype)   lse_swa, lse_gsa [T_tot, HQ] fp32 (either may be NULL)
+ *   h0k [N,H,K,M], h0v [N,H,M,V] fp32 or NULL;  hkt, hvt same shapes, or NULL when not wanted
+ *   cu_seqlens int32 [N+1] (batched mode: arange(0,(B+1)T,T), chunk.py:660)
+ *   chunk_indices int32 [NT,2] rows (sequence, chunk-in-sequence), chunk_offsets int32 [N+1]:
+ *     as produced by nha_varlen_indices() with chunk size 64.
+ * Semantics per token t of a sequence [bos,eos): window keys j in [max(bos, t-wl), t] (wl < 0:
+ * unbounded); the slots have absorbed tokens bos .. t-shift (shift >= 0); one softmax over
+ * [M slot logits | window logits]; q-head hq reads kv-head hq / (HQ/H).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct NhaPrefillArgs {
+  const void* q_swa;
+  const void* k_swa;
+  const void* q_gsa;
+  const void* k_gsa;
+  const void* v;
+  const void* s;
+  const void* g;
+  void* o;
+  float* lse_swa;
+  float* lse_gsa;
+  const float* h0k;
+  const float* h0v;
+  float* hkt;
+  float* hvt;
+  const int32_t* cu_seqlens;
+  const int32_t* chunk_indices;
+  const int32_t* chunk_offsets;
+  void* scratch;
+  size_t scratch_bytes;
+  int32_t T_tot, N, NT, HQ, H, K, V, M;
+  int32_t wl;     /* window_size_left; < 0 = unbounded */
+  int32_t shift;  /* gsa_kv_shift */
+  int32_t dtype;  /* NHA_DTYPE_* of q/k/v/s/g/o */
+  int32_t impl;   /* NHA_IMPL_* */
+  float scale;
+  void* stream;
+} NhaPrefillArgs;
+
+/* Bytes of device scratch nha_prefill_fwd needs for these dims (chunk-start slot states, gate
+ * cumsums, staging).  Only the integer/dtype/impl fields of `a` are read. */
+size_t nha_prefill_scratch_bytes(const NhaPrefillArgs* a);
+int nha_prefill_fwd(const NhaPrefillArgs* a);
+
+/* ------------------------------------------------------------------------------------------
+ * Single-token decode step.  Replaces the k/v kernel pair of fused_recurrent_nha_decode
+ * (nha_fla/ops/nha/fused_recurrent.py:228-428, host :431-584) and, with `win_logits`, the
+ * kernel pair + host softmax of fused_recurrent_nha (:47-225).  One launch; a workgroup owns a
+ * (sequence, kv-head) and serves all HQ/H query heads, so state and window are read once.
+ *
+ * mode NHA_DECODE_WINDOW: explicit popped entry k_pop/v_pop/g_pop [B,H,*] (s_pop optional,
+ *   else 1-exp(g), :282-285) and a time-ordered window win_k/win_v [B,W,H,*], all W rows valid
+ *   (:287-288).  Either `sq` (pre-rotated query, pre-rotated win_k) or cos/sin tables
+ *   [B|1, W, K] (row stride cos_sw, batch stride cos_sb = 0 to broadcast; row W-1 is the query
+ *   position) for in-kernel rotate-half RoPE of raw q / win_k (:309-329).
+ * mode NHA_DECODE_LOGITS: explicit popped entry and caller-supplied window logits
+ *   win_logits [B,HQ,W] (input dtype); writes the window probabilities win_probs [B,HQ,W] fp32
+ *   and the slot part of the output only (:200-205, :143-145).
+ * mode NHA_DECODE_RING: W-slot ring buffers ring_k (window keys), ring_kg (slot-branch keys),
+ *   ring_v, ring_g [B,W,H,*] resident in HBM and count[b] = tokens cached so far.  The step
+ *   pops slot count%W into the slots when count >= W, stores the new token (k_new, kg_new,
+ *   v_new, g_new [B,H,*]) there, and attends over the min(count+1, W) valid entries.  The
+ *   caller advances count (nha_decode_advance) after the step.  No reference counterpart: it
+ *   replaces the cat-shift cache of nha_fla/models/nha_cache.py:105-131, :143-154.
+ * State hk [B,H,K,M], hv [B,H,M,V] fp32: read from hk_in/hv_in (NULL = zeros), written to
+ * hk_out/hv_out (NULL = not written; may alias the inputs, fused_recurrent.py:541-545).
+ * o [B,HQ,V] in the input dtype.
+ * ------------------------------------------------------------------------------------------ */
+enum { NHA_DECODE_WINDOW = 0, NHA_DECODE_LOGITS = 1, NHA_DECODE_RING = 2 };
+
+typedef struct NhaDecodeArgs {
+  int32_t mode;
+  int32_t dtype;
+  int32_t B, HQ, H, K, V, M, W;
+  float scale;
+  const void* q;   /* [B,HQ,K] raw query: slot logits (and the rotated window query when cos/sin) */
+  const void* sq;  /* [B,HQ,K] pre-rotated window query, or NULL */
+  const void* k_pop;
+  const void* v_pop;
+  const void* g_pop;
+  const void* s_pop;
+  const void* win_k;
+  const void* win_v;
+  const void* cos;
+  const void* sin;
+  int64_t cos_sb, cos_sw;
+  const void* win_logits;
+  float* win_probs;
+  void* ring_k;
+  void* ring_kg;
+  void* ring_v;
+  void* ring_g;
+  const void* k_new;
+  const void* kg_new;
+  const void* v_new;
+  const void* g_new;
+  const int32_t* count;
+  const float* hk_in;
+  const float* hv_in;
+  float* hk_out;
+  float* hv_out;
+  void* o;
+  void* stream;
+} NhaDecodeArgs;
+
+int nha_decode_step(const NhaDecodeArgs* a);
+/* count[b] += 1 for b < B (ring mode bookkeeping between steps). */
+int nha_decode_advance(int32_t* count, int32_t B, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Varlen chunk tables (HOST pointers, pure integer, no GPU).  Replaces fla's
+ * prepare_chunk_indices / prepare_chunk_offsets as consumed at
+ * nha_fla/ops/nha_naive/chunk.py:59-64, :557-558: rows (i_n, i_t) in sequence-major order,
+ * NT = sum_n ceil(L_n / BT); chunk_off is the exclusive prefix sum of ceil(L_n / BT).
+ * nha_varlen_num_chunks returns NT (or a negative error for a non-increasing cu_seqlens).
+ * ------------------------------------------------------------------------------------------ */
+int32_t nha_varlen_num_chunks(const int32_t* cu_seqlens_host, int32_t N, int32_t BT);
+int nha_varlen_indices(const int32_t* cu_seqlens_host, int32_t N, int32_t BT,
+                       int32_t* chunk_idx_host /* [NT,2] */, int32_t* chunk_off_host /* [N+1] */);
+
+const char* nha_last_error(void);
+int nha_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NHA_HIP_H */

@@ -1,0 +1,56 @@
+"""Build libnha_hip.so (gfx950) in-tree with hipcc.  `python -m nha_amd.build` or build_library()."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libnha_hip.so")
+SOURCES = ["abi.hip", "decode.hip", "prefill_simple.hip", "prefill_mfma.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math" if False else "-fno-fast-math",
+    # hipcc -O3 may otherwise emit packed-fp32 VALU forms from ordinary float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result", "-Wno-unknown-warning-option",
+]
+
+
+def build_library(verbose: bool = False, jobs: int = 4) -> str:
+    objs = []
+    procs = []
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    for src in SOURCES:
+        obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+        if len(procs) >= jobs:
+            _drain(procs)
+    _drain(procs)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        raise RuntimeError("link failed:\n" + out.stdout)
+    return LIB
+
+
+def _drain(procs):
+    while procs:
+        src, p = procs.pop(0)
+        out, _ = p.communicate()
+        real = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l and l.strip())
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+        if real and os.environ.get("NHA_BUILD_VERBOSE"):
+            print(real)
+
+
+if __name__ == "__main__":
+    print(build_library(verbose="-v" in sys.argv))

@@ -1,0 +1,126 @@
+// extern "C" surface of libnha_hip.so (declared in include/nha_hip.h): argument validation,
+// implementation choice, the host-side varlen chunk tables and the error string.
+#include "common.h"
+
+#include <string.h>
+
+namespace nha {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+static int check_prefill(const NhaPrefillArgs* a, bool pointers) {
+  NHA_CHECK_ARG(a != nullptr, "nha_prefill: null args");
+  NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->NT > 0 && a->HQ > 0 && a->H > 0 && a->K > 0 && a->V > 0 && a->M > 0,
+                "nha_prefill: non-positive dimension");
+  NHA_CHECK_ARG(a->HQ % a->H == 0, "nha_prefill: HQ (%d) must be a multiple of H (%d)", a->HQ, a->H);
+  NHA_CHECK_ARG(a->shift >= 0, "nha_prefill: gsa_kv_shift must be >= 0, got %d", a->shift);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_prefill: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->impl >= NHA_IMPL_AUTO && a->impl <= NHA_IMPL_MFMA, "nha_prefill: bad impl %d", a->impl);
+  if (pointers) {
+    NHA_CHECK_ARG(a->q_swa && a->k_swa && a->q_gsa && a->k_gsa && a->v && a->s && a->g && a->o,
+                  "nha_prefill_fwd: q_swa, k_swa, q_gsa, k_gsa, v, s, g, o are required");
+    NHA_CHECK_ARG(a->cu_seqlens && a->chunk_indices && a->chunk_offsets,
+                  "nha_prefill_fwd: cu_seqlens, chunk_indices and chunk_offsets are required");
+    NHA_CHECK_ARG((a->h0k == nullptr) == (a->h0v == nullptr), "nha_prefill_fwd: pass both initial states or neither");
+    NHA_CHECK_ARG((a->hkt == nullptr) == (a->hvt == nullptr), "nha_prefill_fwd: pass both final states or neither");
+    NHA_CHECK_ARG(a->scratch != nullptr, "nha_prefill_fwd: scratch is required");
+  }
+  return NHA_OK;
+}
+
+static bool use_mfma(const NhaPrefillArgs* a) {
+  if (a->impl == NHA_IMPL_SIMPLE) return false;
+  return prefill_mfma_supported(a);
+}
+
+}  // namespace nha
+
+using namespace nha;
+
+extern "C" {
+
+size_t nha_prefill_scratch_bytes(const NhaPrefillArgs* a) {
+  if (check_prefill(a, false) != NHA_OK) return 0;
+  return use_mfma(a) ? prefill_mfma_scratch_bytes(a) : prefill_simple_scratch_bytes(a);
+}
+
+int nha_prefill_fwd(const NhaPrefillArgs* a) {
+  int rc = check_prefill(a, true);
+  if (rc != NHA_OK) return rc;
+  const bool mfma = use_mfma(a);
+  if (a->impl == NHA_IMPL_MFMA && !mfma) {
+    set_error("nha_prefill_fwd: the MFMA kernels are not built for dtype=%d K=%d V=%d M=%d HQ/H=%d", a->dtype, a->K,
+              a->V, a->M, a->HQ / a->H);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  const size_t need = mfma ? prefill_mfma_scratch_bytes(a) : prefill_simple_scratch_bytes(a);
+  if (a->scratch_bytes < need) {
+    set_error("nha_prefill_fwd: scratch has %zu bytes, %zu needed", a->scratch_bytes, need);
+    return NHA_ERR_SCRATCH;
+  }
+  return mfma ? prefill_mfma_impl(a) : prefill_simple_impl(a);
+}
+
+int nha_decode_step(const NhaDecodeArgs* a) { return decode_step_impl(a); }
+
+int nha_decode_advance(int32_t* count, int32_t B, void* stream) { return decode_advance_impl(count, B, stream); }
+
+int32_t nha_varlen_num_chunks(const int32_t* cu, int32_t N, int32_t BT) {
+  if (!cu || N <= 0 || BT <= 0) {
+    set_error("nha_varlen_num_chunks: bad arguments");
+    return NHA_ERR_INVALID;
+  }
+  if (cu[0] != 0) {
+    set_error("nha_varlen_num_chunks: cu_seqlens[0] must be 0, got %d", cu[0]);
+    return NHA_ERR_INVALID;
+  }
+  int64_t nt = 0;
+  for (int n = 0; n < N; ++n) {
+    const int64_t len = (int64_t)cu[n + 1] - cu[n];
+    if (len <= 0) {
+      set_error("nha_varlen_num_chunks: cu_seqlens must be strictly increasing (sequence %d has length %lld)", n,
+                (long long)len);
+      return NHA_ERR_INVALID;
+    }
+    nt += (len + BT - 1) / BT;
+  }
+  if (nt > INT32_MAX) {
+    set_error("nha_varlen_num_chunks: too many chunks");
+    return NHA_ERR_INVALID;
+  }
+  return (int32_t)nt;
+}
+
+int nha_varlen_indices(const int32_t* cu, int32_t N, int32_t BT, int32_t* chunk_idx, int32_t* chunk_off) {
+  const int32_t nt = nha_varlen_num_chunks(cu, N, BT);
+  if (nt < 0) return nt;
+  if (!chunk_idx || !chunk_off) {
+    set_error("nha_varlen_indices: null output");
+    return NHA_ERR_INVALID;
+  }
+  int32_t row = 0;
+  for (int32_t n = 0; n < N; ++n) {
+    chunk_off[n] = row;
+    const int32_t nc = (int32_t)(((int64_t)cu[n + 1] - cu[n] + BT - 1) / BT);
+    for (int32_t i = 0; i < nc; ++i) {
+      chunk_idx[2 * row] = n;
+      chunk_idx[2 * row + 1] = i;
+      ++row;
+    }
+  }
+  chunk_off[N] = row;
+  return NHA_OK;
+}
+
+const char* nha_last_error(void) { return g_err; }
+
+int nha_abi_version(void) { return NHA_ABI_VERSION; }
+
+}  // extern "C"

@@ -1,0 +1,107 @@
+// Shared device/host helpers for the gfx950 NHA kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/nha_hip.h"
+
+namespace nha {
+
+typedef uint16_t bf16_t;  // raw bf16 bit pattern
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t x) {
+  return __uint_as_float(((uint32_t)x) << 16);
+}
+// round-to-nearest-even, NaN preserved
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  // 8 consecutive elements, p 16-byte aligned
+  static __device__ __forceinline__ void ld8(const float* p, float* o) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+  static __device__ __forceinline__ void st8(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct Elem<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+  static __device__ __forceinline__ void ld8(const bf16_t* p, float* o) {
+    uint4 a = *reinterpret_cast<const uint4*>(p);
+    o[0] = __uint_as_float(a.x << 16); o[1] = __uint_as_float(a.x & 0xffff0000u);
+    o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
+    o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
+    o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
+    uint4 a;
+    a.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+    a.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    a.z = (uint32_t)f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
+    a.w = (uint32_t)f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
+    *reinterpret_cast<uint4*>(p) = a;
+  }
+};
+
+__device__ __forceinline__ float wave_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+
+static inline int next_pow2_i(int x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+// host-side error plumbing (thread-local message)
+void set_error(const char* fmt, ...);
+
+int decode_step_impl(const NhaDecodeArgs* a);
+int decode_advance_impl(int32_t* count, int32_t B, void* stream);
+size_t prefill_simple_scratch_bytes(const NhaPrefillArgs* a);
+int prefill_simple_impl(const NhaPrefillArgs* a);
+bool prefill_mfma_supported(const NhaPrefillArgs* a);
+size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
+int prefill_mfma_impl(const NhaPrefillArgs* a);
+
+}  // namespace nha
+
+#define NHA_CHECK_ARG(cond, ...)            \
+  do {                                      \
+    if (!(cond)) {                          \
+      nha::set_error(__VA_ARGS__);          \
+      return NHA_ERR_INVALID;               \
+    }                                       \
+  } while (0)
+
+#define NHA_CHECK_LAUNCH(what)                                             \
+  do {                                                                     \
+    hipError_t e__ = hipGetLastError();                                    \
+    if (e__ != hipSuccess) {                                               \
+      nha::set_error("%s: %s", what, hipGetErrorString(e__));              \
+      return NHA_ERR_LAUNCH;                                               \
+    }                                                                      \
+  } while (0)

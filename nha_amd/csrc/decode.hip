@@ -1,0 +1,423 @@
+// Single-token NHA decode step for gfx950: one launch, one workgroup per (sequence, kv-head)
+// serving all HQ/H query heads, so the fp32 slot state and the W-row K/V window are each read
+// from HBM exactly once per step.  HBM-bound: every global access below is a 16- or 32-byte
+// per-lane vector access over contiguous rows.
+//
+// Semantics follow nha_fla/ops/nha/fused_recurrent.py:228-428 (decode k/v kernels: state write
+// :305/:416, fused softmax over [M | W] :342-349, rotate-half pairing :309-329) and :47-149
+// (caller-supplied window logits).  fp32 math on bf16/fp32 loads, state fp32.
+#include "common.h"
+
+namespace nha {
+
+namespace {
+
+struct Lds {
+  float *eg, *s, *kp, *vp, *q, *sq, *ok, *inv, *part, *logit;
+};
+
+template <int G>
+__device__ __forceinline__ Lds carve(float* base, int K, int V, int M, int W) {
+  Lds l;
+  float* p = base;
+  l.eg = p; p += M;
+  l.s = p; p += M;
+  l.kp = p; p += K;
+  l.vp = p; p += V;
+  l.q = p; p += G * K;
+  l.sq = p; p += G * K;
+  l.ok = p; p += G * M;
+  l.inv = p; p += 16;
+  const int mv = M > V ? M : V;
+  l.part = p; p += 4 * G * mv;
+  l.logit = p;
+  return l;
+}
+
+static size_t lds_floats(int G, int K, int V, int M, int W) {
+  const int mv = M > V ? M : V;
+  return (size_t)2 * M + K + V + (size_t)2 * G * K + (size_t)G * M + 16 + (size_t)4 * G * mv + (size_t)G * W;
+}
+
+template <typename T, int G>
+__global__ __launch_bounds__(256) void decode_kernel(const NhaDecodeArgs a, const int LK, const int LV,
+                                                     const int LM) {
+  extern __shared__ __align__(16) float lds_raw[];
+  const int K = a.K, V = a.V, M = a.M, W = a.W, H = a.H, HQ = a.HQ;
+  const int NG = HQ / H;
+  const Lds L = carve<G>(lds_raw, K, V, M, W);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = blockIdx.x / H, h = blockIdx.x % H;
+  const int64_t bh = (int64_t)b * H + h;
+
+  // ---- phase 0: popped entry, gates, queries -> LDS ---------------------------------------
+  int slot = -1, nvalid = W;
+  bool has_pop = true;
+  const T *kp, *vp, *gp, *sp = nullptr;
+  if (a.mode == NHA_DECODE_RING) {
+    const int c = a.count[b];
+    slot = c % W;
+    has_pop = c >= W;
+    nvalid = c + 1 < W ? c + 1 : W;
+    const int64_t row = ((int64_t)b * W + slot) * H + h;
+    kp = (const T*)a.ring_kg + row * K;
+    vp = (const T*)a.ring_v + row * V;
+    gp = (const T*)a.ring_g + row * M;
+  } else {
+    kp = (const T*)a.k_pop + bh * K;
+    vp = (const T*)a.v_pop + bh * V;
+    gp = (const T*)a.g_pop + bh * M;
+    if (a.s_pop) sp = (const T*)a.s_pop + bh * M;
+  }
+  for (int i = tid; i < M; i += 256) {
+    float e = 1.f, s = 0.f;
+    if (has_pop) {
+      e = expf(Elem<T>::ld(gp + i));
+      s = sp ? Elem<T>::ld(sp + i) : 1.f - e;
+    }
+    L.eg[i] = e;
+    L.s[i] = s;
+  }
+  for (int i = tid; i < K; i += 256) L.kp[i] = has_pop ? Elem<T>::ld(kp + i) : 0.f;
+  for (int i = tid; i < V; i += 256) L.vp[i] = has_pop ? Elem<T>::ld(vp + i) : 0.f;
+  for (int i = tid; i < G * K; i += 256) {
+    const int gq = i / K, kk = i - gq * K;
+    float qv = 0.f, sv = 0.f;
+    if (gq < NG) {
+      const T* qrow = (const T*)a.q + ((int64_t)b * HQ + h * NG + gq) * K;
+      qv = Elem<T>::ld(qrow + kk);
+      if (a.cos) {
+        const int half = K >> 1;
+        const int pr = kk < half ? kk + half : kk - half;
+        const float sgn = kk < half ? -1.f : 1.f;
+        const int64_t co = (int64_t)b * a.cos_sb + (int64_t)(W - 1) * a.cos_sw + kk;
+        sv = qv * Elem<T>::ld((const T*)a.cos + co) + sgn * Elem<T>::ld(qrow + pr) * Elem<T>::ld((const T*)a.sin + co);
+      } else if (a.sq) {
+        sv = Elem<T>::ld((const T*)a.sq + ((int64_t)b * HQ + h * NG + gq) * K + kk);
+      }
+    }
+    L.q[i] = qv * a.scale;
+    L.sq[i] = sv * a.scale;
+  }
+  __syncthreads();
+
+  // ring mode: the popped entry now lives in LDS; store the new token in its slot.  The window
+  // loops below read the new token from k_new / v_new, never back from the ring.
+  if (a.mode == NHA_DECODE_RING) {
+    const int64_t row = ((int64_t)b * W + slot) * H + h;
+    for (int i = tid; i < K; i += 256) {
+      ((T*)a.ring_k)[row * K + i] = ((const T*)a.k_new)[bh * K + i];
+      ((T*)a.ring_kg)[row * K + i] = ((const T*)a.kg_new)[bh * K + i];
+    }
+    for (int i = tid; i < V; i += 256) ((T*)a.ring_v)[row * V + i] = ((const T*)a.v_new)[bh * V + i];
+    for (int i = tid; i < M; i += 256) ((T*)a.ring_g)[row * M + i] = ((const T*)a.g_new)[bh * M + i];
+  }
+
+  // ---- phase 1: hk <- hk*exp(g) + k s^T ; slot logits ok[g][m] = scale q . hk[:,m] ----------
+  {
+    const int cm = lane % LM, rm = lane / LM, RM = 64 / LM;
+    const int m0 = cm * 8;
+    const bool act = m0 < M;
+    float eg8[8], s8[8], acc[G][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      eg8[e] = act ? L.eg[m0 + e] : 0.f;
+      s8[e] = act ? L.s[m0 + e] : 0.f;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    if (act) {
+      const float* hin = a.hk_in ? a.hk_in + bh * K * M + m0 : nullptr;
+      float* hout = a.hk_out ? a.hk_out + bh * K * M + m0 : nullptr;
+#pragma unroll 4
+      for (int kk = wave * RM + rm; kk < K; kk += 4 * RM) {
+        float hr[8];
+        if (hin) {
+          Elem<float>::ld8(hin + (int64_t)kk * M, hr);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) hr[e] = 0.f;
+        }
+        const float kv = L.kp[kk];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hr[e] = hr[e] * eg8[e] + kv * s8[e];
+        if (hout) Elem<float>::st8(hout + (int64_t)kk * M, hr);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const float qg = L.q[g * K + kk];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[g][e] += qg * hr[e];
+        }
+      }
+    }
+    for (int mask = LM; mask < 64; mask <<= 1)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] += __shfl_xor(acc[g][e], mask, 64);
+    if (rm == 0 && act)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) L.part[(wave * G + g) * M + m0 + e] = acc[g][e];
+  }
+  __syncthreads();
+  for (int i = tid; i < G * M; i += 256)
+    L.ok[i] = L.part[i] + L.part[G * M + i] + L.part[2 * G * M + i] + L.part[3 * G * M + i];
+
+  // ---- phase 2: window logits --------------------------------------------------------------
+  if (a.mode == NHA_DECODE_LOGITS) {
+    for (int i = tid; i < G * W; i += 256) {
+      const int g = i / W, w = i - g * W;
+      if (g < NG) L.logit[i] = Elem<T>::ld((const T*)a.win_logits + ((int64_t)b * HQ + h * NG + g) * W + w);
+    }
+  } else {
+    const int ck = lane % LK, rk = lane / LK, RK = 64 / LK;
+    const int k0 = ck * 8;
+    const bool act = k0 < K;
+    float qr[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qr[g][e] = act ? L.sq[g * K + k0 + e] : 0.f;
+    const T* kbase = (const T*)(a.mode == NHA_DECODE_RING ? a.ring_k : a.win_k) + ((int64_t)b * W * H + h) * K + k0;
+    const T* knew = a.mode == NHA_DECODE_RING ? (const T*)a.k_new + bh * K + k0 : nullptr;
+    const bool rot = a.cos != nullptr;
+    const float sgn = ck < (LK >> 1) ? -1.f : 1.f;
+#pragma unroll 4
+    for (int wb = wave * RK; wb < nvalid; wb += 4 * RK) {
+      const int w = wb + rk;
+      const bool ok = act && w < nvalid;
+      float kv[8];
+      if (ok) {
+        const T* row = (w == slot) ? knew : kbase + (int64_t)w * H * K;
+        Elem<T>::ld8(row, kv);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) kv[e] = 0.f;
+      }
+      if (rot) {
+        float cs[8], sn[8];
+        if (ok) {
+          const int64_t co = (int64_t)b * a.cos_sb + (int64_t)w * a.cos_sw + k0;
+          Elem<T>::ld8((const T*)a.cos + co, cs);
+          Elem<T>::ld8((const T*)a.sin + co, sn);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float pr = __shfl_xor(kv[e], LK >> 1, 64);
+          if (ok) kv[e] = kv[e] * cs[e] + sgn * pr * sn[e];
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d += qr[g][e] * kv[e];
+        for (int mask = 1; mask < LK; mask <<= 1) d += __shfl_xor(d, mask, 64);
+        if (ck == 0 && w < nvalid) L.logit[g * W + w] = d;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 3: ONE softmax over [M slot logits | window logits] per query head ------------
+  for (int g = wave; g < NG; g += 4) {
+    float mx = -INFINITY;
+    for (int i = lane; i < M; i += 64) mx = fmaxf(mx, L.ok[g * M + i]);
+    for (int i = lane; i < nvalid; i += 64) mx = fmaxf(mx, L.logit[g * W + i]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int i = lane; i < M; i += 64) {
+      const float e = expf(L.ok[g * M + i] - mx);
+      L.ok[g * M + i] = e;
+      sum += e;
+    }
+    for (int i = lane; i < nvalid; i += 64) {
+      const float e = expf(L.logit[g * W + i] - mx);
+      L.logit[g * W + i] = e;
+      sum += e;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    if (lane == 0) L.inv[g] = inv;
+    if (a.mode == NHA_DECODE_LOGITS && a.win_probs) {
+      float* pr = a.win_probs + ((int64_t)b * HQ + h * NG + g) * W;
+      for (int i = lane; i < W; i += 64) pr[i] = L.logit[g * W + i] * inv;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 4: hv <- hv*exp(g) + s v^T ; o = p_slots . hv + p_win . V_win -------------------
+  {
+    const int cv = lane % LV, rv = lane / LV, RV = 64 / LV;
+    const int v0 = cv * 8;
+    const bool act = v0 < V;
+    float acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    if (act) {
+      float vp8[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vp8[e] = L.vp[v0 + e];
+      const float* hin = a.hv_in ? a.hv_in + bh * M * V + v0 : nullptr;
+      float* hout = a.hv_out ? a.hv_out + bh * M * V + v0 : nullptr;
+#pragma unroll 4
+      for (int m = wave * RV + rv; m < M; m += 4 * RV) {
+        float hr[8];
+        if (hin) {
+          Elem<float>::ld8(hin + (int64_t)m * V, hr);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) hr[e] = 0.f;
+        }
+        const float eg = L.eg[m], sm = L.s[m];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hr[e] = hr[e] * eg + sm * vp8[e];
+        if (hout) Elem<float>::st8(hout + (int64_t)m * V, hr);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const float p = L.ok[g * M + m];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[g][e] += p * hr[e];
+        }
+      }
+      if (a.mode != NHA_DECODE_LOGITS) {
+        const T* vbase = (const T*)(a.mode == NHA_DECODE_RING ? a.ring_v : a.win_v) + ((int64_t)b * W * H + h) * V + v0;
+        const T* vnew = a.mode == NHA_DECODE_RING ? (const T*)a.v_new + bh * V + v0 : nullptr;
+#pragma unroll 4
+        for (int w = wave * RV + rv; w < nvalid; w += 4 * RV) {
+          float vv[8];
+          const T* row = (w == slot) ? vnew : vbase + (int64_t)w * H * V;
+          Elem<T>::ld8(row, vv);
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            const float p = L.logit[g * W + w];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] += p * vv[e];
+          }
+        }
+      }
+    }
+    for (int mask = LV; mask < 64; mask <<= 1)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] += __shfl_xor(acc[g][e], mask, 64);
+    if (rv == 0 && act)
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) L.part[(wave * G + g) * V + v0 + e] = acc[g][e];
+  }
+  __syncthreads();
+  for (int i = tid; i < G * V; i += 256) {
+    const int g = i / V, vv = i - g * V;
+    if (g < NG) {
+      const float r = (L.part[i] + L.part[G * V + i] + L.part[2 * G * V + i] + L.part[3 * G * V + i]) * L.inv[g];
+      Elem<T>::st((T*)a.o + ((int64_t)b * HQ + h * NG + g) * V + vv, r);
+    }
+  }
+}
+
+__global__ void advance_kernel(int32_t* count, int B) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < B) count[i] += 1;
+}
+
+template <typename T, int G>
+int launch(const NhaDecodeArgs* a, int LK, int LV, int LM, size_t lds_bytes) {
+  static size_t configured = 0;
+  if (lds_bytes > configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)decode_kernel<T, G>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes);
+    if (e != hipSuccess) {
+      set_error("decode: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+      return NHA_ERR_LAUNCH;
+    }
+    configured = lds_bytes;
+  }
+  hipLaunchKernelGGL((decode_kernel<T, G>), dim3(a->B * a->H), dim3(256), lds_bytes, (hipStream_t)a->stream, *a, LK,
+                     LV, LM);
+  NHA_CHECK_LAUNCH("nha_decode_step");
+  return NHA_OK;
+}
+
+template <typename T>
+int dispatch_g(const NhaDecodeArgs* a, int G, int LK, int LV, int LM, size_t lds_bytes) {
+  switch (G) {
+    case 1: return launch<T, 1>(a, LK, LV, LM, lds_bytes);
+    case 2: return launch<T, 2>(a, LK, LV, LM, lds_bytes);
+    case 4: return launch<T, 4>(a, LK, LV, LM, lds_bytes);
+    case 8: return launch<T, 8>(a, LK, LV, LM, lds_bytes);
+    default: return launch<T, 16>(a, LK, LV, LM, lds_bytes);
+  }
+}
+
+}  // namespace
+
+int decode_step_impl(const NhaDecodeArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_decode_step: null args");
+  NHA_CHECK_ARG(a->B > 0 && a->H > 0 && a->HQ > 0 && a->K > 0 && a->V > 0 && a->M > 0 && a->W > 0,
+                "nha_decode_step: non-positive dimension");
+  NHA_CHECK_ARG(a->HQ % a->H == 0, "nha_decode_step: HQ (%d) must be a multiple of H (%d)", a->HQ, a->H);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_decode_step: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->q && a->o, "nha_decode_step: q and o are required");
+  if (a->mode == NHA_DECODE_RING) {
+    NHA_CHECK_ARG(a->ring_k && a->ring_kg && a->ring_v && a->ring_g && a->k_new && a->kg_new && a->v_new && a->g_new &&
+                      a->count && a->sq,
+                  "nha_decode_step: ring mode needs ring_k/kg/v/g, k/kg/v/g_new, count and sq");
+    NHA_CHECK_ARG(!a->cos, "nha_decode_step: ring mode stores rotated keys; cos/sin are not accepted");
+  } else if (a->mode == NHA_DECODE_WINDOW || a->mode == NHA_DECODE_LOGITS) {
+    NHA_CHECK_ARG(a->k_pop && a->v_pop && a->g_pop, "nha_decode_step: k_pop, v_pop, g_pop are required");
+    if (a->mode == NHA_DECODE_WINDOW) {
+      NHA_CHECK_ARG(a->win_k && a->win_v, "nha_decode_step: win_k and win_v are required");
+      NHA_CHECK_ARG((a->sq != nullptr) != (a->cos != nullptr),
+                    "nha_decode_step: pass either sq (pre-rotated) or cos/sin (in-kernel rotary), not both");
+      NHA_CHECK_ARG(!a->cos || a->sin, "nha_decode_step: cos without sin");
+      NHA_CHECK_ARG(!a->cos || a->K % 2 == 0, "nha_decode_step: in-kernel rotate-half requires an even head dim");
+    } else {
+      NHA_CHECK_ARG(a->win_logits, "nha_decode_step: win_logits is required");
+    }
+  } else {
+    NHA_CHECK_ARG(false, "nha_decode_step: unknown mode %d", a->mode);
+  }
+  const int NG = a->HQ / a->H;
+  if (NG > 16 || a->K % 8 || a->V % 8 || a->M % 8 || a->K > 512 || a->V > 512 || a->M > 512) {
+    set_error("nha_decode_step: unsupported shape (need HQ/H <= 16 and K, V, M multiples of 8 up to 512; got NG=%d K=%d V=%d M=%d)",
+              NG, a->K, a->V, a->M);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  const int LK = next_pow2_i(a->K / 8), LV = next_pow2_i(a->V / 8), LM = next_pow2_i(a->M / 8);
+  if (a->cos && LK * 8 != a->K) {
+    set_error("nha_decode_step: in-kernel rotary needs a power-of-two head dim, got K=%d", a->K);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  if (a->cos && (a->cos_sw % 8 || a->cos_sb % 8)) {
+    set_error("nha_decode_step: cos/sin strides must be multiples of 8 elements");
+    return NHA_ERR_UNSUPPORTED;
+  }
+  int G = 1;
+  while (G < NG) G <<= 1;
+  const size_t lds_bytes = lds_floats(G, a->K, a->V, a->M, a->W) * sizeof(float);
+  if (lds_bytes > 160 * 1024) {
+    set_error("nha_decode_step: window of %d rows x %d query heads per kv-head needs %zu bytes of LDS (limit 163840)",
+              a->W, NG, lds_bytes);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  if (a->dtype == NHA_DTYPE_BF16) return dispatch_g<bf16_t>(a, G, LK, LV, LM, lds_bytes);
+  return dispatch_g<float>(a, G, LK, LV, LM, lds_bytes);
+}
+
+int decode_advance_impl(int32_t* count, int32_t B, void* stream) {
+  NHA_CHECK_ARG(count && B > 0, "nha_decode_advance: bad arguments");
+  hipLaunchKernelGGL(advance_kernel, dim3((B + 255) / 256), dim3(256), 0, (hipStream_t)stream, count, B);
+  NHA_CHECK_LAUNCH("nha_decode_advance");
+  return NHA_OK;
+}
+
+}  // namespace nha

@@ -1,0 +1,377 @@
+"""Host-side mirror of the reference op API for the NHA hot path, bound to libnha_hip.so.
+
+Same names, argument meaning, return tuples and error behaviour as
+  nha_fla/ops/nha/chunk.py:568-690            chunk_nha
+  nha_fla/ops/nha/chunk_fused.py:291-380      fused_chunk_nha_prefill
+  nha_fla/ops/nha/fused_recurrent.py:431-584  fused_recurrent_nha_decode
+  nha_fla/ops/nha/fused_recurrent.py:588-682  fused_recurrent_nha
+Differences, all widening: k/v/s/g may carry fewer (kv) heads than q in chunk_nha (the reference
+needs them pre-expanded); window and head-dim limits of the fused prefill are lifted.  Forward
+only: inputs that require grad are rejected (the reference's backward is not part of this path).
+PyTorch is used for device memory and the current stream only; every tensor op on the hot path
+is a HIP kernel behind the C ABI.  There is no CPU / eager fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from .varlen import CHUNK, chunk_tables
+
+__all__ = ["chunk_nha", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
+           "prefill_tables", "nha_prefill"]
+
+_DT = {torch.float32: _lib.NHA_DTYPE_F32, torch.bfloat16: _lib.NHA_DTYPE_BF16}
+_IMPL = {None: _lib.NHA_IMPL_AUTO, "auto": _lib.NHA_IMPL_AUTO, "simple": _lib.NHA_IMPL_SIMPLE,
+         "mfma": _lib.NHA_IMPL_MFMA}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise TypeError(f"NHA HIP kernels take bfloat16 or float32 tensors, got {t.dtype}")
+    return _DT[t.dtype]
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("NHA ops run on the GPU only (tensor on %s); there is no CPU fallback" % t.device)
+
+
+def _no_grad_inputs(name, *ts):
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts):
+        raise NotImplementedError(f"{name}: forward only -- the backward of the reference op is not implemented; "
+                                  "call under torch.no_grad() or detach the inputs")
+
+
+# ---------------------------------------------------------------------------------------------
+# varlen tables, cached per cu_seqlens content
+# ---------------------------------------------------------------------------------------------
+_TABLE_CACHE: dict = {}
+
+
+def prefill_tables(cu_host: np.ndarray, device) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]:
+    """(cu_seqlens, chunk_indices [NT,2], chunk_offsets [N+1]) as int32 device tensors + NT."""
+    key = (cu_host.tobytes(), str(device))
+    hit = _TABLE_CACHE.get(key)
+    if hit is not None:
+        return hit
+    idx, off = chunk_tables(cu_host, CHUNK)
+    out = (torch.from_numpy(cu_host.astype(np.int32)).to(device), torch.from_numpy(idx).to(device),
+           torch.from_numpy(off).to(device), int(idx.shape[0]))
+    if len(_TABLE_CACHE) > 64:
+        _TABLE_CACHE.clear()
+    _TABLE_CACHE[key] = out
+    return out
+
+
+def nha_prefill(q_swa, k_swa, q_gsa, k_gsa, v, s, g, cu_host: np.ndarray, *, wl: int, shift: int, scale: float,
+                h0=None, want_state: bool = False, want_lse: bool = True, impl=None):
+    """Packed prefill on token-major tensors ``[T_tot, heads, dim]`` (one nha_prefill_fwd call).
+    Returns (o, lse_swa, lse_gsa, hkt, hvt)."""
+    lib = _lib.load()
+    T_tot, HQ, K = q_swa.shape
+    H, V, M = k_swa.shape[1], v.shape[-1], s.shape[-1]
+    dev = q_swa.device
+    N = cu_host.size - 1
+    cu_d, idx_d, off_d, NT = prefill_tables(cu_host, dev)
+    o = torch.empty(T_tot, HQ, V, dtype=q_swa.dtype, device=dev)
+    lse_swa = torch.empty(T_tot, HQ, dtype=torch.float32, device=dev) if want_lse else None
+    lse_gsa = torch.empty(T_tot, HQ, dtype=torch.float32, device=dev) if want_lse else None
+    hkt = torch.empty(N, H, K, M, dtype=torch.float32, device=dev) if want_state else None
+    hvt = torch.empty(N, H, M, V, dtype=torch.float32, device=dev) if want_state else None
+    h0k = h0v = None
+    if h0 is not None and h0[0] is not None:
+        h0k = h0[0].to(torch.float32).contiguous()
+        h0v = h0[1].to(torch.float32).contiguous()
+        if tuple(h0k.shape) != (N, H, K, M) or tuple(h0v.shape) != (N, H, M, V):
+            raise ValueError(f"initial_state must be ([{N},{H},{K},{M}], [{N},{H},{M},{V}]) (kv-head count), "
+                             f"got {tuple(h0k.shape)} / {tuple(h0v.shape)}")
+    a = _lib.NhaPrefillArgs()
+    a.q_swa, a.k_swa, a.q_gsa, a.k_gsa = _ptr(q_swa), _ptr(k_swa), _ptr(q_gsa), _ptr(k_gsa)
+    a.v, a.s, a.g, a.o = _ptr(v), _ptr(s), _ptr(g), _ptr(o)
+    a.lse_swa, a.lse_gsa = _ptr(lse_swa), _ptr(lse_gsa)
+    a.h0k, a.h0v, a.hkt, a.hvt = _ptr(h0k), _ptr(h0v), _ptr(hkt), _ptr(hvt)
+    a.cu_seqlens, a.chunk_indices, a.chunk_offsets = _ptr(cu_d), _ptr(idx_d), _ptr(off_d)
+    a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = T_tot, N, NT, HQ, H, K, V, M
+    a.wl, a.shift = int(wl), int(shift)
+    a.dtype = _dtype_code(q_swa)
+    a.impl = _IMPL[impl]
+    a.scale = float(scale)
+    a.stream = _stream(dev)
+    nbytes = lib.nha_prefill_scratch_bytes(C.byref(a))
+    if nbytes == 0:
+        _lib.check(_lib.NHA_ERR_INVALID)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
+    _lib.check(lib.nha_prefill_fwd(C.byref(a)))
+    return o, lse_swa, lse_gsa, hkt, hvt
+
+
+def _flat(x):
+    return x.reshape(x.shape[0] * x.shape[1], *x.shape[2:]).contiguous()
+
+
+@torch.compiler.disable
+def chunk_nha(
+    q_swa: torch.Tensor,
+    k_swa: torch.Tensor,
+    q_gsa: torch.Tensor,
+    k_gsa: torch.Tensor,
+    v: torch.Tensor,
+    s: torch.Tensor,
+    g: torch.Tensor,
+    cu_seqlens: Optional[torch.Tensor] = None,
+    max_seqlen: Optional[int] = None,
+    scale: Optional[float] = None,
+    window_size_left: int = -1,
+    window_size_right: int = -1,
+    head_first: Optional[bool] = False,
+    gsa_kv_shift: int = 0,
+    initial_state: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    output_final_state: bool = False,
+    impl: Optional[str] = None,
+):
+    r"""Chunk-level Native Hybrid Attention forward (nha_fla/ops/nha/chunk.py:568-690).
+
+    q_swa/q_gsa ``[B,T,HQ,D]``; k_swa/k_gsa ``[B,T,H,D]``, v ``[B,T,H,V]``, s/g ``[B,T,H,M]`` with
+    ``HQ % H == 0`` (the reference takes ``H == HQ``).  ``cu_seqlens`` ``[N+1]`` selects varlen
+    packing (then ``B == 1``).  The SWA branch is causal: ``window_size_right`` is accepted and
+    has no effect, as in the reference's ``causal=True`` flash-attn call (chunk.py:423-431).
+    Returns ``(o [B,T,HQ,V], lse_swa [B,T,HQ], lse_gsa [B,T,HQ])`` plus ``(hkt [N,H,K,M],
+    hvt [N,H,M,V])`` fp32 when ``output_final_state`` (chunk.py:688-690).
+    """
+    if head_first:
+        raise DeprecationWarning(
+            "head_first is deprecated and will be removed in a future version. "
+            "Please use head_first=False for now instead.",
+        )
+    assert q_swa.dim() == 4, "Expected [B, T, H, D] for input"
+    _need_cuda(q_swa, k_swa, q_gsa, k_gsa, v, s, g)
+    _no_grad_inputs("chunk_nha", q_swa, k_swa, q_gsa, k_gsa, v, s, g)
+    B, T, HQ, D = q_swa.shape
+    H = k_swa.shape[2]
+    if scale is None:
+        scale = D ** -0.5
+    if HQ % H:
+        raise ValueError(f"query heads ({HQ}) must be a multiple of kv heads ({H})")
+    for name, x, hh in (("q_gsa", q_gsa, HQ), ("k_gsa", k_gsa, H), ("v", v, H), ("s", s, H), ("g", g, H)):
+        if x.shape[0] != B or x.shape[1] != T or x.shape[2] != hh:
+            raise ValueError(f"{name} has shape {tuple(x.shape)}, expected [{B},{T},{hh},*]")
+    if cu_seqlens is not None:
+        if B != 1:
+            raise ValueError("varlen (cu_seqlens) inputs must be packed with batch size 1")
+        cu_host = cu_seqlens.detach().to("cpu", torch.int32).numpy()
+        if int(cu_host[-1]) != T:
+            raise ValueError(f"cu_seqlens[-1] = {int(cu_host[-1])} does not match the packed length {T}")
+    else:
+        cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)          # chunk.py:660
+    dt = q_swa.dtype
+    args = [_flat(x.to(dt)) for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)]
+    o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(
+        *args, cu_host, wl=window_size_left, shift=gsa_kv_shift, scale=scale,
+        h0=initial_state, want_state=output_final_state, impl=impl)
+    o = o.view(B, T, HQ, -1)
+    lse_swa = lse_swa.view(B, T, HQ)
+    lse_gsa = lse_gsa.view(B, T, HQ)
+    if output_final_state:
+        return o, lse_swa, lse_gsa, (hkt, hvt)
+    return o, lse_swa, lse_gsa
+
+
+@torch.no_grad()
+def fused_chunk_nha_prefill(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    rotary_q: torch.Tensor,
+    rotary_k: torch.Tensor,
+    s: torch.Tensor,
+    g: torch.Tensor,
+    window_size: int,
+    initial_state: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    output_final_state: bool = False,
+    scale: Optional[float] = None,
+    impl: Optional[str] = None,
+) -> Tuple[torch.Tensor, Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]]:
+    r"""Fused NHA prefill, inference only (nha_fla/ops/nha/chunk_fused.py:291-380): window covers
+    raw tokens ``[t-W+1, t]``, the slots hold tokens ``<= t-W``.  q/rotary_q ``[B,T,HQ,K]``;
+    k/rotary_k/v/s/g ``[B,T,H,*]``.  Returns ``(o [B,T,HQ,V], (hkt, hvt))`` (Nones unless
+    ``output_final_state``).  The reference's limits ``W <= 64`` and power-of-two dims <= 128
+    (:331-332) do not apply here."""
+    B, T, HQ, K = q.shape
+    H = k.shape[2]
+    W = int(window_size)
+    assert k.shape[1] == T and v.shape[1] == T and s.shape[1] == T and g.shape[1] == T
+    assert rotary_q.shape == q.shape and rotary_k.shape == k.shape
+    assert HQ % H == 0
+    assert W >= 1
+    _need_cuda(q, k, v, rotary_q, rotary_k, s, g)
+    if initial_state is not None and initial_state[0] is not None:
+        hk0, hv0 = initial_state
+        assert tuple(hk0.shape) == (B, H, K, s.shape[-1]) and tuple(hv0.shape) == (B, H, s.shape[-1], v.shape[-1]), \
+            f"initial_state must be at the kv-head count [B, {H}, ...], got {tuple(hk0.shape)} / {tuple(hv0.shape)}"
+    else:
+        initial_state = None
+    if scale is None:
+        scale = K ** -0.5
+    cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)
+    dt = q.dtype
+    args = [_flat(x.to(dt)) for x in (rotary_q, rotary_k, q, k, v, s, g)]
+    o, _, _, hkt, hvt = nha_prefill(*args, cu_host, wl=W - 1, shift=W, scale=scale, h0=initial_state,
+                                    want_state=output_final_state, want_lse=False, impl=impl)
+    return o.view(B, T, HQ, -1), (hkt, hvt)
+
+
+def _decode_state(initial_state, output_final_state, NG, B, H, K, V, M, dev):
+    """State plumbing shared by the two T == 1 ops (fused_recurrent.py:169-179, :533-545)."""
+    if initial_state is not None and initial_state != (None, None) and initial_state[0] is not None:
+        hk0, hv0 = initial_state
+        if hk0.dtype != torch.float32 or hv0.dtype != torch.float32:
+            raise TypeError("the slot state must be float32")
+        hk0, hv0 = hk0.contiguous(), hv0.contiguous()
+        assert tuple(hk0.shape) == (B, H, K, M) and tuple(hv0.shape) == (B, H, M, V), \
+            f"initial_state must be ([{B},{H},{K},{M}], [{B},{H},{M},{V}]), got {tuple(hk0.shape)} / {tuple(hv0.shape)}"
+    else:
+        hk0 = hv0 = None
+    hkt = hvt = None
+    if output_final_state:
+        if NG == 1 and hk0 is not None:
+            hkt, hvt = hk0, hv0                                          # in place, as the reference
+        else:
+            hkt = torch.empty(B, H, K, M, dtype=torch.float32, device=dev)
+            hvt = torch.empty(B, H, M, V, dtype=torch.float32, device=dev)
+    return hk0, hv0, hkt, hvt
+
+
+def fused_recurrent_nha_decode(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    sw_k: torch.Tensor,
+    sw_v: torch.Tensor,
+    sq: Optional[torch.Tensor] = None,
+    s: Optional[torch.Tensor] = None,
+    cos: Optional[torch.Tensor] = None,
+    sin: Optional[torch.Tensor] = None,
+    initial_state: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    output_final_state: bool = False,
+    scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]]:
+    r"""Single-token fused NHA decode step with GQA (nha_fla/ops/nha/fused_recurrent.py:431-584).
+
+    q ``[B,1,HQ,K]`` raw; popped k/v/g ``[B,1,H,*]``; ``sw_k/sw_v [B,W,H,*]`` ascending in time;
+    either ``sq`` (pre-rotated, with pre-rotated ``sw_k``) or ``cos/sin [B|1, W2>=W, K]``
+    (in-kernel rotate-half on raw ``q``/``sw_k``; last W rows used, row W-1 = query position).
+    Returns ``(o [B,1,HQ,V], (hkt, hvt))``; the state is updated in place when ``HQ == H``."""
+    B, T, HQ, K = q.shape
+    H = sw_k.shape[2]
+    V = v.shape[-1]
+    M = g.shape[-1]
+    W = sw_k.shape[1]
+    assert T == 1 and k.shape[1] == 1 and g.shape[1] == 1
+    assert k.shape[2] == H and v.shape[2] == H and g.shape[2] == H, \
+        f"popped-entry head count must match the kv-head count ({H}) of the window tensors"
+    assert sw_v.shape[1] == W and sw_v.shape[2] == H
+    assert HQ % H == 0
+    assert K >= 16 and V >= 16
+    _need_cuda(q, k, v, g, sw_k, sw_v, sq, s, cos, sin)
+    NG = HQ // H
+    if scale is None:
+        scale = K ** -0.5
+    dt = q.dtype
+    rotary = cos is not None
+    c_sb = c_sw = 0
+    if rotary:
+        assert sq is None, "pass either sq (pre-rotated) or cos/sin (in-kernel rotary), not both"
+        assert sin is not None and cos.shape == sin.shape
+        assert cos.shape[0] in (1, B) and cos.shape[1] >= W and cos.shape[2] == K, \
+            f"rotary cos/sin must be [1|{B}, W2>={W}, K={K}], got {tuple(cos.shape)}"
+        assert K % 2 == 0, "in-kernel rotate-half requires an even head dim"
+        cos = cos[:, -W:].to(dt).contiguous()
+        sin = sin[:, -W:].to(dt).contiguous()
+        c_sb = cos.stride(0) if cos.shape[0] == B else 0
+        c_sw = cos.stride(1)
+    else:
+        assert sq is not None and sq.shape == q.shape
+    if s is not None:
+        assert s.shape == g.shape
+    dev = q.device
+    cont = lambda x: None if x is None else x.to(dt).contiguous()
+    q_, sq_, k_, v_, g_, s_, swk_, swv_ = map(cont, (q, sq, k, v, g, s, sw_k, sw_v))
+    hk0, hv0, hkt, hvt = _decode_state(initial_state, output_final_state, NG, B, H, K, V, M, dev)
+    o = torch.empty(B, 1, HQ, V, dtype=dt, device=dev)
+    a = _lib.NhaDecodeArgs()
+    a.mode, a.dtype = _lib.NHA_DECODE_WINDOW, _dtype_code(q_)
+    a.B, a.HQ, a.H, a.K, a.V, a.M, a.W = B, HQ, H, K, V, M, W
+    a.scale = float(scale)
+    a.q, a.sq = _ptr(q_), _ptr(sq_)
+    a.k_pop, a.v_pop, a.g_pop, a.s_pop = _ptr(k_), _ptr(v_), _ptr(g_), _ptr(s_)
+    a.win_k, a.win_v = _ptr(swk_), _ptr(swv_)
+    a.cos, a.sin, a.cos_sb, a.cos_sw = _ptr(cos), _ptr(sin), c_sb, c_sw
+    a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(hk0), _ptr(hv0), _ptr(hkt), _ptr(hvt)
+    a.o, a.stream = _ptr(o), _stream(dev)
+    _lib.check(_lib.load().nha_decode_step(C.byref(a)))
+    return o, (hkt, hvt)
+
+
+@torch.compiler.disable
+def fused_recurrent_nha(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    sliding_window: torch.Tensor,
+    s: torch.Tensor,
+    g: torch.Tensor,
+    scale: Optional[float] = None,
+    initial_state: Optional[Tuple[torch.Tensor]] = None,
+    output_final_state: Optional[bool] = False,
+) -> Tuple[torch.Tensor, torch.Tensor, list]:
+    r"""Single-token NHA inference step with caller-supplied window logits
+    (nha_fla/ops/nha/fused_recurrent.py:588-682).  q ``[B,1,HQ,K]``; k/v/s/g ``[B,1,H,*]``;
+    ``sliding_window [B,1,HQ,W]`` logits.  Returns ``(o [B,1,HQ,V]`` slot part only,
+    ``swa_score [B,1,HQ,W]`` fp32 window probabilities of the mixing softmax, ``[hkt, hvt])``."""
+    T = q.shape[1]
+    if T != 1:
+        raise ValueError(
+            f"fused_recurrent_nha is the single-token inference path and expects T == 1, got T = {T}."
+        )
+    assert not q.requires_grad, "fused_recurrent_nha is inference-only (no autograd)"
+    _need_cuda(q, k, v, sliding_window, s, g)
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    B, _, HQ, K = q.shape
+    H, V, M, W = k.shape[2], v.shape[-1], s.shape[-1], sliding_window.shape[-1]
+    assert HQ % H == 0
+    NG = HQ // H
+    dt = q.dtype
+    dev = q.device
+    cont = lambda x: x.to(dt).contiguous()
+    q_, k_, v_, sw_, s_, g_ = map(cont, (q, k, v, sliding_window, s, g))
+    hk0, hv0, hkt, hvt = _decode_state(initial_state, output_final_state, NG, B, H, K, V, M, dev)
+    o = torch.empty(B, 1, HQ, V, dtype=dt, device=dev)
+    probs = torch.empty(B, 1, HQ, W, dtype=torch.float32, device=dev)
+    a = _lib.NhaDecodeArgs()
+    a.mode, a.dtype = _lib.NHA_DECODE_LOGITS, _dtype_code(q_)
+    a.B, a.HQ, a.H, a.K, a.V, a.M, a.W = B, HQ, H, K, V, M, W
+    a.scale = float(scale)
+    a.q = _ptr(q_)
+    a.k_pop, a.v_pop, a.g_pop, a.s_pop = _ptr(k_), _ptr(v_), _ptr(g_), _ptr(s_)
+    a.win_logits, a.win_probs = _ptr(sw_), _ptr(probs)
+    a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(hk0), _ptr(hv0), _ptr(hkt), _ptr(hvt)
+    a.o, a.stream = _ptr(o), _stream(dev)
+    _lib.check(_lib.load().nha_decode_step(C.byref(a)))
+    return o, probs, [hkt, hvt]

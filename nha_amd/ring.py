@@ -1,0 +1,78 @@
+"""Resident decode state: fp32 slot state + W-slot K/V/gate ring buffers, stepped by ONE kernel.
+
+Replaces the cat-shift window cache and the pop/update choreography around the decode op in the
+reference (nha_fla/models/nha_cache.py:105-131, :143-154; models/qwen3_moe_nha/qwennha.py:151-176,
+:351-365): the kernel pops the oldest ring entry into the slots, stores the new token in its
+slot and attends over the valid entries, reading state and window once per kv-head."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .ops import _dtype_code, _need_cuda, _ptr, _stream
+
+
+@dataclass
+class NHARingState:
+    """Per-layer decode state for B sequences.  ``ring_k`` holds the window keys as the window
+    branch reads them (already rotated), ``ring_kg`` the slot-branch keys (raw), ``ring_g`` the
+    log forget gates of the cached tokens; ``count[b]`` tokens have been cached so far."""
+    hk: torch.Tensor        # [B,H,K,M] fp32
+    hv: torch.Tensor        # [B,H,M,V] fp32
+    ring_k: torch.Tensor    # [B,W,H,K]
+    ring_kg: torch.Tensor   # [B,W,H,K]
+    ring_v: torch.Tensor    # [B,W,H,V]
+    ring_g: torch.Tensor    # [B,W,H,M]
+    count: torch.Tensor     # [B] int32
+
+    @classmethod
+    def empty(cls, B, H, K, V, M, W, dtype=torch.bfloat16, device="cuda") -> "NHARingState":
+        z = lambda *s, dt=dtype: torch.zeros(*s, dtype=dt, device=device)
+        return cls(z(B, H, K, M, dt=torch.float32), z(B, H, M, V, dt=torch.float32), z(B, W, H, K), z(B, W, H, K),
+                   z(B, W, H, V), z(B, W, H, M), z(B, dt=torch.int32))
+
+    @property
+    def window(self) -> int:
+        return self.ring_k.shape[1]
+
+
+def ring_decode_step(state: NHARingState, q: torch.Tensor, sq: torch.Tensor, k_new: torch.Tensor,
+                     kg_new: torch.Tensor, v_new: torch.Tensor, g_new: torch.Tensor,
+                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                     advance: bool = True) -> torch.Tensor:
+    """One decode step for every sequence of ``state`` (updated in place).
+
+    q (slot-branch query) and sq (window query, rotated) ``[B,HQ,K]``; the new token's window key
+    ``k_new`` (rotated), slot key ``kg_new`` ``[B,H,K]``, value ``[B,H,V]`` and log gate
+    ``g_new [B,H,M]``.  Returns ``o [B,HQ,V]``."""
+    _need_cuda(q, sq, k_new, kg_new, v_new, g_new, state.hk)
+    B, HQ, K = q.shape
+    _, W, H, _ = state.ring_k.shape
+    V, M = state.ring_v.shape[-1], state.ring_g.shape[-1]
+    dt = state.ring_k.dtype
+    for name, x, shp in (("q", q, (B, HQ, K)), ("sq", sq, (B, HQ, K)), ("k_new", k_new, (B, H, K)),
+                         ("kg_new", kg_new, (B, H, K)), ("v_new", v_new, (B, H, V)), ("g_new", g_new, (B, H, M))):
+        if tuple(x.shape) != shp or x.dtype != dt or not x.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous {dt} tensor of shape {shp}, got {tuple(x.shape)} {x.dtype}")
+    if scale is None:
+        scale = K ** -0.5
+    o = out if out is not None else torch.empty(B, HQ, V, dtype=dt, device=q.device)
+    a = _lib.NhaDecodeArgs()
+    a.mode, a.dtype = _lib.NHA_DECODE_RING, _dtype_code(q)
+    a.B, a.HQ, a.H, a.K, a.V, a.M, a.W = B, HQ, H, K, V, M, W
+    a.scale = float(scale)
+    a.q, a.sq = _ptr(q), _ptr(sq)
+    a.ring_k, a.ring_kg, a.ring_v, a.ring_g = map(_ptr, (state.ring_k, state.ring_kg, state.ring_v, state.ring_g))
+    a.k_new, a.kg_new, a.v_new, a.g_new = _ptr(k_new), _ptr(kg_new), _ptr(v_new), _ptr(g_new)
+    a.count = _ptr(state.count)
+    a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(state.hk), _ptr(state.hv), _ptr(state.hk), _ptr(state.hv)
+    a.o, a.stream = _ptr(o), _stream(q.device)
+    lib = _lib.load()
+    _lib.check(lib.nha_decode_step(C.byref(a)))
+    if advance:
+        _lib.check(lib.nha_decode_advance(_ptr(state.count), B, a.stream))
+    return o

@@ -1,0 +1,67 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol include/nha_hip.h
+declares, validates arguments, and its host-only varlen tables equal the integer oracle."""
+import ctypes as C
+import os
+import random
+import re
+
+import numpy as np
+import pytest
+
+from nha_amd import _lib
+from nha_amd.varlen import chunk_tables
+from oracle import varlen_index as VI
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_header_symbols():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "nha_hip.h")).read()
+    declared = set(re.findall(r"\b(nha_[a-z_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.nha_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_sizes_match_the_header():
+    # a tiny C program would be the strict check; here: field count and pointer-size sanity
+    assert C.sizeof(_lib.NhaPrefillArgs) == 18 * 8 + 8 + 12 * 4 + 4 + 4 + 8  # ptrs, size_t, ints, scale(+pad), stream
+    assert C.sizeof(_lib.NhaDecodeArgs) % 8 == 0
+
+
+def test_argument_validation_without_gpu():
+    lib = _lib.load()
+    a = _lib.NhaPrefillArgs()
+    assert lib.nha_prefill_fwd(C.byref(a)) == _lib.NHA_ERR_INVALID
+    assert b"non-positive" in lib.nha_last_error()
+    d = _lib.NhaDecodeArgs()
+    assert lib.nha_decode_step(C.byref(d)) == _lib.NHA_ERR_INVALID
+    d.B = d.H = d.K = d.V = d.M = d.W = 8
+    d.HQ = 12
+    assert lib.nha_decode_step(C.byref(d)) == _lib.NHA_ERR_INVALID and b"multiple" in lib.nha_last_error()
+    with pytest.raises(_lib.NhaError):
+        chunk_tables([0, 5, 5])          # zero-length sequence
+    with pytest.raises(_lib.NhaError):
+        chunk_tables([1, 5])             # does not start at 0
+
+
+def test_varlen_tables_bit_exact_vs_oracle():
+    random.seed(0)
+    cases = [[128] * 4, [128, 64, 200, 10], [4096, 2048, 1, 1024, 2],
+             [random.randint(1, 100) for _ in range(256)], [1, 2000, 3, 50, 4, 3000, 2, 7], [1], [64], [65]]
+    rng = np.random.default_rng(0)
+    lens, tot = [], 0
+    while tot < 32768:                       # the varlen benchmark config's draw rule
+        L = int(rng.integers(64, 4097))
+        L = min(L, 32768 - tot)
+        lens.append(L); tot += L
+    cases.append(lens)
+    for lens in cases:
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        for bt in (16, 64):
+            idx, off = chunk_tables(cu, bt)
+            ridx, roff = VI.chunk_tables_closed(cu, bt)
+            assert idx.dtype == np.int32 and off.dtype == np.int32
+            assert np.array_equal(idx, ridx) and np.array_equal(off, roff)

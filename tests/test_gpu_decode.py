@@ -1,0 +1,128 @@
+"""GPU parity of the decode kernels (through the C ABI via nha_amd.ops / nha_amd.ring) against
+the fp64 oracle, on the reference's own case grid (scripts/verify_opt_parity.py:278-285, :322-329)."""
+import itertools
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import nha_ref as R
+from tests.util import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+
+GRID = list(itertools.product((1, 4, 8), (16, 64, 80), (32, 64), (64, 128), (1, 4)))
+
+
+def decode_inputs(seed, B, H, NG, K, V, M, W, dtype):
+    gen = torch.Generator().manual_seed(seed)
+    HQ = H * NG
+    d = dict(q=randn(gen, B, 1, HQ, K, dtype=dtype), k=randn(gen, B, 1, H, K, dtype=dtype),
+             v=randn(gen, B, 1, H, V, dtype=dtype), sliding_window=randn(gen, B, 1, HQ, W, dtype=dtype),
+             hk0=randn(gen, B, H, K, M, dtype=torch.float32, scale=0.5),
+             hv0=randn(gen, B, H, M, V, dtype=torch.float32, scale=0.5))
+    d["g"] = (F.logsigmoid(torch.randn(B, 1, H, M, generator=gen)) / 8.0).to(dtype)
+    d["s"] = (1 - d["g"].float().exp()).to(dtype)
+    d["sw_k_raw"] = randn(gen, B, W, H, K, dtype=dtype)
+    d["vw"] = randn(gen, B, W, H, V, dtype=dtype)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, K, 2, dtype=torch.float32) / K))
+    fr = torch.outer(torch.arange(100, 100 + W, dtype=torch.float32), inv)
+    emb = torch.cat([fr, fr], -1)
+    d["cos"], d["sin"] = emb.cos().to(dtype)[None], emb.sin().to(dtype)[None]
+    d["sq"] = R.rope_rotate_half(d["q"].float(), d["cos"][:, -1:].float(), d["sin"][:, -1:].float()).to(dtype)
+    d["sk"] = R.rope_rotate_half(d["sw_k_raw"].float(), d["cos"].float(), d["sin"].float()).to(dtype)
+    return d
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_grid(dtype):
+    from nha_amd import fused_recurrent_nha, fused_recurrent_nha_decode
+    dev = "cuda"
+    for idx, (NG, M, W, K, B) in enumerate(GRID):
+        H, V = 2, K
+        d = decode_inputs(2000 + idx, B, H, NG, K, V, M, W, dtype)
+        c = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
+        tag = f"ng{NG}_m{M}_w{W}_k{K}_b{B}"
+        print("case", tag, dtype, flush=True)
+        # eager mode: pre-rotated sq / sk, caller-supplied s
+        o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], s=c["s"],
+                                                   sw_k=c["sk"], sw_v=c["vw"],
+                                                   initial_state=(c["hk0"].clone(), c["hv0"].clone()),
+                                                   output_final_state=True)
+        ro, rhk, rhv, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sk"], d["vw"], sq=d["sq"], s=d["s"],
+                                          initial_state=(d["hk0"], d["hv0"]))
+        assert_close(tag + " o", o, ro, dtype)
+        assert_close(tag + " hk", hkt, rhk, torch.float32 if dtype == torch.float32 else dtype)
+        assert_close(tag + " hv", hvt, rhv, torch.float32 if dtype == torch.float32 else dtype)
+        # rotary mode: raw q / keys + cos/sin, s recomputed in-kernel
+        o2, (hk2, hv2) = fused_recurrent_nha_decode(q=c["q"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sw_k_raw"],
+                                                    sw_v=c["vw"], cos=c["cos"], sin=c["sin"],
+                                                    initial_state=(c["hk0"].clone(), c["hv0"].clone()),
+                                                    output_final_state=True)
+        ro2, rhk2, rhv2, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sw_k_raw"], d["vw"], cos=d["cos"],
+                                             sin=d["sin"], initial_state=(d["hk0"], d["hv0"]))
+        assert_close(tag + " rot o", o2, ro2, dtype)
+        assert_close(tag + " rot hk", hk2, rhk2, torch.float32 if dtype == torch.float32 else dtype)
+        # caller-supplied window logits
+        o3, sc, (hk3, hv3) = fused_recurrent_nha(c["q"], c["k"], c["v"], c["sliding_window"], c["s"], c["g"],
+                                                 initial_state=(c["hk0"].clone(), c["hv0"].clone()),
+                                                 output_final_state=True)
+        ro3, rsc, rhk3, rhv3 = R.fused_recurrent_ref(d["q"], d["k"], d["v"], d["sliding_window"], d["s"], d["g"],
+                                                     initial_state=(d["hk0"], d["hv0"]))
+        assert_close(tag + " fr o", o3, ro3, dtype)
+        assert_close(tag + " fr p", sc, rsc, dtype)
+        assert_close(tag + " fr hv", hv3, rhv3, torch.float32 if dtype == torch.float32 else dtype)
+
+
+def test_decode_state_aliasing_and_errors():
+    from nha_amd import fused_recurrent_nha, fused_recurrent_nha_decode
+    d = decode_inputs(7, 2, 2, 1, 64, 64, 16, 32, torch.bfloat16)
+    c = {k: v.cuda() for k, v in d.items()}
+    hk0, hv0 = c["hk0"].clone(), c["hv0"].clone()
+    o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sk"],
+                                               sw_v=c["vw"], initial_state=(hk0, hv0), output_final_state=True)
+    assert hkt.data_ptr() == hk0.data_ptr() and hvt.data_ptr() == hv0.data_ptr()      # in place when NG == 1
+    assert not torch.equal(hk0, c["hk0"])
+    o2, st = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sk"],
+                                        sw_v=c["vw"], initial_state=(c["hk0"], c["hv0"]))
+    assert st == (None, None)
+    with pytest.raises(ValueError):
+        fused_recurrent_nha(c["q"].expand(-1, 2, -1, -1), c["k"], c["v"], c["sliding_window"], c["s"], c["g"])
+    with pytest.raises(AssertionError):
+        fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sk"], sw_v=c["vw"],
+                                   cos=c["cos"], sin=c["sin"])
+
+
+@pytest.mark.parametrize("NG,K,M,W", [(4, 128, 64, 48), (1, 64, 16, 8), (8, 64, 80, 33)])
+def test_ring_decode_steps(NG, K, M, W):
+    """Consecutive ring-buffer steps from random fill levels == the oracle's ring recurrence."""
+    from nha_amd import NHARingState, ring_decode_step
+    dtype, B, H, V = torch.bfloat16, 3, 2, K
+    HQ = H * NG
+    gen = torch.Generator().manual_seed(99)
+    st = NHARingState.empty(B, H, K, V, M, W, dtype=dtype)
+    st.hk.copy_(randn(gen, B, H, K, M, dtype=torch.float32, scale=0.1))
+    st.hv.copy_(randn(gen, B, H, M, V, dtype=torch.float32, scale=0.1))
+    st.ring_k.copy_(randn(gen, B, W, H, K, dtype=dtype))
+    st.ring_kg.copy_(randn(gen, B, W, H, K, dtype=dtype))
+    st.ring_v.copy_(randn(gen, B, W, H, V, dtype=dtype))
+    st.ring_g.copy_((F.logsigmoid(torch.randn(B, W, H, M, generator=gen)) / 8).to(dtype))
+    counts = torch.tensor([0, W - 2, 5 * W + 3], dtype=torch.int32)
+    st.count.copy_(counts)
+    ref = dict(hk=st.hk.cpu().double(), hv=st.hv.cpu().double(),
+               rings=tuple(x.cpu().double() for x in (st.ring_k, st.ring_kg, st.ring_v, st.ring_g)),
+               count=counts.clone())
+    for step in range(6):
+        q, sq = randn(gen, B, HQ, K, dtype=dtype), randn(gen, B, HQ, K, dtype=dtype)
+        kn, kgn, vn = randn(gen, B, H, K, dtype=dtype), randn(gen, B, H, K, dtype=dtype), randn(gen, B, H, V, dtype=dtype)
+        gn = (F.logsigmoid(torch.randn(B, H, M, generator=gen)) / 8).to(dtype)
+        o = ring_decode_step(st, q.cuda(), sq.cuda(), kn.cuda(), kgn.cuda(), vn.cuda(), gn.cuda())
+        ro, ref["hk"], ref["hv"], ref["rings"] = R.decode_ring_ref(q, sq, kn, kgn, vn, gn, *ref["rings"], ref["count"],
+                                                                   ref["hk"], ref["hv"])
+        ref["count"] += 1
+        assert_close(f"ring step {step} o", o, ro, dtype)
+    assert torch.equal(st.count.cpu(), ref["count"])
+    assert_close("ring hk", st.hk, ref["hk"], dtype)
+    assert_close("ring hv", st.hv, ref["hv"], dtype)
+    assert torch.equal(st.ring_k.cpu().double(), ref["rings"][0])
+    assert torch.equal(st.ring_g.cpu().double(), ref["rings"][3])
