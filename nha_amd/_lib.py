@@ -32,7 +32,7 @@ class NhaPrefillArgs(C.Structure):
         ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t),
         ("T_tot", C.c_int32), ("N", C.c_int32), ("NT", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32),
         ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
-        ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32), ("impl", C.c_int32),
+        ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32), ("impl", C.c_int32), ("phases", C.c_int32),
         ("scale", C.c_float), ("stream", C.c_void_p),
     ]
 

@@ -23,6 +23,7 @@ static int check_prefill(const NhaPrefillArgs* a, bool pointers) {
   NHA_CHECK_ARG(a->shift >= 0, "nha_prefill: gsa_kv_shift must be >= 0, got %d", a->shift);
   NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_prefill: bad dtype %d", a->dtype);
   NHA_CHECK_ARG(a->impl >= NHA_IMPL_AUTO && a->impl <= NHA_IMPL_MFMA, "nha_prefill: bad impl %d", a->impl);
+  NHA_CHECK_ARG(a->phases >= 0 && a->phases <= 3, "nha_prefill: bad phases %d", a->phases);
   if (pointers) {
     NHA_CHECK_ARG(a->q_swa && a->k_swa && a->q_gsa && a->k_gsa && a->v && a->s && a->g && a->o,
                   "nha_prefill_fwd: q_swa, k_swa, q_gsa, k_gsa, v, s, g, o are required");

@@ -334,10 +334,14 @@ static int run_simple(const NhaPrefillArgs* a) {
     set_error("nha_prefill_fwd(simple): head dims too large for the generic kernels (K=%d V=%d M=%d)", a->K, a->V, a->M);
     return NHA_ERR_UNSUPPORTED;
   }
-  hipLaunchKernelGGL((simple_state_kernel<T>), dim3(a->N * a->H, (a->M + BMS - 1) / BMS), dim3(256), lds1, st, p);
-  NHA_CHECK_LAUNCH("nha_prefill_fwd(simple state pass)");
-  hipLaunchKernelGGL((simple_out_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds2, st, p);
-  NHA_CHECK_LAUNCH("nha_prefill_fwd(simple output pass)");
+  if (a->phases != 2) {
+    hipLaunchKernelGGL((simple_state_kernel<T>), dim3(a->N * a->H, (a->M + BMS - 1) / BMS), dim3(256), lds1, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_fwd(simple state pass)");
+  }
+  if (a->phases != 1) {
+    hipLaunchKernelGGL((simple_out_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds2, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_fwd(simple output pass)");
+  }
   return NHA_OK;
 }
 

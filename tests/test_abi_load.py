@@ -27,7 +27,7 @@ def test_library_loads_and_exports_header_symbols():
 
 def test_struct_sizes_match_the_header():
     # a tiny C program would be the strict check; here: field count and pointer-size sanity
-    assert C.sizeof(_lib.NhaPrefillArgs) == 18 * 8 + 8 + 12 * 4 + 4 + 4 + 8  # ptrs, size_t, ints, scale(+pad), stream
+    assert C.sizeof(_lib.NhaPrefillArgs) == 18 * 8 + 8 + 13 * 4 + 4 + 8  # ptrs, size_t, ints, scale, stream
     assert C.sizeof(_lib.NhaDecodeArgs) % 8 == 0
 
 

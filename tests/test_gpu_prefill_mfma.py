@@ -1,0 +1,69 @@
+"""GPU parity of the bf16 MFMA prefill kernels against the fp64 oracle (small/medium shapes) and
+against the independent fp32-math HIP kernels (larger shapes), through the C ABI."""
+import itertools
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import nha_ref as R
+from tests.test_gpu_prefill import KEYS, run_case
+from tests.util import assert_close, prefill_inputs
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def test_mfma_reference_grid():
+    """The reference's prefill grid shapes that the MFMA kernels serve (M = 64)."""
+    seed = 3100
+    for T, B, W in itertools.product((63, 128, 257, 1000), (1, 4), (32, 64)):
+        d = prefill_inputs(seed, B, T, 8, 2, 64, 64, 64, dtype=BF, with_state=(T == 128))
+        seed += 1
+        run_case(f"mfma_t{T}_b{B}_w{W} shifted", d, wl=W - 1, shift=W, dtype=BF, impl="mfma")
+        if B == 1:
+            run_case(f"mfma_t{T}_b{B}_w{W} layer", d, wl=W, shift=0, dtype=BF, impl="mfma")
+
+
+@pytest.mark.parametrize("D,NG", [(128, 4), (128, 1), (128, 2), (128, 8), (64, 1), (64, 3)])
+def test_mfma_head_shapes_and_windows(D, NG):
+    H = 2
+    for li, (T, wl, shift) in enumerate([(200, 99, 100), (333, 100, 0), (130, -1, 0), (260, 255, 256), (70, 500, 0),
+                                         (192, 63, 0), (192, 64, 64), (150, 0, 1)]):
+        d = prefill_inputs(500 + 10 * D + NG + li, 2, T, H * NG, H, D, D, 64, dtype=BF, with_state=(li % 2 == 0))
+        run_case(f"mfma D{D} NG{NG} T{T} wl{wl} sh{shift}", d, wl=wl, shift=shift, dtype=BF, impl="mfma")
+
+
+def test_mfma_varlen():
+    random.seed(1)
+    for li, lens in enumerate([[128, 64, 200, 10], [300, 1, 129, 2, 64], [random.randint(1, 100) for _ in range(40)],
+                               [1, 200, 3, 50, 4, 130, 2, 7]]):
+        cu = [0] + list(np.cumsum(lens))
+        T, H, NG, D = cu[-1], 2, 4, 128
+        d = prefill_inputs(700 + li, 1, T, H * NG, H, D, D, 64, dtype=BF, with_state=True, N=len(lens))
+        run_case(f"mfma varlen{li} shifted", d, wl=31, shift=32, dtype=BF, impl="mfma", cu=cu)
+        run_case(f"mfma varlen{li} layer", d, wl=100, shift=0, dtype=BF, impl="mfma", cu=cu)
+
+
+def test_mfma_slow_forgetting_gates():
+    """Gate logits ~ N(-1,1) -> logsigmoid with no /8 normaliser (the long-context config's
+    distribution): sum of g over a 16-row sub-block is about -22."""
+    d = prefill_inputs(800, 2, 400, 8, 2, 128, 128, 64, dtype=BF, gate_div=1.0, gate_mean=-1.0, qk_scale=128 ** -0.5)
+    run_case("slow-forgetting", d, wl=127, shift=128, dtype=BF, impl="mfma")
+    run_case("slow-forgetting layer", d, wl=128, shift=0, dtype=BF, impl="mfma")
+
+
+def test_mfma_matches_simple_kernels_at_size():
+    """A shape the CPU recurrence cannot reach in seconds: MFMA kernels vs the fp32-math kernels."""
+    from nha_amd import chunk_nha
+    B, T, HQ, H, D, W = 2, 4096, 8, 2, 128, 1024
+    d = prefill_inputs(900, B, T, HQ, H, D, D, 64, dtype=BF, qk_scale=D ** -0.5, gate_div=1.0, gate_mean=-1.0)
+    c = [d[k].cuda() for k in KEYS]
+    a = chunk_nha(*c, window_size_left=W - 1, gsa_kv_shift=W, output_final_state=True, impl="mfma")
+    b = chunk_nha(*c, window_size_left=W - 1, gsa_kv_shift=W, output_final_state=True, impl="simple")
+    assert_close("o", a[0], b[0].double(), BF)
+    assert_close("lse_swa", a[1], b[1].double(), BF)
+    assert_close("lse_gsa", a[2], b[2].double(), BF)
+    assert_close("hk", a[3][0], b[3][0].double(), BF)
+    assert_close("hv", a[3][1], b[3][1].double(), BF)
