@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the NHA hot path on ONE MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  `value` is prefill tokens/s of one NHA attention layer at the
+long-context head shape (32 q heads, 8 kv heads, D=128, M=64 slots, W=2048, B=2) at T=8192,
+bf16, whole op (state pass + output pass), inputs resident in HBM.  The same line carries the
+decode leg (B=128 sequences, 32/8 heads, D=128, M=64, W=1024 ring buffer, 256 consecutive
+steps, us/step), each with its roofline object, and the CPU baseline (the oracle's naive
+per-token PyTorch recurrence timed on the host cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+
+PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
+DECODE = dict(B=128, HQ=32, H=8, D=128, M=64, W=1024, steps=256)
+
+
+def w_eff(T, W):
+    return sum(min(t + 1, W) for t in range(T)) / T
+
+
+def prefill_flops(B, T, HQ, H, D, M, W):
+    """Algorithmic (recurrent-form) flops: slot logits + slot read per q-head, window QK^T + PV
+    per q-head over the in-window keys, slot write per kv-head."""
+    return B * T * HQ * (2 * (D * M + M * D) + 2 * w_eff(T, W) * (D + D)) + B * T * H * 2 * (D * M + M * D)
+
+
+def decode_bytes(B, HQ, H, D, M, W):
+    """Algorithmic HBM bytes of one decode step: fp32 state read+write, bf16 K/V window read,
+    q/o/new-token/popped-entry traffic."""
+    state = 2 * 4 * B * H * (D * M + M * D)
+    window = 2 * B * W * H * (D + D)
+    small = 2 * B * (2 * HQ * D + HQ * D) + 2 * 2 * B * H * (3 * D + M)
+    return state + window + small
+
+
+def make_prefill_inputs(torch, cfg, device, seed=0, B=None, T=None):
+    B = cfg["B"] if B is None else B
+    T = cfg["T"] if T is None else T
+    HQ, H, D, M = cfg["HQ"], cfg["H"], cfg["D"], cfg["M"]
+    gen = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    q = (r(B, T, HQ, D) * D ** -0.5).to(torch.bfloat16)
+    k = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
+    v = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
+    g = torch.nn.functional.logsigmoid(r(B, T, H, M) - 1.0).to(torch.bfloat16)   # slow-forgetting gates
+    s = (1 - g.float().exp()).to(torch.bfloat16)
+    # the window branch and the slot branch see different (rotated / raw) q and k in the hybrid
+    # models; a second draw keeps the two operand streams distinct as they are in production
+    q2 = (r(B, T, HQ, D) * D ** -0.5).to(torch.bfloat16)
+    k2 = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
+    return [x.to(device) for x in (q2, k2, q, k, v, s, g)]
+
+
+def bench_prefill(torch, steps, warmup):
+    import numpy as np
+    from nha_amd import _lib
+    from nha_amd.ops import prefill_tables, _ptr
+    cfg = PREFILL
+    dev = torch.device("cuda:0")
+    B, T, HQ, H, D, M, W = (cfg[k] for k in ("B", "T", "HQ", "H", "D", "M", "W"))
+    xs = [x.reshape(B * T, *x.shape[2:]).contiguous() for x in make_prefill_inputs(torch, cfg, dev)]
+    cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)
+    cu_d, idx_d, off_d, NT = prefill_tables(cu_host, dev)
+    lib = _lib.load()
+    o = torch.empty(B * T, HQ, D, dtype=torch.bfloat16, device=dev)
+    lse_s = torch.empty(B * T, HQ, dtype=torch.float32, device=dev)
+    lse_g = torch.empty(B * T, HQ, dtype=torch.float32, device=dev)
+    hkt = torch.empty(B, H, D, M, dtype=torch.float32, device=dev)
+    hvt = torch.empty(B, H, M, D, dtype=torch.float32, device=dev)
+    a = _lib.NhaPrefillArgs()
+    a.q_swa, a.k_swa, a.q_gsa, a.k_gsa, a.v, a.s, a.g = (_ptr(x) for x in xs)
+    a.o, a.lse_swa, a.lse_gsa, a.hkt, a.hvt = _ptr(o), _ptr(lse_s), _ptr(lse_g), _ptr(hkt), _ptr(hvt)
+    a.cu_seqlens, a.chunk_indices, a.chunk_offsets = _ptr(cu_d), _ptr(idx_d), _ptr(off_d)
+    a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = B * T, B, NT, HQ, H, D, D, M
+    a.wl, a.shift, a.dtype, a.impl, a.scale = W - 1, W, _lib.NHA_DTYPE_BF16, _lib.NHA_IMPL_MFMA, D ** -0.5
+    stream = torch.cuda.current_stream(dev)
+    a.stream = stream.cuda_stream
+    nbytes = lib.nha_prefill_scratch_bytes(C.byref(a))
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
+
+    def run(phases):
+        a.phases = phases
+        _lib.check(lib.nha_prefill_fwd(C.byref(a)))
+
+    for _ in range(warmup):
+        run(0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run(0)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    # per-kernel durations with events on the launch stream: state pass alone, output pass alone
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_state = t_out = 0.0
+    for _ in range(steps):
+        ev[0].record(stream)
+        run(1)
+        ev[1].record(stream)
+        run(2)
+        ev[2].record(stream)
+        torch.cuda.synchronize()
+        t_state += ev[0].elapsed_time(ev[1]) * 1e-3
+        t_out += ev[1].elapsed_time(ev[2]) * 1e-3
+    t_state /= steps
+    t_out /= steps
+    flops = prefill_flops(B, T, HQ, H, D, M, W)
+    # the output pass carries everything but the slot write (the state pass's flops)
+    flops_out = flops - B * T * H * 2 * (D * M + M * D)
+    return dict(tokens_per_s=B * T / wall, ms_per_step=wall * 1e3, t_state_ms=t_state * 1e3, t_out_ms=t_out * 1e3,
+                flops=flops, achieved_tflops=flops_out / t_out / 1e12, whole_op_tflops=flops / wall / 1e12)
+
+
+def bench_decode(torch, warmup):
+    from nha_amd import NHARingState, ring_decode_step
+    cfg = DECODE
+    dev = torch.device("cuda:0")
+    B, HQ, H, D, M, W, steps = (cfg[k] for k in ("B", "HQ", "H", "D", "M", "W", "steps"))
+    gen = torch.Generator().manual_seed(0)
+    r = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    st = NHARingState.empty(B, H, D, D, M, W, dtype=torch.bfloat16, device=dev)
+    st.hk.copy_(r(B, H, D, M) * 0.1)
+    st.hv.copy_(r(B, H, M, D) * 0.1)
+    st.ring_k.copy_(r(B, W, H, D))
+    st.ring_kg.copy_(r(B, W, H, D))
+    st.ring_v.copy_(r(B, W, H, D))
+    st.ring_g.copy_(torch.nn.functional.logsigmoid(r(B, W, H, M)))
+    # full windows at random ring positions
+    st.count.copy_(torch.randint(W, 3 * W, (B,), generator=gen, dtype=torch.int32))
+    pool = 8
+    q = [(r(B, HQ, D) * D ** -0.5).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    sq = [(r(B, HQ, D) * D ** -0.5).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    kn = [r(B, H, D).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    kgn = [r(B, H, D).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    vn = [r(B, H, D).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    gn = [torch.nn.functional.logsigmoid(r(B, H, M)).to(torch.bfloat16).to(dev) for _ in range(pool)]
+    o = torch.empty(B, HQ, D, dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def loop(n, advance):
+        for i in range(n):
+            j = i % pool
+            ring_decode_step(st, q[j], sq[j], kn[j], kgn[j], vn[j], gn[j], out=o, advance=advance)
+
+    loop(warmup, True)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    loop(steps, True)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    us_step = e0.elapsed_time(e1) * 1e3 / steps
+    # decode kernel alone (no count-advance launch in between)
+    e0.record(stream)
+    loop(steps, False)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    us_kernel = e0.elapsed_time(e1) * 1e3 / steps
+    nbytes = decode_bytes(B, HQ, H, D, M, W)
+    return dict(us_per_step=us_step, us_kernel=us_kernel, bytes=nbytes, achieved_gbs=nbytes / (us_kernel * 1e-6) / 1e9)
+
+
+def cpu_baseline(torch):
+    """Oracle (naive per-token PyTorch recurrence, fp32) on the host cores, bounded sample."""
+    from oracle import nha_ref as R
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    cfg = PREFILL
+    W = cfg["W"]
+
+    def timed(T):
+        xs = make_prefill_inputs(torch, cfg, "cpu", B=1, T=T)
+        t0 = time.perf_counter()
+        R.prefill_ref(*xs, window_size_left=W - 1, gsa_kv_shift=W, dtype=torch.float32)
+        return time.perf_counter() - t0
+
+    t_probe = timed(256)
+    # cost per token grows with the window fill; aim at ~15 s of CPU work, at most the full T
+    T = 256
+    est = t_probe
+    while T < cfg["T"] and est * 4.5 < 15.0:
+        T *= 2
+        est *= 4.5 if T <= W else 2.2
+    t = timed(T)
+    pre = dict(value=T / t, unit="tokens/s", cores=cores, kind="port",
+               sample=f"B=1 slice, first {T} tokens of the T={cfg['T']} workload, fp32, {t:.1f} s")
+    d = DECODE
+    B, HQ, H, D, M, Wd = (d[k] for k in ("B", "HQ", "H", "D", "M", "W"))
+    gen = torch.Generator().manual_seed(1)
+    r = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    args = dict(q=r(B, 1, HQ, D), k=r(B, 1, H, D), v=r(B, 1, H, D), g=torch.nn.functional.logsigmoid(r(B, 1, H, M)),
+                sw_k=r(B, Wd, H, D), sw_v=r(B, Wd, H, D))
+    h0 = (r(B, H, D, M) * 0.1, r(B, H, M, D) * 0.1)
+    R.decode_ref(**args, sq=args["q"], initial_state=h0, dtype=torch.float32)
+    t0 = time.perf_counter()
+    nrep = 3
+    for _ in range(nrep):
+        R.decode_ref(**args, sq=args["q"], initial_state=h0, dtype=torch.float32)
+    pre["decode_us_per_step"] = (time.perf_counter() - t0) / nrep * 1e6
+    pre["decode_sample"] = f"{nrep} steps of the B={B} decode workload, fp32"
+    return pre
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="development aid: time one leg only and print its raw numbers")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path shards by sequence / kv-head with no communication and "
+              "no multi-GPU figure is produced (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the NHA ops have no CPU fallback)", file=sys.stderr)
+        sys.exit(3)
+    if args.only:
+        res = bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else bench_decode(torch, args.warmup)
+        print(json.dumps(res))
+        return
+    pf = bench_prefill(torch, args.steps, args.warmup)
+    dc = bench_decode(torch, args.warmup)
+    cpu = None if args.no_cpu_baseline else cpu_baseline(torch)
+    out = {
+        "metric": "NHA prefill tokens/s @T=8K bf16",
+        "value": pf["tokens_per_s"],
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": pf["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "one NHA layer prefill, B=2 T=8192 HQ=32 H=8 D=128 M=64 W=2048 "
+                               "(window W keys, slots hold tokens <= t-W), gate logits N(-1,1)->logsigmoid",
+                   "decode_workload": "B=128 HQ=32 H=8 D=128 M=64 W=1024 ring buffer, full windows at random "
+                                      "ring positions, 256 consecutive steps"},
+        "roofline": {"bound": "mfma", "kernel": "mfma_out_kernel<128,4>", "achieved": pf["achieved_tflops"],
+                     "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": pf["achieved_tflops"] / PEAK_MFMA_BF16_TFLOPS,
+                     "traffic": None, "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
+                     "whole_op_tflops": pf["whole_op_tflops"], "algorithmic_flop": pf["flops"]},
+        "decode": {"metric": "decode step us @B=128", "value": dc["us_per_step"], "unit": "us/step",
+                   "higher_is_better": False,
+                   "roofline": {"bound": "hbm", "kernel": "decode_kernel<bf16,4>", "achieved": dc["achieved_gbs"],
+                                "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
+                                "traffic": None, "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

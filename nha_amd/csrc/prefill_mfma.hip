@@ -40,9 +40,13 @@ struct MP {
   const float *h0k, *h0v;
   float *hkt, *hvt;
   const int32_t *cu, *cidx, *coff;
-  bf16_t* hkT;   // [NT][H][MS][D]   chunk-start k-state, transposed
-  bf16_t* hvc;   // [NT][H][MS][D]   chunk-start v-state
+  bf16_t* hkT;   // [NT][H][MS][D]   segment-local chunk-start k-state, transposed ([m][d])
+  bf16_t* hvc;   // [NT][H][MS][D]   segment-local chunk-start v-state ([m][d])
   float* gc;     // [NT][H][BT][MS]  chunk-local inclusive gate cumsum
+  float* dcum;   // [NT][H][MS]      decay from the segment start to the chunk start
+  float *hend_k, *hend_v;   // [NSLOT][H][MS][D]  segment-local end states
+  float *hseg_k, *hseg_v;   // [NSLOT][H][MS][D]  true segment-start states
+  float* dtot;   // [NSLOT][H][MS]   total decay of a segment
   int T_tot, N, NT, HQ, H, NG, wl, shift;
   float scale;
 };
@@ -110,40 +114,51 @@ __device__ __forceinline__ void tile_r2l(bf16_t* lds, const TileRegs<D>& t, int 
 }
 
 // ==========================================================================================
-// state pass
+// state pass, two levels
 // ==========================================================================================
+// The slot recurrence is sequential over the chunks of a sequence, so it is cut into segments of
+// SEG chunks.  Level 1 (mfma_state_local_kernel, one workgroup per (segment, kv-head), one wave
+// per 16-slot block) runs the recurrence of chunk_fused.py:30-113 from a ZERO state over its
+// segment and stores, per chunk, the local chunk-start states, the gate cumsum table and the
+// decay accumulated since the segment start; per segment, the local end state and total decay.
+// Level 2 (state_scan_kernel) carries the true state across segments element-wise:
+//   h_seg[s+1] = h_seg[s] * dtot[s] + hend[s].
+// The true chunk-start state, h_loc + h_seg * dcum, is formed by the output pass while it stages
+// the state tiles into LDS.  Both states are kept as C[d][m] accumulators (slot m = lane % 16).
+constexpr int SEG = 4;
+
+__device__ __forceinline__ int seg_slot(const int32_t* coff, int n, int it) { return coff[n] / SEG + it / SEG + n; }
+
 template <int D>
-__global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
+__global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   constexpr int LDT = D + 16;
-  constexpr int BPW = D / 64;   // 16-wide blocks of the head dim per wave
-  __shared__ __align__(16) bf16_t Kt[2][BT * LDT];
-  __shared__ __align__(16) bf16_t Vt[2][BT * LDT];
+  constexpr int NB = D / 16;
+  __shared__ __align__(16) bf16_t Kt[BT * LDT];
+  __shared__ __align__(16) bf16_t Vt[BT * LDT];
+  __shared__ __align__(16) bf16_t St[BT * SLD];
+  __shared__ __align__(16) bf16_t Gt[BT * SLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
-  const int n = blockIdx.x / H, h = blockIdx.x % H;
-  const int mb = blockIdx.y * 16;
+  const int chunk0 = blockIdx.x, h = blockIdx.y;
+  const int n = p.cidx[2 * chunk0], it0 = p.cidx[2 * chunk0 + 1];
+  if (it0 % SEG != 0) return;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int L = eos - bos;
   const int nchunks = (L + BT - 1) / BT;
-  const int c0g = p.coff[n];
-  const int m = mb + l16;   // this lane's slot in the B/A fragments and in hk's accumulator columns
+  const int nloc = (nchunks - it0) < SEG ? (nchunks - it0) : SEG;
+  const int m = wave * 16 + l16;   // this lane's slot
 
-  // accumulators: hk[kk block][.] : C[kk = 4*kb + r][m = l16];  hv[.][vv block] : C[m = 4*kb + r][vv = l16]
-  f32x4 hk[BPW], hv[BPW];
+  f32x4 hk[NB], hv[NB];
 #pragma unroll
-  for (int b = 0; b < BPW; ++b) {
-    const int d0 = (wave * BPW + b) * 16;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      hk[b][r] = p.h0k ? p.h0k[(((int64_t)n * H + h) * D + d0 + 4 * kb + r) * MS + m] : 0.f;
-      hv[b][r] = p.h0v ? p.h0v[(((int64_t)n * H + h) * MS + mb + 4 * kb + r) * D + d0 + l16] : 0.f;
-    }
+  for (int b = 0; b < NB; ++b) {
+    hk[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    hv[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
+  float gsum = 0.f;   // sum of the chunk-end gate cumsums since the segment start, this lane's slot
 
   TileRegs<D> rk, rv;
-  // this lane's g / s values: element e = 4*q + r is row t = 16*q + 4*kb + r of the chunk
-  float gq[16], sq[16];
+  uint4 rs[2], rg[2];
   auto issue = [&](int it) {
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     const int64_t grow0 = (int64_t)bos + it * BT - p.shift;
@@ -152,26 +167,37 @@ __global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
     tile_g2r<D>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
     tile_g2r<D>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int t = 16 * (e >> 2) + 4 * kb + (e & 3);
-      float gv = 0.f, sv = 0.f;
-      if (t >= vlo && t < rows) {
-        const int64_t off = ((grow0 + t) * H + h) * MS + m;
-        gv = bf16_to_f32(p.g[off]);
-        sv = bf16_to_f32(p.s[off]);
+    for (int u = 0; u < 2; ++u) {
+      const int c8 = tid + 256 * u;
+      const int j = c8 >> 3, m8 = (c8 & 7) * 8;
+      uint4 xs = make_uint4(0, 0, 0, 0), xg = xs;
+      if (j >= vlo && j < rows) {
+        xs = *reinterpret_cast<const uint4*>(p.s + ((grow0 + j) * H + h) * MS + m8);
+        xg = *reinterpret_cast<const uint4*>(p.g + ((grow0 + j) * H + h) * MS + m8);
       }
-      gq[e] = gv;
-      sq[e] = sv;
+      rs[u] = xs;
+      rg[u] = xg;
     }
   };
 
-  if (nchunks > 0) issue(0);
-  for (int it = 0; it < nchunks; ++it) {
-    const int cur = it & 1;
+  issue(it0);
+  for (int jc = 0; jc < nloc; ++jc) {
+    const int it = it0 + jc;
+    const int chunk = chunk0 + jc;
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
-    tile_r2l<D>(Kt[cur], rk, tid);
-    tile_r2l<D>(Vt[cur], rv, tid);
-    // inclusive cumsum over t for this lane's slot: four runs of 4 rows per lane, 16 runs per slot
+    if (jc > 0) __syncthreads();   // everyone is done reading the previous chunk's tiles
+    tile_r2l<D>(Kt, rk, tid);
+    tile_r2l<D>(Vt, rv, tid);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c8 = tid + 256 * u;
+      const int j = c8 >> 3, m8 = (c8 & 7) * 8;
+      *reinterpret_cast<uint4*>(St + j * SLD + m8) = rs[u];
+      *reinterpret_cast<uint4*>(Gt + j * SLD + m8) = rg[u];
+    }
+    if (jc + 1 < nloc) issue(it + 1);
+    __syncthreads();
+    // this lane's rows: element e = 4*q + r is row t = 16*q + 4*kb + r
     float gcv[16], sg[16];
     {
       float run[4], base = 0.f;
@@ -180,7 +206,7 @@ __global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
         float a = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          a += gq[4 * q + r];
+          a += bf16_to_f32(Gt[(16 * q + 4 * kb + r) * SLD + m]);
           gcv[4 * q + r] = a;
         }
         run[q] = a;
@@ -198,7 +224,6 @@ __global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
         for (int r = 0; r < 4; ++r) gcv[4 * q + r] += off;
       }
     }
-    // gc of the chunk's last valid row, for this lane's slot
     float glast;
     {
       const int tl = rows - 1;
@@ -209,18 +234,17 @@ __global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
         if (x == e) cand = gcv[x];
       glast = __shfl(cand, l16 + 16 * src_kb, 64);
     }
-    if (wave == 0) {
-      float* gout = p.gc + (((int64_t)(c0g + it) * H + h) * BT) * MS + m;
+    const int64_t cg = (int64_t)chunk * H + h;
+    {
+      float* gout = p.gc + cg * BT * MS + m;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int t = 16 * (e >> 2) + 4 * kb + (e & 3);
-        gout[(int64_t)t * MS] = gcv[e];
-      }
+      for (int e = 0; e < 16; ++e) gout[(16 * (e >> 2) + 4 * kb + (e & 3)) * MS] = gcv[e];
+      if (kb == 0) p.dcum[cg * MS + m] = fexp(gsum);
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int t = 16 * (e >> 2) + 4 * kb + (e & 3);
-      sg[e] = (t < rows) ? sq[e] * fexp(glast - gcv[e]) : 0.f;
+      sg[e] = (t < rows) ? bf16_to_f32(St[t * SLD + m]) * fexp(glast - gcv[e]) : 0.f;
     }
     bf16x8 sg0, sg1;   // contraction steps over rows [0,32) and [32,64)
 #pragma unroll
@@ -228,56 +252,72 @@ __global__ __launch_bounds__(256) void mfma_state_kernel(const MP p) {
       sg0[e] = (__bf16)sg[e];
       sg1[e] = (__bf16)sg[8 + e];
     }
-    // chunk-start states (bf16), before the update
-    {
-      const int64_t cg = (int64_t)(c0g + it) * H + h;
+    // local chunk-start states (bf16), before the update: rows m, 4 consecutive d per lane
 #pragma unroll
-      for (int b = 0; b < BPW; ++b) {
-        const int d0 = (wave * BPW + b) * 16;
-        bf16x4 pk;
+    for (int b = 0; b < NB; ++b) {
+      bf16x4 pk, pv;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) pk[r] = (__bf16)hk[b][r];
-        *reinterpret_cast<bf16x4*>(p.hkT + (cg * MS + m) * D + d0 + 4 * kb) = pk;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) p.hvc[(cg * MS + mb + 4 * kb + r) * D + d0 + l16] = f32_to_bf16(hv[b][r]);
+      for (int r = 0; r < 4; ++r) {
+        pk[r] = (__bf16)hk[b][r];
+        pv[r] = (__bf16)hv[b][r];
       }
+      *reinterpret_cast<bf16x4*>(p.hkT + (cg * MS + m) * D + 16 * b + 4 * kb) = pk;
+      *reinterpret_cast<bf16x4*>(p.hvc + (cg * MS + m) * D + 16 * b + 4 * kb) = pv;
     }
-    if (it + 1 < nchunks) issue(it + 1);
-    __syncthreads();
-    // decay, then accumulate this chunk
     const float dk = fexp(glast);
-    float dv[4];
+    gsum += glast;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) dv[r] = __shfl(dk, 4 * kb + r, 64);
-#pragma unroll
-    for (int b = 0; b < BPW; ++b) {
-      const int d0 = (wave * BPW + b) * 16;
+    for (int b = 0; b < NB; ++b) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         hk[b][r] *= dk;
-        hv[b][r] *= dv[r];
+        hv[b][r] *= dk;
       }
-      // hk[kk][m] += sum_t k[t][kk] sg[t][m]      A = k^T (transposed read), B = sg
-      hk[b] = mfma16(lds_frag_tr(Kt[cur], LDT, 0, 16, d0, lane), sg0, hk[b]);
-      hk[b] = mfma16(lds_frag_tr(Kt[cur], LDT, 32, 48, d0, lane), sg1, hk[b]);
-      // hv[m][vv] += sum_t sg[t][m] v[t][vv]      A = sg^T (same registers), B = v (transposed read)
-      hv[b] = mfma16(sg0, lds_frag_tr(Vt[cur], LDT, 0, 16, d0, lane), hv[b]);
-      hv[b] = mfma16(sg1, lds_frag_tr(Vt[cur], LDT, 32, 48, d0, lane), hv[b]);
+      // h[d][m] += sum_t x[t][d] sg[t][m]     A = x^T (transposed LDS read), B = sg
+      hk[b] = mfma16(lds_frag_tr(Kt, LDT, 0, 16, 16 * b, lane), sg0, hk[b]);
+      hk[b] = mfma16(lds_frag_tr(Kt, LDT, 32, 48, 16 * b, lane), sg1, hk[b]);
+      hv[b] = mfma16(lds_frag_tr(Vt, LDT, 0, 16, 16 * b, lane), sg0, hv[b]);
+      hv[b] = mfma16(lds_frag_tr(Vt, LDT, 32, 48, 16 * b, lane), sg1, hv[b]);
     }
   }
-  if (p.hkt) {
+  // segment end: local state (fp32, [m][d]) and total decay
+  const int64_t sl = (int64_t)seg_slot(p.coff, n, it0) * H + h;
 #pragma unroll
-    for (int b = 0; b < BPW; ++b) {
-      const int d0 = (wave * BPW + b) * 16;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        p.hkt[(((int64_t)n * H + h) * D + d0 + 4 * kb + r) * MS + m] = hk[b][r];
-        p.hvt[(((int64_t)n * H + h) * MS + mb + 4 * kb + r) * D + d0 + l16] = hv[b][r];
-      }
-    }
+  for (int b = 0; b < NB; ++b) {
+    *reinterpret_cast<float4*>(p.hend_k + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hk[b][0], hk[b][1], hk[b][2], hk[b][3]);
+    *reinterpret_cast<float4*>(p.hend_v + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hv[b][0], hv[b][1], hv[b][2], hv[b][3]);
   }
+  if (kb == 0) p.dtot[sl * MS + m] = fexp(gsum);
 }
 
+// Level 2: one thread per state element, sequential over the segments of its sequence.
+// grid (N*H, 2*MS*D/256): the first MS*D elements are the k-state ([m][d]), the rest the v-state.
+template <int D>
+__global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
+  const int H = p.H;
+  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  const bool isv = e >= MS * D;
+  const int em = isv ? e - MS * D : e;
+  const int m = em / D, d = em % D;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int nchunks = (eos - bos + BT - 1) / BT;
+  const int nseg = (nchunks + SEG - 1) / SEG;
+  float hcur = 0.f;
+  if (p.h0k) hcur = isv ? p.h0v[(((int64_t)n * H + h) * MS + m) * D + d] : p.h0k[(((int64_t)n * H + h) * D + d) * MS + m];
+  const float* hend = isv ? p.hend_v : p.hend_k;
+  float* hseg = isv ? p.hseg_v : p.hseg_k;
+  const int slot0 = p.coff[n] / SEG + n;
+  for (int sg = 0; sg < nseg; ++sg) {
+    const int64_t sl = (int64_t)(slot0 + sg) * H + h;
+    hseg[(sl * MS + m) * D + d] = hcur;
+    hcur = hcur * p.dtot[sl * MS + m] + hend[(sl * MS + m) * D + d];
+  }
+  if (p.hkt) {
+    if (isv) p.hvt[(((int64_t)n * H + h) * MS + m) * D + d] = hcur;
+    else p.hkt[(((int64_t)n * H + h) * D + d) * MS + m] = hcur;
+  }
+}
 
 // ==========================================================================================
 // output pass
@@ -347,14 +387,39 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
     const int64_t grow0 = (int64_t)c0 - p.shift;
-    TileRegs<D> a, b, c, d;
-    tile_g2r<D>(a, p.hkT + cg * MS * D, D, 0, 0, BT, tid);
+    TileRegs<D> b, d;
     tile_g2r<D>(b, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<D>(c, p.hvc + cg * MS * D, D, 0, 0, BT, tid);
     tile_g2r<D>(d, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_r2l<D>(Kb[0], a, tid);
+    // true chunk-start states: segment-local state + decayed segment-start state, as bf16 tiles
+    {
+      const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
+#pragma unroll
+      for (int u = 0; u < D / 32; ++u) {
+        const int c = tid + 256 * u;
+        const int row = c / (D / 8), col = (c % (D / 8)) * 8;
+        const float dc = p.dcum[cg * MS + row];
+        const uint4 lk = *reinterpret_cast<const uint4*>(p.hkT + (cg * MS + row) * D + col);
+        const uint4 lv = *reinterpret_cast<const uint4*>(p.hvc + (cg * MS + row) * D + col);
+        const float* sk = p.hseg_k + (sl * MS + row) * D + col;
+        const float* sv = p.hseg_v + (sl * MS + row) * D + col;
+        const float4 k0 = *reinterpret_cast<const float4*>(sk), k1 = *reinterpret_cast<const float4*>(sk + 4);
+        const float4 v0 = *reinterpret_cast<const float4*>(sv), v1 = *reinterpret_cast<const float4*>(sv + 4);
+        const float kf[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const float vf[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+        const uint32_t lkw[4] = {lk.x, lk.y, lk.z, lk.w}, lvw[4] = {lv.x, lv.y, lv.z, lv.w};
+        bf16x8 ok8, ov8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float a0 = __uint_as_float((e & 1) ? (lkw[e >> 1] & 0xffff0000u) : (lkw[e >> 1] << 16));
+          const float a1 = __uint_as_float((e & 1) ? (lvw[e >> 1] & 0xffff0000u) : (lvw[e >> 1] << 16));
+          ok8[e] = (__bf16)(a0 + kf[e] * dc);
+          ov8[e] = (__bf16)(a1 + vf[e] * dc);
+        }
+        *reinterpret_cast<bf16x8*>(Kb[0] + row * LDT + col) = ok8;
+        *reinterpret_cast<bf16x8*>(Vb[0] + row * LDT + col) = ov8;
+      }
+    }
     tile_r2l<D>(Kb[1], b, tid);
-    tile_r2l<D>(Vb[0], c, tid);
     tile_r2l<D>(Vb[1], d, tid);
     // gate cumsum table (fp32 [64][64]) in both orientations; rows past the sequence end are zero
     const float* gsrc = p.gc + cg * BT * MS;
@@ -730,8 +795,10 @@ int launch_out(const MP& p, hipStream_t st) {
 template <int D>
 int run_mfma(const MP& p, int phases, hipStream_t st) {
   if (phases != 2) {
-    hipLaunchKernelGGL((mfma_state_kernel<D>), dim3(p.N * p.H, MS / 16), dim3(256), 0, st, p);
-    NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass)");
+    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT, p.H), dim3(256), 0, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
+    hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
   }
   if (phases != 1) {
     const int G = (p.NG % 4 == 0) ? 4 : (p.NG % 2 == 0) ? 2 : 1;
@@ -750,10 +817,31 @@ bool prefill_mfma_supported(const NhaPrefillArgs* a) {
   return a->dtype == NHA_DTYPE_BF16 && a->K == a->V && (a->K == 64 || a->K == 128) && a->M == MS;
 }
 
-size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a) {
+namespace {
+struct ScratchPlan {
+  size_t hkT, hvc, gc, dcum, hend_k, hend_v, hseg_k, hseg_v, dtot, total;
+};
+ScratchPlan plan_scratch(const NhaPrefillArgs* a) {
   const size_t per = (size_t)a->NT * a->H;
-  return aligned(per * MS * a->K * 2) + aligned(per * MS * a->V * 2) + aligned(per * BT * MS * 4);
+  const size_t nslot = (size_t)a->NT / SEG + a->N + 1;
+  const size_t seg = aligned(nslot * a->H * MS * a->K * 4);
+  ScratchPlan s;
+  size_t off = 0;
+  s.hkT = off; off += aligned(per * MS * a->K * 2);
+  s.hvc = off; off += aligned(per * MS * a->V * 2);
+  s.gc = off; off += aligned(per * BT * MS * 4);
+  s.dcum = off; off += aligned(per * MS * 4);
+  s.hend_k = off; off += seg;
+  s.hend_v = off; off += seg;
+  s.hseg_k = off; off += seg;
+  s.hseg_v = off; off += seg;
+  s.dtot = off; off += aligned(nslot * a->H * MS * 4);
+  s.total = off;
+  return s;
 }
+}  // namespace
+
+size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a) { return plan_scratch(a).total; }
 
 int prefill_mfma_impl(const NhaPrefillArgs* a) {
   MP p;
@@ -764,13 +852,17 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
   p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa;
   p.h0k = a->h0k; p.h0v = a->h0v; p.hkt = a->hkt; p.hvt = a->hvt;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
-  const size_t per = (size_t)a->NT * a->H;
+  const ScratchPlan sp = plan_scratch(a);
   char* sc = (char*)a->scratch;
-  p.hkT = (bf16_t*)sc;
-  sc += aligned(per * MS * a->K * 2);
-  p.hvc = (bf16_t*)sc;
-  sc += aligned(per * MS * a->V * 2);
-  p.gc = (float*)sc;
+  p.hkT = (bf16_t*)(sc + sp.hkT);
+  p.hvc = (bf16_t*)(sc + sp.hvc);
+  p.gc = (float*)(sc + sp.gc);
+  p.dcum = (float*)(sc + sp.dcum);
+  p.hend_k = (float*)(sc + sp.hend_k);
+  p.hend_v = (float*)(sc + sp.hend_v);
+  p.hseg_k = (float*)(sc + sp.hseg_k);
+  p.hseg_v = (float*)(sc + sp.hseg_v);
+  p.dtot = (float*)(sc + sp.dtot);
   p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H;
   p.wl = a->wl; p.shift = a->shift; p.scale = a->scale;
   hipStream_t st = (hipStream_t)a->stream;

@@ -74,6 +74,28 @@ def test_decode_grid(dtype):
         assert_close(tag + " fr hv", hv3, rhv3, torch.float32 if dtype == torch.float32 else dtype)
 
 
+def test_decode_long_window_streaming_kernel():
+    """A window too long for the logits-in-LDS kernel takes the single-pass streaming kernel."""
+    from nha_amd import fused_recurrent_nha_decode
+    for dtype, NG, W, K, rot in ((torch.bfloat16, 4, 3000, 128, False), (torch.float32, 2, 5000, 64, True)):
+        d = decode_inputs(77, 2, 2, NG, K, K, 64, W, dtype)
+        c = {k: v.cuda() for k, v in d.items()}
+        if rot:
+            o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sw_k_raw"],
+                                                       sw_v=c["vw"], cos=c["cos"], sin=c["sin"],
+                                                       initial_state=(c["hk0"], c["hv0"]), output_final_state=True)
+            ro, rhk, rhv, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sw_k_raw"], d["vw"], cos=d["cos"],
+                                              sin=d["sin"], initial_state=(d["hk0"], d["hv0"]))
+        else:
+            o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sk"],
+                                                       sw_v=c["vw"], initial_state=(c["hk0"], c["hv0"]),
+                                                       output_final_state=True)
+            ro, rhk, rhv, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sk"], d["vw"], sq=d["sq"],
+                                              initial_state=(d["hk0"], d["hv0"]))
+        assert_close("long-window o", o, ro, dtype)
+        assert_close("long-window hv", hvt, rhv, dtype)
+
+
 def test_decode_state_aliasing_and_errors():
     from nha_amd import fused_recurrent_nha, fused_recurrent_nha_decode
     d = decode_inputs(7, 2, 2, 1, 64, 64, 16, 32, torch.bfloat16)
