@@ -25,6 +25,18 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
+// explicit LDS address space: keeps every tile access a ds_* instruction (never a flat access)
+#define NHA_LDS __attribute__((address_space(3)))
+typedef NHA_LDS bf16_t lbf16;
+typedef NHA_LDS float lfloat;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void lds_st16(lbf16* p, uint4 v) { *reinterpret_cast<NHA_LDS u32x4*>(p) = (u32x4){v.x, v.y, v.z, v.w}; }
+__device__ __forceinline__ float4 lds_ld_f4(const lfloat* p) {
+  const f32x4 v = *reinterpret_cast<const NHA_LDS f32x4*>(p);
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+
 constexpr int BT = 64;        // chunk rows == window tile keys
 constexpr int MS = 64;        // slots
 constexpr int GLD = 68;       // LDS row stride (floats) of the gate-cumsum tables
@@ -66,50 +78,50 @@ __device__ __forceinline__ bf16x8 pack8(f32x4 a, f32x4 b) {
 }
 
 // A/B fragment of a row-major LDS tile: 8 consecutive elements of row `row` starting at `col`.
-__device__ __forceinline__ bf16x8 lds_frag(const bf16_t* tile, int ld, int row, int col) {
-  return as_bf16x8(*reinterpret_cast<const uint4*>(tile + row * ld + col));
+__device__ __forceinline__ bf16x8 lds_frag(const lbf16* tile, int ld, int row, int col) {
+  return *reinterpret_cast<const NHA_LDS bf16x8*>(tile + row * ld + col);
 }
 
 // Transposed fragment of a row-major [rows][ld] bf16 LDS tile: the lane (c = l%16, kb = l/16)
 // receives X[r0a + 4*kb + e][col0 + c] for e = 0..3 and X[r0b + 4*kb + e][col0 + c] for e = 4..7.
-__device__ __forceinline__ bf16x8 lds_frag_tr(const bf16_t* tile, int ld, int r0a, int r0b, int col0, int lane) {
+__device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a, int r0b, int col0, int lane) {
   const int l16 = lane & 15, kb = lane >> 4;
-  const bf16_t* pa = tile + (r0a + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
-  const bf16_t* pb = tile + (r0b + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
+  const lbf16* pa = tile + (r0a + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
+  const lbf16* pb = tile + (r0b + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
   struct { s16x4 a, b; } t;
-  t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)pa);
-  t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)pb);
+  t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+  t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pb);
   return __builtin_bit_cast(bf16x8, t);
 }
 
 // ------------------------------------------------------------------------------------------
 // cooperative 64-row tile copy, global -> registers -> LDS (16-byte pieces, zero fill)
 // ------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int NTHR>
 struct TileRegs {
-  uint4 r[D / 32];
+  uint4 r[8 * D / NTHR];
 };
 
 // rows of the tile map to global rows grow0 + j; rows outside [vlo, vhi) are zero
-template <int D>
-__device__ __forceinline__ void tile_g2r(TileRegs<D>& t, const bf16_t* base, int64_t row_stride, int64_t grow0,
+template <int D, int NTHR>
+__device__ __forceinline__ void tile_g2r(TileRegs<D, NTHR>& t, const bf16_t* base, int64_t row_stride, int64_t grow0,
                                          int vlo, int vhi, int tid) {
 #pragma unroll
-  for (int u = 0; u < D / 32; ++u) {
-    const int c = tid + 256 * u;
+  for (int u = 0; u < 8 * D / NTHR; ++u) {
+    const int c = tid + NTHR * u;
     const int row = c / (D / 8), col = (c % (D / 8)) * 8;
     uint4 x = make_uint4(0, 0, 0, 0);
     if (row >= vlo && row < vhi) x = *reinterpret_cast<const uint4*>(base + (grow0 + row) * row_stride + col);
     t.r[u] = x;
   }
 }
-template <int D>
-__device__ __forceinline__ void tile_r2l(bf16_t* lds, const TileRegs<D>& t, int tid) {
+template <int D, int NTHR>
+__device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<D, NTHR>& t, int tid) {
 #pragma unroll
-  for (int u = 0; u < D / 32; ++u) {
-    const int c = tid + 256 * u;
+  for (int u = 0; u < 8 * D / NTHR; ++u) {
+    const int c = tid + NTHR * u;
     const int row = c / (D / 8), col = (c % (D / 8)) * 8;
-    *reinterpret_cast<uint4*>(lds + row * (D + 16) + col) = t.r[u];
+    lds_st16(lds + row * (D + 16) + col, t.r[u]);
   }
 }
 
@@ -133,10 +145,14 @@ template <int D>
 __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   constexpr int LDT = D + 16;
   constexpr int NB = D / 16;
-  __shared__ __align__(16) bf16_t Kt[BT * LDT];
-  __shared__ __align__(16) bf16_t Vt[BT * LDT];
-  __shared__ __align__(16) bf16_t St[BT * SLD];
-  __shared__ __align__(16) bf16_t Gt[BT * SLD];
+  __shared__ __align__(16) bf16_t Kt_[BT * LDT];
+  __shared__ __align__(16) bf16_t Vt_[BT * LDT];
+  __shared__ __align__(16) bf16_t St_[BT * SLD];
+  __shared__ __align__(16) bf16_t Gt_[BT * SLD];
+  lbf16* Kt = (lbf16*)Kt_;
+  lbf16* Vt = (lbf16*)Vt_;
+  lbf16* St = (lbf16*)St_;
+  lbf16* Gt = (lbf16*)Gt_;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
@@ -157,15 +173,15 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   }
   float gsum = 0.f;   // sum of the chunk-end gate cumsums since the segment start, this lane's slot
 
-  TileRegs<D> rk, rv;
+  TileRegs<D, 256> rk, rv;
   uint4 rs[2], rg[2];
   auto issue = [&](int it) {
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     const int64_t grow0 = (int64_t)bos + it * BT - p.shift;
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
-    tile_g2r<D>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<D>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<D, 256>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<D, 256>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -186,14 +202,14 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     const int chunk = chunk0 + jc;
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     if (jc > 0) __syncthreads();   // everyone is done reading the previous chunk's tiles
-    tile_r2l<D>(Kt, rk, tid);
-    tile_r2l<D>(Vt, rv, tid);
+    tile_r2l<D, 256>(Kt, rk, tid);
+    tile_r2l<D, 256>(Vt, rv, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
       const int j = c8 >> 3, m8 = (c8 & 7) * 8;
-      *reinterpret_cast<uint4*>(St + j * SLD + m8) = rs[u];
-      *reinterpret_cast<uint4*>(Gt + j * SLD + m8) = rg[u];
+      lds_st16(St + j * SLD + m8, rs[u]);
+      lds_st16(Gt + j * SLD + m8, rg[u]);
     }
     if (jc + 1 < nloc) issue(it + 1);
     __syncthreads();
@@ -333,24 +349,26 @@ struct OutSmem {
   static constexpr size_t bytes = 4 * tile_bytes + 2 * (size_t)BT * GLD * 4 + 2 * (size_t)BT * SLD * 2;
 };
 
-template <int D, int G>
-__global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
-  constexpr int RQB = G;
-  constexpr int WPU = 4 / G;
+template <int D, int G, int NW>
+__global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
+  constexpr int NTHR = 64 * NW;      // threads per workgroup
+  constexpr int WPU = NW / G;        // waves per (chunk, head)
+  constexpr int RQB = 4 / WPU;       // 16-row query blocks per wave
+  static_assert(WPU >= 1 && WPU <= 4 && RQB * WPU == 4, "bad wave split");
   constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   constexpr int LDT = D + 16;
   extern __shared__ __align__(16) unsigned char smem[];
-  bf16_t* Kb[2];
-  bf16_t* Vb[2];
-  Kb[0] = (bf16_t*)smem;
-  Kb[1] = Kb[0] + BT * LDT;
-  Vb[0] = Kb[1] + BT * LDT;
-  Vb[1] = Vb[0] + BT * LDT;
-  float* gcR = (float*)(Vb[1] + BT * LDT);   // [row j][slot m]
-  float* gcT = gcR + BT * GLD;               // [slot m][row j]
-  bf16_t* sR = (bf16_t*)(gcT + BT * GLD);    // [row j][slot m]
-  bf16_t* sT = sR + BT * SLD;                // [slot m][row j]
+  constexpr int TILE = BT * LDT;
+  lbf16* const tiles = (lbf16*)smem;           // K0, K1, V0, V1
+  lbf16* const Kb0 = tiles;
+  lbf16* const Kb1 = tiles + TILE;
+  lbf16* const Vb0 = tiles + 2 * TILE;
+  lbf16* const Vb1 = tiles + 3 * TILE;
+  lfloat* const gcR = (lfloat*)(tiles + 4 * TILE);   // [row j][slot m]
+  lfloat* const gcT = gcR + BT * GLD;                // [slot m][row j]
+  lbf16* const sR = (lbf16*)(gcT + BT * GLD);        // [row j][slot m]
+  lbf16* const sT = sR + BT * SLD;                   // [slot m][row j]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
@@ -373,12 +391,12 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     n_last = w < n_last ? w : n_last;
   }
   const int ntiles = n_last + 1;
-  TileRegs<D> rk, rv;
+  TileRegs<D, NTHR> rk, rv;
   auto issue_window = [&](int i) {
     const int64_t grow0 = (int64_t)c0 - 64 * i;
     const int vhi = i == 0 ? rows : BT;
-    tile_g2r<D>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
-    tile_g2r<D>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    tile_g2r<D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    tile_g2r<D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
   };
 
   // ---- phase 0: slot-branch operands -> LDS --------------------------------------------------
@@ -387,15 +405,15 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
     const int64_t grow0 = (int64_t)c0 - p.shift;
-    TileRegs<D> b, d;
-    tile_g2r<D>(b, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<D>(d, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    TileRegs<D, NTHR> b, d;
+    tile_g2r<D, NTHR>(b, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<D, NTHR>(d, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
     // true chunk-start states: segment-local state + decayed segment-start state, as bf16 tiles
     {
       const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
 #pragma unroll
-      for (int u = 0; u < D / 32; ++u) {
-        const int c = tid + 256 * u;
+      for (int u = 0; u < 8 * D / NTHR; ++u) {
+        const int c = tid + NTHR * u;
         const int row = c / (D / 8), col = (c % (D / 8)) * 8;
         const float dc = p.dcum[cg * MS + row];
         const uint4 lk = *reinterpret_cast<const uint4*>(p.hkT + (cg * MS + row) * D + col);
@@ -415,21 +433,21 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
           ok8[e] = (__bf16)(a0 + kf[e] * dc);
           ov8[e] = (__bf16)(a1 + vf[e] * dc);
         }
-        *reinterpret_cast<bf16x8*>(Kb[0] + row * LDT + col) = ok8;
-        *reinterpret_cast<bf16x8*>(Vb[0] + row * LDT + col) = ov8;
+        *reinterpret_cast<NHA_LDS bf16x8*>(Kb0 + row * LDT + col) = ok8;
+        *reinterpret_cast<NHA_LDS bf16x8*>(Vb0 + row * LDT + col) = ov8;
       }
     }
-    tile_r2l<D>(Kb[1], b, tid);
-    tile_r2l<D>(Vb[1], d, tid);
+    tile_r2l<D, NTHR>(Kb1, b, tid);
+    tile_r2l<D, NTHR>(Vb1, d, tid);
     // gate cumsum table (fp32 [64][64]) in both orientations; rows past the sequence end are zero
     const float* gsrc = p.gc + cg * BT * MS;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int cidx4 = tid + 256 * u;
+    for (int u = 0; u < 1024 / NTHR; ++u) {
+      const int cidx4 = tid + NTHR * u;
       const int j = cidx4 >> 4, m4 = (cidx4 & 15) * 4;
       float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
       if (j < rows) x = *reinterpret_cast<const float4*>(gsrc + j * MS + m4);
-      *reinterpret_cast<float4*>(gcR + j * GLD + m4) = x;
+      *reinterpret_cast<NHA_LDS f32x4*>(gcR + j * GLD + m4) = (f32x4){x.x, x.y, x.z, x.w};
       gcT[(m4 + 0) * GLD + j] = x.x;
       gcT[(m4 + 1) * GLD + j] = x.y;
       gcT[(m4 + 2) * GLD + j] = x.z;
@@ -437,12 +455,12 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     }
     // s rows of the slot branch (shifted), both orientations
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c8 = tid + 256 * u;
+    for (int u = 0; u < 512 / NTHR; ++u) {
+      const int c8 = tid + NTHR * u;
       const int j = c8 >> 3, m8 = (c8 & 7) * 8;
       uint4 x = make_uint4(0, 0, 0, 0);
       if (j >= vlo && j < rows) x = *reinterpret_cast<const uint4*>(p.s + ((grow0 + j) * H + h) * MS + m8);
-      *reinterpret_cast<uint4*>(sR + j * SLD + m8) = x;
+      lds_st16(sR + j * SLD + m8, x);
       const uint32_t w4[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
       for (int e = 0; e < 8; ++e) sT[(m8 + e) * SLD + j] = (bf16_t)(w4[e >> 1] >> (16 * (e & 1)));
@@ -480,7 +498,7 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     for (int mb = 0; mb < 4; ++mb) {
       ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ok[mb] = mfma16(lds_frag(Kb[0], LDT, 16 * mb + l16, 32 * ks + 8 * kb), qf[ks], ok[mb]);
+      for (int ks = 0; ks < KS; ++ks) ok[mb] = mfma16(lds_frag(Kb0, LDT, 16 * mb + l16, 32 * ks + 8 * kb), qf[ks], ok[mb]);
     }
     // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
     bf16x8 bA[2];
@@ -492,7 +510,7 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
         if (jb <= Q) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
-            at[jb] = mfma16(lds_frag(Kb[1], LDT, 16 * jb + l16, 32 * ks + 8 * kb), qf[ks], at[jb]);
+            at[jb] = mfma16(lds_frag(Kb1, LDT, 16 * jb + l16, 32 * ks + 8 * kb), qf[ks], at[jb]);
           if (jb == Q) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -520,8 +538,8 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
           for (int half = 0; half < 2; ++half) {
             const int jb = 2 * pr + half;
             const int j0 = 16 * jb + 4 * kb;
-            const float4 gj = *reinterpret_cast<const float4*>(gcT + mrow * GLD + j0);
-            const bf16x4 sj = *reinterpret_cast<const bf16x4*>(sT + mrow * SLD + j0);
+            const float4 gj = lds_ld_f4(gcT + mrow * GLD + j0);
+            const bf16x4 sj = *reinterpret_cast<const NHA_LDS bf16x4*>(sT + mrow * SLD + j0);
             const float gv[4] = {gj.x, gj.y, gj.z, gj.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -539,9 +557,9 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
-      const float4 gi = *reinterpret_cast<const float4*>(gcR + irow * GLD + 16 * mb + 4 * kb);
+      const float4 gi = lds_ld_f4(gcR + irow * GLD + 16 * mb + 4 * kb);
       float4 gr4 = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (Q > 0) gr4 = *reinterpret_cast<const float4*>(gcR + rref * GLD + 16 * mb + 4 * kb);
+      if (Q > 0) gr4 = lds_ld_f4(gcR + rref * GLD + 16 * mb + 4 * kb);
       const float giv[4] = {gi.x, gi.y, gi.z, gi.w};
       const float grv[4] = {gr4.x, gr4.y, gr4.z, gr4.w};
 #pragma unroll
@@ -583,7 +601,7 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
       const bf16x8 bp = pack8(x0, x1);
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        O[db][qb] = mfma16(lds_frag_tr(Vb[0], LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bp, O[db][qb]);
+        O[db][qb] = mfma16(lds_frag_tr(Vb0, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bp, O[db][qb]);
     }
     // slot read, intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m]))
     bf16x8 bpr[2];
@@ -611,10 +629,10 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
               const int m0 = 32 * pr + 16 * half + 4 * kb;
-              const float4 gj = *reinterpret_cast<const float4*>(gcR + jrow * GLD + m0);
+              const float4 gj = lds_ld_f4(gcR + jrow * GLD + m0);
               float4 gr4 = make_float4(0.f, 0.f, 0.f, 0.f);
-              if (Q > 0) gr4 = *reinterpret_cast<const float4*>(gcR + rref * GLD + m0);
-              const bf16x4 sj = *reinterpret_cast<const bf16x4*>(sR + jrow * SLD + m0);
+              if (Q > 0) gr4 = lds_ld_f4(gcR + rref * GLD + m0);
+              const bf16x4 sj = *reinterpret_cast<const NHA_LDS bf16x4*>(sR + jrow * SLD + m0);
               const float gv[4] = {gj.x, gj.y, gj.z, gj.w};
               const float grv[4] = {gr4.x, gr4.y, gr4.z, gr4.w};
 #pragma unroll
@@ -638,7 +656,7 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
       if (2 * pr <= Q) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          O[db][qb] = mfma16(lds_frag_tr(Vb[1], LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bAv[pr], O[db][qb]);
+          O[db][qb] = mfma16(lds_frag_tr(Vb1, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bAv[pr], O[db][qb]);
       }
     }
   }
@@ -657,95 +675,102 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
     }
   }
   __syncthreads();   // every wave is done with the slot-branch tiles
-  tile_r2l<D>(Kb[0], rk, tid);
-  tile_r2l<D>(Vb[0], rv, tid);
+  tile_r2l<D, NTHR>(Kb0, rk, tid);
+  tile_r2l<D, NTHR>(Vb0, rv, tid);
   if (ntiles > 1) issue_window(1);
   __syncthreads();
 
+  // lazy rescaling: the running reference max only moves when a tile exceeds it by more than
+  // 2^RESCALE_LOG2 in probability units, so O is rescaled a handful of times per chunk
+  constexpr float RESCALE_LOG2 = 8.f;
+  const float thr = RESCALE_LOG2 / cs;
   for (int i = 0; i < ntiles; ++i) {
     const int cur = i & 1;
-    const bf16_t* Kt = Kb[cur];
-    const bf16_t* Vt = Vb[cur];
-    // S^T[key][q] for 4 key blocks x RQB query blocks
-    f32x4 S[4][RQB];
-#pragma unroll
-    for (int kblk = 0; kblk < 4; ++kblk) {
-#pragma unroll
-      for (int qb = 0; qb < RQB; ++qb) S[kblk][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const bf16x8 a = lds_frag(Kt, LDT, 16 * kblk + l16, 32 * ks + 8 * kb);
-#pragma unroll
-        for (int qb = 0; qb < RQB; ++qb) S[kblk][qb] = mfma16(a, qs[qb][ks], S[kblk][qb]);
-      }
-    }
+    const lbf16* Kt = cur ? Kb1 : Kb0;
+    const lbf16* Vt = cur ? Vb1 : Vb0;
     const bool edge = (i == 0) || (p.wl >= 0 && 64 * i + 63 > p.wl);
-    if (edge) {
 #pragma unroll
-      for (int kblk = 0; kblk < 4; ++kblk)
+    for (int hf = 0; hf < 2; ++hf) {
+      // S^T[key][q] for the 32 keys of this half: 2 key blocks x RQB query blocks
+      f32x4 S[2][RQB];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+        for (int qb = 0; qb < RQB; ++qb) S[kk][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8 a = lds_frag(Kt, LDT, 32 * hf + 16 * kk + l16, 32 * ks + 8 * kb);
+#pragma unroll
+          for (int qb = 0; qb < RQB; ++qb) S[kk][qb] = mfma16(a, qs[qb][ks], S[kk][qb]);
+        }
+      }
+      if (edge) {
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int qb = 0; qb < RQB; ++qb) {
+            const int y = 16 * (qb0 + qb) + l16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int x = 32 * hf + 16 * kk + 4 * kb + r - 64 * i;   // key offset relative to the chunk start
+              const bool ok = (x <= y) && (p.wl < 0 || x >= y - p.wl);
+              if (!ok) S[kk][qb][r] = -INFINITY;
+            }
+          }
+      }
+      // online softmax per query column
+      bf16x8 P[RQB];
+      bool need = false;
+      float rmax[RQB];
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) {
+        float x = fmaxf(fmaxf(S[0][qb][0], S[0][qb][1]), fmaxf(S[0][qb][2], S[0][qb][3]));
+        x = fmaxf(x, fmaxf(fmaxf(S[1][qb][0], S[1][qb][1]), fmaxf(S[1][qb][2], S[1][qb][3])));
+        x = fmaxf(x, __shfl_xor(x, 16, 64));
+        x = fmaxf(x, __shfl_xor(x, 32, 64));
+        rmax[qb] = x;
+        need |= x > mrun[qb] + thr;
+      }
+      if (__any(need)) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) {
-          const int y = 16 * (qb0 + qb) + l16;
+          const float mnew = fmaxf(mrun[qb], rmax[qb]);
+          const float alpha = fexp2((mrun[qb] - mnew) * cs);
+          mrun[qb] = mnew;
+          lw[qb] *= alpha;
+          lg[qb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) O[db][qb][r] *= alpha;
+        }
+      }
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) {
+        const float mc = mrun[qb] * cs;
+        float psum = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int x = 16 * kblk + 4 * kb + r - 64 * i;   // key offset relative to the chunk start
-            const bool ok = (x <= y) && (p.wl < 0 || x >= y - p.wl);
-            if (!ok) S[kblk][qb][r] = -INFINITY;
+            const float e = fexp2(S[kk][qb][r] * cs - mc);
+            S[kk][qb][r] = e;
+            psum += e;
           }
-        }
-    }
-    // online softmax per query column
-    bf16x8 P[2][RQB];
-    bool any_rescale = false;
-    float alpha[RQB];
-#pragma unroll
-    for (int qb = 0; qb < RQB; ++qb) {
-      float rmax = S[0][qb][0];
-#pragma unroll
-      for (int kblk = 0; kblk < 4; ++kblk)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) rmax = fmaxf(rmax, S[kblk][qb][r]);
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 16, 64));
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
-      const float mnew = fmaxf(mrun[qb], rmax);
-      alpha[qb] = fexp2((mrun[qb] - mnew) * cs);
-      any_rescale |= (mnew != mrun[qb]);
-      mrun[qb] = mnew;
-      const float mc = mnew * cs;
-      float psum = 0.f;
-#pragma unroll
-      for (int kblk = 0; kblk < 4; ++kblk)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float e = fexp2(S[kblk][qb][r] * cs - mc);
-          S[kblk][qb][r] = e;
-          psum += e;
-        }
-      lw[qb] = lw[qb] * alpha[qb] + psum;
-      lg[qb] *= alpha[qb];
-      P[0][qb] = pack8(S[0][qb], S[1][qb]);
-      P[1][qb] = pack8(S[2][qb], S[3][qb]);
-    }
-    if (__any(any_rescale)) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int qb = 0; qb < RQB; ++qb)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) O[db][qb][r] *= alpha[qb];
-    }
-    // O^T[d][q] += V^T P^T
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
+        lw[qb] += psum;
+        P[qb] = pack8(S[0][qb], S[1][qb]);
+      }
+      // O^T[d][q] += V^T P^T over the 32 keys of this half
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const bf16x8 a = lds_frag_tr(Vt, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane);
+        const bf16x8 a = lds_frag_tr(Vt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);
 #pragma unroll
-        for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(a, P[pr][qb], O[db][qb]);
+        for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(a, P[qb], O[db][qb]);
       }
+    }
     if (i + 1 < ntiles) {
-      tile_r2l<D>(Kb[cur ^ 1], rk, tid);
-      tile_r2l<D>(Vb[cur ^ 1], rv, tid);
+      tile_r2l<D, NTHR>(cur ? Kb0 : Kb1, rk, tid);
+      tile_r2l<D, NTHR>(cur ? Vb0 : Vb1, rv, tid);
       if (i + 2 < ntiles) issue_window(i + 2);
     }
     __syncthreads();
@@ -775,19 +800,19 @@ __global__ __launch_bounds__(256, 1) void mfma_out_kernel(const MP p) {
   }
 }
 
-template <int D, int G>
+template <int D, int G, int NW>
 int launch_out(const MP& p, hipStream_t st) {
   static bool configured = false;
   const size_t lds = OutSmem<D>::bytes;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
       set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
       return NHA_ERR_LAUNCH;
     }
     configured = true;
   }
-  hipLaunchKernelGGL((mfma_out_kernel<D, G>), dim3(p.NT, p.H * (p.NG / G)), dim3(256), lds, st, p);
+  hipLaunchKernelGGL((mfma_out_kernel<D, G, NW>), dim3(p.NT, p.H * (p.NG / G)), dim3(64 * NW), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass)");
   return NHA_OK;
 }
@@ -801,10 +826,12 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
   }
   if (phases != 1) {
+    // G query heads of one kv-head share a workgroup; 8 waves (two per SIMD, 32 or 16 query rows
+    // each) when the group is large enough, else 4
     const int G = (p.NG % 4 == 0) ? 4 : (p.NG % 2 == 0) ? 2 : 1;
-    if (G == 4) return launch_out<D, 4>(p, st);
-    if (G == 2) return launch_out<D, 2>(p, st);
-    return launch_out<D, 1>(p, st);
+    if (G == 4) return launch_out<D, 4, 8>(p, st);
+    if (G == 2) return launch_out<D, 2, 8>(p, st);
+    return launch_out<D, 1, 4>(p, st);
   }
   return NHA_OK;
 }
