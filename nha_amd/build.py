@@ -18,13 +18,19 @@ FLAGS = [
 ]
 
 
+# the MFMA kernels never produce NaN on purpose; without this flag every fmaxf operand is
+# canonicalised by an extra VALU instruction in the softmax inner loop
+EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"]}
+
+
 def build_library(verbose: bool = False, jobs: int = 4) -> str:
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     for src in SOURCES:
         obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
-        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *FLAGS, *EXTRA.get(src, []), *os.environ.get("NHA_EXTRA_FLAGS", "").split(),
+               "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

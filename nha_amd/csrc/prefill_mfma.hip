@@ -77,6 +77,20 @@ __device__ __forceinline__ bf16x8 pack8(f32x4 a, f32x4 b) {
   return r;
 }
 
+// workgroup barrier that orders LDS traffic only: outstanding global loads (tile prefetches) stay
+// in flight across it
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// max over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), VALU only
+__device__ __forceinline__ float max_over_rows(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned v = __float_as_uint(x);
+  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 // A/B fragment of a row-major LDS tile: 8 consecutive elements of row `row` starting at `col`.
 __device__ __forceinline__ bf16x8 lds_frag(const lbf16* tile, int ld, int row, int col) {
   return *reinterpret_cast<const NHA_LDS bf16x8*>(tile + row * ld + col);
@@ -337,6 +351,13 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
 
 // ==========================================================================================
 // output pass
+#ifdef NHA_PROF
+#define PROF_DECL long long pt_[8] = {0,0,0,0,0,0,0,0}; long long pl_ = __builtin_amdgcn_s_memtime();
+#define PROF_MARK(k) { __builtin_amdgcn_sched_barrier(0); long long n_ = __builtin_amdgcn_s_memtime(); pt_[k] += n_ - pl_; pl_ = n_; }
+#else
+#define PROF_DECL
+#define PROF_MARK(k)
+#endif
 // ==========================================================================================
 // One workgroup = one 64-row chunk x G query heads of one kv-head (G in {1,2,4}); wave w owns
 // RQB = G blocks of 16 query rows of head w / (4/G).  LDS: two K-tile and two V-tile buffers
@@ -684,26 +705,42 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   // 2^RESCALE_LOG2 in probability units, so O is rescaled a handful of times per chunk
   constexpr float RESCALE_LOG2 = 8.f;
   const float thr = RESCALE_LOG2 / cs;
+  f32x4 Lw[RQB];
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) Lw[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
+  // every load issued so far (queries, first tiles) lands here, so inside the loop only the tile
+  // prefetches of the previous iteration are ever outstanding
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0), other counters untouched
+  PROF_DECL
   for (int i = 0; i < ntiles; ++i) {
+    PROF_MARK(7)
     const int cur = i & 1;
     const lbf16* Kt = cur ? Kb1 : Kb0;
     const lbf16* Vt = cur ? Vb1 : Vb0;
     const bool edge = (i == 0) || (p.wl >= 0 && 64 * i + 63 > p.wl);
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      // S^T[key][q] for the 32 keys of this half: 2 key blocks x RQB query blocks
+      // S^T[key][q] for the 32 keys of this half: 2 key blocks x RQB query blocks, the
+      // 2 * RQB accumulators advance together so consecutive MFMAs are independent
       f32x4 S[2][RQB];
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
+      for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) S[kk][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 a = lds_frag(Kt, LDT, 32 * hf + 16 * kk + l16, 32 * ks + 8 * kb);
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 a0 = lds_frag(Kt, LDT, 32 * hf + l16, 32 * ks + 8 * kb);
+        const bf16x8 a1 = lds_frag(Kt, LDT, 32 * hf + 16 + l16, 32 * ks + 8 * kb);
 #pragma unroll
-          for (int qb = 0; qb < RQB; ++qb) S[kk][qb] = mfma16(a, qs[qb][ks], S[kk][qb]);
+        for (int qb = 0; qb < RQB; ++qb) {
+          S[0][qb] = mfma16(a0, qs[qb][ks], S[0][qb]);
+          S[1][qb] = mfma16(a1, qs[qb][ks], S[1][qb]);
         }
       }
+      PROF_MARK(0)
       if (edge) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
@@ -726,19 +763,20 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       for (int qb = 0; qb < RQB; ++qb) {
         float x = fmaxf(fmaxf(S[0][qb][0], S[0][qb][1]), fmaxf(S[0][qb][2], S[0][qb][3]));
         x = fmaxf(x, fmaxf(fmaxf(S[1][qb][0], S[1][qb][1]), fmaxf(S[1][qb][2], S[1][qb][3])));
-        x = fmaxf(x, __shfl_xor(x, 16, 64));
-        x = fmaxf(x, __shfl_xor(x, 32, 64));
+        x = max_over_rows(x);
         rmax[qb] = x;
         need |= x > mrun[qb] + thr;
       }
+      PROF_MARK(1)
       if (__any(need)) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) {
           const float mnew = fmaxf(mrun[qb], rmax[qb]);
           const float alpha = fexp2((mrun[qb] - mnew) * cs);
           mrun[qb] = mnew;
-          lw[qb] *= alpha;
           lg[qb] *= alpha;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) Lw[qb][r] *= alpha;
 #pragma unroll
           for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -748,18 +786,15 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
 #pragma unroll
       for (int qb = 0; qb < RQB; ++qb) {
         const float mc = mrun[qb] * cs;
-        float psum = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float e = fexp2(S[kk][qb][r] * cs - mc);
-            S[kk][qb][r] = e;
-            psum += e;
-          }
-        lw[qb] += psum;
+          for (int r = 0; r < 4; ++r) S[kk][qb][r] = fexp2(S[kk][qb][r] * cs - mc);
         P[qb] = pack8(S[0][qb], S[1][qb]);
+        // window row sums on the matrix core: every row of ones^T P is the sum over the 32 keys
+        Lw[qb] = mfma16(ones, P[qb], Lw[qb]);
       }
+      PROF_MARK(2)
       // O^T[d][q] += V^T P^T over the 32 keys of this half
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
@@ -767,21 +802,29 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(a, P[qb], O[db][qb]);
       }
+      PROF_MARK(3)
     }
     if (i + 1 < ntiles) {
       tile_r2l<D, NTHR>(cur ? Kb0 : Kb1, rk, tid);
       tile_r2l<D, NTHR>(cur ? Vb0 : Vb1, rv, tid);
       if (i + 2 < ntiles) issue_window(i + 2);
     }
-    __syncthreads();
+    PROF_MARK(4)
+    lds_barrier();
+    PROF_MARK(5)
   }
+#ifdef NHA_PROF
+  if (blockIdx.x == 200 && blockIdx.y == 3 && lane == 0) {
+    long long* dbg = (long long*)p.lse_gsa;
+    for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
+  }
+#endif
 
   // ---- epilogue -------------------------------------------------------------------------------
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
     const int irow = 16 * (qb0 + qb) + l16;
-    float lwt = lw[qb] + __shfl_xor(lw[qb], 16, 64);
-    lwt += __shfl_xor(lwt, 32, 64);
+    const float lwt = Lw[qb][0];
     float lgt = lg[qb] + __shfl_xor(lg[qb], 16, 64);
     lgt += __shfl_xor(lgt, 32, 64);
     const float inv = 1.f / (lwt + lgt);
