@@ -258,7 +258,7 @@ def main():
                                "(window W keys, slots hold tokens <= t-W), gate logits N(-1,1)->logsigmoid",
                    "decode_workload": "B=128 HQ=32 H=8 D=128 M=64 W=1024 ring buffer, full windows at random "
                                       "ring positions, 256 consecutive steps"},
-        "roofline": {"bound": "mfma", "kernel": "mfma_out_kernel<128,4>", "achieved": pf["achieved_tflops"],
+        "roofline": {"bound": "mfma", "kernel": "mfma_out_kernel<128,4,8,64>", "achieved": pf["achieved_tflops"],
                      "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": pf["achieved_tflops"] / PEAK_MFMA_BF16_TFLOPS,
                      "traffic": None, "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
                      "whole_op_tflops": pf["whole_op_tflops"], "algorithmic_flop": pf["flops"]},

@@ -1,4 +1,4 @@
-// bf16 MFMA prefill for gfx950 (K == V == D in {64,128}, M == 64 slots), fp32 accumulation.
+// bf16 MFMA prefill for gfx950 (K == V == D in {64,128,256}, M == 64 slots), fp32 accumulation.
 //
 // Everything is computed "transposed" so that each lane owns ONE query column of a 16x16
 // accumulator block (v_mfma_f32_16x16x32_bf16: A[i][8*(l/16)+e], B[8*(l/16)+e][j], C[4*(l/16)+r][l%16]):
@@ -111,17 +111,17 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a
 // ------------------------------------------------------------------------------------------
 // cooperative 64-row tile copy, global -> registers -> LDS (16-byte pieces, zero fill)
 // ------------------------------------------------------------------------------------------
-template <int D, int NTHR>
+template <int ROWS, int D, int NTHR>
 struct TileRegs {
-  uint4 r[8 * D / NTHR];
+  uint4 r[ROWS * D / 8 / NTHR];
 };
 
 // rows of the tile map to global rows grow0 + j; rows outside [vlo, vhi) are zero
-template <int D, int NTHR>
-__device__ __forceinline__ void tile_g2r(TileRegs<D, NTHR>& t, const bf16_t* base, int64_t row_stride, int64_t grow0,
-                                         int vlo, int vhi, int tid) {
+template <int ROWS, int D, int NTHR>
+__device__ __forceinline__ void tile_g2r(TileRegs<ROWS, D, NTHR>& t, const bf16_t* base, int64_t row_stride,
+                                         int64_t grow0, int vlo, int vhi, int tid) {
 #pragma unroll
-  for (int u = 0; u < 8 * D / NTHR; ++u) {
+  for (int u = 0; u < ROWS * D / 8 / NTHR; ++u) {
     const int c = tid + NTHR * u;
     const int row = c / (D / 8), col = (c % (D / 8)) * 8;
     uint4 x = make_uint4(0, 0, 0, 0);
@@ -129,10 +129,10 @@ __device__ __forceinline__ void tile_g2r(TileRegs<D, NTHR>& t, const bf16_t* bas
     t.r[u] = x;
   }
 }
-template <int D, int NTHR>
-__device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<D, NTHR>& t, int tid) {
+template <int ROWS, int D, int NTHR>
+__device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<ROWS, D, NTHR>& t, int tid) {
 #pragma unroll
-  for (int u = 0; u < 8 * D / NTHR; ++u) {
+  for (int u = 0; u < ROWS * D / 8 / NTHR; ++u) {
     const int c = tid + NTHR * u;
     const int row = c / (D / 8), col = (c % (D / 8)) * 8;
     lds_st16(lds + row * (D + 16) + col, t.r[u]);
@@ -159,20 +159,30 @@ template <int D>
 __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   constexpr int LDT = D + 16;
   constexpr int NB = D / 16;
-  __shared__ __align__(16) bf16_t Kt_[BT * LDT];
-  __shared__ __align__(16) bf16_t Vt_[BT * LDT];
-  __shared__ __align__(16) bf16_t St_[BT * SLD];
-  __shared__ __align__(16) bf16_t Gt_[BT * SLD];
-  lbf16* Kt = (lbf16*)Kt_;
-  lbf16* Vt = (lbf16*)Vt_;
-  lbf16* St = (lbf16*)St_;
-  lbf16* Gt = (lbf16*)Gt_;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* Kt = (lbf16*)smem;
+  lbf16* Vt = Kt + BT * LDT;
+  lbf16* St = Vt + BT * LDT;
+  lbf16* Gt = St + BT * SLD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
-  const int chunk0 = blockIdx.x, h = blockIdx.y;
-  const int n = p.cidx[2 * chunk0], it0 = p.cidx[2 * chunk0 + 1];
-  if (it0 % SEG != 0) return;
+  // blockIdx.x is a segment slot (seg_slot); slots are dense up to a few gaps per sequence, so
+  // every XCD receives the same share of working workgroups
+  const int slot = blockIdx.x, h = blockIdx.y;
+  int n = 0;
+  {
+    int lo = 0, hi = p.N - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.coff[mid] / SEG + mid <= slot) lo = mid; else hi = mid - 1;
+    }
+    n = lo;
+  }
+  const int kseg = slot - (p.coff[n] / SEG + n);
+  const int it0 = kseg * SEG;
+  if (it0 >= p.coff[n + 1] - p.coff[n]) return;
+  const int chunk0 = p.coff[n] + it0;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int L = eos - bos;
   const int nchunks = (L + BT - 1) / BT;
@@ -187,15 +197,15 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   }
   float gsum = 0.f;   // sum of the chunk-end gate cumsums since the segment start, this lane's slot
 
-  TileRegs<D, 256> rk, rv;
+  TileRegs<BT, D, 256> rk, rv;
   uint4 rs[2], rg[2];
   auto issue = [&](int it) {
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     const int64_t grow0 = (int64_t)bos + it * BT - p.shift;
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
-    tile_g2r<D, 256>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<D, 256>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<BT, D, 256>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<BT, D, 256>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -216,8 +226,8 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     const int chunk = chunk0 + jc;
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     if (jc > 0) __syncthreads();   // everyone is done reading the previous chunk's tiles
-    tile_r2l<D, 256>(Kt, rk, tid);
-    tile_r2l<D, 256>(Vt, rv, tid);
+    tile_r2l<BT, D, 256>(Kt, rk, tid);
+    tile_r2l<BT, D, 256>(Vt, rv, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -359,44 +369,64 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
 #define PROF_MARK(k)
 #endif
 // ==========================================================================================
-// One workgroup = one 64-row chunk x G query heads of one kv-head (G in {1,2,4}); wave w owns
-// RQB = G blocks of 16 query rows of head w / (4/G).  LDS: two K-tile and two V-tile buffers
-// (double buffered window stream; they first hold hkT, k_gsa rows, hv, v rows of the slot branch)
-// plus the chunk's gate-cumsum / s tables in both orientations.
-template <int D>
+// One workgroup = one 64-row chunk x G query heads of one kv-head; its NW waves split the
+// 64 x G query rows into RQB blocks of 16 rows per wave.  Window K/V stream through four LDS
+// buffers of TK keys (two K, two V, double buffered); TK = 64 for D <= 128, 32 for D = 256.
+// The slot branch runs first on the same buffers: its four 64-row operand tiles (transposed
+// chunk-start k-state, k_gsa rows, chunk-start v-state, v rows) fit at once when TK = 64 and
+// in two stages when TK = 32.  The decay factors s_j[m] exp(gr[m] - gc_j[m]) that every wave
+// needs are computed once per workgroup into LDS, already in MFMA fragment order.
+constexpr int NSEA = 24;   // fragments s*decay with rows = slots  (A operand of the logit update)
+constexpr int NSEB = 20;   // fragments s*decay with rows = tokens (A operand of the slot-read weights)
+
+template <int D, int TK>
 struct OutSmem {
   static constexpr int LDT = D + 16;
-  static constexpr size_t tile_bytes = (size_t)BT * LDT * 2;
-  static constexpr size_t bytes = 4 * tile_bytes + 2 * (size_t)BT * GLD * 4 + 2 * (size_t)BT * SLD * 2;
+  static constexpr size_t tile_bytes = (size_t)TK * LDT * 2;
+  static constexpr size_t bytes =
+      4 * tile_bytes + (size_t)BT * GLD * 4 + (size_t)BT * SLD * 2 + (size_t)(NSEA + NSEB) * 512 * 2;
 };
 
-template <int D, int G, int NW>
+__device__ __forceinline__ int sea_base(int Q) { return Q == 0 ? 0 : Q == 1 ? 4 : Q == 2 ? 8 : 16; }
+__device__ __forceinline__ int seb_base(int Q) { return Q == 0 ? 0 : Q == 1 ? 2 : Q == 2 ? 6 : 12; }
+
+template <int D, int G, int NW, int TK>
 __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   constexpr int NTHR = 64 * NW;      // threads per workgroup
   constexpr int WPU = NW / G;        // waves per (chunk, head)
   constexpr int RQB = 4 / WPU;       // 16-row query blocks per wave
   static_assert(WPU >= 1 && WPU <= 4 && RQB * WPU == 4, "bad wave split");
+  static_assert(TK == 64 || TK == 32, "bad tile size");
   constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   constexpr int LDT = D + 16;
+  constexpr int NH = TK / 32;        // 32-key halves per tile
+  constexpr int TILE = TK * LDT;
   extern __shared__ __align__(16) unsigned char smem[];
-  constexpr int TILE = BT * LDT;
   lbf16* const tiles = (lbf16*)smem;           // K0, K1, V0, V1
   lbf16* const Kb0 = tiles;
   lbf16* const Kb1 = tiles + TILE;
   lbf16* const Vb0 = tiles + 2 * TILE;
   lbf16* const Vb1 = tiles + 3 * TILE;
-  lfloat* const gcR = (lfloat*)(tiles + 4 * TILE);   // [row j][slot m]
-  lfloat* const gcT = gcR + BT * GLD;                // [slot m][row j]
-  lbf16* const sR = (lbf16*)(gcT + BT * GLD);        // [row j][slot m]
-  lbf16* const sT = sR + BT * SLD;                   // [slot m][row j]
+  lfloat* const gcR = (lfloat*)(tiles + 4 * TILE);   // gate cumsum [row j][slot m]
+  lbf16* const sR = (lbf16*)(gcR + BT * GLD);        // s [row j][slot m]
+  lbf16* const SEa = sR + BT * SLD;                  // NSEA fragments of 64 lanes x 8
+  lbf16* const SEb = SEa + NSEA * 512;               // NSEB fragments
+  // 64-row slot-branch tiles: TK = 64 -> four buffers; TK = 32 -> two double-height buffers
+  lbf16* const tA = Kb0;                                 // hkT, then (TK = 32) hv
+  lbf16* const tB = TK == 64 ? Kb1 : Vb0;                // k_gsa rows, then (TK = 32) v rows
+  lbf16* const tC = TK == 64 ? Vb0 : Kb0;                // hv
+  lbf16* const tD = TK == 64 ? Vb1 : Vb0;                // v rows
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
-  const int chunk = blockIdx.x;
+  // grid = (kv-head x head-group, chunk): consecutive workgroup ids are the heads of one chunk, so
+  // with 8 (kv-head, group) pairs each XCD (id % 8) streams the chunks of ONE kv-head in order and
+  // the window tiles its resident workgroups share stay in that XCD's L2
+  const int chunk = blockIdx.y;
   const int ngrp = NG / G;
-  const int h = blockIdx.y / ngrp, grp = blockIdx.y % ngrp;
+  const int h = blockIdx.x / ngrp, grp = blockIdx.x % ngrp;
   const int hq = h * NG + grp * G + wave / WPU;
   const int qb0 = (wave % WPU) * RQB;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
@@ -404,101 +434,126 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   const int c0 = bos + it * BT;
   const int rows = (eos - c0) < BT ? (eos - c0) : BT;
   const float cs = p.scale * LOG2E;   // logits are kept unscaled; p = exp2(cs * (s - m))
+  const int64_t cg = (int64_t)chunk * H + h;
 
-  // ---- window tile schedule: tile i covers keys [c0 - 64 i, c0 - 64 i + 63] -----------------
-  int n_last = it;   // tiles may not start before bos
-  if (p.wl >= 0) {
-    const int w = (p.wl + 63) / 64;
-    n_last = w < n_last ? w : n_last;
-  }
-  const int ntiles = n_last + 1;
-  TileRegs<D, NTHR> rk, rv;
+  // ---- window tile schedule: tile i covers keys [c0 + 64 - TK (i+1), c0 + 64 - TK i) ----------
+  int lowest = bos;
+  if (p.wl >= 0 && c0 - p.wl > bos) lowest = c0 - p.wl;
+  const int ntiles = (c0 + 64 - lowest + TK - 1) / TK;
+  TileRegs<TK, D, NTHR> rk, rv;
   auto issue_window = [&](int i) {
-    const int64_t grow0 = (int64_t)c0 - 64 * i;
-    const int vhi = i == 0 ? rows : BT;
-    tile_g2r<D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
-    tile_g2r<D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    const int64_t grow0 = (int64_t)c0 + 64 - TK * (i + 1);
+    int vhi = eos - (int)grow0;
+    vhi = vhi < 0 ? 0 : (vhi > TK ? TK : vhi);
+    tile_g2r<TK, D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    tile_g2r<TK, D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
   };
 
   // ---- phase 0: slot-branch operands -> LDS --------------------------------------------------
-  {
-    const int64_t cg = (int64_t)chunk * H + h;
-    int vlo = p.shift - it * BT;
-    vlo = vlo < 0 ? 0 : vlo;
-    const int64_t grow0 = (int64_t)c0 - p.shift;
-    TileRegs<D, NTHR> b, d;
-    tile_g2r<D, NTHR>(b, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<D, NTHR>(d, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    // true chunk-start states: segment-local state + decayed segment-start state, as bf16 tiles
-    {
-      const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
+  int vlo = p.shift - it * BT;
+  vlo = vlo < 0 ? 0 : vlo;
+  const int64_t grow_s = (int64_t)c0 - p.shift;
+  // true chunk-start state (segment-local state + decayed segment-start state) as a bf16 tile
+  auto load_state_tile = [&](lbf16* dst, const bf16_t* hloc, const float* hseg) {
+    const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
 #pragma unroll
-      for (int u = 0; u < 8 * D / NTHR; ++u) {
-        const int c = tid + NTHR * u;
-        const int row = c / (D / 8), col = (c % (D / 8)) * 8;
-        const float dc = p.dcum[cg * MS + row];
-        const uint4 lk = *reinterpret_cast<const uint4*>(p.hkT + (cg * MS + row) * D + col);
-        const uint4 lv = *reinterpret_cast<const uint4*>(p.hvc + (cg * MS + row) * D + col);
-        const float* sk = p.hseg_k + (sl * MS + row) * D + col;
-        const float* sv = p.hseg_v + (sl * MS + row) * D + col;
-        const float4 k0 = *reinterpret_cast<const float4*>(sk), k1 = *reinterpret_cast<const float4*>(sk + 4);
-        const float4 v0 = *reinterpret_cast<const float4*>(sv), v1 = *reinterpret_cast<const float4*>(sv + 4);
-        const float kf[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-        const float vf[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-        const uint32_t lkw[4] = {lk.x, lk.y, lk.z, lk.w}, lvw[4] = {lv.x, lv.y, lv.z, lv.w};
-        bf16x8 ok8, ov8;
+    for (int u = 0; u < BT * D / 8 / NTHR; ++u) {
+      const int c = tid + NTHR * u;
+      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
+      const float dc = p.dcum[cg * MS + row];
+      const uint4 lk = *reinterpret_cast<const uint4*>(hloc + (cg * MS + row) * D + col);
+      const float* sk = hseg + (sl * MS + row) * D + col;
+      const float4 k0 = *reinterpret_cast<const float4*>(sk), k1 = *reinterpret_cast<const float4*>(sk + 4);
+      const float kf[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+      const uint32_t lkw[4] = {lk.x, lk.y, lk.z, lk.w};
+      bf16x8 o8;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float a0 = __uint_as_float((e & 1) ? (lkw[e >> 1] & 0xffff0000u) : (lkw[e >> 1] << 16));
-          const float a1 = __uint_as_float((e & 1) ? (lvw[e >> 1] & 0xffff0000u) : (lvw[e >> 1] << 16));
-          ok8[e] = (__bf16)(a0 + kf[e] * dc);
-          ov8[e] = (__bf16)(a1 + vf[e] * dc);
-        }
-        *reinterpret_cast<NHA_LDS bf16x8*>(Kb0 + row * LDT + col) = ok8;
-        *reinterpret_cast<NHA_LDS bf16x8*>(Vb0 + row * LDT + col) = ov8;
+      for (int e = 0; e < 8; ++e) {
+        const float a0 = __uint_as_float((e & 1) ? (lkw[e >> 1] & 0xffff0000u) : (lkw[e >> 1] << 16));
+        o8[e] = (__bf16)(a0 + kf[e] * dc);
       }
+      *reinterpret_cast<NHA_LDS bf16x8*>(dst + row * LDT + col) = o8;
     }
-    tile_r2l<D, NTHR>(Kb1, b, tid);
-    tile_r2l<D, NTHR>(Vb1, d, tid);
-    // gate cumsum table (fp32 [64][64]) in both orientations; rows past the sequence end are zero
+  };
+  auto load_rows_tile = [&](lbf16* dst, const bf16_t* src) {
+    TileRegs<BT, D, NTHR> t;
+    tile_g2r<BT, D, NTHR>(t, src + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
+    tile_r2l<BT, D, NTHR>(dst, t, tid);
+  };
+  load_state_tile(tA, p.hkT, p.hseg_k);
+  load_rows_tile(tB, p.k_gsa);
+  if (TK == 64) {
+    load_state_tile(tC, p.hvc, p.hseg_v);
+    load_rows_tile(tD, p.v);
+  }
+  {
+    // gate cumsum table (fp32 [64][64]); rows past the sequence end are zero
     const float* gsrc = p.gc + cg * BT * MS;
-#pragma unroll
-    for (int u = 0; u < 1024 / NTHR; ++u) {
-      const int cidx4 = tid + NTHR * u;
-      const int j = cidx4 >> 4, m4 = (cidx4 & 15) * 4;
+    for (int c4 = tid; c4 < 1024; c4 += NTHR) {
+      const int j = c4 >> 4, m4 = (c4 & 15) * 4;
       float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
       if (j < rows) x = *reinterpret_cast<const float4*>(gsrc + j * MS + m4);
       *reinterpret_cast<NHA_LDS f32x4*>(gcR + j * GLD + m4) = (f32x4){x.x, x.y, x.z, x.w};
-      gcT[(m4 + 0) * GLD + j] = x.x;
-      gcT[(m4 + 1) * GLD + j] = x.y;
-      gcT[(m4 + 2) * GLD + j] = x.z;
-      gcT[(m4 + 3) * GLD + j] = x.w;
     }
-    // s rows of the slot branch (shifted), both orientations
-#pragma unroll
-    for (int u = 0; u < 512 / NTHR; ++u) {
-      const int c8 = tid + NTHR * u;
+    // s rows of the slot branch (shifted)
+    for (int c8 = tid; c8 < 512; c8 += NTHR) {
       const int j = c8 >> 3, m8 = (c8 & 7) * 8;
       uint4 x = make_uint4(0, 0, 0, 0);
-      if (j >= vlo && j < rows) x = *reinterpret_cast<const uint4*>(p.s + ((grow0 + j) * H + h) * MS + m8);
+      if (j >= vlo && j < rows) x = *reinterpret_cast<const uint4*>(p.s + ((grow_s + j) * H + h) * MS + m8);
       lds_st16(sR + j * SLD + m8, x);
-      const uint32_t w4[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sT[(m8 + e) * SLD + j] = (bf16_t)(w4[e >> 1] >> (16 * (e & 1)));
     }
   }
   issue_window(0);
   __syncthreads();
+  // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
+  // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows
+  // j of earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.
+  for (int item = tid; item < (NSEA + NSEB) * 64; item += NTHR) {
+    const int f = item >> 6, ln = item & 63;
+    const int fl16 = ln & 15, fkb = ln >> 4;
+    bf16x8 out;
+    if (f < NSEA) {
+      const int Q = f < 4 ? 0 : f < 8 ? 1 : f < 16 ? 2 : 3;
+      const int rem = f - sea_base(Q);
+      const int pr = rem >> 2, mb = rem & 3;
+      const int m = 16 * mb + fl16;
+      const float gr = Q > 0 ? gcR[(16 * Q - 1) * GLD + m] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int jb = 2 * pr + (e >> 2);
+        const int j = 16 * jb + 4 * fkb + (e & 3);
+        float val = 0.f;
+        if (jb <= Q) val = bf16_to_f32(sR[j * SLD + m]) * fexp(fminf(gr - gcR[j * GLD + m], DECAY_CLAMP));
+        out[e] = (__bf16)val;
+      }
+      *reinterpret_cast<NHA_LDS bf16x8*>(SEa + f * 512 + ln * 8) = out;
+    } else {
+      const int g2 = f - NSEA;
+      const int Q = g2 < 2 ? 0 : g2 < 6 ? 1 : g2 < 12 ? 2 : 3;
+      const int rem = g2 - seb_base(Q);
+      const int jb = rem >> 1, pr = rem & 1;
+      const int j = 16 * jb + fl16;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int m = 32 * pr + 16 * (e >> 2) + 4 * fkb + (e & 3);
+        const float gr = Q > 0 ? gcR[(16 * Q - 1) * GLD + m] : 0.f;
+        out[e] = (__bf16)(bf16_to_f32(sR[j * SLD + m]) * fexp(fminf(gr - gcR[j * GLD + m], DECAY_CLAMP)));
+      }
+      *reinterpret_cast<NHA_LDS bf16x8*>(SEb + g2 * 512 + ln * 8) = out;
+    }
+  }
+  __syncthreads();
 
   // per-lane softmax state for the RQB queries (l16 + 16*(qb0+qb)) this lane serves
-  float mrun[RQB], lg[RQB], lw[RQB];
+  float mrun[RQB], lg[RQB];
   f32x4 O[DB][RQB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int qb = 0; qb < RQB; ++qb) O[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  bf16x8 bp[RQB][2], bpr[RQB][2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
 
-  // ---- phase 1: slot branch, one 16-row query block at a time --------------------------------
+  // ---- phase 1a: slot logits and the slot "tile" of the softmax, one 16-row block at a time ----
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
     const int Q = qb0 + qb;                // sub-block index inside the chunk
@@ -516,64 +571,46 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
     f32x4 ok[4];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < 4; ++mb) ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ok[mb] = mfma16(lds_frag(Kb0, LDT, 16 * mb + l16, 32 * ks + 8 * kb), qf[ks], ok[mb]);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(lds_frag(tA, LDT, 16 * mb + l16, 32 * ks + 8 * kb), qf[ks], ok[mb]);
     // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
     bf16x8 bA[2];
     {
       f32x4 at[4];
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
-        at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        if (jb <= Q) {
+      for (int jb = 0; jb < 4; ++jb) at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks)
-            at[jb] = mfma16(lds_frag(Kb1, LDT, 16 * jb + l16, 32 * ks + 8 * kb), qf[ks], at[jb]);
-          if (jb == Q) {
+      for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (4 * kb + r > l16) at[jb][r] = 0.f;
-          }
+        for (int jb = 0; jb < 4; ++jb)
+          if (jb <= Q) at[jb] = mfma16(lds_frag(tB, LDT, 16 * jb + l16, 32 * ks + 8 * kb), qf[ks], at[jb]);
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+        if (jb == Q) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (4 * kb + r > l16) at[jb][r] = 0.f;
         }
-      }
       bA[0] = pack8(at[0], at[1]);
       bA[1] = pack8(at[2], at[3]);
     }
-    // decay reference of this sub-block: gc at the row before it (0 for the first sub-block)
-    const int rref = 16 * Q - 1;
     // okT_intra[m][i] = sum_j s_j[m] exp(gr[m] - gc_j[m]) AT[j][i]
     f32x4 oki[4];
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
       oki[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      const int mrow = 16 * mb + l16;
-      const float gr = Q > 0 ? gcT[mrow * GLD + rref] : 0.f;
 #pragma unroll
-      for (int pr = 0; pr < 2; ++pr) {
+      for (int pr = 0; pr < 2; ++pr)
         if (2 * pr <= Q) {
-          bf16x8 se;
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int jb = 2 * pr + half;
-            const int j0 = 16 * jb + 4 * kb;
-            const float4 gj = lds_ld_f4(gcT + mrow * GLD + j0);
-            const bf16x4 sj = *reinterpret_cast<const NHA_LDS bf16x4*>(sT + mrow * SLD + j0);
-            const float gv[4] = {gj.x, gj.y, gj.z, gj.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float val = 0.f;
-              if (jb <= Q) val = (float)sj[e] * fexp(fminf(gr - gv[e], DECAY_CLAMP));
-              se[4 * half + e] = (__bf16)val;
-            }
-          }
+          const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(SEa + (sea_base(Q) + 4 * pr + mb) * 512 + lane * 8);
           oki[mb] = mfma16(se, bA[pr], oki[mb]);
         }
-      }
     }
     // combine, then the slot "tile" of the online softmax (logits unscaled, exponent scale cs)
+    const int rref = 16 * Q - 1;
     float rmax = -INFINITY;
     f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
 #pragma unroll
@@ -591,8 +628,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
         rmax = fmaxf(rmax, ok[mb][r]);
       }
     }
-    rmax = fmaxf(rmax, __shfl_xor(rmax, 16, 64));
-    rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
+    rmax = max_over_rows(rmax);
     mrun[qb] = rmax;
     float psum = 0.f;
     const float mc = rmax * cs;
@@ -604,38 +640,43 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
         psum += ok[mb][r];
       }
     lg[qb] = psum;   // partial over this lane's 16 slots
-    lw[qb] = 0.f;
     if (p.lse_gsa) {
       float tot = psum + __shfl_xor(psum, 16, 64);
       tot += __shfl_xor(tot, 32, 64);
       if (kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (mc + __builtin_amdgcn_logf(tot)) * LN2;
     }
-    // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr) {
-      f32x4 x0, x1;
+      f32x4 x0, x1, y0, y1;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         x0[r] = ok[2 * pr][r] * egi[2 * pr][r];
         x1[r] = ok[2 * pr + 1][r] * egi[2 * pr + 1][r];
+        y0[r] = ok[2 * pr][r] * egr[2 * pr][r];
+        y1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
       }
-      const bf16x8 bp = pack8(x0, x1);
+      bp[qb][pr] = pack8(x0, x1);
+      bpr[qb][pr] = pack8(y0, y1);
+    }
+  }
+  if (TK == 32) {
+    // second stage of the slot-branch tiles: the state / row tiles of the value side
+    __syncthreads();
+    load_state_tile(tC, p.hvc, p.hseg_v);
+    load_rows_tile(tD, p.v);
+    __syncthreads();
+  }
+  // ---- phase 1b: slot read ----------------------------------------------------------------------
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const int Q = qb0 + qb;
+    // inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        O[db][qb] = mfma16(lds_frag_tr(Vb0, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bp, O[db][qb]);
-    }
-    // slot read, intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m]))
-    bf16x8 bpr[2];
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
-      f32x4 x0, x1;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        x0[r] = ok[2 * pr][r] * egr[2 * pr][r];
-        x1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
-      }
-      bpr[pr] = pack8(x0, x1);
-    }
+        O[db][qb] = mfma16(lds_frag_tr(tC, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bp[qb][pr], O[db][qb]);
+    // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
     bf16x8 bAv[2];
     {
       f32x4 av[4];
@@ -643,24 +684,10 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       for (int jb = 0; jb < 4; ++jb) {
         av[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (jb <= Q) {
-          const int jrow = 16 * jb + l16;
 #pragma unroll
           for (int pr = 0; pr < 2; ++pr) {
-            bf16x8 se;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              const int m0 = 32 * pr + 16 * half + 4 * kb;
-              const float4 gj = lds_ld_f4(gcR + jrow * GLD + m0);
-              float4 gr4 = make_float4(0.f, 0.f, 0.f, 0.f);
-              if (Q > 0) gr4 = lds_ld_f4(gcR + rref * GLD + m0);
-              const bf16x4 sj = *reinterpret_cast<const NHA_LDS bf16x4*>(sR + jrow * SLD + m0);
-              const float gv[4] = {gj.x, gj.y, gj.z, gj.w};
-              const float grv[4] = {gr4.x, gr4.y, gr4.z, gr4.w};
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                se[4 * half + e] = (__bf16)((float)sj[e] * fexp(fminf(grv[e] - gv[e], DECAY_CLAMP)));
-            }
-            av[jb] = mfma16(se, bpr[pr], av[jb]);
+            const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(SEb + (seb_base(Q) + 2 * jb + pr) * 512 + lane * 8);
+            av[jb] = mfma16(se, bpr[qb][pr], av[jb]);
           }
           if (jb == Q) {
 #pragma unroll
@@ -673,16 +700,15 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       bAv[1] = pack8(av[2], av[3]);
     }
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
+    for (int pr = 0; pr < 2; ++pr)
       if (2 * pr <= Q) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          O[db][qb] = mfma16(lds_frag_tr(Vb1, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bAv[pr], O[db][qb]);
+          O[db][qb] = mfma16(lds_frag_tr(tD, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bAv[pr], O[db][qb]);
       }
-    }
   }
 
-  // ---- phase 2: sliding window, streamed in 64-key tiles --------------------------------------
+  // ---- phase 2: sliding window, streamed in TK-key tiles --------------------------------------
   bf16x8 qs[RQB][KS];
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -696,12 +722,12 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     }
   }
   __syncthreads();   // every wave is done with the slot-branch tiles
-  tile_r2l<D, NTHR>(Kb0, rk, tid);
-  tile_r2l<D, NTHR>(Vb0, rv, tid);
+  tile_r2l<TK, D, NTHR>(Kb0, rk, tid);
+  tile_r2l<TK, D, NTHR>(Vb0, rv, tid);
   if (ntiles > 1) issue_window(1);
   __syncthreads();
 
-  // lazy rescaling: the running reference max only moves when a tile exceeds it by more than
+  // lazy rescaling: the running reference max only moves when a half tile exceeds it by more than
   // 2^RESCALE_LOG2 in probability units, so O is rescaled a handful of times per chunk
   constexpr float RESCALE_LOG2 = 8.f;
   const float thr = RESCALE_LOG2 / cs;
@@ -720,9 +746,10 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     const int cur = i & 1;
     const lbf16* Kt = cur ? Kb1 : Kb0;
     const lbf16* Vt = cur ? Vb1 : Vb0;
-    const bool edge = (i == 0) || (p.wl >= 0 && 64 * i + 63 > p.wl);
+    const int xbase = 64 - TK * (i + 1);   // key offset of the tile's first key relative to the chunk start
+    const bool edge = (xbase + TK - 1 > 0) || (p.wl >= 0 && p.wl < TK * (i + 1) - 1);
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
+    for (int hf = 0; hf < NH; ++hf) {
       // S^T[key][q] for the 32 keys of this half: 2 key blocks x RQB query blocks, the
       // 2 * RQB accumulators advance together so consecutive MFMAs are independent
       f32x4 S[2][RQB];
@@ -749,7 +776,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
             const int y = 16 * (qb0 + qb) + l16;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int x = 32 * hf + 16 * kk + 4 * kb + r - 64 * i;   // key offset relative to the chunk start
+              const int x = xbase + 32 * hf + 16 * kk + 4 * kb + r;
               const bool ok = (x <= y) && (p.wl < 0 || x >= y - p.wl);
               if (!ok) S[kk][qb][r] = -INFINITY;
             }
@@ -805,8 +832,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       PROF_MARK(3)
     }
     if (i + 1 < ntiles) {
-      tile_r2l<D, NTHR>(cur ? Kb0 : Kb1, rk, tid);
-      tile_r2l<D, NTHR>(cur ? Vb0 : Vb1, rv, tid);
+      tile_r2l<TK, D, NTHR>(cur ? Kb0 : Kb1, rk, tid);
+      tile_r2l<TK, D, NTHR>(cur ? Vb0 : Vb1, rv, tid);
       if (i + 2 < ntiles) issue_window(i + 2);
     }
     PROF_MARK(4)
@@ -814,7 +841,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     PROF_MARK(5)
   }
 #ifdef NHA_PROF
-  if (blockIdx.x == 200 && blockIdx.y == 3 && lane == 0) {
+  if (blockIdx.y == 200 && blockIdx.x == 3 && lane == 0) {
     long long* dbg = (long long*)p.lse_gsa;
     for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
   }
@@ -843,38 +870,57 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   }
 }
 
-template <int D, int G, int NW>
+template <int D, int G, int NW, int TK>
 int launch_out(const MP& p, hipStream_t st) {
   static bool configured = false;
-  const size_t lds = OutSmem<D>::bytes;
+  const size_t lds = OutSmem<D, TK>::bytes;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G, NW, TK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
       set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
       return NHA_ERR_LAUNCH;
     }
     configured = true;
   }
-  hipLaunchKernelGGL((mfma_out_kernel<D, G, NW>), dim3(p.NT, p.H * (p.NG / G)), dim3(64 * NW), lds, st, p);
+  hipLaunchKernelGGL((mfma_out_kernel<D, G, NW, TK>), dim3(p.H * (p.NG / G), p.NT), dim3(64 * NW), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass)");
   return NHA_OK;
 }
 
 template <int D>
 int run_mfma(const MP& p, int phases, hipStream_t st) {
+  if (p.NT > 65535) {
+    set_error("nha_prefill_fwd(mfma): more than 65535 chunks (%d) in one call", p.NT);
+    return NHA_ERR_UNSUPPORTED;
+  }
   if (phases != 2) {
-    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT, p.H), dim3(256), 0, st, p);
+    static bool configured = false;
+    const size_t lds = (size_t)2 * BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) {
+        set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        return NHA_ERR_LAUNCH;
+      }
+      configured = true;
+    }
+    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H), dim3(256), lds, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
     hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
   }
   if (phases != 1) {
-    // G query heads of one kv-head share a workgroup; 8 waves (two per SIMD, 32 or 16 query rows
-    // each) when the group is large enough, else 4
-    const int G = (p.NG % 4 == 0) ? 4 : (p.NG % 2 == 0) ? 2 : 1;
-    if (G == 4) return launch_out<D, 4, 8>(p, st);
-    if (G == 2) return launch_out<D, 2, 8>(p, st);
-    return launch_out<D, 1, 4>(p, st);
+    // G query heads of one kv-head share a workgroup.  D <= 128: 64-key tiles, 8 waves of 32 (G = 4)
+    // or 16 (G = 2) query rows, two per SIMD; D = 256: 32-key tiles and 16-row waves to fit the
+    // register file and LDS
+    if constexpr (D <= 128) {
+      if (p.NG % 4 == 0) return launch_out<D, 4, 8, 64>(p, st);
+      if (p.NG % 2 == 0) return launch_out<D, 2, 8, 64>(p, st);
+      return launch_out<D, 1, 4, 64>(p, st);
+    } else {
+      if (p.NG % 2 == 0) return launch_out<D, 2, 8, 32>(p, st);
+      return launch_out<D, 1, 4, 32>(p, st);
+    }
   }
   return NHA_OK;
 }
@@ -884,7 +930,7 @@ static size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 }  // namespace
 
 bool prefill_mfma_supported(const NhaPrefillArgs* a) {
-  return a->dtype == NHA_DTYPE_BF16 && a->K == a->V && (a->K == 64 || a->K == 128) && a->M == MS;
+  return a->dtype == NHA_DTYPE_BF16 && a->K == a->V && (a->K == 64 || a->K == 128 || a->K == 256) && a->M == MS;
 }
 
 namespace {
@@ -937,7 +983,8 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
   p.wl = a->wl; p.shift = a->shift; p.scale = a->scale;
   hipStream_t st = (hipStream_t)a->stream;
   if (a->K == 64) return run_mfma<64>(p, a->phases, st);
-  return run_mfma<128>(p, a->phases, st);
+  if (a->K == 128) return run_mfma<128>(p, a->phases, st);
+  return run_mfma<256>(p, a->phases, st);
 }
 
 }  // namespace nha

@@ -26,7 +26,7 @@ def test_mfma_reference_grid():
             run_case(f"mfma_t{T}_b{B}_w{W} layer", d, wl=W, shift=0, dtype=BF, impl="mfma")
 
 
-@pytest.mark.parametrize("D,NG", [(128, 4), (128, 1), (128, 2), (128, 8), (64, 1), (64, 3)])
+@pytest.mark.parametrize("D,NG", [(128, 4), (128, 1), (128, 2), (128, 8), (64, 1), (64, 3), (256, 1), (256, 2), (256, 4)])
 def test_mfma_head_shapes_and_windows(D, NG):
     H = 2
     for li, (T, wl, shift) in enumerate([(200, 99, 100), (333, 100, 0), (130, -1, 0), (260, 255, 256), (70, 500, 0),
@@ -44,6 +44,18 @@ def test_mfma_varlen():
         d = prefill_inputs(700 + li, 1, T, H * NG, H, D, D, 64, dtype=BF, with_state=True, N=len(lens))
         run_case(f"mfma varlen{li} shifted", d, wl=31, shift=32, dtype=BF, impl="mfma", cu=cu)
         run_case(f"mfma varlen{li} layer", d, wl=100, shift=0, dtype=BF, impl="mfma", cu=cu)
+
+
+def test_mfma_varlen_d256():
+    """Scaled-down version of the varlen benchmark config: H=4, D=256, M=64, W=512, random lengths,
+    per-sequence initial state ~ N(0, 0.1)."""
+    rng = np.random.default_rng(3)
+    lens = [int(x) for x in rng.integers(64, 700, size=6)] + [1, 65]
+    cu = [0] + list(np.cumsum(lens))
+    d = prefill_inputs(750, 1, cu[-1], 4, 4, 256, 256, 64, dtype=BF, with_state=True, N=len(lens), state_scale=0.1,
+                       qk_scale=256 ** -0.5, gate_div=1.0)
+    run_case("varlen d256 layer", d, wl=512, shift=0, dtype=BF, impl="mfma", cu=cu)
+    run_case("varlen d256 shifted", d, wl=511, shift=512, dtype=BF, impl="mfma", cu=cu)
 
 
 def test_mfma_slow_forgetting_gates():
