@@ -223,6 +223,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
     args = ap.parse_args()
@@ -234,6 +237,11 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the NHA ops have no CPU fallback)", file=sys.stderr)
         sys.exit(3)
+    if args.copy_calibration:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
     if args.only:
         res = bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else bench_decode(torch, args.warmup)
         print(json.dumps(res))

@@ -1,0 +1,335 @@
+"""NativeHybridAttention layer: the API shell of nha_fla/layers/nha.py:25-343 around chunk_nha.
+
+Constructor arguments, parameter names (q_proj, k_proj, v_proj, f_proj, g_norm, o_proj, optional
+q/k/v_conv1d), forward signature, return tuple and error behaviour follow the reference layer, so a
+checkpoint of the reference loads here.  The op underneath is the HIP chunk_nha; k/v/s/g are handed
+to it at the kv-head count (the reference repeats them to the q-head count first, :229-230).
+
+The reference takes RMSNorm, RotaryEmbedding, ShortConvolution, the feature maps, rms_norm_linear
+and the unpad helpers from flash-linear-attention, which is not vendored; they are restated here in
+plain PyTorch from their published behaviour (elementwise / projection glue around the hot path).
+Forward only: the op has no backward.
+"""
+from __future__ import annotations
+
+import warnings
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .ops import chunk_nha
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden_size: int, elementwise_affine: bool = True, eps: float = 1e-5, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype)) if elementwise_affine else None
+        self.register_parameter("bias", None)
+
+    def forward(self, x):
+        y = x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + self.eps)
+        if self.weight is not None:
+            y = y * self.weight.float()
+        return y.to(x.dtype)
+
+
+def rms_norm_linear(x, norm_weight, norm_bias, linear_weight, linear_bias, eps: float = 1e-5):
+    """linear(rms_norm(x)) -- the fused epilogue of nha_fla/layers/nha.py:278."""
+    y = x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + eps)
+    if norm_weight is not None:
+        y = y * norm_weight.float()
+    if norm_bias is not None:
+        y = y + norm_bias.float()
+    return F.linear(y.to(linear_weight.dtype), linear_weight, linear_bias)
+
+
+class SwishFeatureMap(nn.Module):
+    def forward(self, x):
+        return F.silu(x)
+
+
+class ReLUFeatureMap(nn.Module):
+    def forward(self, x):
+        return F.relu(x)
+
+
+class T2RFeatureMap(nn.Module):
+    def __init__(self, head_dim: int, dot_dim: Optional[int] = None, bias: bool = False):
+        super().__init__()
+        self.layer = nn.Linear(head_dim, head_dim if dot_dim is None else dot_dim, bias=bias)
+
+    def forward(self, x):
+        return F.relu(self.layer(x))
+
+
+class RotaryEmbedding(nn.Module):
+    """Rotate-half RoPE over the whole head dim; positions restart at every cu_seqlens boundary."""
+
+    def __init__(self, dim: int, base: float = 10000.0):
+        super().__init__()
+        self.dim, self.base = dim, base
+
+    def _tables(self, pos: torch.Tensor, dtype):
+        inv = 1.0 / (self.base ** (torch.arange(0, self.dim, 2, device=pos.device, dtype=torch.float32) / self.dim))
+        fr = pos.float()[:, None] * inv[None, :]
+        return fr.cos().to(dtype), fr.sin().to(dtype)
+
+    def forward(self, q, k, seqlen_offset=0, cu_seqlens=None, max_seqlen=None):
+        B, T = q.shape[0], q.shape[1]
+        pos = torch.arange(T, device=q.device)
+        if cu_seqlens is not None:
+            cu = cu_seqlens.to(q.device).long()
+            seq = torch.bucketize(pos, cu[1:], right=True)
+            pos = pos - cu[seq]
+        pos = pos + seqlen_offset
+        cos, sin = self._tables(pos, q.dtype)                     # [T, dim/2]
+
+        def rot(x):
+            x1, x2 = x[..., : self.dim // 2], x[..., self.dim // 2: self.dim]
+            c, s = cos[None, :, None, :], sin[None, :, None, :]
+            out = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1)
+            return out if self.dim == x.shape[-1] else torch.cat([out, x[..., self.dim:]], dim=-1)
+
+        return rot(q), rot(k)
+
+
+class ShortConvolution(nn.Module):
+    """Depthwise causal conv1d (kernel_size taps) + optional SiLU, restarting at cu_seqlens boundaries."""
+
+    def __init__(self, hidden_size: int, kernel_size: int, bias: bool = False, activation: Optional[str] = "silu"):
+        super().__init__()
+        self.hidden_size, self.kernel_size, self.activation = hidden_size, kernel_size, activation
+        self.weight = nn.Parameter(torch.empty(hidden_size, 1, kernel_size).uniform_(-kernel_size ** -0.5, kernel_size ** -0.5))
+        self.bias = nn.Parameter(torch.zeros(hidden_size)) if bias else None
+
+    def forward(self, x, cache=None, output_final_state=False, cu_seqlens=None):
+        B, T, Dm = x.shape
+        xs = x.transpose(1, 2)
+        if cache is not None:
+            xs = torch.cat([cache.to(xs.dtype), xs], dim=-1)
+        else:
+            xs = F.pad(xs, (self.kernel_size - 1, 0))
+        if cu_seqlens is not None and cache is None:
+            # zero the taps that would reach into the previous packed sequence
+            pos = torch.arange(T, device=x.device)
+            cu = cu_seqlens.to(x.device).long()
+            local = pos - cu[torch.bucketize(pos, cu[1:], right=True)]
+            y = torch.zeros_like(x.transpose(1, 2))
+            xin = x.transpose(1, 2)
+            for tap in range(self.kernel_size):
+                back = self.kernel_size - 1 - tap
+                shifted = F.pad(xin, (back, 0))[..., :T]
+                y = y + shifted * (local >= back).to(x.dtype)[None, None, :] * self.weight[:, 0, tap][None, :, None]
+            if self.bias is not None:
+                y = y + self.bias[None, :, None]
+        else:
+            y = F.conv1d(xs, self.weight, self.bias, groups=Dm)
+        final = xs[..., -(self.kernel_size - 1):].contiguous() if output_final_state else None
+        if self.activation in ("silu", "swish"):
+            y = F.silu(y)
+        return y.transpose(1, 2), final
+
+
+def get_unpad_data(attention_mask: torch.Tensor):
+    seqlens = attention_mask.sum(-1, dtype=torch.int32)
+    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    cu = F.pad(torch.cumsum(seqlens, 0, dtype=torch.int32), (1, 0))
+    return indices, cu, int(seqlens.max())
+
+
+def pad_input(x: torch.Tensor, indices: torch.Tensor, batch: int, seqlen: int):
+    out = x.new_zeros(batch * seqlen, *x.shape[1:])
+    out[indices] = x
+    return out.view(batch, seqlen, *x.shape[1:])
+
+
+class NativeHybridAttention(nn.Module):
+    """Drop-in for nha_fla.layers.nha.NativeHybridAttention (forward path)."""
+
+    def __init__(
+        self,
+        mode: str = 'chunk',
+        hidden_size: int = 1024,
+        expand_k: float = 1.,
+        expand_v: float = 1.,
+        num_heads: int = 4,
+        num_kv_heads: Optional[int] = None,
+        use_short_conv: bool = False,
+        conv_size: int = 4,
+        conv_bias: bool = False,
+        num_slots: Optional[int] = None,
+        elementwise_affine: Optional[bool] = True,
+        norm_eps: float = 1e-5,
+        gate_logit_normalizer: int = 8,
+        feature_map: str = 'swish',
+        use_output_gate: bool = False,
+        use_norm: bool = True,
+        fuse_norm: bool = True,
+        layer_idx: Optional[int] = None,
+        scale: Optional[float] = 1.,
+        window_size: int = 2048,
+        rope_theta: float = 10000.,
+        max_position_embeddings: Optional[int] = None,
+        gsa_aux_loss_enable: bool = False,
+        gsa_aux_loss_coeff: Optional[float] = None,
+        gsa_aux_loss_target_ratio: float = 1.0,
+        gsa_kv_shift: int = 0,
+        **kwargs,
+    ):
+        super().__init__()
+        self.mode = mode
+        self.hidden_size = hidden_size
+        self.expand_k, self.expand_v = expand_k, expand_v
+        self.num_heads = num_heads
+        self.num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        self.num_kv_groups = self.num_heads // self.num_kv_heads
+        self.key_dim = int(hidden_size * expand_k)
+        self.value_dim = int(hidden_size * expand_v)
+        self.key_dim_per_group = self.key_dim // self.num_kv_groups
+        self.value_dim_per_group = self.value_dim // self.num_kv_groups
+        self.head_k_dim = self.key_dim // self.num_heads
+        self.head_v_dim = self.value_dim // self.num_heads
+        self.use_short_conv, self.conv_size, self.conv_bias = use_short_conv, conv_size, conv_bias
+        self.gate_logit_normalizer = gate_logit_normalizer
+        self.use_output_gate, self.use_norm, self.fuse_norm = use_output_gate, use_norm, fuse_norm
+        self.scale = scale
+        self.window_size = window_size
+        self.rope_theta = rope_theta
+        self.max_position_embeddings = max_position_embeddings
+        self.gsa_aux_loss_enable = gsa_aux_loss_enable
+        self.gsa_aux_loss_coeff = gsa_aux_loss_coeff
+        self.gsa_aux_loss_target_ratio = gsa_aux_loss_target_ratio
+        self.gsa_kv_shift = gsa_kv_shift
+        self.num_slots = self.head_k_dim if num_slots is None else num_slots
+        self.layer_idx = layer_idx
+        self.norm_eps = norm_eps
+        if layer_idx is None:
+            warnings.warn(
+                f"Instantiating {self.__class__.__name__} without passing `layer_idx` is not recommended and will "
+                "to errors during the forward call, if caching is used. Please make sure to provide a `layer_idx` "
+                "when creating this class.",
+            )
+        self.register_module('feature_map', None)
+        if feature_map == 'swish':
+            self.feature_map = SwishFeatureMap()
+        elif feature_map == 'relu':
+            self.feature_map = ReLUFeatureMap()
+        elif feature_map == 't2r':
+            self.feature_map = T2RFeatureMap(self.head_k_dim, self.head_k_dim)
+        else:
+            raise NotImplementedError(f"Feature map `{feature_map}` is not supported now.")
+        self.q_proj = nn.Linear(self.hidden_size, self.key_dim, bias=False)
+        self.k_proj = nn.Linear(self.hidden_size, self.key_dim_per_group, bias=False)
+        self.v_proj = nn.Linear(self.hidden_size, self.value_dim_per_group, bias=False)
+        self.f_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.num_slots, bias=False)
+        if use_short_conv:
+            self.q_conv1d = ShortConvolution(self.key_dim, conv_size, bias=conv_bias, activation='silu')
+            self.k_conv1d = ShortConvolution(self.key_dim_per_group, conv_size, bias=conv_bias, activation='silu')
+            self.v_conv1d = ShortConvolution(self.value_dim_per_group, conv_size, bias=conv_bias, activation='silu')
+        self.g_norm = RMSNorm(self.hidden_size, elementwise_affine, eps=norm_eps, dtype=torch.float32)
+        self.o_proj = nn.Linear(self.value_dim, self.hidden_size, bias=False)
+        self.rotary = RotaryEmbedding(dim=self.head_k_dim, base=self.rope_theta)
+
+    @torch.no_grad()
+    def forward(
+        self,
+        hidden_states: torch.Tensor,
+        attention_mask: Optional[torch.Tensor] = None,
+        past_key_values=None,
+        use_cache: Optional[bool] = False,
+        output_attentions: Optional[bool] = False,
+        **kwargs,
+    ) -> Tuple[torch.Tensor, None, object]:
+        if attention_mask is not None:
+            assert len(attention_mask.shape) == 2, (
+                "Expected attention_mask as a 0-1 matrix with shape [batch_size, seq_len] "
+                "for padding purposes (0 indicating padding). "
+                "Arbitrary attention masks of shape [batch_size, seq_len, seq_len] are not allowed."
+            )
+        batch_size, q_len, _ = hidden_states.shape
+        last_state = None
+        if past_key_values is not None and len(past_key_values) > self.layer_idx:
+            last_state = past_key_values[self.layer_idx]
+        recurrent_state = last_state['recurrent_state'] if last_state is not None else None
+        if q_len == 1 and last_state is not None:
+            raise NotImplementedError(
+                "Single-token decode for the NHA layer was removed: its only "
+                "implementation called the never-released fused_recurrent_nha_step. "
+                "Run the chunk path (prefill-style) instead."
+            )
+        mode = self.mode
+        cu_seqlens = kwargs.get('cu_seqlens')
+        max_seqlen = kwargs.get('max_seqlen')
+        indices = None
+        if attention_mask is not None:
+            indices, cu_seqlens, max_seqlen = get_unpad_data(attention_mask[:, -q_len:])
+            hidden_states = hidden_states.reshape(batch_size * q_len, -1)[indices].unsqueeze(0)
+        conv_state_q = conv_state_k = conv_state_v = None
+        if self.use_short_conv:
+            if last_state is not None:
+                conv_state_q, conv_state_k, conv_state_v = last_state['conv_state']
+            q, conv_state_q = self.q_conv1d(self.q_proj(hidden_states), conv_state_q, use_cache, cu_seqlens)
+            k, conv_state_k = self.k_conv1d(self.k_proj(hidden_states), conv_state_k, use_cache, cu_seqlens)
+            v, conv_state_v = self.v_conv1d(self.v_proj(hidden_states), conv_state_v, use_cache, cu_seqlens)
+        else:
+            q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+        f = self.f_proj(hidden_states)
+        q = q.unflatten(-1, (-1, self.head_k_dim))
+        k = k.unflatten(-1, (-1, self.head_k_dim))
+        v = v.unflatten(-1, (-1, self.head_v_dim))
+        f = f.unflatten(-1, (-1, self.num_slots))
+        if self.feature_map is not None:
+            q_gsa, k_gsa = self.feature_map(q), self.feature_map(k)
+        else:
+            q_gsa, k_gsa = q, k
+        v = F.silu(v)
+        f = F.logsigmoid(f) / self.gate_logit_normalizer
+        s = (1 - f.exp()).to(f.dtype)
+        g = f
+        seqlen_offset = 0
+        if last_state is not None and 'seqlen_offset' in last_state:
+            seqlen_offset = last_state['seqlen_offset']
+        # rotary on the kv-head keys: identical across the heads of a group, so rotating before the
+        # (implicit, in-kernel) group expansion equals the reference's repeat-then-rotate
+        q_swa, k_swa = self.rotary(q, k, seqlen_offset=seqlen_offset, cu_seqlens=cu_seqlens)
+        if mode == 'chunk':
+            output, lse_swa, lse_gsa = chunk_nha(
+                q_swa=q_swa, k_swa=k_swa, q_gsa=q_gsa, k_gsa=k_gsa, v=v, s=s, g=g,
+                scale=self.scale,
+                window_size_left=self.window_size,
+                window_size_right=0,
+                head_first=False,
+                gsa_kv_shift=self.gsa_kv_shift,
+                cu_seqlens=cu_seqlens,
+                max_seqlen=max_seqlen,
+            )
+            if self.training:
+                lse_max = torch.maximum(lse_swa, lse_gsa)
+                w_swa, w_gsa = torch.exp(lse_swa - lse_max), torch.exp(lse_gsa - lse_max)
+                self._store_compression_stats(w_swa, w_gsa)
+        else:
+            raise NotImplementedError(f"Not supported mode `{mode}`.")
+        if past_key_values is not None:
+            past_key_values.update(
+                recurrent_state=recurrent_state,
+                conv_state=(conv_state_q, conv_state_k, conv_state_v) if self.use_short_conv else None,
+                layer_idx=self.layer_idx,
+                offset=q_len,
+            )
+        o = output[:, :, :, :self.head_v_dim].flatten(-2)
+        o = rms_norm_linear(F.silu(o), self.g_norm.weight, self.g_norm.bias, self.o_proj.weight, self.o_proj.bias,
+                            eps=self.norm_eps)
+        if attention_mask is not None:
+            o = pad_input(o.squeeze(0), indices, batch_size, q_len)
+        return o, None, past_key_values
+
+    @torch.no_grad()
+    def _store_compression_stats(self, w_swa: torch.Tensor, w_gsa: torch.Tensor):
+        """GSA vs SWA share of the softmax mass (nha_fla/layers/nha.py:288-298)."""
+        gsa_ratio = (w_gsa / (w_swa + w_gsa)).mean().item()
+        if not hasattr(self, '_compression_stats'):
+            self._compression_stats = []
+        self._compression_stats.append({'gsa_ratio': gsa_ratio, 'swa_ratio': 1.0 - gsa_ratio})
