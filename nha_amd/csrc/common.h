@@ -81,6 +81,8 @@ void set_error(const char* fmt, ...);
 
 int decode_step_impl(const NhaDecodeArgs* a);
 int decode_advance_impl(int32_t* count, int32_t B, void* stream);
+bool decode_mfma_supported(const NhaDecodeArgs* a);
+int decode_mfma_impl(const NhaDecodeArgs* a);
 size_t prefill_simple_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_simple_impl(const NhaPrefillArgs* a);
 bool prefill_mfma_supported(const NhaPrefillArgs* a);

@@ -7,6 +7,7 @@
 // :305/:416, fused softmax over [M | W] :342-349, rotate-half pairing :309-329) and :47-149
 // (caller-supplied window logits).  fp32 math on bf16/fp32 loads, state fp32.
 #include "common.h"
+#include <stdlib.h>
 
 namespace nha {
 
@@ -683,9 +684,13 @@ int decode_step_impl(const NhaDecodeArgs* a) {
     set_error("nha_decode_step: cos/sin strides must be multiples of 8 elements");
     return NHA_ERR_UNSUPPORTED;
   }
+  // matrix-core kernel for the common bf16 shapes (NHA_DECODE_VALU=1 keeps the VALU kernels, for
+  // comparisons)
+  static const bool valu_only = getenv("NHA_DECODE_VALU") != nullptr;
+  if (!valu_only && decode_mfma_supported(a)) return decode_mfma_impl(a);
   int G = 1;
   while (G < NG) G <<= 1;
-  // two kernels: the two-sweep kernel keeps all window logits in LDS (fewest VALU operations per
+  // two VALU kernels: the two-sweep kernel keeps all window logits in LDS (fewest VALU operations per
   // row); the streaming kernel needs no per-row LDS and serves windows too long for that
   const bool fits_lds = lds_floats(G, a->K, a->V, a->M, a->W) * sizeof(float) <= 40 * 1024;
   if (a->mode != NHA_DECODE_LOGITS && a->K == a->V && !fits_lds) {
