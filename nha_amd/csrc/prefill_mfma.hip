@@ -441,12 +441,43 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   if (p.wl >= 0 && c0 - p.wl > bos) lowest = c0 - p.wl;
   const int ntiles = (c0 + 64 - lowest + TK - 1) / TK;
   TileRegs<TK, D, NTHR> rk, rv;
+  // Tile boundaries are multiples of TK away from bos, so a window tile never starts before its
+  // sequence; only the tiles over the chunk's own rows can run past eos.  Every tile that ends at
+  // or before eos is loaded unconditionally from a wave-uniform base plus per-thread 32-bit
+  // offsets that never change (one scalar subtraction per tile instead of per-load 64-bit
+  // address arithmetic); the others take the row-checked path.
+  constexpr int NPC = TK * D / 8 / NTHR;   // 16-byte pieces per thread and tile
+  uint32_t goff[NPC], loff[NPC];
+#pragma unroll
+  for (int u = 0; u < NPC; ++u) {
+    const int c = tid + NTHR * u;
+    const int row = c / (D / 8), col = (c % (D / 8)) * 8;
+    goff[u] = (uint32_t)row * (uint32_t)(H * D) + col;
+    loff[u] = row * (D + 16) + col;
+  }
   auto issue_window = [&](int i) {
     const int64_t grow0 = (int64_t)c0 + 64 - TK * (i + 1);
-    int vhi = eos - (int)grow0;
-    vhi = vhi < 0 ? 0 : (vhi > TK ? TK : vhi);
-    tile_g2r<TK, D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
-    tile_g2r<TK, D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    if (grow0 + TK > eos) {
+      int vhi = eos - (int)grow0;
+      vhi = vhi < 0 ? 0 : (vhi > TK ? TK : vhi);
+      tile_g2r<TK, D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+      tile_g2r<TK, D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
+    } else {
+      const bf16_t* kb_ = p.k_swa + (grow0 * H + h) * D;
+      const bf16_t* vb_ = p.v + (grow0 * H + h) * D;
+#pragma unroll
+      for (int u = 0; u < NPC; ++u) {
+        rk.r[u] = *reinterpret_cast<const uint4*>(kb_ + goff[u]);
+        rv.r[u] = *reinterpret_cast<const uint4*>(vb_ + goff[u]);
+      }
+    }
+  };
+  auto stage_window = [&](lbf16* kdst, lbf16* vdst) {
+#pragma unroll
+    for (int u = 0; u < NPC; ++u) {
+      lds_st16(kdst + loff[u], rk.r[u]);
+      lds_st16(vdst + loff[u], rv.r[u]);
+    }
   };
 
   // ---- phase 0: slot-branch operands -> LDS --------------------------------------------------
@@ -722,8 +753,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     }
   }
   __syncthreads();   // every wave is done with the slot-branch tiles
-  tile_r2l<TK, D, NTHR>(Kb0, rk, tid);
-  tile_r2l<TK, D, NTHR>(Vb0, rv, tid);
+  stage_window(Kb0, Vb0);
   if (ntiles > 1) issue_window(1);
   __syncthreads();
 
@@ -790,7 +820,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       for (int qb = 0; qb < RQB; ++qb) {
         float x = fmaxf(fmaxf(S[0][qb][0], S[0][qb][1]), fmaxf(S[0][qb][2], S[0][qb][3]));
         x = fmaxf(x, fmaxf(fmaxf(S[1][qb][0], S[1][qb][1]), fmaxf(S[1][qb][2], S[1][qb][3])));
-        x = max_over_rows(x);
+        // the lane's own 8 keys suffice to decide (some lane exceeds the threshold iff the column
+        // maximum does); the cross-lane maximum is only formed on the rare rescale path
         rmax[qb] = x;
         need |= x > mrun[qb] + thr;
       }
@@ -798,7 +829,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       if (__any(need)) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) {
-          const float mnew = fmaxf(mrun[qb], rmax[qb]);
+          const float mnew = fmaxf(mrun[qb], max_over_rows(rmax[qb]));
           const float alpha = fexp2((mrun[qb] - mnew) * cs);
           mrun[qb] = mnew;
           lg[qb] *= alpha;
@@ -832,8 +863,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       PROF_MARK(3)
     }
     if (i + 1 < ntiles) {
-      tile_r2l<TK, D, NTHR>(cur ? Kb0 : Kb1, rk, tid);
-      tile_r2l<TK, D, NTHR>(cur ? Vb0 : Vb1, rv, tid);
+      stage_window(cur ? Kb0 : Kb1, cur ? Vb0 : Vb1);
+      PROF_MARK(6)
       if (i + 2 < ntiles) issue_window(i + 2);
     }
     PROF_MARK(4)

@@ -75,10 +75,13 @@ def test_decode_grid(dtype):
 
 
 def test_decode_long_window_streaming_kernel():
-    """A window too long for the logits-in-LDS kernel takes the single-pass streaming kernel."""
+    """Long windows: the matrix-core kernel (bf16, M == 64, pre-rotated query) and, for the other
+    cases, the single-pass streaming kernel that serves windows too long for logits in LDS."""
     from nha_amd import fused_recurrent_nha_decode
-    for dtype, NG, W, K, rot in ((torch.bfloat16, 4, 3000, 128, False), (torch.float32, 2, 5000, 64, True)):
-        d = decode_inputs(77, 2, 2, NG, K, K, 64, W, dtype)
+    for dtype, NG, W, K, M, rot in ((torch.bfloat16, 4, 3000, 128, 64, False), (torch.bfloat16, 2, 3000, 128, 32, False),
+                                    (torch.bfloat16, 8, 2500, 64, 64, False), (torch.float32, 2, 5000, 64, 64, True)):
+        print("case", dtype, NG, W, K, M, rot, flush=True)
+        d = decode_inputs(77, 2, 2, NG, K, K, M, W, dtype)
         c = {k: v.cuda() for k, v in d.items()}
         if rot:
             o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sw_k_raw"],
