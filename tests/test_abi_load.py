@@ -25,10 +25,24 @@ def test_library_loads_and_exports_header_symbols():
     assert lib.nha_abi_version() == _lib.ABI_VERSION
 
 
-def test_struct_sizes_match_the_header():
-    # a tiny C program would be the strict check; here: field count and pointer-size sanity
-    assert C.sizeof(_lib.NhaPrefillArgs) == 18 * 8 + 8 + 13 * 4 + 4 + 8  # ptrs, size_t, ints, scale, stream
-    assert C.sizeof(_lib.NhaDecodeArgs) % 8 == 0
+def test_struct_sizes_match_the_header(tmp_path):
+    """sizeof and the offsets of the ctypes mirrors against the C compiler's view of the header."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    probes = [("NhaPrefillArgs", f) for f in ("q_swa", "scratch_bytes", "T_tot", "phases", "scale", "stream")]
+    probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream")]
+    src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
+           'printf("%zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs));']
+    src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
+    src += ['return 0; }']
+    cfile = tmp_path / "probe.c"
+    cfile.write_text("\n".join(src))
+    exe = tmp_path / "probe"
+    subprocess.run(["gcc", "-I", os.path.join(root, "include"), str(cfile), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) == C.sizeof(_lib.NhaPrefillArgs) and int(out[1]) == C.sizeof(_lib.NhaDecodeArgs)
+    for (t, f), off in zip(probes, out[2:]):
+        assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 
 def test_argument_validation_without_gpu():

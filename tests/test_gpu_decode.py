@@ -118,7 +118,8 @@ def test_decode_state_aliasing_and_errors():
                                    cos=c["cos"], sin=c["sin"])
 
 
-@pytest.mark.parametrize("NG,K,M,W", [(4, 128, 64, 48), (1, 64, 16, 8), (8, 64, 80, 33)])
+@pytest.mark.parametrize("NG,K,M,W", [(4, 128, 64, 48), (1, 64, 16, 8), (8, 64, 80, 33), (2, 64, 64, 300), (8, 128, 64, 130),
+                                      (1, 128, 64, 1)])
 def test_ring_decode_steps(NG, K, M, W):
     """Consecutive ring-buffer steps from random fill levels == the oracle's ring recurrence."""
     from nha_amd import NHARingState, ring_decode_step
@@ -132,7 +133,7 @@ def test_ring_decode_steps(NG, K, M, W):
     st.ring_kg.copy_(randn(gen, B, W, H, K, dtype=dtype))
     st.ring_v.copy_(randn(gen, B, W, H, V, dtype=dtype))
     st.ring_g.copy_((F.logsigmoid(torch.randn(B, W, H, M, generator=gen)) / 8).to(dtype))
-    counts = torch.tensor([0, W - 2, 5 * W + 3], dtype=torch.int32)
+    counts = torch.tensor([0, max(W - 2, 0), 5 * W + 3], dtype=torch.int32)
     st.count.copy_(counts)
     ref = dict(hk=st.hk.cpu().double(), hv=st.hv.cpu().double(),
                rings=tuple(x.cpu().double() for x in (st.ring_k, st.ring_kg, st.ring_v, st.ring_g)),
