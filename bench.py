@@ -27,6 +27,16 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
 DECODE = dict(B=128, HQ=32, H=8, D=128, M=64, W=1024, steps=256)
+# the other prefill shapes of the reference's configurations (parity-test cases; `--workload NAME`
+# times one of them with the same method as the headline).  wl/shift default to the shifted
+# convention (W-1, W); "layer" = (W, 0).  cfg3 packs sequences of 64..4096 tokens into 32768.
+WORKLOADS = dict(
+    headline=PREFILL,
+    cfg2=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0),
+    cfg2_shifted=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512),
+    cfg3=dict(B=1, T=32768, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0, varlen=True),
+    cfg5=dict(B=2, T=16384, HQ=32, H=8, D=128, M=64, W=2048),
+)
 
 
 def w_eff(T, W):
@@ -37,6 +47,19 @@ def prefill_flops(B, T, HQ, H, D, M, W):
     """Algorithmic (recurrent-form) flops: slot logits + slot read per q-head, window QK^T + PV
     per q-head over the in-window keys, slot write per kv-head."""
     return B * T * HQ * (2 * (D * M + M * D) + 2 * w_eff(T, W) * (D + D)) + B * T * H * 2 * (D * M + M * D)
+
+
+def workload_lengths(torch, cfg):
+    """Sequence lengths of a workload: B equal sequences, or (varlen) draws of 64..4096 tokens
+    until T is filled, the last one truncated."""
+    if not cfg.get("varlen"):
+        return [cfg["T"]] * cfg["B"]
+    gen = torch.Generator().manual_seed(0)
+    lens = []
+    while sum(lens) < cfg["T"]:
+        lens.append(int(torch.randint(64, 4097, (1,), generator=gen)))
+    lens[-1] -= sum(lens) - cfg["T"]
+    return lens
 
 
 def decode_bytes(B, HQ, H, D, M, W):
@@ -66,28 +89,30 @@ def make_prefill_inputs(torch, cfg, device, seed=0, B=None, T=None):
     return [x.to(device) for x in (q2, k2, q, k, v, s, g)]
 
 
-def bench_prefill(torch, steps, warmup):
+def bench_prefill(torch, steps, warmup, cfg=PREFILL):
     import numpy as np
     from nha_amd import _lib
     from nha_amd.ops import prefill_tables, _ptr
-    cfg = PREFILL
     dev = torch.device("cuda:0")
     B, T, HQ, H, D, M, W = (cfg[k] for k in ("B", "T", "HQ", "H", "D", "M", "W"))
+    wl, shift = cfg.get("wl", W - 1), cfg.get("shift", W)
+    lens = workload_lengths(torch, cfg)
     xs = [x.reshape(B * T, *x.shape[2:]).contiguous() for x in make_prefill_inputs(torch, cfg, dev)]
-    cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)
+    cu_host = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = len(lens)
     cu_d, idx_d, off_d, NT = prefill_tables(cu_host, dev)
     lib = _lib.load()
     o = torch.empty(B * T, HQ, D, dtype=torch.bfloat16, device=dev)
     lse_s = torch.empty(B * T, HQ, dtype=torch.float32, device=dev)
     lse_g = torch.empty(B * T, HQ, dtype=torch.float32, device=dev)
-    hkt = torch.empty(B, H, D, M, dtype=torch.float32, device=dev)
-    hvt = torch.empty(B, H, M, D, dtype=torch.float32, device=dev)
+    hkt = torch.empty(N, H, D, M, dtype=torch.float32, device=dev)
+    hvt = torch.empty(N, H, M, D, dtype=torch.float32, device=dev)
     a = _lib.NhaPrefillArgs()
     a.q_swa, a.k_swa, a.q_gsa, a.k_gsa, a.v, a.s, a.g = (_ptr(x) for x in xs)
     a.o, a.lse_swa, a.lse_gsa, a.hkt, a.hvt = _ptr(o), _ptr(lse_s), _ptr(lse_g), _ptr(hkt), _ptr(hvt)
     a.cu_seqlens, a.chunk_indices, a.chunk_offsets = _ptr(cu_d), _ptr(idx_d), _ptr(off_d)
-    a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = B * T, B, NT, HQ, H, D, D, M
-    a.wl, a.shift, a.dtype, a.impl, a.scale = W - 1, W, _lib.NHA_DTYPE_BF16, _lib.NHA_IMPL_MFMA, D ** -0.5
+    a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = B * T, N, NT, HQ, H, D, D, M
+    a.wl, a.shift, a.dtype, a.impl, a.scale = wl, shift, _lib.NHA_DTYPE_BF16, _lib.NHA_IMPL_MFMA, D ** -0.5
     stream = torch.cuda.current_stream(dev)
     a.stream = stream.cuda_stream
     nbytes = lib.nha_prefill_scratch_bytes(C.byref(a))
@@ -120,7 +145,7 @@ def bench_prefill(torch, steps, warmup):
         t_out += ev[1].elapsed_time(ev[2]) * 1e-3
     t_state /= steps
     t_out /= steps
-    flops = prefill_flops(B, T, HQ, H, D, M, W)
+    flops = sum(prefill_flops(1, L, HQ, H, D, M, wl + 1) for L in lens)
     # the output pass carries everything but the slot write (the state pass's flops)
     flops_out = flops - B * T * H * 2 * (D * M + M * D)
     return dict(tokens_per_s=B * T / wall, ms_per_step=wall * 1e3, t_state_ms=t_state * 1e3, t_out_ms=t_out * 1e3,
@@ -228,6 +253,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="time the prefill of another of the reference's configurations and print its raw numbers")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path shards by sequence / kv-head with no communication and "
@@ -242,6 +269,14 @@ def main():
         b = torch.empty_like(a)
         b.copy_(a)
         torch.cuda.synchronize()
+    if args.workload:
+        cfg = WORKLOADS[args.workload]
+        res = bench_prefill(torch, args.steps, args.warmup, cfg)
+        res["workload"] = {k: v for k, v in cfg.items()}
+        res["min_bytes"] = 2 * cfg["B"] * cfg["T"] * (cfg["HQ"] * 3 * cfg["D"] + cfg["H"] * (3 * cfg["D"] + 2 * cfg["M"]))
+        res["min_bytes_gbs"] = res["min_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9
+        print(json.dumps(res))
+        return
     if args.only:
         res = bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else bench_decode(torch, args.warmup)
         print(json.dumps(res))
@@ -272,7 +307,7 @@ def main():
                      "whole_op_tflops": pf["whole_op_tflops"], "algorithmic_flop": pf["flops"]},
         "decode": {"metric": "decode step us @B=128", "value": dc["us_per_step"], "unit": "us/step",
                    "higher_is_better": False,
-                   "roofline": {"bound": "hbm", "kernel": "decode_kernel<bf16,4>", "achieved": dc["achieved_gbs"],
+                   "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel<128,4,2>", "achieved": dc["achieved_gbs"],
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
                                 "traffic": None, "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
         "cpu_baseline": cpu,

@@ -363,9 +363,11 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
 // output pass
 #ifdef NHA_PROF
 #define PROF_DECL long long pt_[8] = {0,0,0,0,0,0,0,0}; long long pl_ = __builtin_amdgcn_s_memtime();
+#define PROF_STAGE(k) { __builtin_amdgcn_sched_barrier(0); ps_[k] = __builtin_amdgcn_s_memtime(); __builtin_amdgcn_sched_barrier(0); }
 #define PROF_MARK(k) { __builtin_amdgcn_sched_barrier(0); long long n_ = __builtin_amdgcn_s_memtime(); pt_[k] += n_ - pl_; pl_ = n_; }
 #else
 #define PROF_DECL
+#define PROF_STAGE(k)
 #define PROF_MARK(k)
 #endif
 // ==========================================================================================
@@ -480,62 +482,115 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     }
   };
 
+#ifdef NHA_PROF
+  long long ps_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+  PROF_STAGE(0)
   // ---- phase 0: slot-branch operands -> LDS --------------------------------------------------
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
   const int64_t grow_s = (int64_t)c0 - p.shift;
-  // true chunk-start state (segment-local state + decayed segment-start state) as a bf16 tile
-  auto load_state_tile = [&](lbf16* dst, const bf16_t* hloc, const float* hseg) {
+  // Every global load of this phase is issued before the first result is used, so the phase costs
+  // one memory latency, not one per tile.
+  constexpr int NPS = BT * D / 8 / NTHR;   // 16-byte pieces per thread of a 64-row tile
+  struct StateRegs {
+    uint4 lk[NPS];        // segment-local state, bf16
+    float4 k0[NPS], k1[NPS];   // segment-start state, fp32
+    float dc[NPS];        // decay from the segment start to the chunk start
+  };
+  // true chunk-start state = segment-local state + decayed segment-start state
+  auto issue_state = [&](StateRegs& r, const bf16_t* hloc, const float* hseg) {
     const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
 #pragma unroll
-    for (int u = 0; u < BT * D / 8 / NTHR; ++u) {
+    for (int u = 0; u < NPS; ++u) {
       const int c = tid + NTHR * u;
       const int row = c / (D / 8), col = (c % (D / 8)) * 8;
-      const float dc = p.dcum[cg * MS + row];
-      const uint4 lk = *reinterpret_cast<const uint4*>(hloc + (cg * MS + row) * D + col);
+      r.dc[u] = p.dcum[cg * MS + row];
+      r.lk[u] = *reinterpret_cast<const uint4*>(hloc + (cg * MS + row) * D + col);
       const float* sk = hseg + (sl * MS + row) * D + col;
-      const float4 k0 = *reinterpret_cast<const float4*>(sk), k1 = *reinterpret_cast<const float4*>(sk + 4);
-      const float kf[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-      const uint32_t lkw[4] = {lk.x, lk.y, lk.z, lk.w};
+      r.k0[u] = *reinterpret_cast<const float4*>(sk);
+      r.k1[u] = *reinterpret_cast<const float4*>(sk + 4);
+    }
+  };
+  auto commit_state = [&](lbf16* dst, const StateRegs& r) {
+#pragma unroll
+    for (int u = 0; u < NPS; ++u) {
+      const int c = tid + NTHR * u;
+      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
+      const float kf[8] = {r.k0[u].x, r.k0[u].y, r.k0[u].z, r.k0[u].w, r.k1[u].x, r.k1[u].y, r.k1[u].z, r.k1[u].w};
+      const uint32_t lkw[4] = {r.lk[u].x, r.lk[u].y, r.lk[u].z, r.lk[u].w};
       bf16x8 o8;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float a0 = __uint_as_float((e & 1) ? (lkw[e >> 1] & 0xffff0000u) : (lkw[e >> 1] << 16));
-        o8[e] = (__bf16)(a0 + kf[e] * dc);
+        o8[e] = (__bf16)(a0 + kf[e] * r.dc[u]);
       }
       *reinterpret_cast<NHA_LDS bf16x8*>(dst + row * LDT + col) = o8;
     }
+  };
+  auto load_state_tile = [&](lbf16* dst, const bf16_t* hloc, const float* hseg) {
+    StateRegs r;
+    issue_state(r, hloc, hseg);
+    commit_state(dst, r);
   };
   auto load_rows_tile = [&](lbf16* dst, const bf16_t* src) {
     TileRegs<BT, D, NTHR> t;
     tile_g2r<BT, D, NTHR>(t, src + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
     tile_r2l<BT, D, NTHR>(dst, t, tid);
   };
-  load_state_tile(tA, p.hkT, p.hseg_k);
-  load_rows_tile(tB, p.k_gsa);
-  if (TK == 64) {
-    load_state_tile(tC, p.hvc, p.hseg_v);
-    load_rows_tile(tD, p.v);
-  }
   {
+    StateRegs ra, rc;
+    TileRegs<BT, D, NTHR> tb, td;
+    constexpr int NG4 = 1024 / NTHR, NS8 = (512 + NTHR - 1) / NTHR;
+    float4 gx[NG4];
+    uint4 sx[NS8];
+    issue_state(ra, p.hkT, p.hseg_k);
+    tile_g2r<BT, D, NTHR>(tb, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
+    if (TK == 64) {
+      issue_state(rc, p.hvc, p.hseg_v);
+      tile_g2r<BT, D, NTHR>(td, p.v + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
+    }
     // gate cumsum table (fp32 [64][64]); rows past the sequence end are zero
     const float* gsrc = p.gc + cg * BT * MS;
-    for (int c4 = tid; c4 < 1024; c4 += NTHR) {
+#pragma unroll
+    for (int u = 0; u < NG4; ++u) {
+      const int c4 = tid + NTHR * u;
       const int j = c4 >> 4, m4 = (c4 & 15) * 4;
-      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (j < rows) x = *reinterpret_cast<const float4*>(gsrc + j * MS + m4);
-      *reinterpret_cast<NHA_LDS f32x4*>(gcR + j * GLD + m4) = (f32x4){x.x, x.y, x.z, x.w};
+      gx[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j < rows) gx[u] = *reinterpret_cast<const float4*>(gsrc + j * MS + m4);
     }
     // s rows of the slot branch (shifted)
-    for (int c8 = tid; c8 < 512; c8 += NTHR) {
+#pragma unroll
+    for (int u = 0; u < NS8; ++u) {
+      const int c8 = tid + NTHR * u;
       const int j = c8 >> 3, m8 = (c8 & 7) * 8;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (j >= vlo && j < rows) x = *reinterpret_cast<const uint4*>(p.s + ((grow_s + j) * H + h) * MS + m8);
-      lds_st16(sR + j * SLD + m8, x);
+      sx[u] = make_uint4(0, 0, 0, 0);
+      if (c8 < 512 && j >= vlo && j < rows) sx[u] = *reinterpret_cast<const uint4*>(p.s + ((grow_s + j) * H + h) * MS + m8);
+    }
+    issue_window(0);
+    PROF_STAGE(6)
+    __builtin_amdgcn_sched_barrier(0);
+    commit_state(tA, ra);
+    tile_r2l<BT, D, NTHR>(tB, tb, tid);
+    if (TK == 64) {
+      commit_state(tC, rc);
+      tile_r2l<BT, D, NTHR>(tD, td, tid);
+    }
+#pragma unroll
+    for (int u = 0; u < NG4; ++u) {
+      const int c4 = tid + NTHR * u;
+      const int j = c4 >> 4, m4 = (c4 & 15) * 4;
+      *reinterpret_cast<NHA_LDS f32x4*>(gcR + j * GLD + m4) = (f32x4){gx[u].x, gx[u].y, gx[u].z, gx[u].w};
+    }
+#pragma unroll
+    for (int u = 0; u < NS8; ++u) {
+      const int c8 = tid + NTHR * u;
+      const int j = c8 >> 3, m8 = (c8 & 7) * 8;
+      if (c8 < 512) lds_st16(sR + j * SLD + m8, sx[u]);
     }
   }
-  issue_window(0);
   __syncthreads();
+  PROF_STAGE(7)
   // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
   // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows
   // j of earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.
@@ -584,6 +639,20 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     for (int qb = 0; qb < RQB; ++qb) O[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
   bf16x8 bp[RQB][2], bpr[RQB][2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
 
+  // window-query fragments: requested here so that they land during the slot branch
+  bf16x8 qs[RQB][KS];
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const int irow = 16 * (qb0 + qb) + l16;
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      qs[qb][ks] = as_bf16x8(x);
+    }
+  }
+  PROF_STAGE(1)
   // ---- phase 1a: slot logits and the slot "tile" of the softmax, one 16-row block at a time ----
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -697,6 +766,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     load_rows_tile(tD, p.v);
     __syncthreads();
   }
+  PROF_STAGE(2)
   // ---- phase 1b: slot read ----------------------------------------------------------------------
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -739,23 +809,12 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       }
   }
 
+  PROF_STAGE(3)
   // ---- phase 2: sliding window, streamed in TK-key tiles --------------------------------------
-  bf16x8 qs[RQB][KS];
-#pragma unroll
-  for (int qb = 0; qb < RQB; ++qb) {
-    const int irow = 16 * (qb0 + qb) + l16;
-    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
-      qs[qb][ks] = as_bf16x8(x);
-    }
-  }
-  __syncthreads();   // every wave is done with the slot-branch tiles
+  lds_barrier();   // every wave is done with the slot-branch tiles
   stage_window(Kb0, Vb0);
   if (ntiles > 1) issue_window(1);
-  __syncthreads();
+  lds_barrier();
 
   // lazy rescaling: the running reference max only moves when a half tile exceeds it by more than
   // 2^RESCALE_LOG2 in probability units, so O is rescaled a handful of times per chunk
@@ -767,9 +826,10 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   bf16x8 ones;
 #pragma unroll
   for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
-  // every load issued so far (queries, first tiles) lands here, so inside the loop only the tile
-  // prefetches of the previous iteration are ever outstanding
-  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0), other counters untouched
+  // every load issued before the prefetch of tile 1 (queries, tile 0) has landed here, so inside
+  // the loop only the tile prefetch of the previous iteration is ever outstanding
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NPC));   // vmcnt(2 * NPC), other counters untouched
+  PROF_STAGE(4)
   PROF_DECL
   for (int i = 0; i < ntiles; ++i) {
     PROF_MARK(7)
@@ -871,10 +931,12 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     lds_barrier();
     PROF_MARK(5)
   }
+  PROF_STAGE(5)
 #ifdef NHA_PROF
   if (blockIdx.y == 200 && blockIdx.x == 3 && lane == 0) {
     long long* dbg = (long long*)p.lse_gsa;
     for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
+    for (int k = 0; k < 8; ++k) dbg[64 + wave * 8 + k] = ps_[k];
   }
 #endif
 
