@@ -24,6 +24,14 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+# HBM bytes per launch of the two dominant kernels on the default workloads, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a 256 MiB
+# device-to-device copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the runs are summarised under
+# profiles/.  Reported as `traffic` only while the workload is the one they were measured on.
+TRAFFIC_BYTES = {
+    "mfma_out_kernel<128,4,8,64>": (283463.0 * 2.0 + 147509.2) * 1024,
+    "decode_mfma_kernel<128,4,2>": (297292.1 * 2.0 + 67619.4) * 1024,
+}
 
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
 DECODE = dict(B=128, HQ=32, H=8, D=128, M=64, W=1024, steps=256)
@@ -303,13 +311,13 @@ def main():
                                       "ring positions, 256 consecutive steps"},
         "roofline": {"bound": "mfma", "kernel": "mfma_out_kernel<128,4,8,64>", "achieved": pf["achieved_tflops"],
                      "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": pf["achieved_tflops"] / PEAK_MFMA_BF16_TFLOPS,
-                     "traffic": None, "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
+                     "traffic": TRAFFIC_BYTES["mfma_out_kernel<128,4,8,64>"], "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
                      "whole_op_tflops": pf["whole_op_tflops"], "algorithmic_flop": pf["flops"]},
         "decode": {"metric": "decode step us @B=128", "value": dc["us_per_step"], "unit": "us/step",
                    "higher_is_better": False,
                    "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel<128,4,2>", "achieved": dc["achieved_gbs"],
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
-                                "traffic": None, "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
+                                "traffic": TRAFFIC_BYTES["decode_mfma_kernel<128,4,2>"], "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
