@@ -457,6 +457,17 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     goff[u] = (uint32_t)row * (uint32_t)(H * D) + col;
     loff[u] = row * (D + 16) + col;
   }
+  auto issue_window_fast = [&](int i) {
+    const int64_t grow0 = (int64_t)c0 + 64 - TK * (i + 1);
+    const bf16_t* kb_ = p.k_swa + (grow0 * H + h) * D;
+    const bf16_t* vb_ = p.v + (grow0 * H + h) * D;
+#pragma unroll
+    for (int u = 0; u < NPC; ++u) {
+      rk.r[u] = *reinterpret_cast<const uint4*>(kb_ + goff[u]);
+      rv.r[u] = *reinterpret_cast<const uint4*>(vb_ + goff[u]);
+    }
+  };
+  // tiles 0 and 1 (issued before the loop) may cover rows of the chunk itself, i.e. run past eos
   auto issue_window = [&](int i) {
     const int64_t grow0 = (int64_t)c0 + 64 - TK * (i + 1);
     if (grow0 + TK > eos) {
@@ -465,13 +476,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       tile_g2r<TK, D, NTHR>(rk, p.k_swa + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
       tile_g2r<TK, D, NTHR>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, 0, vhi, tid);
     } else {
-      const bf16_t* kb_ = p.k_swa + (grow0 * H + h) * D;
-      const bf16_t* vb_ = p.v + (grow0 * H + h) * D;
-#pragma unroll
-      for (int u = 0; u < NPC; ++u) {
-        rk.r[u] = *reinterpret_cast<const uint4*>(kb_ + goff[u]);
-        rv.r[u] = *reinterpret_cast<const uint4*>(vb_ + goff[u]);
-      }
+      issue_window_fast(i);
     }
   };
   auto stage_window = [&](lbf16* kdst, lbf16* vdst) {
@@ -925,7 +930,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     if (i + 1 < ntiles) {
       stage_window(cur ? Kb0 : Kb1, cur ? Vb0 : Vb1);
       PROF_MARK(6)
-      if (i + 2 < ntiles) issue_window(i + 2);
+      if (i + 2 < ntiles) issue_window_fast(i + 2);   // tiles >= 2 lie wholly before the chunk
     }
     PROF_MARK(4)
     lds_barrier();
