@@ -160,13 +160,19 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   constexpr int LDT = D + 16;
   constexpr int NB = D / 16;
   extern __shared__ __align__(16) unsigned char smem[];
-  lbf16* Kt = (lbf16*)smem;
-  lbf16* Vt = Kt + BT * LDT;
-  lbf16* St = Vt + BT * LDT;
+  lbf16* Xt = (lbf16*)smem;
+  lbf16* St = Xt + BT * LDT;
   lbf16* Gt = St + BT * SLD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
+  // blockIdx.z picks the state: 0 = k-state (rows of k_gsa; it also writes the gate tables),
+  // 1 = v-state (rows of v).  The two recurrences share nothing but the gates, and twice the
+  // workgroups of half the size fill the chip better.
+  const bool isv = blockIdx.z != 0;
+  const bf16_t* xsrc = isv ? p.v : p.k_gsa;
+  bf16_t* hloc = isv ? p.hvc : p.hkT;
+  float* hend = isv ? p.hend_v : p.hend_k;
   // blockIdx.x is a segment slot (seg_slot); slots are dense up to a few gaps per sequence, so
   // every XCD receives the same share of working workgroups
   const int slot = blockIdx.x, h = blockIdx.y;
@@ -189,23 +195,19 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   const int nloc = (nchunks - it0) < SEG ? (nchunks - it0) : SEG;
   const int m = wave * 16 + l16;   // this lane's slot
 
-  f32x4 hk[NB], hv[NB];
+  f32x4 hx[NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    hk[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    hv[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  }
+  for (int b = 0; b < NB; ++b) hx[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float gsum = 0.f;   // sum of the chunk-end gate cumsums since the segment start, this lane's slot
 
-  TileRegs<BT, D, 256> rk, rv;
+  TileRegs<BT, D, 256> rx;
   uint4 rs[2], rg[2];
   auto issue = [&](int it) {
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     const int64_t grow0 = (int64_t)bos + it * BT - p.shift;
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
-    tile_g2r<BT, D, 256>(rk, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
-    tile_g2r<BT, D, 256>(rv, p.v + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<BT, D, 256>(rx, xsrc + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -226,8 +228,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     const int chunk = chunk0 + jc;
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     if (jc > 0) __syncthreads();   // everyone is done reading the previous chunk's tiles
-    tile_r2l<BT, D, 256>(Kt, rk, tid);
-    tile_r2l<BT, D, 256>(Vt, rv, tid);
+    tile_r2l<BT, D, 256>(Xt, rx, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
       glast = __shfl(cand, l16 + 16 * src_kb, 64);
     }
     const int64_t cg = (int64_t)chunk * H + h;
-    {
+    if (!isv) {
       float* gout = p.gc + cg * BT * MS + m;
 #pragma unroll
       for (int e = 0; e < 16; ++e) gout[(16 * (e >> 2) + 4 * kb + (e & 3)) * MS] = gcv[e];
@@ -295,39 +296,28 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     // local chunk-start states (bf16), before the update: rows m, 4 consecutive d per lane
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      bf16x4 pk, pv;
+      bf16x4 pk;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pk[r] = (__bf16)hk[b][r];
-        pv[r] = (__bf16)hv[b][r];
-      }
-      *reinterpret_cast<bf16x4*>(p.hkT + (cg * MS + m) * D + 16 * b + 4 * kb) = pk;
-      *reinterpret_cast<bf16x4*>(p.hvc + (cg * MS + m) * D + 16 * b + 4 * kb) = pv;
+      for (int r = 0; r < 4; ++r) pk[r] = (__bf16)hx[b][r];
+      *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + 16 * b + 4 * kb) = pk;
     }
     const float dk = fexp(glast);
     gsum += glast;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        hk[b][r] *= dk;
-        hv[b][r] *= dk;
-      }
+      for (int r = 0; r < 4; ++r) hx[b][r] *= dk;
       // h[d][m] += sum_t x[t][d] sg[t][m]     A = x^T (transposed LDS read), B = sg
-      hk[b] = mfma16(lds_frag_tr(Kt, LDT, 0, 16, 16 * b, lane), sg0, hk[b]);
-      hk[b] = mfma16(lds_frag_tr(Kt, LDT, 32, 48, 16 * b, lane), sg1, hk[b]);
-      hv[b] = mfma16(lds_frag_tr(Vt, LDT, 0, 16, 16 * b, lane), sg0, hv[b]);
-      hv[b] = mfma16(lds_frag_tr(Vt, LDT, 32, 48, 16 * b, lane), sg1, hv[b]);
+      hx[b] = mfma16(lds_frag_tr(Xt, LDT, 0, 16, 16 * b, lane), sg0, hx[b]);
+      hx[b] = mfma16(lds_frag_tr(Xt, LDT, 32, 48, 16 * b, lane), sg1, hx[b]);
     }
   }
   // segment end: local state (fp32, [m][d]) and total decay
   const int64_t sl = (int64_t)seg_slot(p.coff, n, it0) * H + h;
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    *reinterpret_cast<float4*>(p.hend_k + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hk[b][0], hk[b][1], hk[b][2], hk[b][3]);
-    *reinterpret_cast<float4*>(p.hend_v + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hv[b][0], hv[b][1], hv[b][2], hv[b][3]);
-  }
-  if (kb == 0) p.dtot[sl * MS + m] = fexp(gsum);
+  for (int b = 0; b < NB; ++b)
+    *reinterpret_cast<float4*>(hend + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hx[b][0], hx[b][1], hx[b][2], hx[b][3]);
+  if (kb == 0 && !isv) p.dtot[sl * MS + m] = fexp(gsum);
 }
 
 // Level 2: one thread per state element, sequential over the segments of its sequence.
@@ -993,7 +983,7 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
   }
   if (phases != 2) {
     static bool configured = false;
-    const size_t lds = (size_t)2 * BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
+    const size_t lds = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
     if (!configured) {
       hipError_t e = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) {
@@ -1002,7 +992,7 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
       }
       configured = true;
     }
-    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H), dim3(256), lds, st, p);
+    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H, 2), dim3(256), lds, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
     hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
