@@ -69,6 +69,13 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int col
 
 __host__ __device__ constexpr int imax(int a, int b) { return a > b ? a : b; }
 
+// 16 bytes of a window row: read once per step and never again, so the load is marked
+// non-temporal (it does not displace the state lines in L2; measured 145 -> 134 us per step)
+__device__ __forceinline__ uint4 ld16_stream(const bf16_t* p) {
+  const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(x[0], x[1], x[2], x[3]);
+}
+
 constexpr int MS = 64;   // slots
 
 static size_t lds_bytes_for(int D, int G, int NW) {
@@ -149,7 +156,7 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
       const bf16_t* pw = kwin + (uint32_t)w * rstride;
       const bf16_t* row = (w == slot ? knew : pw) + 8 * qd;
 #pragma unroll
-      for (int j = 0; j < KS; ++j) kr[t * KS + j] = *reinterpret_cast<const uint4*>(row + 32 * j);
+      for (int j = 0; j < KS; ++j) kr[t * KS + j] = ld16_stream(row + 32 * j);
     }
 #pragma unroll
     for (int u = 0; u < NVT; ++u) {
@@ -157,7 +164,7 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
       w = w < nvalid ? w : nvalid - 1;
       const bf16_t* pw = vwin + (uint32_t)w * rstride;
       const bf16_t* row = (w == slot ? vnew : pw) + 8 * (lane % LV);
-      vr[u] = *reinterpret_cast<const uint4*>(row);
+      vr[u] = ld16_stream(row);
     }
   };
 
