@@ -199,7 +199,7 @@ def bench_decode(torch, warmup):
     e1.record(stream)
     torch.cuda.synchronize()
     us_step = e0.elapsed_time(e1) * 1e3 / steps
-    # decode kernel alone (no count-advance launch in between)
+    # decode kernel alone, counters left where they are
     e0.record(stream)
     loop(steps, False)
     e1.record(stream)

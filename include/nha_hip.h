@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 1
+#define NHA_ABI_VERSION 2
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -110,7 +110,9 @@ int nha_prefill_fwd(const NhaPrefillArgs* a);
  *   ring_v, ring_g [B,W,H,*] resident in HBM and count[b] = tokens cached so far.  The step
  *   pops slot count%W into the slots when count >= W, stores the new token (k_new, kg_new,
  *   v_new, g_new [B,H,*]) there, and attends over the min(count+1, W) valid entries.  The
- *   caller advances count (nha_decode_advance) after the step.  No reference counterpart: it
+ *   counters advance either in the same launch, into a second array (count_next[b] = count[b]+1;
+ *   the caller then swaps the two arrays), or by nha_decode_advance after the step; count itself
+ *   is never written by nha_decode_step.  No reference counterpart: it
  *   replaces the cat-shift cache of nha_fla/models/nha_cache.py:105-131, :143-154.
  * State hk [B,H,K,M], hv [B,H,M,V] fp32: read from hk_in/hv_in (NULL = zeros), written to
  * hk_out/hv_out (NULL = not written; may alias the inputs, fused_recurrent.py:541-545).
@@ -151,6 +153,7 @@ typedef struct NhaDecodeArgs {
   float* hv_out;
   void* o;
   void* stream;
+  int32_t* count_next; /* ring mode, optional: receives count[b] + 1 (must not alias count) */
 } NhaDecodeArgs;
 
 int nha_decode_step(const NhaDecodeArgs* a);

@@ -14,7 +14,7 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTS = (
     "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_decode_step", "nha_decode_advance",
@@ -51,7 +51,7 @@ class NhaDecodeArgs(C.Structure):
         ("k_new", C.c_void_p), ("kg_new", C.c_void_p), ("v_new", C.c_void_p), ("g_new", C.c_void_p),
         ("count", C.c_void_p),
         ("hk_in", C.c_void_p), ("hv_in", C.c_void_p), ("hk_out", C.c_void_p), ("hv_out", C.c_void_p),
-        ("o", C.c_void_p), ("stream", C.c_void_p),
+        ("o", C.c_void_p), ("stream", C.c_void_p), ("count_next", C.c_void_p),
     ]
 
 

@@ -79,6 +79,7 @@ __device__ __forceinline__ Ctx decode_prologue(const NhaDecodeArgs& a, const Lds
     slot = c % W;
     has_pop = c >= W;
     nvalid = c + 1 < W ? c + 1 : W;
+    if (a.count_next && h == 0 && tid == 0) a.count_next[b] = c + 1;
     const int64_t row = ((int64_t)b * W + slot) * H + h;
     kp = (const T*)a.ring_kg + row * K;
     vp = (const T*)a.ring_v + row * V;
@@ -655,6 +656,7 @@ int decode_step_impl(const NhaDecodeArgs* a) {
                       a->count && a->sq,
                   "nha_decode_step: ring mode needs ring_k/kg/v/g, k/kg/v/g_new, count and sq");
     NHA_CHECK_ARG(!a->cos, "nha_decode_step: ring mode stores rotated keys; cos/sin are not accepted");
+    NHA_CHECK_ARG((const int32_t*)a->count_next != a->count, "nha_decode_step: count_next must not alias count");
   } else if (a->mode == NHA_DECODE_WINDOW || a->mode == NHA_DECODE_LOGITS) {
     NHA_CHECK_ARG(a->k_pop && a->v_pop && a->g_pop, "nha_decode_step: k_pop, v_pop, g_pop are required");
     if (a->mode == NHA_DECODE_WINDOW) {

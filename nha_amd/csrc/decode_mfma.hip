@@ -134,6 +134,7 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
     cnt = a.count[b];
     slot = cnt % W;
     nvalid = cnt + 1 < W ? cnt + 1 : W;
+    if (a.count_next && h == 0 && tid == 0) a.count_next[b] = cnt + 1;
   }
   const bf16_t* kwin = (const bf16_t*)(ring ? a.ring_k : a.win_k) + ((int64_t)b * W * H + h) * D;
   const bf16_t* vwin = (const bf16_t*)(ring ? a.ring_v : a.win_v) + ((int64_t)b * W * H + h) * D;

@@ -27,7 +27,8 @@ class NHARingState:
     ring_kg: torch.Tensor   # [B,W,H,K]
     ring_v: torch.Tensor    # [B,W,H,V]
     ring_g: torch.Tensor    # [B,W,H,M]
-    count: torch.Tensor     # [B] int32
+    count: torch.Tensor     # [B] int32; the tensor bound to this name changes with every step
+    count_alt: Optional[torch.Tensor] = None   # the other counter array (the step writes count + 1 there)
 
     @classmethod
     def empty(cls, B, H, K, V, M, W, dtype=torch.bfloat16, device="cuda") -> "NHARingState":
@@ -71,8 +72,13 @@ def ring_decode_step(state: NHARingState, q: torch.Tensor, sq: torch.Tensor, k_n
     a.count = _ptr(state.count)
     a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(state.hk), _ptr(state.hv), _ptr(state.hk), _ptr(state.hv)
     a.o, a.stream = _ptr(o), _stream(q.device)
+    if advance:
+        # the kernel writes count + 1 into the second array; the two arrays then trade places
+        if state.count_alt is None:
+            state.count_alt = torch.empty_like(state.count)
+        a.count_next = _ptr(state.count_alt)
     lib = _lib.load()
     _lib.check(lib.nha_decode_step(C.byref(a)))
     if advance:
-        _lib.check(lib.nha_decode_advance(_ptr(state.count), B, a.stream))
+        state.count, state.count_alt = state.count_alt, state.count
     return o

@@ -30,7 +30,7 @@ def test_struct_sizes_match_the_header(tmp_path):
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     probes = [("NhaPrefillArgs", f) for f in ("q_swa", "scratch_bytes", "T_tot", "phases", "scale", "stream")]
-    probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream")]
+    probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream", "count_next")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
            'printf("%zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
