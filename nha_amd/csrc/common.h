@@ -22,6 +22,8 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return (bf16_t)(u >> 16);
 }
 
+typedef unsigned int nha_u32x4 __attribute__((ext_vector_type(4)));
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static __device__ __forceinline__ float ld(const float* p) { return *p; }
@@ -36,6 +38,13 @@ template <> struct Elem<float> {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
     *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
   }
+  // ld8 of data that is read once (non-temporal: it does not displace reused lines in L2)
+  static __device__ __forceinline__ void ld8_stream(const float* p, float* o) {
+    const nha_u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const nha_u32x4*>(p));
+    const nha_u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const nha_u32x4*>(p + 4));
+    o[0] = __uint_as_float(a[0]); o[1] = __uint_as_float(a[1]); o[2] = __uint_as_float(a[2]); o[3] = __uint_as_float(a[3]);
+    o[4] = __uint_as_float(b[0]); o[5] = __uint_as_float(b[1]); o[6] = __uint_as_float(b[2]); o[7] = __uint_as_float(b[3]);
+  }
 };
 template <> struct Elem<bf16_t> {
   static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
@@ -46,6 +55,13 @@ template <> struct Elem<bf16_t> {
     o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
     o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
     o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void ld8_stream(const bf16_t* p, float* o) {
+    const nha_u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const nha_u32x4*>(p));
+    o[0] = __uint_as_float(a[0] << 16); o[1] = __uint_as_float(a[0] & 0xffff0000u);
+    o[2] = __uint_as_float(a[1] << 16); o[3] = __uint_as_float(a[1] & 0xffff0000u);
+    o[4] = __uint_as_float(a[2] << 16); o[5] = __uint_as_float(a[2] & 0xffff0000u);
+    o[6] = __uint_as_float(a[3] << 16); o[7] = __uint_as_float(a[3] & 0xffff0000u);
   }
   static __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
     uint4 a;

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256, G <= 4 ? 4 : 2) void decode_kernel(const NhaDe
         const int w = wb + u * RK + rk;
         if (act && w < nvalid) {
           const T* row = (w == slot) ? knew : kbase + (int64_t)w * H * K;
-          Elem<T>::ld8(row, kv[u]);
+          Elem<T>::ld8_stream(row, kv[u]);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) kv[u][e] = 0.f;
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256, G <= 4 ? 4 : 2) void decode_kernel(const NhaDe
             const int w = wb + u * RV + rv;
             if (w < nvalid) {
               const T* row = (w == slot) ? vnew : vbase + (int64_t)w * H * V;
-              Elem<T>::ld8(row, vv[u]);
+              Elem<T>::ld8_stream(row, vv[u]);
             } else {
 #pragma unroll
               for (int e = 0; e < 8; ++e) vv[u][e] = 0.f;
@@ -483,8 +483,8 @@ __global__ __launch_bounds__(256, G <= 4 ? 4 : 2) void decode_stream_kernel(cons
       for (int u = 0; u < UNR; ++u) {
         const int w = wb + u * R + r;
         if (act && w < nvalid) {
-          Elem<T>::ld8((w == slot) ? knew : kbase + (int64_t)w * H * K, kv[u]);
-          Elem<T>::ld8((w == slot) ? vnew : vbase + (int64_t)w * H * V, vv[u]);
+          Elem<T>::ld8_stream((w == slot) ? knew : kbase + (int64_t)w * H * K, kv[u]);
+          Elem<T>::ld8_stream((w == slot) ? vnew : vbase + (int64_t)w * H * V, vv[u]);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
