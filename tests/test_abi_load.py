@@ -79,3 +79,12 @@ def test_varlen_tables_bit_exact_vs_oracle():
             ridx, roff = VI.chunk_tables_closed(cu, bt)
             assert idx.dtype == np.int32 and off.dtype == np.int32
             assert np.array_equal(idx, ridx) and np.array_equal(off, roff)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; --gpus N > 1 exits with a message instead of a number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
