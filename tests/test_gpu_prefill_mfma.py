@@ -66,6 +66,18 @@ def test_mfma_slow_forgetting_gates():
     run_case("slow-forgetting layer", d, wl=128, shift=0, dtype=BF, impl="mfma")
 
 
+@pytest.mark.parametrize("gate_mean", [-3.0, -4.5])
+def test_mfma_fast_forgetting_gates(gate_mean):
+    """Strong forgetting inside the range the matrix-core slot branch represents exactly: gate
+    logits ~ N(gate_mean, 1) -> logsigmoid, so a 16-row sub-block decays by about e^-50 / e^-72
+    (the factored decays are clamped at e^80) and a chunk by far more than fp32 can hold: decayed
+    terms must underflow to zero, not to NaN, and the recent rows must stay exact."""
+    d = prefill_inputs(850, 2, 300, 8, 2, 128, 128, 64, dtype=BF, gate_div=1.0, gate_mean=gate_mean, qk_scale=128 ** -0.5,
+                       with_state=True)
+    run_case(f"fast-forgetting {gate_mean}", d, wl=63, shift=64, dtype=BF, impl="mfma")
+    run_case(f"fast-forgetting {gate_mean} layer", d, wl=100, shift=0, dtype=BF, impl="mfma")
+
+
 def test_mfma_matches_simple_kernels_at_size():
     """A shape the CPU recurrence cannot reach in seconds: MFMA kernels vs the fp32-math kernels."""
     from nha_amd import chunk_nha
