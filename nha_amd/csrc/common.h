@@ -86,6 +86,40 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// reductions over a 256-thread workgroup (red: 4 floats of LDS) and a dot product of an fp32 LDS
+// vector with one global row
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <typename T>
+__device__ __forceinline__ float dot_row(const float* q, const T* row, int K) {
+  float acc = 0.f;
+  int kk = 0;
+  if ((K & 7) == 0 && ((reinterpret_cast<uintptr_t>(row) & 15) == 0)) {
+    for (; kk < K; kk += 8) {
+      float x[8];
+      Elem<T>::ld8(row + kk, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += q[kk + e] * x[e];
+    }
+    return acc;
+  }
+  for (; kk < K; ++kk) acc += q[kk] * Elem<T>::ld(row + kk);
+  return acc;
+}
+
 static inline int next_pow2_i(int x) {
   int p = 1;
   while (p < x) p <<= 1;

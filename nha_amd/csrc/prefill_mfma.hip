@@ -59,6 +59,7 @@ struct MP {
   float *hend_k, *hend_v;   // [NSLOT][H][MS][D]  segment-local end states
   float *hseg_k, *hseg_v;   // [NSLOT][H][MS][D]  true segment-start states
   float* dtot;   // [NSLOT][H][MS]   total decay of a segment
+  int* flags;    // [NT][H][4]       per 16-slot block: bit q = sub-block q decays past DECAY_CLAMP
   int T_tot, N, NT, HQ, H, NG, wl, shift;
   float scale;
 };
@@ -281,6 +282,19 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) gout[(16 * (e >> 2) + 4 * kb + (e & 3)) * MS] = gcv[e];
       if (kb == 0) p.dcum[cg * MS + m] = fexp(gsum);
+      // 16-row sub-blocks over which some slot decays by more than exp(DECAY_CLAMP): the output
+      // pass cannot factor their intra-block decay; mfma_repair_kernel recomputes their rows
+      int bits = 0;
+      if (kb == 3) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float ref = q > 0 ? gcv[4 * q - 1] : 0.f;
+          if (ref - gcv[4 * q + 3] > DECAY_CLAMP) bits |= 1 << q;
+        }
+      }
+#pragma unroll
+      for (int x = 32; x >= 1; x >>= 1) bits |= __shfl_xor(bits, x, 64);
+      if (lane == 0) p.flags[cg * 4 + wave] = bits;
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -958,6 +972,165 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   }
 }
 
+// ==========================================================================================
+// exact recomputation of rows the output pass cannot factor
+// ==========================================================================================
+// The output pass writes the intra-chunk decay exp(gc_i - gc_j) as exp(gc_i - gr) * exp(gr - gc_j)
+// with gr the gate cumsum at the start of j's 16-row sub-block, and caps the second exponent at
+// DECAY_CLAMP.  Where a slot forgets faster than that (flags from the state pass), the rows of
+// that sub-block are recomputed here token by token with the unfactored decay (<= 1), in fp32
+// VALU arithmetic, from the same chunk-start states and gate table: slot logits
+// (nha_fla/ops/nha/chunk_fused.py:186-222), window logits, one softmax (:233-240), both reads
+// (:242-283) and the branch LSEs (nha_fla/ops/nha/chunk.py:459-470).  grid (chunk, q-head);
+// workgroups of unflagged chunks leave at once.
+template <int D>
+struct RepairSmem {
+  static constexpr int LDH = D + 1;
+  static constexpr size_t floats = (size_t)MS * LDH + (size_t)MS * D + (size_t)BT * MS + 2 * D + 2 * MS + 2 * BT + 256 + 4 + BT;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void mfma_repair_kernel(const MP p) {
+  constexpr int LDH = RepairSmem<D>::LDH;
+  const int chunk = blockIdx.x, hq = blockIdx.y;
+  const int H = p.H, HQ = p.HQ, h = hq / p.NG;
+  const int64_t cg = (int64_t)chunk * H + h;
+  const int* fl = p.flags + cg * 4;
+  const int bits = fl[0] | fl[1] | fl[2] | fl[3];
+  if (bits == 0) return;
+  extern __shared__ __align__(16) float rsm[];
+  float* hk = rsm;                // [MS][LDH] true chunk-start k-state, transposed
+  float* hv = hk + MS * LDH;      // [MS][D]   true chunk-start v-state
+  float* gcl = hv + MS * D;       // [BT][MS]  gate cumsum
+  float* qg = gcl + BT * MS;      // [D] scaled slot-branch query
+  float* qs = qg + D;             // [D] scaled window query
+  float* okl = qs + D;            // [MS] slot logits -> probabilities
+  float* gct = okl + MS;          // [MS] gate cumsum of the row
+  float* Aj = gct + MS;           // [BT]
+  float* Avj = Aj + BT;           // [BT]
+  float* pw = Avj + BT;           // [256]
+  float* red = pw + 256;          // [4]
+  int* src = (int*)(red + 4);     // [BT]
+  const int tid = threadIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int rows = (eos - c0) < BT ? (eos - c0) : BT;
+  const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
+  for (int e = tid; e < MS * D; e += 256) {
+    const int m = e / D, d = e % D;
+    const float dc = p.dcum[cg * MS + m];
+    hk[m * LDH + d] = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
+    hv[m * D + d] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+  }
+  for (int e = tid; e < BT * MS; e += 256) gcl[e] = p.gc[cg * BT * MS + e];
+
+  for (int r = 0; r < rows; ++r) {
+    if (!((bits >> (r >> 4)) & 1)) continue;
+    const int t = c0 + r;
+    __syncthreads();   // state tables are in place; the previous row is finished
+    const bf16_t* qsw = p.q_swa + ((int64_t)t * HQ + hq) * D;
+    const bf16_t* qgs = p.q_gsa + ((int64_t)t * HQ + hq) * D;
+    for (int i = tid; i < D; i += 256) {
+      qg[i] = bf16_to_f32(qgs[i]) * p.scale;
+      qs[i] = bf16_to_f32(qsw[i]) * p.scale;
+    }
+    if (tid < MS) gct[tid] = gcl[r * MS + tid];
+    if (tid < BT) {
+      const int tl = it * BT + tid - p.shift;
+      src[tid] = (tid <= r && tl >= 0) ? bos + tl : -1;
+    }
+    __syncthreads();
+    if (tid < BT) {
+      const int sj = src[tid];
+      Aj[tid] = sj >= 0 ? dot_row<bf16_t>(qg, p.k_gsa + ((int64_t)sj * H + h) * D, D) : 0.f;
+    }
+    __syncthreads();
+    float lmax = -INFINITY;
+    if (tid < MS) {
+      const int m = tid;
+      float acc = 0.f;
+      for (int d = 0; d < D; ++d) acc += qg[d] * hk[m * LDH + d];
+      acc *= expf(gct[m]);
+      for (int j = 0; j <= r; ++j) {
+        const int sj = src[j];
+        if (sj >= 0) acc += Aj[j] * bf16_to_f32(p.s[((int64_t)sj * H + h) * MS + m]) * expf(gct[m] - gcl[j * MS + m]);
+      }
+      okl[m] = acc;
+      lmax = acc;
+    }
+    const float mg = block_max(lmax, red);
+    const float lg = block_sum(tid < MS ? expf(okl[tid] - mg) : 0.f, red);
+    const int lo = p.wl < 0 ? bos : (t - p.wl > bos ? t - p.wl : bos);
+    float wm = -INFINITY, wsum = 0.f;
+    for (int j = lo + tid; j <= t; j += 256) {
+      const float d = dot_row<bf16_t>(qs, p.k_swa + ((int64_t)j * H + h) * D, D);
+      if (d > wm) {
+        wsum = wsum * expf(wm - d) + 1.f;
+        wm = d;
+      } else {
+        wsum += expf(d - wm);
+      }
+    }
+    const float mw = block_max(wm, red);
+    const float lw = block_sum(wm == -INFINITY ? 0.f : wsum * expf(wm - mw), red);
+    if (tid == 0) {
+      if (p.lse_gsa) p.lse_gsa[(int64_t)t * HQ + hq] = mg + logf(lg);
+      if (p.lse_swa) p.lse_swa[(int64_t)t * HQ + hq] = mw + logf(lw);
+    }
+    const float mt = fmaxf(mg, mw);
+    const float inv = 1.f / (lg * expf(mg - mt) + lw * expf(mw - mt));
+    __syncthreads();
+    if (tid < MS) okl[tid] = expf(okl[tid] - mt) * inv;
+    __syncthreads();
+    if (tid < BT) {
+      const int sj = src[tid];
+      float acc = 0.f;
+      if (sj >= 0) {
+        const bf16_t* srow = p.s + ((int64_t)sj * H + h) * MS;
+        for (int m = 0; m < MS; ++m) acc += okl[m] * bf16_to_f32(srow[m]) * expf(gct[m] - gcl[tid * MS + m]);
+      }
+      Avj[tid] = acc;
+    }
+    __syncthreads();
+    float acc = 0.f;   // value column tid (D <= 256 == threads)
+    if (tid < D) {
+      for (int m = 0; m < MS; ++m) acc += okl[m] * expf(gct[m]) * hv[m * D + tid];
+      for (int j = 0; j <= r; ++j) {
+        const int sj = src[j];
+        if (sj >= 0) acc += Avj[j] * bf16_to_f32(p.v[((int64_t)sj * H + h) * D + tid]);
+      }
+    }
+    for (int jb = lo; jb <= t; jb += 256) {
+      const int j = jb + tid;
+      __syncthreads();
+      pw[tid] = j <= t ? expf(dot_row<bf16_t>(qs, p.k_swa + ((int64_t)j * H + h) * D, D) - mt) * inv : 0.f;
+      __syncthreads();
+      const int cnt = (t - jb + 1) < 256 ? (t - jb + 1) : 256;
+      if (tid < D)
+        for (int x = 0; x < cnt; ++x) acc += pw[x] * bf16_to_f32(p.v[((int64_t)(jb + x) * H + h) * D + tid]);
+    }
+    if (tid < D) p.o[((int64_t)t * HQ + hq) * D + tid] = f32_to_bf16(acc);
+  }
+}
+
+template <int D>
+int launch_repair(const MP& p, hipStream_t st) {
+  static bool configured = false;
+  const size_t lds = RepairSmem<D>::floats * 4;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)mfma_repair_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) {
+      set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+      return NHA_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL((mfma_repair_kernel<D>), dim3(p.NT, p.HQ), dim3(256), lds, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma repair pass)");
+  return NHA_OK;
+}
+
 template <int D, int G, int NW, int TK>
 int launch_out(const MP& p, hipStream_t st) {
   static bool configured = false;
@@ -1001,14 +1174,17 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     // G query heads of one kv-head share a workgroup.  D <= 128: 64-key tiles, 8 waves of 32 (G = 4)
     // or 16 (G = 2) query rows, two per SIMD; D = 256: 32-key tiles and 16-row waves to fit the
     // register file and LDS
+    int rc;
     if constexpr (D <= 128) {
-      if (p.NG % 4 == 0) return launch_out<D, 4, 8, 64>(p, st);
-      if (p.NG % 2 == 0) return launch_out<D, 2, 8, 64>(p, st);
-      return launch_out<D, 1, 4, 64>(p, st);
+      if (p.NG % 4 == 0) rc = launch_out<D, 4, 8, 64>(p, st);
+      else if (p.NG % 2 == 0) rc = launch_out<D, 2, 8, 64>(p, st);
+      else rc = launch_out<D, 1, 4, 64>(p, st);
     } else {
-      if (p.NG % 2 == 0) return launch_out<D, 2, 8, 32>(p, st);
-      return launch_out<D, 1, 4, 32>(p, st);
+      if (p.NG % 2 == 0) rc = launch_out<D, 2, 8, 32>(p, st);
+      else rc = launch_out<D, 1, 4, 32>(p, st);
     }
+    if (rc != NHA_OK) return rc;
+    return launch_repair<D>(p, st);
   }
   return NHA_OK;
 }
@@ -1023,7 +1199,7 @@ bool prefill_mfma_supported(const NhaPrefillArgs* a) {
 
 namespace {
 struct ScratchPlan {
-  size_t hkT, hvc, gc, dcum, hend_k, hend_v, hseg_k, hseg_v, dtot, total;
+  size_t hkT, hvc, gc, dcum, hend_k, hend_v, hseg_k, hseg_v, dtot, flags, total;
 };
 ScratchPlan plan_scratch(const NhaPrefillArgs* a) {
   const size_t per = (size_t)a->NT * a->H;
@@ -1040,6 +1216,7 @@ ScratchPlan plan_scratch(const NhaPrefillArgs* a) {
   s.hseg_k = off; off += seg;
   s.hseg_v = off; off += seg;
   s.dtot = off; off += aligned(nslot * a->H * MS * 4);
+  s.flags = off; off += aligned(per * 4 * 4);
   s.total = off;
   return s;
 }
@@ -1067,6 +1244,7 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
   p.hseg_k = (float*)(sc + sp.hseg_k);
   p.hseg_v = (float*)(sc + sp.hseg_v);
   p.dtot = (float*)(sc + sp.dtot);
+  p.flags = (int*)(sc + sp.flags);
   p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H;
   p.wl = a->wl; p.shift = a->shift; p.scale = a->scale;
   hipStream_t st = (hipStream_t)a->stream;

@@ -131,38 +131,6 @@ __global__ __launch_bounds__(256) void simple_state_kernel(const SP p) {
     }
 }
 
-__device__ __forceinline__ float block_max(float v, float* red) {
-  v = wave_max(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-}
-__device__ __forceinline__ float block_sum(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
-}
-
-template <typename T>
-__device__ __forceinline__ float dot_row(const float* q, const T* row, int K) {
-  float acc = 0.f;
-  int kk = 0;
-  if ((K & 7) == 0 && ((reinterpret_cast<uintptr_t>(row) & 15) == 0)) {
-    for (; kk < K; kk += 8) {
-      float x[8];
-      Elem<T>::ld8(row + kk, x);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc += q[kk + e] * x[e];
-    }
-    return acc;
-  }
-  for (; kk < K; ++kk) acc += q[kk] * Elem<T>::ld(row + kk);
-  return acc;
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void simple_out_kernel(const SP p) {
   extern __shared__ __align__(16) float lds[];

@@ -66,16 +66,35 @@ def test_mfma_slow_forgetting_gates():
     run_case("slow-forgetting layer", d, wl=128, shift=0, dtype=BF, impl="mfma")
 
 
-@pytest.mark.parametrize("gate_mean", [-3.0, -4.5])
+@pytest.mark.parametrize("gate_mean", [-3.0, -4.5, -6.0, -8.0, -12.0])
 def test_mfma_fast_forgetting_gates(gate_mean):
-    """Strong forgetting inside the range the matrix-core slot branch represents exactly: gate
-    logits ~ N(gate_mean, 1) -> logsigmoid, so a 16-row sub-block decays by about e^-50 / e^-72
-    (the factored decays are clamped at e^80) and a chunk by far more than fp32 can hold: decayed
-    terms must underflow to zero, not to NaN, and the recent rows must stay exact."""
+    """Strong forgetting: gate logits ~ N(gate_mean, 1) -> logsigmoid, so a 16-row sub-block decays
+    by about e^-50 ... e^-190 and a chunk by far more than fp32 can hold.  Up to e^-80 per sub-block
+    the matrix-core slot branch factors the decay exactly; beyond that the state pass flags the
+    sub-block and its rows are recomputed with the unfactored decay.  Decayed terms must underflow
+    to zero, not to NaN, and the recent rows must stay exact."""
     d = prefill_inputs(850, 2, 300, 8, 2, 128, 128, 64, dtype=BF, gate_div=1.0, gate_mean=gate_mean, qk_scale=128 ** -0.5,
                        with_state=True)
     run_case(f"fast-forgetting {gate_mean}", d, wl=63, shift=64, dtype=BF, impl="mfma")
     run_case(f"fast-forgetting {gate_mean} layer", d, wl=100, shift=0, dtype=BF, impl="mfma")
+
+
+@pytest.mark.parametrize("D,HQ,H", [(64, 4, 4), (128, 8, 2), (256, 4, 2)])
+def test_mfma_isolated_strong_decay(D, HQ, H):
+    """A few slots forget abruptly in a few rows of otherwise ordinary, packed sequences: only the
+    16-row sub-blocks that contain them take the exact path, everything else the matrix-core path,
+    and both must agree with the recurrence."""
+    cu = [0, 100, 333, 400]
+    d = prefill_inputs(860 + D, 1, cu[-1], HQ, H, D, D, 64, dtype=BF, gate_div=8.0, qk_scale=D ** -0.5, with_state=True,
+                       N=3)
+    g = d["g"].float()
+    g[0, 70:73, 0, 5] = -40.0       # sequence 0, chunk 1, sub-block 0
+    g[0, 150, :, 17] = -90.0        # sequence 1 (rows 100..332): row 50 -> chunk 0, sub-block 3
+    g[0, 331:333, H - 1, 63] = -60.0   # last rows of sequence 1, ragged chunk
+    g[0, 399, 0, :] = -100.0        # the very last row
+    d["g"] = g.to(BF)
+    run_case("isolated decay layer", d, wl=64, shift=0, dtype=BF, impl="mfma", cu=cu)
+    run_case("isolated decay shifted", d, wl=31, shift=32, dtype=BF, impl="mfma", cu=cu)
 
 
 def test_mfma_matches_simple_kernels_at_size():
