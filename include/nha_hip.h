@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 2
+#define NHA_ABI_VERSION 3
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -91,6 +91,64 @@ typedef struct NhaPrefillArgs {
  * cumsums, staging).  Only the integer/dtype/impl fields of `a` are read. */
 size_t nha_prefill_scratch_bytes(const NhaPrefillArgs* a);
 int nha_prefill_fwd(const NhaPrefillArgs* a);
+
+/* ------------------------------------------------------------------------------------------
+ * Chunked prefill backward.  Replaces ChunkNativeHybridAttentionFunction.backward
+ * (nha_fla/ops/nha/chunk.py:490-564: window-branch backward :499-511, slot-branch backward with
+ * the LSE coupling of the merged softmax :514-530 and nha_fla/ops/nha/chunk_gsa.py:52-122,
+ * un-shifting of the slot-branch gradients :533-543, dv accumulated over both branches :559).
+ *
+ * Inputs: the forward's inputs (same layouts and dims as NhaPrefillArgs), its outputs o, lse_swa,
+ * lse_gsa (all three required), the initial states if the forward had them, and the cotangents
+ * dout [T_tot,HQ,V] (input dtype; required), dlse_swa / dlse_gsa [T_tot,HQ] fp32 and dhkt
+ * [N,H,K,M] / dhvt [N,H,M,V] fp32 (each NULL = zero).  Outputs: dq_swa, dq_gsa [T_tot,HQ,K],
+ * dk_swa, dk_gsa [T_tot,H,K], dv [T_tot,H,V], ds, dg [T_tot,H,M] in the input dtype (all
+ * required, fully written), and dh0k / dh0v fp32 (NULL = not wanted).  fp32 arithmetic
+ * throughout; K, V <= 256 (multiples of 8), M <= 64.  The slot states are recomputed from the
+ * inputs into the scratch, nothing else is kept from the forward.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct NhaPrefillBwdArgs {
+  const void* q_swa;
+  const void* k_swa;
+  const void* q_gsa;
+  const void* k_gsa;
+  const void* v;
+  const void* s;
+  const void* g;
+  const void* o;
+  const float* lse_swa;
+  const float* lse_gsa;
+  const float* h0k;
+  const float* h0v;
+  const void* dout;
+  const float* dlse_swa;
+  const float* dlse_gsa;
+  const float* dhkt;
+  const float* dhvt;
+  void* dq_swa;
+  void* dk_swa;
+  void* dq_gsa;
+  void* dk_gsa;
+  void* dv;
+  void* ds;
+  void* dg;
+  float* dh0k;
+  float* dh0v;
+  const int32_t* cu_seqlens;
+  const int32_t* chunk_indices;
+  const int32_t* chunk_offsets;
+  void* scratch;
+  size_t scratch_bytes;
+  int32_t T_tot, N, NT, HQ, H, K, V, M;
+  int32_t wl;
+  int32_t shift;
+  int32_t dtype;
+  float scale;
+  void* stream;
+} NhaPrefillBwdArgs;
+
+size_t nha_prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
+int nha_prefill_bwd(const NhaPrefillBwdArgs* a);
 
 /* ------------------------------------------------------------------------------------------
  * Single-token decode step.  Replaces the k/v kernel pair of fused_recurrent_nha_decode

@@ -14,10 +14,11 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EXPORTS = (
-    "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_decode_step", "nha_decode_advance",
+    "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
+    "nha_decode_step", "nha_decode_advance",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
 )
 
@@ -33,6 +34,26 @@ class NhaPrefillArgs(C.Structure):
         ("T_tot", C.c_int32), ("N", C.c_int32), ("NT", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32),
         ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
         ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32), ("impl", C.c_int32), ("phases", C.c_int32),
+        ("scale", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
+class NhaPrefillBwdArgs(C.Structure):
+    _fields_ = [
+        ("q_swa", C.c_void_p), ("k_swa", C.c_void_p), ("q_gsa", C.c_void_p), ("k_gsa", C.c_void_p),
+        ("v", C.c_void_p), ("s", C.c_void_p), ("g", C.c_void_p),
+        ("o", C.c_void_p), ("lse_swa", C.c_void_p), ("lse_gsa", C.c_void_p),
+        ("h0k", C.c_void_p), ("h0v", C.c_void_p),
+        ("dout", C.c_void_p), ("dlse_swa", C.c_void_p), ("dlse_gsa", C.c_void_p),
+        ("dhkt", C.c_void_p), ("dhvt", C.c_void_p),
+        ("dq_swa", C.c_void_p), ("dk_swa", C.c_void_p), ("dq_gsa", C.c_void_p), ("dk_gsa", C.c_void_p),
+        ("dv", C.c_void_p), ("ds", C.c_void_p), ("dg", C.c_void_p),
+        ("dh0k", C.c_void_p), ("dh0v", C.c_void_p),
+        ("cu_seqlens", C.c_void_p), ("chunk_indices", C.c_void_p), ("chunk_offsets", C.c_void_p),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t),
+        ("T_tot", C.c_int32), ("N", C.c_int32), ("NT", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32),
+        ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
+        ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32),
         ("scale", C.c_float), ("stream", C.c_void_p),
     ]
 
@@ -77,6 +98,10 @@ def load() -> C.CDLL:
     lib.nha_prefill_scratch_bytes.argtypes = [C.POINTER(NhaPrefillArgs)]
     lib.nha_prefill_fwd.restype = C.c_int
     lib.nha_prefill_fwd.argtypes = [C.POINTER(NhaPrefillArgs)]
+    lib.nha_prefill_bwd_scratch_bytes.restype = C.c_size_t
+    lib.nha_prefill_bwd_scratch_bytes.argtypes = [C.POINTER(NhaPrefillBwdArgs)]
+    lib.nha_prefill_bwd.restype = C.c_int
+    lib.nha_prefill_bwd.argtypes = [C.POINTER(NhaPrefillBwdArgs)]
     lib.nha_decode_step.restype = C.c_int
     lib.nha_decode_step.argtypes = [C.POINTER(NhaDecodeArgs)]
     lib.nha_decode_advance.restype = C.c_int

@@ -36,6 +36,29 @@ static int check_prefill(const NhaPrefillArgs* a, bool pointers) {
   return NHA_OK;
 }
 
+static int check_prefill_bwd(const NhaPrefillBwdArgs* a, bool pointers) {
+  NHA_CHECK_ARG(a != nullptr, "nha_prefill_bwd: null args");
+  NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->NT > 0 && a->HQ > 0 && a->H > 0 && a->K > 0 && a->V > 0 && a->M > 0,
+                "nha_prefill_bwd: non-positive dimension");
+  NHA_CHECK_ARG(a->HQ % a->H == 0, "nha_prefill_bwd: HQ (%d) must be a multiple of H (%d)", a->HQ, a->H);
+  NHA_CHECK_ARG(a->shift >= 0, "nha_prefill_bwd: gsa_kv_shift must be >= 0, got %d", a->shift);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_prefill_bwd: bad dtype %d", a->dtype);
+  if (pointers) {
+    NHA_CHECK_ARG(a->q_swa && a->k_swa && a->q_gsa && a->k_gsa && a->v && a->s && a->g,
+                  "nha_prefill_bwd: q_swa, k_swa, q_gsa, k_gsa, v, s, g are required");
+    NHA_CHECK_ARG(a->o && a->lse_swa && a->lse_gsa && a->dout, "nha_prefill_bwd: o, lse_swa, lse_gsa and dout are required");
+    NHA_CHECK_ARG(a->dq_swa && a->dk_swa && a->dq_gsa && a->dk_gsa && a->dv && a->ds && a->dg,
+                  "nha_prefill_bwd: dq_swa, dk_swa, dq_gsa, dk_gsa, dv, ds, dg are required");
+    NHA_CHECK_ARG(a->cu_seqlens && a->chunk_indices && a->chunk_offsets,
+                  "nha_prefill_bwd: cu_seqlens, chunk_indices and chunk_offsets are required");
+    NHA_CHECK_ARG((a->h0k == nullptr) == (a->h0v == nullptr), "nha_prefill_bwd: pass both initial states or neither");
+    NHA_CHECK_ARG((a->dhkt == nullptr) == (a->dhvt == nullptr), "nha_prefill_bwd: pass both final-state cotangents or neither");
+    NHA_CHECK_ARG((a->dh0k == nullptr) == (a->dh0v == nullptr), "nha_prefill_bwd: pass both initial-state gradients or neither");
+    NHA_CHECK_ARG(a->scratch != nullptr, "nha_prefill_bwd: scratch is required");
+  }
+  return NHA_OK;
+}
+
 static bool use_mfma(const NhaPrefillArgs* a) {
   if (a->impl == NHA_IMPL_SIMPLE) return false;
   return prefill_mfma_supported(a);
@@ -67,6 +90,26 @@ int nha_prefill_fwd(const NhaPrefillArgs* a) {
     return NHA_ERR_SCRATCH;
   }
   return mfma ? prefill_mfma_impl(a) : prefill_simple_impl(a);
+}
+
+size_t nha_prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a) {
+  if (check_prefill_bwd(a, false) != NHA_OK) return 0;
+  return prefill_bwd_scratch_bytes(a);
+}
+
+int nha_prefill_bwd(const NhaPrefillBwdArgs* a) {
+  int rc = check_prefill_bwd(a, true);
+  if (rc != NHA_OK) return rc;
+  if (!prefill_bwd_supported(a)) {
+    set_error("nha_prefill_bwd: built for K, V <= 256 (multiples of 8) and M <= 64, got K=%d V=%d M=%d", a->K, a->V, a->M);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  const size_t need = prefill_bwd_scratch_bytes(a);
+  if (a->scratch_bytes < need) {
+    set_error("nha_prefill_bwd: scratch has %zu bytes, %zu needed", a->scratch_bytes, need);
+    return NHA_ERR_SCRATCH;
+  }
+  return prefill_bwd_impl(a);
 }
 
 int nha_decode_step(const NhaDecodeArgs* a) { return decode_step_impl(a); }

@@ -1,0 +1,661 @@
+// Backward of the chunked NHA prefill for gfx950, fp32 VALU arithmetic (any K, V <= 256, M <= 64;
+// fp32 or bf16 tensors; GQA; varlen).  Replaces ChunkNativeHybridAttentionFunction.backward
+// (nha_fla/ops/nha/chunk.py:490-564): window-branch gradients (:499-511), slot-branch gradients
+// with the merged-softmax coupling (:514-530; chunk_gsa.py:52-122), un-shifting (:533-543) and the
+// accumulation of dv over both branches (:559) -- as ONE differentiation of the merged softmax
+// instead of two branch backwards glued by an LSE correction.
+//
+// Per token t and q-head a (kv-head h, slot-branch rows read at src = t - shift):
+//   u[m] = scale q_gsa . hk_t[:,m]      w[j] = scale q_swa . k_swa_j       lse = log(sum e^u + sum e^w)
+//   p = e^(u-lse)   pi = e^(w-lse)      o = p hv_t + pi v
+//   delta = do . o      dp[m] = do . hv_t[m,:]      dpi[j] = do . v_j
+//   du = p (dp - delta) + dlse_gsa e^(u-lse_gsa)     dw = pi (dpi - delta) + dlse_swa e^(w-lse_swa)
+// and the state recurrences hk_t = hk_(t-1) e^g + k' s^T, hv_t = e^g hv_(t-1) + s v'^T run backward
+// in chunk form.  With Dh_r the total gradient of the state after row r,
+//   dk'_r = Dhk_r s_r     dv'_r = s_r^T Dhv_r     ds_r = k'_r^T Dhk_r + Dhv_r v'_r
+//   dg_r  = dg_(r+1) + sum_a (du u + p dp)_r - s_r ds_r        (dg past the end = <dh_T, h_T>)
+// (the last line is the usual reverse cumulative sum of gated linear attention: <Dh_r, h_r> telescopes).
+//
+// Launches: forward state pass (chunk-start states, gate cumsums) -> bwd_q_kernel (per token: dq's and
+// the per-token vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra
+// part of ds) -> bwd_state_kernel (reverse sweep over chunks, one workgroup per 32 state columns:
+// dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_kernel (reverse scan: ds, dg)
+// -> bwd_kv_window_kernel (per key: dk_swa, dv).
+#include "common.h"
+
+namespace nha {
+namespace {
+
+constexpr int BT = 64;   // chunk rows
+constexpr int CB = 32;   // state columns per workgroup of the state-gradient sweep
+
+struct BP {
+  const void *q_swa, *k_swa, *q_gsa, *k_gsa, *v, *s, *g, *o, *dout;
+  const float *lse_swa, *lse_gsa, *dlse_swa, *dlse_gsa, *dhkt, *dhvt;
+  void *dq_swa, *dk_swa, *dq_gsa, *dk_gsa, *dv, *ds, *dg;
+  float *dh0k, *dh0v;
+  const int32_t *cu, *cidx, *coff;
+  // forward recomputation (layout of the generic forward state pass)
+  float *gc;          // [T_tot][H][M]      chunk-local inclusive gate cumsum, indexed by row token
+  float *hkc, *hvc;   // [NT][H][K][M], [NT][H][M][V]   chunk-start states
+  float *hkT, *hvT;   // [N][H][K][M], [N][H][M][V]     final states (for the end term of dg)
+  // per-token vectors of the slot branch
+  float *dus, *pp, *xg;   // [T_tot][HQ][M]   scale*du, p, du*u + p*dp
+  float *delta;           // [T_tot][HQ]
+  float *ck, *cv;         // [NT][HQ][BT][BT]  sum_m dus_i s_r e^(gc_i-gc_r), same with p   (i >= r)
+  float *dsi;             // [T_tot][H][M]     intra-chunk part of ds, indexed by row token
+  float *dsp;             // [nbk+nbv][T_tot][H][M]  inter-chunk part of ds per column block
+  float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
+  int T_tot, N, NT, HQ, H, K, V, M, wl, shift, nbk, nbv;
+  float scale;
+};
+
+__device__ __forceinline__ float logaddexp_f(float a, float b) {
+  const float mx = fmaxf(a, b);
+  return mx + logf(expf(a - mx) + expf(b - mx));
+}
+
+// ------------------------------------------------------------------------------------------
+// per (token, q-head): dq_swa, dq_gsa and the vectors du, p the state gradients are built from
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  float* qg = lds;             // [K] scaled slot-branch query
+  float* qs = qg + K;          // [K] scaled window query
+  float* dov = qs + K;         // [V]
+  float* gct = dov + V;        // [M]
+  float* okl = gct + M;        // [M] slot logits u
+  float* dpl = okl + M;        // [M] dp
+  float* dul = dpl + M;        // [M] scale * du
+  float* Aj = dul + M;         // [BT] q_gsa . k'_j
+  float* Bj = Aj + BT;         // [BT] do . v'_j
+  float* Wj = Bj + BT;         // [BT]
+  float* pw = Wj + BT;         // [256]
+  float* red = pw + 256;       // [4]
+  int* src = (int*)(red + 4);  // [BT]
+  const int tid = threadIdx.x;
+  const int chunk = blockIdx.x / BT, r = blockIdx.x % BT;
+  const int hq = blockIdx.y, h = hq / NG;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int t = bos + it * BT + r;
+  if (t >= eos) return;
+  const T* ksw = (const T*)p.k_swa;
+  const T* kgs = (const T*)p.k_gsa;
+  const T* vv_ = (const T*)p.v;
+  const T* ss = (const T*)p.s;
+  const int64_t tq = (int64_t)t * HQ + hq;
+  for (int i = tid; i < K; i += 256) {
+    qg[i] = Elem<T>::ld((const T*)p.q_gsa + tq * K + i) * p.scale;
+    qs[i] = Elem<T>::ld((const T*)p.q_swa + tq * K + i) * p.scale;
+  }
+  float dl = 0.f;
+  for (int i = tid; i < V; i += 256) {
+    const float d = Elem<T>::ld((const T*)p.dout + tq * V + i);
+    dov[i] = d;
+    dl += d * Elem<T>::ld((const T*)p.o + tq * V + i);
+  }
+  for (int i = tid; i < M; i += 256) gct[i] = p.gc[((int64_t)t * H + h) * M + i];
+  if (tid < BT) {
+    const int tl = it * BT + tid - p.shift;
+    src[tid] = (tid <= r && tl >= 0) ? bos + tl : -1;
+  }
+  const float delta = block_sum(dl, red);   // includes the barrier that publishes the tables
+  if (tid < BT) {
+    const int sj = src[tid];
+    Aj[tid] = sj >= 0 ? dot_row<T>(qg, kgs + ((int64_t)sj * H + h) * K, K) : 0.f;
+  } else if (tid < 2 * BT) {
+    const int sj = src[tid - BT];
+    Bj[tid - BT] = sj >= 0 ? dot_row<T>(dov, vv_ + ((int64_t)sj * H + h) * V, V) : 0.f;
+  }
+  __syncthreads();
+  const float* hk0 = p.hkc + ((int64_t)chunk * H + h) * K * M;
+  const float* hv0 = p.hvc + ((int64_t)chunk * H + h) * M * V;
+  const float* gcb = p.gc + ((int64_t)(bos + it * BT) * H + h) * M;
+  const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
+  const float lt = logaddexp_f(ls, lg);
+  const float dlg = p.dlse_gsa ? p.dlse_gsa[tq] : 0.f;
+  const float dls = p.dlse_swa ? p.dlse_swa[tq] : 0.f;
+  for (int m = tid; m < M; m += 256) {
+    float au = 0.f, ad = 0.f;
+    for (int kk = 0; kk < K; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
+    for (int c = 0; c < V; ++c) ad += dov[c] * hv0[(int64_t)m * V + c];
+    const float e = expf(gct[m]);
+    au *= e;
+    ad *= e;
+    for (int j = 0; j <= r; ++j) {
+      const int sj = src[j];
+      if (sj >= 0) {
+        const float w = Elem<T>::ld(ss + ((int64_t)sj * H + h) * M + m) * expf(gct[m] - gcb[(int64_t)j * H * M + m]);
+        au += Aj[j] * w;
+        ad += Bj[j] * w;
+      }
+    }
+    const float pm = expf(au - lt);
+    const float du = pm * (ad - delta) + dlg * expf(au - lg);
+    okl[m] = au;
+    dpl[m] = ad;
+    dul[m] = p.scale * du;
+    p.dus[tq * M + m] = p.scale * du;
+    p.pp[tq * M + m] = pm;
+    p.xg[tq * M + m] = du * au + pm * ad;
+  }
+  if (tid == 0) p.delta[tq] = delta;
+  __syncthreads();
+  if (tid < BT) {
+    const int sj = src[tid];
+    float acc = 0.f;
+    if (sj >= 0) {
+      const T* srow = ss + ((int64_t)sj * H + h) * M;
+      const float* gj = gcb + (int64_t)tid * H * M;
+      for (int m = 0; m < M; ++m) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
+    }
+    Wj[tid] = acc;
+  }
+  __syncthreads();
+  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]
+  for (int d = tid; d < K; d += 256) {
+    float acc = 0.f;
+    for (int m = 0; m < M; ++m) acc += dul[m] * expf(gct[m]) * hk0[(int64_t)d * M + m];
+    for (int j = 0; j <= r; ++j) {
+      const int sj = src[j];
+      if (sj >= 0) acc += Wj[j] * Elem<T>::ld(kgs + ((int64_t)sj * H + h) * K + d);
+    }
+    Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
+  }
+  // window: dq_swa[d] = scale sum_j dw[j] k_swa_j[d]   (K <= 256: one column per thread)
+  const int lo = p.wl < 0 ? bos : (t - p.wl > bos ? t - p.wl : bos);
+  float acc = 0.f;
+  for (int jb = lo; jb <= t; jb += 256) {
+    const int j = jb + tid;
+    float val = 0.f;
+    if (j <= t) {
+      const float w = dot_row<T>(qs, ksw + ((int64_t)j * H + h) * K, K);
+      const float pi = expf(w - lt);
+      const float dpi = dot_row<T>(dov, vv_ + ((int64_t)j * H + h) * V, V);
+      val = p.scale * (pi * (dpi - delta) + dls * expf(w - ls));
+    }
+    __syncthreads();
+    pw[tid] = val;
+    __syncthreads();
+    const int cnt = (t - jb + 1) < 256 ? (t - jb + 1) : 256;
+    if (tid < K)
+      for (int x = 0; x < cnt; ++x) acc += pw[x] * Elem<T>::ld(ksw + ((int64_t)(jb + x) * H + h) * K + tid);
+  }
+  if (tid < K) Elem<T>::st((T*)p.dq_swa + tq * K + tid, acc);
+}
+
+// ------------------------------------------------------------------------------------------
+// per (chunk, kv-head): intra-chunk matrices ck, cv and the intra-chunk part of ds
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  const int LM = M + 1;
+  float* gcl = lds;              // [BT][LM]
+  float* sl = gcl + BT * LM;     // [BT][LM]
+  float* du = sl + BT * LM;      // [BT][LM]
+  float* pl = du + BT * LM;      // [BT][LM]
+  float* dsl = pl + BT * LM;     // [BT][LM]
+  float* Am = dsl + BT * LM;     // [BT][BT+1]  q_gsa_i . k'_r
+  float* Bm = Am + BT * (BT + 1);   // [BT][BT+1]  do_i . v'_r
+  int* src = (int*)(Bm + BT * (BT + 1));   // [BT]
+  const int tid = threadIdx.x;
+  const int chunk = blockIdx.x, h = blockIdx.y;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const T* ss = (const T*)p.s;
+  if (tid < BT) {
+    const int tl = it * BT + tid - p.shift;
+    src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
+  }
+  __syncthreads();
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
+    const int sj = src[r];
+    sl[r * LM + m] = sj >= 0 ? Elem<T>::ld(ss + ((int64_t)sj * H + h) * M + m) : 0.f;
+    dsl[r * LM + m] = 0.f;
+  }
+  for (int a = 0; a < NG; ++a) {
+    const int hq = h * NG + a;
+    __syncthreads();
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      du[r * LM + m] = p.dus[((int64_t)(c0 + r) * HQ + hq) * M + m];
+      pl[r * LM + m] = p.pp[((int64_t)(c0 + r) * HQ + hq) * M + m];
+    }
+    for (int e = tid; e < R * R; e += 256) {
+      const int i = e / R, r = e - i * R;
+      if (i < r) continue;
+      const int sj = src[r];
+      float av = 0.f, bv = 0.f;
+      if (sj >= 0) {
+        const T* qrow = (const T*)p.q_gsa + ((int64_t)(c0 + i) * HQ + hq) * K;
+        const T* krow = (const T*)p.k_gsa + ((int64_t)sj * H + h) * K;
+        for (int d = 0; d < K; ++d) av += Elem<T>::ld(qrow + d) * Elem<T>::ld(krow + d);
+        const T* drow = (const T*)p.dout + ((int64_t)(c0 + i) * HQ + hq) * V;
+        const T* vrow = (const T*)p.v + ((int64_t)sj * H + h) * V;
+        for (int c = 0; c < V; ++c) bv += Elem<T>::ld(drow + c) * Elem<T>::ld(vrow + c);
+      }
+      Am[i * (BT + 1) + r] = av;
+      Bm[i * (BT + 1) + r] = bv;
+    }
+    __syncthreads();
+    float* ckp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
+    float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
+    for (int e = tid; e < R * R; e += 256) {
+      const int i = e / R, r = e - i * R;
+      if (i < r) continue;
+      float a1 = 0.f, a2 = 0.f;
+      for (int m = 0; m < M; ++m) {
+        const float w = sl[r * LM + m] * expf(gcl[i * LM + m] - gcl[r * LM + m]);
+        a1 += du[i * LM + m] * w;
+        a2 += pl[i * LM + m] * w;
+      }
+      ckp[i * BT + r] = a1;
+      cvp[i * BT + r] = a2;
+    }
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      float acc = 0.f;
+      const float gr = gcl[r * LM + m];
+      for (int i = r; i < R; ++i)
+        acc += (Am[i * (BT + 1) + r] * du[i * LM + m] + Bm[i * (BT + 1) + r] * pl[i * LM + m]) * expf(gcl[i * LM + m] - gr);
+      dsl[r * LM + m] += acc;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    p.dsi[((int64_t)(c0 + r) * H + h) * M + m] = dsl[r * LM + m];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// reverse sweep over the chunks of one (sequence, kv-head), one workgroup per CB state columns.
+// blockIdx.z = 0: k-state (columns d of hk; rows of q_gsa / k_gsa, weights dus, matrix ck, output
+// dk_gsa); 1: v-state (columns c of hv; rows of do / v, weights p, matrix cv, output dvs).
+// E[x][m] is the gradient of the state at the end of the current chunk coming from later chunks.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_state_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int M = p.M, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  const int LM = M + 1;
+  const bool isv = blockIdx.z != 0;
+  const int X = isv ? p.V : p.K;
+  const int nb = isv ? p.nbv : p.nbk;
+  if ((int)blockIdx.y >= nb) return;
+  const int slab = isv ? p.nbk + blockIdx.y : blockIdx.y;
+  const int x0 = blockIdx.y * CB;
+  float* E = lds;                    // [CB][LM]
+  float* En = E + CB * LM;           // [CB][LM]  update accumulated over the heads
+  float* gcl = En + CB * LM;         // [BT][LM]
+  float* dec = gcl + BT * LM;        // [BT][LM]  e^(gl - gc_r)
+  float* sE = dec + BT * LM;         // [BT][LM]  s_r e^(gl - gc_r)
+  float* Lw = sE + BT * LM;          // [BT][LM]  per head: weight_i[m] e^(gc_i[m])
+  float* Cm = Lw + BT * LM;          // [BT][BT+1] per head
+  float* xq = Cm + BT * (BT + 1);    // [BT][CB+1] per head: q_gsa / do columns
+  float* xk = xq + BT * (CB + 1);    // [BT][CB+1] k' / v' columns
+  float* acc = xk + BT * (CB + 1);   // [BT][CB+1] dk' / dv'
+  float* eg = acc + BT * (CB + 1);   // [M] e^(gl)
+  int* src = (int*)(eg + M);         // [BT]
+  const int tid = threadIdx.x;
+  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int L = eos - bos;
+  const int nchunks = (L + BT - 1) / BT;
+  const T* xrow_src = isv ? (const T*)p.v : (const T*)p.k_gsa;     // [T_tot][H][X]
+  const T* qrow_src = isv ? (const T*)p.dout : (const T*)p.q_gsa;  // [T_tot][HQ][X]
+  const float* wsrc = isv ? p.pp : p.dus;
+  const float* csrc = isv ? p.cv : p.ck;
+  const float* dht = isv ? p.dhvt : p.dhkt;
+  for (int e = tid; e < CB * M; e += 256) {
+    const int x = e / M, m = e - x * M;
+    float val = 0.f;
+    if (dht && x0 + x < X)
+      val = isv ? dht[(((int64_t)n * H + h) * M + m) * X + x0 + x] : dht[(((int64_t)n * H + h) * X + x0 + x) * M + m];
+    E[x * LM + m] = val;
+  }
+  for (int it = nchunks - 1; it >= 0; --it) {
+    const int chunk = p.coff[n] + it;
+    const int c0 = bos + it * BT;
+    const int R = (L - it * BT) < BT ? (L - it * BT) : BT;
+    __syncthreads();   // previous chunk finished, E updated
+    if (tid < BT) {
+      const int tl = it * BT + tid - p.shift;
+      src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
+    }
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
+    }
+    for (int e = tid; e < CB * M; e += 256) En[(e / M) * LM + (e % M)] = 0.f;
+    __syncthreads();
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      const float d = expf(gcl[(R - 1) * LM + m] - gcl[r * LM + m]);
+      const int sj = src[r];
+      dec[r * LM + m] = d;
+      sE[r * LM + m] = sj >= 0 ? d * Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m) : 0.f;
+    }
+    for (int m = tid; m < M; m += 256) eg[m] = expf(gcl[(R - 1) * LM + m]);
+    for (int e = tid; e < R * CB; e += 256) {
+      const int r = e / CB, x = e - r * CB;
+      const int sj = src[r];
+      xk[r * (CB + 1) + x] = (sj >= 0 && x0 + x < X) ? Elem<T>::ld(xrow_src + ((int64_t)sj * H + h) * X + x0 + x) : 0.f;
+    }
+    __syncthreads();
+    // inter-chunk parts: dk'_r[x] = sum_m sE_r[m] E[x][m];  ds part = dec_r[m] sum_x k'_r[x] E[x][m]
+    for (int e = tid; e < R * CB; e += 256) {
+      const int r = e / CB, x = e - r * CB;
+      float a = 0.f;
+      for (int m = 0; m < M; ++m) a += sE[r * LM + m] * E[x * LM + m];
+      acc[r * (CB + 1) + x] = a;
+    }
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      float a = 0.f;
+      for (int x = 0; x < CB; ++x) a += xk[r * (CB + 1) + x] * E[x * LM + m];
+      p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a * dec[r * LM + m];
+    }
+    for (int a = 0; a < NG; ++a) {
+      const int hq = h * NG + a;
+      __syncthreads();
+      const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
+      for (int e = tid; e < R * R; e += 256) {
+        const int i = e / R, r = e - i * R;
+        Cm[i * (BT + 1) + r] = i >= r ? cp[i * BT + r] : 0.f;
+      }
+      for (int e = tid; e < R * CB; e += 256) {
+        const int i = e / CB, x = e - i * CB;
+        xq[i * (CB + 1) + x] = (x0 + x < X) ? Elem<T>::ld(qrow_src + ((int64_t)(c0 + i) * HQ + hq) * X + x0 + x) : 0.f;
+      }
+      for (int e = tid; e < R * M; e += 256) {
+        const int i = e / M, m = e - i * M;
+        Lw[i * LM + m] = wsrc[((int64_t)(c0 + i) * HQ + hq) * M + m] * expf(gcl[i * LM + m]);
+      }
+      __syncthreads();
+      for (int e = tid; e < R * CB; e += 256) {
+        const int r = e / CB, x = e - r * CB;
+        float s2 = 0.f;
+        for (int i = r; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Cm[i * (BT + 1) + r];
+        acc[r * (CB + 1) + x] += s2;
+      }
+      for (int e = tid; e < CB * M; e += 256) {
+        const int x = e / M, m = e - x * M;
+        float s2 = 0.f;
+        for (int i = 0; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Lw[i * LM + m];
+        En[x * LM + m] += s2;
+      }
+    }
+    __syncthreads();
+    for (int e = tid; e < R * CB; e += 256) {
+      const int r = e / CB, x = e - r * CB;
+      const int sj = src[r];
+      if (sj < 0 || x0 + x >= X) continue;
+      const float val = acc[r * (CB + 1) + x];
+      if (isv) p.dvs[((int64_t)sj * H + h) * X + x0 + x] = val;
+      else Elem<T>::st((T*)p.dk_gsa + ((int64_t)sj * H + h) * X + x0 + x, val);
+    }
+    for (int e = tid; e < CB * M; e += 256) {
+      const int x = e / M, m = e - x * M;
+      E[x * LM + m] = E[x * LM + m] * eg[m] + En[x * LM + m];
+    }
+  }
+  __syncthreads();
+  float* dh0 = isv ? p.dh0v : p.dh0k;
+  if (dh0)
+    for (int e = tid; e < CB * M; e += 256) {
+      const int x = e / M, m = e - x * M;
+      if (x0 + x >= X) continue;
+      if (isv) dh0[(((int64_t)n * H + h) * M + m) * X + x0 + x] = E[x * LM + m];
+      else dh0[(((int64_t)n * H + h) * X + x0 + x) * M + m] = E[x * LM + m];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// per (sequence, kv-head), one thread per slot: ds and the reverse cumulative sum that is dg;
+// zero gradients for the tokens that never reach the slots (the last `shift` of a sequence)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void bwd_gate_kernel(const BP p) {
+  const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int tid = threadIdx.x;
+  const int nslab = p.nbk + p.nbv;
+  // tokens without a slot-branch row
+  int z0 = eos - p.shift;
+  z0 = z0 < bos ? bos : z0;
+  for (int j = z0; j < eos; ++j) {
+    for (int m = tid; m < M; m += blockDim.x) {
+      Elem<T>::st((T*)p.ds + ((int64_t)j * H + h) * M + m, 0.f);
+      Elem<T>::st((T*)p.dg + ((int64_t)j * H + h) * M + m, 0.f);
+    }
+    for (int d = tid; d < K; d += blockDim.x) Elem<T>::st((T*)p.dk_gsa + ((int64_t)j * H + h) * K + d, 0.f);
+    for (int c = tid; c < V; c += blockDim.x) p.dvs[((int64_t)j * H + h) * V + c] = 0.f;
+  }
+  const int m = tid;
+  if (m >= M) return;
+  float run = 0.f;
+  if (p.dhkt) {
+    const float* a = p.dhkt + ((int64_t)n * H + h) * K * M;
+    const float* b = p.hkT + ((int64_t)n * H + h) * K * M;
+    for (int d = 0; d < K; ++d) run += a[d * M + m] * b[d * M + m];
+  }
+  if (p.dhvt) {
+    const float* a = p.dhvt + (((int64_t)n * H + h) * M + m) * V;
+    const float* b = p.hvT + (((int64_t)n * H + h) * M + m) * V;
+    for (int c = 0; c < V; ++c) run += a[c] * b[c];
+  }
+  for (int t = eos - 1; t - p.shift >= bos; --t) {
+    const int sj = t - p.shift;
+    const int64_t rt = ((int64_t)t * H + h) * M + m;
+    float dstot = p.dsi[rt];
+    for (int b = 0; b < nslab; ++b) dstot += p.dsp[(int64_t)b * p.T_tot * H * M + rt];
+    float x = 0.f;
+    for (int a = 0; a < NG; ++a) x += p.xg[((int64_t)t * HQ + h * NG + a) * M + m];
+    const float sval = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m);
+    run += x - sval * dstot;
+    Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m, dstot);
+    Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, run);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// per (key token, kv-head): dk_swa and dv (window part + slot-branch part)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int K = p.K, V = p.V, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  float* kj = lds;          // [K] scale * k_swa_j
+  float* vj = kj + K;       // [V]
+  float* pwk = vj + V;      // [256] scale * dw
+  float* ppi = pwk + 256;   // [256] pi
+  const int tid = threadIdx.x;
+  const int j = blockIdx.x, h = blockIdx.y;
+  int n = 0;
+  {
+    int lo = 0, hi = p.N - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.cu[mid] <= j) lo = mid; else hi = mid - 1;
+    }
+    n = lo;
+  }
+  const int eos = p.cu[n + 1];
+  int tmax = eos - 1;
+  if (p.wl >= 0 && j + p.wl < tmax) tmax = j + p.wl;
+  for (int i = tid; i < K; i += 256) kj[i] = Elem<T>::ld((const T*)p.k_swa + ((int64_t)j * H + h) * K + i) * p.scale;
+  for (int i = tid; i < V; i += 256) vj[i] = Elem<T>::ld((const T*)p.v + ((int64_t)j * H + h) * V + i);
+  __syncthreads();
+  const int npairs = (tmax - j + 1) * NG;
+  float acck = 0.f, accv = 0.f;
+  for (int pb = 0; pb < npairs; pb += 256) {
+    const int x = pb + tid;
+    float dwv = 0.f, piv = 0.f;
+    if (x < npairs) {
+      const int t = j + x / NG, hq = h * NG + x % NG;
+      const int64_t tq = (int64_t)t * HQ + hq;
+      const float w = dot_row<T>(kj, (const T*)p.q_swa + tq * K, K);
+      const float ls = p.lse_swa[tq];
+      const float lt = logaddexp_f(ls, p.lse_gsa[tq]);
+      piv = expf(w - lt);
+      const float dpi = dot_row<T>(vj, (const T*)p.dout + tq * V, V);
+      dwv = p.scale * (piv * (dpi - p.delta[tq]) + (p.dlse_swa ? p.dlse_swa[tq] * expf(w - ls) : 0.f));
+    }
+    __syncthreads();
+    pwk[tid] = dwv;
+    ppi[tid] = piv;
+    __syncthreads();
+    const int cnt = (npairs - pb) < 256 ? (npairs - pb) : 256;
+    if (tid < K)
+      for (int y = 0; y < cnt; ++y) {
+        const int t = j + (pb + y) / NG, hq = h * NG + (pb + y) % NG;
+        acck += pwk[y] * Elem<T>::ld((const T*)p.q_swa + ((int64_t)t * HQ + hq) * K + tid);
+      }
+    if (tid < V)
+      for (int y = 0; y < cnt; ++y) {
+        const int t = j + (pb + y) / NG, hq = h * NG + (pb + y) % NG;
+        accv += ppi[y] * Elem<T>::ld((const T*)p.dout + ((int64_t)t * HQ + hq) * V + tid);
+      }
+  }
+  if (tid < K) Elem<T>::st((T*)p.dk_swa + ((int64_t)j * H + h) * K + tid, acck);
+  if (tid < V) Elem<T>::st((T*)p.dv + ((int64_t)j * H + h) * V + tid, accv + p.dvs[((int64_t)j * H + h) * V + tid]);
+}
+
+size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
+
+struct BwdPlan {
+  size_t fwd, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, total;
+  int nbk, nbv;
+};
+BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
+  BwdPlan s;
+  s.nbk = (a->K + CB - 1) / CB;
+  s.nbv = (a->V + CB - 1) / CB;
+  size_t off = 0;
+  s.fwd = off; off += aligned(prefill_simple_scratch_bytes(&f));
+  s.hkT = off; off += aligned((size_t)a->N * a->H * a->K * a->M * 4);
+  s.hvT = off; off += aligned((size_t)a->N * a->H * a->M * a->V * 4);
+  const size_t tqm = aligned((size_t)a->T_tot * a->HQ * a->M * 4);
+  s.dus = off; off += tqm;
+  s.pp = off; off += tqm;
+  s.xg = off; off += tqm;
+  s.delta = off; off += aligned((size_t)a->T_tot * a->HQ * 4);
+  const size_t cc = aligned((size_t)a->NT * a->HQ * BT * BT * 4);
+  s.ck = off; off += cc;
+  s.cv = off; off += cc;
+  const size_t thm = (size_t)a->T_tot * a->H * a->M * 4;
+  s.dsi = off; off += aligned(thm);
+  s.dsp = off; off += aligned(thm * (s.nbk + s.nbv));
+  s.dvs = off; off += aligned((size_t)a->T_tot * a->H * a->V * 4);
+  s.total = off;
+  return s;
+}
+
+NhaPrefillArgs forward_args(const NhaPrefillBwdArgs* a) {
+  NhaPrefillArgs f = {};
+  f.q_swa = a->q_swa; f.k_swa = a->k_swa; f.q_gsa = a->q_gsa; f.k_gsa = a->k_gsa;
+  f.v = a->v; f.s = a->s; f.g = a->g;
+  f.h0k = a->h0k; f.h0v = a->h0v;
+  f.cu_seqlens = a->cu_seqlens; f.chunk_indices = a->chunk_indices; f.chunk_offsets = a->chunk_offsets;
+  f.T_tot = a->T_tot; f.N = a->N; f.NT = a->NT; f.HQ = a->HQ; f.H = a->H; f.K = a->K; f.V = a->V; f.M = a->M;
+  f.wl = a->wl; f.shift = a->shift; f.dtype = a->dtype; f.impl = NHA_IMPL_SIMPLE; f.phases = 1;
+  f.scale = a->scale; f.stream = a->stream;
+  return f;
+}
+
+template <typename T>
+int run_bwd(const NhaPrefillBwdArgs* a) {
+  NhaPrefillArgs f = forward_args(a);
+  const BwdPlan sp = plan_bwd(a, f);
+  char* sc = (char*)a->scratch;
+  f.scratch = sc + sp.fwd;
+  f.scratch_bytes = prefill_simple_scratch_bytes(&f);
+  f.hkt = (float*)(sc + sp.hkT);
+  f.hvt = (float*)(sc + sp.hvT);
+  int rc = prefill_simple_impl(&f);
+  if (rc != NHA_OK) return rc;
+
+  BP p;
+  p.q_swa = a->q_swa; p.k_swa = a->k_swa; p.q_gsa = a->q_gsa; p.k_gsa = a->k_gsa;
+  p.v = a->v; p.s = a->s; p.g = a->g; p.o = a->o; p.dout = a->dout;
+  p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa; p.dlse_swa = a->dlse_swa; p.dlse_gsa = a->dlse_gsa;
+  p.dhkt = a->dhkt; p.dhvt = a->dhvt;
+  p.dq_swa = a->dq_swa; p.dk_swa = a->dk_swa; p.dq_gsa = a->dq_gsa; p.dk_gsa = a->dk_gsa;
+  p.dv = a->dv; p.ds = a->ds; p.dg = a->dg; p.dh0k = a->dh0k; p.dh0v = a->dh0v;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
+  // layout of the generic forward state pass: gc | hkc | hvc, each aligned to 256 bytes
+  char* fs = sc + sp.fwd;
+  p.gc = (float*)fs;
+  fs += aligned((size_t)a->T_tot * a->H * a->M * 4);
+  p.hkc = (float*)fs;
+  fs += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
+  p.hvc = (float*)fs;
+  p.hkT = (float*)(sc + sp.hkT); p.hvT = (float*)(sc + sp.hvT);
+  p.dus = (float*)(sc + sp.dus); p.pp = (float*)(sc + sp.pp); p.xg = (float*)(sc + sp.xg);
+  p.delta = (float*)(sc + sp.delta);
+  p.ck = (float*)(sc + sp.ck); p.cv = (float*)(sc + sp.cv);
+  p.dsi = (float*)(sc + sp.dsi); p.dsp = (float*)(sc + sp.dsp); p.dvs = (float*)(sc + sp.dvs);
+  p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.K = a->K; p.V = a->V; p.M = a->M;
+  p.wl = a->wl; p.shift = a->shift; p.nbk = sp.nbk; p.nbv = sp.nbv; p.scale = a->scale;
+  hipStream_t st = (hipStream_t)a->stream;
+  const int K = a->K, V = a->V, M = a->M, LM = M + 1;
+
+  const size_t lds_q = ((size_t)2 * K + V + 4 * M + 3 * BT + 256 + 4) * 4 + BT * 4;
+  const size_t lds_i = ((size_t)5 * BT * LM + 2 * BT * (BT + 1)) * 4 + BT * 4;
+  const size_t lds_s = ((size_t)2 * CB * LM + 4 * BT * LM + BT * (BT + 1) + 3 * BT * (CB + 1) + M) * 4 + BT * 4;
+  const size_t lds_w = ((size_t)K + V + 512) * 4;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e1 = hipFuncSetAttribute((const void*)bwd_intra_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e2 = hipFuncSetAttribute((const void*)bwd_state_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("nha_prefill_bwd: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+      return NHA_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_q, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
+  hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(256), lds_i, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
+  const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
+  hipLaunchKernelGGL((bwd_state_kernel<T>), dim3(a->N * a->H, nbmax, 2), dim3(256), lds_s, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(state sweep)");
+  hipLaunchKernelGGL((bwd_gate_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(gate scan)");
+  hipLaunchKernelGGL((bwd_kv_window_kernel<T>), dim3(a->T_tot, a->H), dim3(256), lds_w, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(key pass)");
+  return NHA_OK;
+}
+
+}  // namespace
+
+size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a) {
+  NhaPrefillArgs f = forward_args(a);
+  return plan_bwd(a, f).total;
+}
+
+bool prefill_bwd_supported(const NhaPrefillBwdArgs* a) { return a->K <= 256 && a->V <= 256 && a->M <= 64 && a->K % 8 == 0 && a->V % 8 == 0; }
+
+int prefill_bwd_impl(const NhaPrefillBwdArgs* a) {
+  if (a->dtype == NHA_DTYPE_BF16) return run_bwd<bf16_t>(a);
+  return run_bwd<float>(a);
+}
+
+}  // namespace nha

@@ -8,7 +8,7 @@ to it at the kv-head count (the reference repeats them to the q-head count first
 The reference takes RMSNorm, RotaryEmbedding, ShortConvolution, the feature maps, rms_norm_linear
 and the unpad helpers from flash-linear-attention, which is not vendored; they are restated here in
 plain PyTorch from their published behaviour (elementwise / projection glue around the hot path).
-Forward only: the op has no backward.
+The layer is trainable: chunk_nha carries its own backward, the glue around it is plain autograd.
 """
 from __future__ import annotations
 
@@ -233,7 +233,6 @@ class NativeHybridAttention(nn.Module):
         self.o_proj = nn.Linear(self.value_dim, self.hidden_size, bias=False)
         self.rotary = RotaryEmbedding(dim=self.head_k_dim, base=self.rope_theta)
 
-    @torch.no_grad()
     def forward(
         self,
         hidden_states: torch.Tensor,

@@ -6,8 +6,9 @@ Same names, argument meaning, return tuples and error behaviour as
   nha_fla/ops/nha/fused_recurrent.py:431-584  fused_recurrent_nha_decode
   nha_fla/ops/nha/fused_recurrent.py:588-682  fused_recurrent_nha
 Differences, all widening: k/v/s/g may carry fewer (kv) heads than q in chunk_nha (the reference
-needs them pre-expanded); window and head-dim limits of the fused prefill are lifted.  Forward
-only: inputs that require grad are rejected (the reference's backward is not part of this path).
+needs them pre-expanded); window and head-dim limits of the fused prefill are lifted.  chunk_nha
+is differentiable (nha_prefill_bwd behind nha_fla/ops/nha/chunk.py:490-564); the inference ops
+reject inputs that require grad, as the reference's do.
 PyTorch is used for device memory and the current stream only; every tensor op on the hot path
 is a HIP kernel behind the C ABI.  There is no CPU / eager fallback.
 """
@@ -23,7 +24,7 @@ from . import _lib
 from .varlen import CHUNK, chunk_tables
 
 __all__ = ["chunk_nha", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
-           "prefill_tables", "nha_prefill"]
+           "prefill_tables", "nha_prefill", "nha_prefill_bwd"]
 
 _DT = {torch.float32: _lib.NHA_DTYPE_F32, torch.bfloat16: _lib.NHA_DTYPE_BF16}
 _IMPL = {None: _lib.NHA_IMPL_AUTO, "auto": _lib.NHA_IMPL_AUTO, "simple": _lib.NHA_IMPL_SIMPLE,
@@ -120,6 +121,84 @@ def nha_prefill(q_swa, k_swa, q_gsa, k_gsa, v, s, g, cu_host: np.ndarray, *, wl:
     return o, lse_swa, lse_gsa, hkt, hvt
 
 
+def nha_prefill_bwd(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, dout, cu_host: np.ndarray, *,
+                    wl: int, shift: int, scale: float, h0=None, dlse_swa=None, dlse_gsa=None, dht=None,
+                    want_dh0: bool = False):
+    """Packed prefill backward on token-major tensors (one nha_prefill_bwd call).  Returns
+    (dq_swa, dk_swa, dq_gsa, dk_gsa, dv, ds, dg, dh0k, dh0v) -- the last two None unless wanted."""
+    lib = _lib.load()
+    T_tot, HQ, K = q_swa.shape
+    H, V, M = k_swa.shape[1], v.shape[-1], s.shape[-1]
+    dev = q_swa.device
+    N = cu_host.size - 1
+    cu_d, idx_d, off_d, NT = prefill_tables(cu_host, dev)
+    f32 = lambda x: None if x is None else x.to(torch.float32).contiguous()
+    h0k, h0v = (None, None) if h0 is None or h0[0] is None else (f32(h0[0]), f32(h0[1]))
+    dhkt, dhvt = (None, None) if dht is None else dht
+    if (dhkt is None) != (dhvt is None):      # one final state unused downstream: its cotangent is zero
+        dhkt = torch.zeros(N, H, K, M, dtype=torch.float32, device=dev) if dhkt is None else dhkt
+        dhvt = torch.zeros(N, H, M, V, dtype=torch.float32, device=dev) if dhvt is None else dhvt
+    dhkt, dhvt, dlse_swa, dlse_gsa = f32(dhkt), f32(dhvt), f32(dlse_swa), f32(dlse_gsa)
+    dout = dout.to(q_swa.dtype).contiguous()
+    outs = [torch.empty_like(x) for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)]
+    dh0k = torch.empty(N, H, K, M, dtype=torch.float32, device=dev) if want_dh0 else None
+    dh0v = torch.empty(N, H, M, V, dtype=torch.float32, device=dev) if want_dh0 else None
+    a = _lib.NhaPrefillBwdArgs()
+    a.q_swa, a.k_swa, a.q_gsa, a.k_gsa = _ptr(q_swa), _ptr(k_swa), _ptr(q_gsa), _ptr(k_gsa)
+    a.v, a.s, a.g = _ptr(v), _ptr(s), _ptr(g)
+    a.o, a.lse_swa, a.lse_gsa = _ptr(o), _ptr(lse_swa), _ptr(lse_gsa)
+    a.h0k, a.h0v = _ptr(h0k), _ptr(h0v)
+    a.dout, a.dlse_swa, a.dlse_gsa, a.dhkt, a.dhvt = _ptr(dout), _ptr(dlse_swa), _ptr(dlse_gsa), _ptr(dhkt), _ptr(dhvt)
+    a.dq_swa, a.dk_swa, a.dq_gsa, a.dk_gsa, a.dv, a.ds, a.dg = [_ptr(x) for x in outs]
+    a.dh0k, a.dh0v = _ptr(dh0k), _ptr(dh0v)
+    a.cu_seqlens, a.chunk_indices, a.chunk_offsets = _ptr(cu_d), _ptr(idx_d), _ptr(off_d)
+    a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = T_tot, N, NT, HQ, H, K, V, M
+    a.wl, a.shift = int(wl), int(shift)
+    a.dtype = _dtype_code(q_swa)
+    a.scale = float(scale)
+    a.stream = _stream(dev)
+    nbytes = lib.nha_prefill_bwd_scratch_bytes(C.byref(a))
+    if nbytes == 0:
+        _lib.check(_lib.NHA_ERR_INVALID)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
+    _lib.check(lib.nha_prefill_bwd(C.byref(a)))
+    return (*outs, dh0k, dh0v)
+
+
+class _ChunkNHAFunction(torch.autograd.Function):
+    """Autograd node of chunk_nha on packed tensors: same outputs and gradient set as
+    ChunkNativeHybridAttentionFunction (nha_fla/ops/nha/chunk.py:364-564)."""
+
+    @staticmethod
+    def forward(ctx, q_swa, k_swa, q_gsa, k_gsa, v, s, g, h0k, h0v, cu_host, wl, shift, scale, want_state, impl):
+        h0 = None if h0k is None else (h0k, h0v)
+        o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(q_swa, k_swa, q_gsa, k_gsa, v, s, g, cu_host, wl=wl, shift=shift,
+                                                    scale=scale, h0=h0, want_state=want_state, impl=impl)
+        ctx.save_for_backward(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, h0k, h0v)
+        ctx.cu_host, ctx.wl, ctx.shift, ctx.scale = cu_host, wl, shift, scale
+        ctx.set_materialize_grads(False)
+        if not want_state:
+            return o, lse_swa, lse_gsa, None, None
+        return o, lse_swa, lse_gsa, hkt, hvt
+
+    @staticmethod
+    def backward(ctx, do, dlse_swa, dlse_gsa, dhkt, dhvt):
+        q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, h0k, h0v = ctx.saved_tensors
+        if do is None:
+            do = torch.zeros_like(o)
+        want_dh0 = h0k is not None and (ctx.needs_input_grad[7] or ctx.needs_input_grad[8])
+        dht = None if dhkt is None and dhvt is None else (dhkt, dhvt)
+        grads = nha_prefill_bwd(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, do, ctx.cu_host,
+                                wl=ctx.wl, shift=ctx.shift, scale=ctx.scale,
+                                h0=None if h0k is None else (h0k, h0v), dlse_swa=dlse_swa, dlse_gsa=dlse_gsa,
+                                dht=dht, want_dh0=want_dh0)
+        dh0k, dh0v = grads[7], grads[8]
+        if dh0k is not None:
+            dh0k, dh0v = dh0k.to(h0k.dtype), dh0v.to(h0v.dtype)
+        return (*grads[:7], dh0k, dh0v, None, None, None, None, None, None)
+
+
 def _flat(x):
     return x.reshape(x.shape[0] * x.shape[1], *x.shape[2:]).contiguous()
 
@@ -160,7 +239,6 @@ def chunk_nha(
         )
     assert q_swa.dim() == 4, "Expected [B, T, H, D] for input"
     _need_cuda(q_swa, k_swa, q_gsa, k_gsa, v, s, g)
-    _no_grad_inputs("chunk_nha", q_swa, k_swa, q_gsa, k_gsa, v, s, g)
     B, T, HQ, D = q_swa.shape
     H = k_swa.shape[2]
     if scale is None:
@@ -180,9 +258,14 @@ def chunk_nha(
         cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)          # chunk.py:660
     dt = q_swa.dtype
     args = [_flat(x.to(dt)) for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)]
-    o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(
-        *args, cu_host, wl=window_size_left, shift=gsa_kv_shift, scale=scale,
-        h0=initial_state, want_state=output_final_state, impl=impl)
+    h0 = (None, None) if initial_state is None or initial_state[0] is None else tuple(initial_state)
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (*args, *h0)):
+        o, lse_swa, lse_gsa, hkt, hvt = _ChunkNHAFunction.apply(
+            *args, h0[0], h0[1], cu_host, window_size_left, gsa_kv_shift, scale, output_final_state, impl)
+    else:
+        o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(
+            *args, cu_host, wl=window_size_left, shift=gsa_kv_shift, scale=scale,
+            h0=initial_state, want_state=output_final_state, impl=impl)
     o = o.view(B, T, HQ, -1)
     lse_swa = lse_swa.view(B, T, HQ)
     lse_gsa = lse_gsa.view(B, T, HQ)

@@ -38,6 +38,7 @@ __all__ = [
     "gsa_step",
     "prefill_ref",
     "prefill_chunked_ref",
+    "prefill_grad_ref",
     "decode_ref",
     "decode_ring_ref",
     "fused_recurrent_ref",
@@ -240,6 +241,63 @@ def prefill_chunked_ref(q_swa, k_swa, q_gsa, k_gsa, v, s, g, *, window_size_left
         hk = hk * glast.exp()[:, :, None, :] + torch.einsum("bjhk,bjhm->bhkm", kg[:, c0:c1], sdec)
         hv = hv * glast.exp()[:, :, :, None] + torch.einsum("bjhm,bjhv->bhmv", sdec, vg[:, c0:c1])
     return o, lse_swa, lse_gsa, hk, hv
+
+
+def prefill_grad_ref(q_swa, k_swa, q_gsa, k_gsa, v, s, g, do, *, window_size_left, gsa_kv_shift=0,
+                     cu_seqlens=None, initial_state=None, scale=None, dlse_swa=None, dlse_gsa=None,
+                     dht=None, dtype=torch.float64):
+    """Gradients of the prefill op: reverse-mode differentiation of the per-token recurrence of
+    ``prefill_ref`` itself (no second formula), which is what
+    ChunkNativeHybridAttentionFunction.backward (nha_fla/ops/nha/chunk.py:490-564) has to equal:
+    window-branch gradients (:499-511), slot-branch gradients with the merged-softmax coupling
+    (:514-530), un-shifting of the slot-branch gradients (:533-543), dv accumulated over both
+    branches (:559), initial-state gradients.  The scalar differentiated is
+    ``<o, do> + <lse_swa, dlse_swa> + <lse_gsa, dlse_gsa> + <hkt, dht[0]> + <hvt, dht[1]>``.
+    Pinned by central finite differences of ``prefill_ref`` (tests/test_oracle_pins.py).
+
+    Returns a dict with dq_swa, dk_swa, dq_gsa, dk_gsa, dv, ds, dg and, when an initial state is
+    given, dh0k, dh0v (all ``dtype``, shapes of the corresponding inputs)."""
+    B, T, HQ, K = q_swa.shape
+    H = k_swa.shape[2]
+    M = s.shape[-1]
+    V = v.shape[-1]
+    if scale is None:
+        scale = K ** -0.5
+    leaf = lambda x: x.detach().to("cpu", dtype).clone().requires_grad_(True)
+    names = ["q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g"]
+    xs = [leaf(x) for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)]
+    h0 = None
+    if initial_state is not None:
+        h0 = (leaf(initial_state[0]), leaf(initial_state[1]))
+    cu = [0, T] if cu_seqlens is None else [int(c) for c in cu_seqlens]
+    total = torch.zeros((), dtype=dtype)
+    seqs = [(b, 0, T, b) for b in range(B)] if cu_seqlens is None else \
+        [(0, cu[n], cu[n + 1], n) for n in range(len(cu) - 1)]
+    cst = lambda x: None if x is None else x.detach().to("cpu", dtype)
+    do, dlse_swa, dlse_gsa = cst(do), cst(dlse_swa), cst(dlse_gsa)
+    dht = None if dht is None else (cst(dht[0]), cst(dht[1]))
+    for b, st, en, n in seqs:
+        sl = slice(st, en)
+        part = [x[b:b + 1, sl] for x in xs]
+        if h0 is not None:
+            hk, hv = h0[0][n:n + 1], h0[1][n:n + 1]
+        else:
+            hk = torch.zeros(1, H, K, M, dtype=dtype)
+            hv = torch.zeros(1, H, M, V, dtype=dtype)
+        o, ls, lg, hk, hv = _prefill_equal_len(*part, window_size_left, gsa_kv_shift, scale, hk, hv)
+        total = total + (o * do[b:b + 1, sl]).sum()
+        if dlse_swa is not None:
+            total = total + (ls * dlse_swa[b:b + 1, sl]).sum()
+        if dlse_gsa is not None:
+            total = total + (lg * dlse_gsa[b:b + 1, sl]).sum()
+        if dht is not None:
+            total = total + (hk[0] * dht[0][n]).sum() + (hv[0] * dht[1][n]).sum()
+    wrt = xs + (list(h0) if h0 is not None else [])
+    grads = torch.autograd.grad(total, wrt, allow_unused=True)
+    out = {"d" + nm: (gr if gr is not None else torch.zeros_like(x)) for nm, gr, x in zip(names, grads[:7], xs)}
+    if h0 is not None:
+        out["dh0k"], out["dh0v"] = grads[7], grads[8]
+    return out
 
 
 def decode_ref(q, k, v, g, sw_k, sw_v, *, sq=None, s=None, cos=None, sin=None,

@@ -31,8 +31,10 @@ def test_struct_sizes_match_the_header(tmp_path):
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     probes = [("NhaPrefillArgs", f) for f in ("q_swa", "scratch_bytes", "T_tot", "phases", "scale", "stream")]
     probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream", "count_next")]
+    probes += [("NhaPrefillBwdArgs", f) for f in ("q_swa", "o", "dout", "dhvt", "dq_swa", "dg", "dh0v", "cu_seqlens",
+                                                  "scratch_bytes", "T_tot", "dtype", "scale", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
-           'printf("%zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs));']
+           'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
     src += ['return 0; }']
     cfile = tmp_path / "probe.c"
@@ -41,7 +43,8 @@ def test_struct_sizes_match_the_header(tmp_path):
     subprocess.run(["gcc", "-I", os.path.join(root, "include"), str(cfile), "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert int(out[0]) == C.sizeof(_lib.NhaPrefillArgs) and int(out[1]) == C.sizeof(_lib.NhaDecodeArgs)
-    for (t, f), off in zip(probes, out[2:]):
+    assert int(out[2]) == C.sizeof(_lib.NhaPrefillBwdArgs)
+    for (t, f), off in zip(probes, out[3:]):
         assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 
@@ -50,6 +53,14 @@ def test_argument_validation_without_gpu():
     a = _lib.NhaPrefillArgs()
     assert lib.nha_prefill_fwd(C.byref(a)) == _lib.NHA_ERR_INVALID
     assert b"non-positive" in lib.nha_last_error()
+    b = _lib.NhaPrefillBwdArgs()
+    assert lib.nha_prefill_bwd(C.byref(b)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
+    b.T_tot, b.N, b.NT, b.HQ, b.H, b.K, b.V, b.M = 64, 1, 1, 3, 2, 64, 64, 64
+    assert lib.nha_prefill_bwd(C.byref(b)) == _lib.NHA_ERR_INVALID and b"multiple" in lib.nha_last_error()
+    assert lib.nha_prefill_bwd_scratch_bytes(C.byref(b)) == 0
+    b.HQ = 4
+    assert lib.nha_prefill_bwd(C.byref(b)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    assert lib.nha_prefill_bwd_scratch_bytes(C.byref(b)) > 0
     d = _lib.NhaDecodeArgs()
     assert lib.nha_decode_step(C.byref(d)) == _lib.NHA_ERR_INVALID
     d.B = d.H = d.K = d.V = d.M = d.W = 8

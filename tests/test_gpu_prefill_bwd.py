@@ -1,0 +1,107 @@
+"""Backward of chunk_nha on the GPU (nha_prefill_bwd through autograd) against reverse-mode
+differentiation of the fp64 recurrence (oracle.nha_ref.prefill_grad_ref, pinned by finite
+differences on the CPU).  The inputs the oracle sees are the rounded tensors the kernels see.
+
+Tolerances: fp32 tensors 1e-4 of each gradient's scale (max norm), as for the forward; bf16 tensors
+(gradients are returned in bf16, o and do enter in bf16): relative L2 error <= 1e-2 -- half the
+reference's own 2e-2 relative-L2 bar against fp64 (scripts/verify_opt_parity.py:753) -- and every
+element within 3e-2 of the gradient's max norm."""
+import pytest
+import torch
+
+from oracle import nha_ref as R
+from tests.util import prefill_inputs
+
+pytestmark = pytest.mark.gpu
+
+KEYS = ["q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g"]
+BF = torch.bfloat16
+
+
+def check_grad(name, got, ref, dtype):
+    got = got.detach().double().cpu()
+    ref = ref.detach().double()
+    assert got.shape == ref.shape, (name, got.shape, ref.shape)
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    scale = max(ref.abs().max().item(), 1e-30)
+    err = (got - ref).abs().max().item()
+    if dtype == BF:
+        rel = ((got - ref).norm() / max(ref.norm().item(), 1e-30)).item()
+        assert rel <= 1e-2, f"{name}: relative L2 error {rel:.3e}"
+        assert err <= 3e-2 * scale, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
+    else:
+        assert err <= 1e-4 * scale, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
+
+
+def run_bwd_case(tag, d, *, wl, shift, dtype, cu=None, scale=None, with_lse=False, with_dht=False, impl=None, seed=0):
+    from nha_amd import chunk_nha
+    print("case", tag, dtype, flush=True)
+    gen = torch.Generator().manual_seed(seed)
+    B, T, HQ, _ = d["q_swa"].shape
+    H, V, M = d["v"].shape[2], d["v"].shape[3], d["s"].shape[3]
+    N = B if cu is None else len(cu) - 1
+    K = d["q_swa"].shape[3]
+    do = torch.randn(B, T, HQ, V, generator=gen).to(dtype)
+    dl1 = torch.randn(B, T, HQ, generator=gen) if with_lse else None
+    dl2 = torch.randn(B, T, HQ, generator=gen) if with_lse else None
+    dht = (torch.randn(N, H, K, M, generator=gen), torch.randn(N, H, M, V, generator=gen)) if with_dht else None
+    h0 = d.get("h0")
+    x = [d[k].cuda().requires_grad_(True) for k in KEYS]
+    h0c = None if h0 is None else tuple(t.cuda().requires_grad_(True) for t in h0)
+    out = chunk_nha(*x, cu_seqlens=None if cu is None else torch.tensor(cu, dtype=torch.int32).cuda(), scale=scale,
+                    window_size_left=wl, gsa_kv_shift=shift, initial_state=h0c, output_final_state=with_dht, impl=impl)
+    loss = (out[0].float() * do.cuda().float()).sum()
+    if with_lse:
+        loss = loss + (out[1] * dl1.cuda()).sum() + (out[2] * dl2.cuda()).sum()
+    if with_dht:
+        loss = loss + (out[3][0] * dht[0].cuda()).sum() + (out[3][1] * dht[1].cuda()).sum()
+    loss.backward()
+    G = R.prefill_grad_ref(*[d[k] for k in KEYS], do, window_size_left=wl, gsa_kv_shift=shift, cu_seqlens=cu,
+                           initial_state=h0, scale=scale, dlse_swa=dl1, dlse_gsa=dl2, dht=dht)
+    for k, t in zip(KEYS, x):
+        assert t.grad is not None and t.grad.dtype == dtype, k
+        check_grad(f"{tag} d{k}", t.grad, G["d" + k], dtype)
+    if h0 is not None:
+        # fp32 tensors, but computed from the same rounded o / do as the other gradients
+        check_grad(f"{tag} dh0k", h0c[0].grad, G["dh0k"], dtype)
+        check_grad(f"{tag} dh0v", h0c[1].grad, G["dh0v"], dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, BF])
+def test_bwd_small_grid(dtype):
+    """Both call conventions, GQA and not, chunk-ragged lengths, with and without initial state."""
+    seed = 7000
+    for T, W, NG, M in ((63, 32, 1, 16), (130, 64, 4, 64), (257, 100, 2, 64)):
+        H, K, V = 2, 64, 64
+        d = prefill_inputs(seed, 2, T, H * NG, H, K, V, M, dtype=dtype, qk_scale=1.0, with_state=(T == 130))
+        seed += 1
+        run_bwd_case(f"T{T} shifted", d, wl=W - 1, shift=W, dtype=dtype, scale=K ** -0.5)
+        run_bwd_case(f"T{T} layer", d, wl=W, shift=0, dtype=dtype, scale=K ** -0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, BF])
+def test_bwd_all_cotangents_and_varlen(dtype):
+    """Cotangents on both LSEs and on the final states, packed sequences (one shorter than the
+    shift, one ending mid-chunk), initial states, K != V."""
+    cu = [0, 70, 90, 300, 333]
+    d = prefill_inputs(7100, 1, cu[-1], 4, 2, 32, 64, 32, dtype=dtype, qk_scale=1.0, with_state=True, N=4)
+    run_bwd_case("varlen shifted", d, wl=31, shift=32, dtype=dtype, cu=cu, scale=32 ** -0.5, with_lse=True, with_dht=True)
+    run_bwd_case("varlen layer", d, wl=48, shift=0, dtype=dtype, cu=cu, scale=32 ** -0.5, with_lse=True, with_dht=True)
+    run_bwd_case("varlen unbounded window", d, wl=-1, shift=5, dtype=dtype, cu=cu, scale=32 ** -0.5, with_dht=True)
+
+
+def test_bwd_head_dims_of_the_models():
+    """D = 128 (hybrid LLM heads, 4 query heads per kv-head) and D = 256 (the 340M layer)."""
+    d = prefill_inputs(7200, 1, 200, 8, 2, 128, 128, 64, dtype=BF, qk_scale=128 ** -0.5, gate_div=1.0, gate_mean=-1.0)
+    run_bwd_case("D128 GQA", d, wl=63, shift=64, dtype=BF, impl="mfma")
+    d = prefill_inputs(7201, 2, 150, 2, 2, 256, 256, 64, dtype=BF, qk_scale=256 ** -0.5)
+    run_bwd_case("D256", d, wl=64, shift=0, dtype=BF, impl="mfma")
+
+
+def test_bwd_rejects_unsupported_shapes():
+    from nha_amd import NhaError, chunk_nha
+    d = prefill_inputs(7300, 1, 64, 2, 2, 64, 64, 128, dtype=torch.float32)
+    x = [d[k].cuda().requires_grad_(True) for k in KEYS]
+    out = chunk_nha(*x, window_size_left=16, gsa_kv_shift=0)
+    with pytest.raises(NhaError, match="M <= 64"):
+        out[0].sum().backward()

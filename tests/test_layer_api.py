@@ -50,3 +50,55 @@ def test_layer_forward_matches_oracle_layer():
     ref = y @ w["o_proj.weight"].T
     err = (o.cpu().double() - ref).abs().max().item()
     assert err <= 3e-2 * max(1.0, ref.abs().max().item()), err
+
+
+def _oracle_layer(w, xc, H, HKV, M, W, D):
+    """fp64 restatement of nha_fla/layers/nha.py:209-278 (differentiable: built on the oracle's
+    per-token recurrence without detaching)."""
+    from oracle import nha_ref as R
+    T = xc.shape[1]
+    q = (xc @ w["q_proj.weight"].T).unflatten(-1, (H, D))
+    k = (xc @ w["k_proj.weight"].T).unflatten(-1, (HKV, D))
+    v = F.silu((xc @ w["v_proj.weight"].T).unflatten(-1, (HKV, D)))
+    f = F.logsigmoid((xc @ w["f_proj.weight"].T).unflatten(-1, (HKV, M))) / 8
+    s, g = 1 - f.exp(), f
+    pos = torch.arange(T, dtype=torch.float64)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))
+    fr = torch.outer(pos, inv)
+    cos, sin = torch.cat([fr.cos(), fr.cos()], -1)[None], torch.cat([fr.sin(), fr.sin()], -1)[None]
+    q_swa, k_swa = R.rope_rotate_half(q, cos, sin), R.rope_rotate_half(k, cos, sin)
+    B = xc.shape[0]
+    hk = torch.zeros(B, HKV, D, M, dtype=torch.float64)
+    hv = torch.zeros(B, HKV, M, D, dtype=torch.float64)
+    out = R._prefill_equal_len(q_swa, k_swa, F.silu(q), F.silu(k), v, s, g, W, 0, 1.0, hk, hv)[0]
+    y = F.silu(out.flatten(-2))
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + 1e-5) * w["g_norm.weight"]
+    return y @ w["o_proj.weight"].T
+
+
+@pytest.mark.gpu
+def test_layer_training_step_matches_oracle_layer():
+    """One forward + backward through the layer in fp32: the gradient of every parameter and of the
+    input against autograd through the fp64 restatement (1e-3 of each gradient's scale: fp32
+    projections and normalisation around the op)."""
+    from nha_amd.layer import NativeHybridAttention
+    torch.manual_seed(1)
+    hid, H, HKV, M, W = 128, 4, 2, 32, 16
+    D = hid // H
+    layer = NativeHybridAttention(hidden_size=hid, num_heads=H, num_kv_heads=HKV, num_slots=M, layer_idx=0,
+                                  window_size=W, scale=1.0).cuda().float().train()
+    x = (torch.randn(2, 100, hid) * 0.5).cuda().requires_grad_(True)
+    tgt = torch.randn(2, 100, hid)
+    o, _, _ = layer(x)
+    (o * tgt.cuda()).sum().backward()
+    w = {k: v.detach().cpu().double().requires_grad_(True) for k, v in layer.state_dict().items()}
+    xc = x.detach().cpu().double().requires_grad_(True)
+    ref = _oracle_layer(w, xc, H, HKV, M, W, D)
+    (ref * tgt.double()).sum().backward()
+    assert (o.detach().cpu().double() - ref.detach()).abs().max() <= 1e-3 * max(1.0, ref.abs().max().item())
+    named = dict(layer.named_parameters())
+    for name, p in list(named.items()) + [("input", x)]:
+        rg = xc.grad if name == "input" else w[name].grad
+        assert p.grad is not None, name
+        err = (p.grad.cpu().double() - rg).abs().max().item()
+        assert err <= 1e-3 * max(rg.abs().max().item(), 1e-6), (name, err, rg.abs().max().item())

@@ -275,3 +275,50 @@ def test_fused_recurrent_consistent_with_decode():
     assert torch.allclose(p2[:, 0], pw, atol=1e-12)
     o_full = o2[:, 0] + torch.einsum("bqw,bwqv->bqv", p2[:, 0], swv.repeat_interleave(NG, 2))
     assert torch.allclose(o_full, o[:, 0], atol=1e-12) and torch.allclose(hk, hk2) and torch.allclose(hv, hv2)
+
+
+@pytest.mark.parametrize("wl,shift,varlen", [(2, 3, False), (3, 0, False), (-1, 1, False), (2, 3, True), (4, 0, True)])
+def test_gradients_match_finite_differences(wl, shift, varlen):
+    """prefill_grad_ref against central differences of prefill_ref (the forward is pinned above;
+    this pins the plumbing of the gradient oracle: cotangents of o, both LSEs and the final states,
+    every input incl. the initial state, batched and packed).  A dropped cotangent, a wrong
+    sequence slice or a missing un-shift fails it."""
+    torch.manual_seed(11)
+    f64 = torch.float64
+    HQ, H, K, V, M = 4, 2, 4, 6, 3
+    if varlen:
+        cu, B, T = [0, 5, 6, 13], 1, 13        # one sequence shorter than the shift
+        N = 3
+    else:
+        cu, B, T = None, 2, 9
+        N = B
+    r = lambda *s: torch.randn(*s, dtype=f64)
+    g = F.logsigmoid(r(B, T, H, M))
+    x = [r(B, T, HQ, K), r(B, T, H, K), r(B, T, HQ, K), r(B, T, H, K), r(B, T, H, V), 1 - g.exp() + 0.1 * r(B, T, H, M), g]
+    h0 = (r(N, H, K, M), r(N, H, M, V))
+    do, dl1, dl2 = r(B, T, HQ, V), r(B, T, HQ), r(B, T, HQ)
+    dht = (r(N, H, K, M), r(N, H, M, V))
+    kw = dict(window_size_left=wl, gsa_kv_shift=shift, cu_seqlens=cu)
+    G = R.prefill_grad_ref(*x, do, initial_state=h0, dlse_swa=dl1, dlse_gsa=dl2, dht=dht, **kw)
+
+    def f(xs, h):
+        o, ls, lg, hk, hv = R.prefill_ref(*xs, initial_state=h, **kw)
+        return float((o * do).sum() + (ls * dl1).sum() + (lg * dl2).sum() + (hk * dht[0]).sum() + (hv * dht[1]).sum())
+
+    eps = 1e-6
+    names = ["q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g"]
+    gen = torch.Generator().manual_seed(5)
+    for i, nm in enumerate(names + ["h0k", "h0v"]):
+        tgt = x[i] if i < 7 else h0[i - 7]
+        for _ in range(6):
+            idx = tuple(int(torch.randint(0, d, (1,), generator=gen)) for d in tgt.shape)
+            xp, xm = [t.clone() for t in x], [t.clone() for t in x]
+            hp, hm = [t.clone() for t in h0], [t.clone() for t in h0]
+            (xp[i] if i < 7 else hp[i - 7])[idx] += eps
+            (xm[i] if i < 7 else hm[i - 7])[idx] -= eps
+            fd = (f(xp, tuple(hp)) - f(xm, tuple(hm))) / (2 * eps)
+            an = float(G["d" + nm][idx])
+            assert abs(fd - an) <= 1e-6 * max(1.0, abs(fd)), (nm, idx, fd, an)
+    if varlen and shift >= 1:
+        # tokens of a sequence no longer than the shift never reach the slots: no slot-branch gradient
+        assert G["dk_gsa"][0, 5:6].abs().max() == 0 and G["dg"][0, 5:6].abs().max() == 0
