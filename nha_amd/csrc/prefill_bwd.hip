@@ -19,7 +19,7 @@
 // Launches: forward state pass (chunk-start states, gate cumsums) -> bwd_q_kernel (per token: dq's and
 // the per-token vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra
 // part of ds) -> bwd_state_kernel (reverse sweep over chunks, one workgroup per 32 state columns:
-// dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_kernel (reverse scan: ds, dg)
+// dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_*_kernel (reverse scan: ds, dg)
 // -> bwd_kv_window_kernel (per key: dk_swa, dv).
 #include "common.h"
 
@@ -46,6 +46,7 @@ struct BP {
   float *dsi;             // [T_tot][H][M]     intra-chunk part of ds, indexed by row token
   float *dsp;             // [nbk+nbv][T_tot][H][M]  inter-chunk part of ds per column block
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
+  float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
   int T_tot, N, NT, HQ, H, K, V, M, wl, shift, nbk, nbv;
   float scale;
 };
@@ -424,18 +425,47 @@ __global__ __launch_bounds__(256) void bwd_state_kernel(const BP p) {
 }
 
 // ------------------------------------------------------------------------------------------
-// per (sequence, kv-head), one thread per slot: ds and the reverse cumulative sum that is dg;
-// zero gradients for the tokens that never reach the slots (the last `shift` of a sequence)
+// ds and dg.  dg is a reverse cumulative sum over the rows of a sequence; three small launches:
+// per chunk the summand, ds and the chunk-local sums (bwd_gate_local_kernel), per sequence the
+// sums of all later chunks plus the end term (bwd_gate_scan_kernel, which also zeroes the
+// gradients of the tokens that never reach the slots: the last `shift` of a sequence), per chunk
+// the final values (bwd_gate_final_kernel).  One thread per slot.
 // ------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void bwd_gate_kernel(const BP p) {
-  const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
+__global__ void bwd_gate_local_kernel(const BP p) {
+  const int M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
+  const int chunk = blockIdx.x, h = blockIdx.y;
+  const int m = threadIdx.x;
+  if (m >= M) return;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const int nslab = p.nbk + p.nbv;
+  float run = 0.f;
+  for (int r = R - 1; r >= 0; --r) {
+    const int t = c0 + r, sj = t - p.shift;
+    if (sj < bos) break;
+    const int64_t rt = ((int64_t)t * H + h) * M + m;
+    float dstot = p.dsi[rt];
+    for (int b = 0; b < nslab; ++b) dstot += p.dsp[(int64_t)b * p.T_tot * H * M + rt];
+    float x = 0.f;
+    for (int a = 0; a < NG; ++a) x += p.xg[((int64_t)t * HQ + h * NG + a) * M + m];
+    const float sval = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m);
+    run += x - sval * dstot;
+    Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m, dstot);
+    p.dsi[rt] = run;   // chunk-local reverse cumulative sum
+  }
+  p.gtot[((int64_t)chunk * H + h) * M + m] = run;
+}
+
+template <typename T>
+__global__ void bwd_gate_scan_kernel(const BP p) {
+  const int K = p.K, V = p.V, M = p.M, H = p.H;
   const int n = blockIdx.x / H, h = blockIdx.x % H;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int tid = threadIdx.x;
-  const int nslab = p.nbk + p.nbv;
-  // tokens without a slot-branch row
   int z0 = eos - p.shift;
   z0 = z0 < bos ? bos : z0;
   for (int j = z0; j < eos; ++j) {
@@ -448,7 +478,7 @@ __global__ void bwd_gate_kernel(const BP p) {
   }
   const int m = tid;
   if (m >= M) return;
-  float run = 0.f;
+  float run = 0.f;   // <dh_T, h_T>: what the gates past the end of the sequence would receive
   if (p.dhkt) {
     const float* a = p.dhkt + ((int64_t)n * H + h) * K * M;
     const float* b = p.hkT + ((int64_t)n * H + h) * K * M;
@@ -459,17 +489,29 @@ __global__ void bwd_gate_kernel(const BP p) {
     const float* b = p.hvT + (((int64_t)n * H + h) * M + m) * V;
     for (int c = 0; c < V; ++c) run += a[c] * b[c];
   }
-  for (int t = eos - 1; t - p.shift >= bos; --t) {
-    const int sj = t - p.shift;
-    const int64_t rt = ((int64_t)t * H + h) * M + m;
-    float dstot = p.dsi[rt];
-    for (int b = 0; b < nslab; ++b) dstot += p.dsp[(int64_t)b * p.T_tot * H * M + rt];
-    float x = 0.f;
-    for (int a = 0; a < NG; ++a) x += p.xg[((int64_t)t * HQ + h * NG + a) * M + m];
-    const float sval = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m);
-    run += x - sval * dstot;
-    Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m, dstot);
-    Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, run);
+  const int nchunks = (eos - bos + BT - 1) / BT;
+  for (int it = nchunks - 1; it >= 0; --it) {
+    const int64_t idx = ((int64_t)(p.coff[n] + it) * H + h) * M + m;
+    const float tot = p.gtot[idx];
+    p.gtot[idx] = run;
+    run += tot;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_gate_final_kernel(const BP p) {
+  const int M = p.M, H = p.H;
+  const int chunk = blockIdx.x, h = blockIdx.y;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  for (int e = threadIdx.x; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    const int t = c0 + r, sj = t - p.shift;
+    if (sj < bos) continue;
+    const float val = p.dsi[((int64_t)t * H + h) * M + m] + p.gtot[((int64_t)chunk * H + h) * M + m];
+    Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, val);
   }
 }
 
@@ -540,7 +582,8 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, total;
+  size_t fwd, mfma, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, total;
+  bool use_mfma;
   int nbk, nbv;
 };
 BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
@@ -549,6 +592,10 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   s.nbv = (a->V + CB - 1) / CB;
   size_t off = 0;
   s.fwd = off; off += aligned(prefill_simple_scratch_bytes(&f));
+  // bf16 shapes the matrix-core state pass covers: recompute the states with it and convert
+  s.use_mfma = prefill_mfma_supported(&f);
+  s.mfma = off;
+  if (s.use_mfma) off += aligned(prefill_mfma_scratch_bytes(&f));
   s.hkT = off; off += aligned((size_t)a->N * a->H * a->K * a->M * 4);
   s.hvT = off; off += aligned((size_t)a->N * a->H * a->M * a->V * 4);
   const size_t tqm = aligned((size_t)a->T_tot * a->HQ * a->M * 4);
@@ -563,6 +610,7 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   s.dsi = off; off += aligned(thm);
   s.dsp = off; off += aligned(thm * (s.nbk + s.nbv));
   s.dvs = off; off += aligned((size_t)a->T_tot * a->H * a->V * 4);
+  s.gtot = off; off += aligned((size_t)a->NT * a->H * a->M * 4);
   s.total = off;
   return s;
 }
@@ -584,11 +632,27 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   NhaPrefillArgs f = forward_args(a);
   const BwdPlan sp = plan_bwd(a, f);
   char* sc = (char*)a->scratch;
-  f.scratch = sc + sp.fwd;
-  f.scratch_bytes = prefill_simple_scratch_bytes(&f);
   f.hkt = (float*)(sc + sp.hkT);
   f.hvt = (float*)(sc + sp.hvT);
-  int rc = prefill_simple_impl(&f);
+  // layout of the generic forward state pass: gc | hkc | hvc, each aligned to 256 bytes
+  char* fs = sc + sp.fwd;
+  float* gc = (float*)fs;
+  fs += aligned((size_t)a->T_tot * a->H * a->M * 4);
+  float* hkc = (float*)fs;
+  fs += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
+  float* hvc = (float*)fs;
+  int rc;
+  if (sp.use_mfma) {
+    f.impl = NHA_IMPL_MFMA;
+    f.scratch = sc + sp.mfma;
+    f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
+    rc = prefill_mfma_impl(&f);
+    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, hvc);
+  } else {
+    f.scratch = sc + sp.fwd;
+    f.scratch_bytes = prefill_simple_scratch_bytes(&f);
+    rc = prefill_simple_impl(&f);
+  }
   if (rc != NHA_OK) return rc;
 
   BP p;
@@ -599,18 +663,13 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.dq_swa = a->dq_swa; p.dk_swa = a->dk_swa; p.dq_gsa = a->dq_gsa; p.dk_gsa = a->dk_gsa;
   p.dv = a->dv; p.ds = a->ds; p.dg = a->dg; p.dh0k = a->dh0k; p.dh0v = a->dh0v;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
-  // layout of the generic forward state pass: gc | hkc | hvc, each aligned to 256 bytes
-  char* fs = sc + sp.fwd;
-  p.gc = (float*)fs;
-  fs += aligned((size_t)a->T_tot * a->H * a->M * 4);
-  p.hkc = (float*)fs;
-  fs += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
-  p.hvc = (float*)fs;
+  p.gc = gc; p.hkc = hkc; p.hvc = hvc;
   p.hkT = (float*)(sc + sp.hkT); p.hvT = (float*)(sc + sp.hvT);
   p.dus = (float*)(sc + sp.dus); p.pp = (float*)(sc + sp.pp); p.xg = (float*)(sc + sp.xg);
   p.delta = (float*)(sc + sp.delta);
   p.ck = (float*)(sc + sp.ck); p.cv = (float*)(sc + sp.cv);
   p.dsi = (float*)(sc + sp.dsi); p.dsp = (float*)(sc + sp.dsp); p.dvs = (float*)(sc + sp.dvs);
+  p.gtot = (float*)(sc + sp.gtot);
   p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.K = a->K; p.V = a->V; p.M = a->M;
   p.wl = a->wl; p.shift = a->shift; p.nbk = sp.nbk; p.nbv = sp.nbv; p.scale = a->scale;
   hipStream_t st = (hipStream_t)a->stream;
@@ -637,7 +696,9 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
   hipLaunchKernelGGL((bwd_state_kernel<T>), dim3(a->N * a->H, nbmax, 2), dim3(256), lds_s, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state sweep)");
-  hipLaunchKernelGGL((bwd_gate_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
+  hipLaunchKernelGGL((bwd_gate_local_kernel<T>), dim3(a->NT, a->H), dim3(64), 0, st, p);
+  hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
+  hipLaunchKernelGGL((bwd_gate_final_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(gate scan)");
   hipLaunchKernelGGL((bwd_kv_window_kernel<T>), dim3(a->T_tot, a->H), dim3(256), lds_w, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(key pass)");

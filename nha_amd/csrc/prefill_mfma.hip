@@ -1131,6 +1131,30 @@ int launch_repair(const MP& p, hipStream_t st) {
   return NHA_OK;
 }
 
+// ==========================================================================================
+// fp32 copies of what the state pass left in the scratch, in the layout of the generic kernels
+// (true chunk-start states hk [K][M], hv [M][V]; gate cumsums per row token): the backward pass
+// reads those
+// ==========================================================================================
+template <int D>
+__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hvc) {
+  const int chunk = blockIdx.x, h = blockIdx.y, H = p.H;
+  const int tid = threadIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const int64_t cg = (int64_t)chunk * H + h;
+  const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
+  for (int e = tid; e < MS * D; e += 256) {
+    const int m = e / D, d = e % D;
+    const float dc = p.dcum[cg * MS + m];
+    hkc[(cg * D + d) * MS + m] = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
+    hvc[(cg * MS + m) * D + d] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+  }
+  for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
+}
+
 template <int D, int G, int NW, int TK>
 int launch_out(const MP& p, hipStream_t st) {
   static bool configured = false;
@@ -1224,7 +1248,8 @@ ScratchPlan plan_scratch(const NhaPrefillArgs* a) {
 
 size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a) { return plan_scratch(a).total; }
 
-int prefill_mfma_impl(const NhaPrefillArgs* a) {
+namespace {
+MP make_mp(const NhaPrefillArgs* a) {
   MP p;
   p.q_swa = (const bf16_t*)a->q_swa; p.k_swa = (const bf16_t*)a->k_swa;
   p.q_gsa = (const bf16_t*)a->q_gsa; p.k_gsa = (const bf16_t*)a->k_gsa;
@@ -1247,10 +1272,29 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
   p.flags = (int*)(sc + sp.flags);
   p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H;
   p.wl = a->wl; p.shift = a->shift; p.scale = a->scale;
+  return p;
+}
+}  // namespace
+
+int prefill_mfma_impl(const NhaPrefillArgs* a) {
+  const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
   if (a->K == 64) return run_mfma<64>(p, a->phases, st);
   if (a->K == 128) return run_mfma<128>(p, a->phases, st);
   return run_mfma<256>(p, a->phases, st);
+}
+
+// `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
+// [NT][H][K][M], hvc [NT][H][M][V] receive fp32 copies in the layout of the generic kernels
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hvc) {
+  const MP p = make_mp(a);
+  hipStream_t st = (hipStream_t)a->stream;
+  const dim3 grid(a->NT, a->H);
+  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
+  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
+  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(state export)");
+  return NHA_OK;
 }
 
 }  // namespace nha
