@@ -8,7 +8,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnha_hip.so")
-SOURCES = ["abi.hip", "decode.hip", "decode_mfma.hip", "prefill_simple.hip", "prefill_mfma.hip", "prefill_bwd.hip"]
+SOURCES = ["abi.hip", "decode.hip", "decode_mfma.hip", "prefill_simple.hip", "prefill_mfma.hip", "prefill_bwd.hip", "prefill_bwd_mfma.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math" if False else "-fno-fast-math",
@@ -20,7 +20,8 @@ FLAGS = [
 
 # the MFMA kernels never produce NaN on purpose; without this flag every fmaxf operand is
 # canonicalised by an extra VALU instruction in the softmax inner loop
-EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "decode_mfma.hip": ["-fno-honor-nans"]}
+EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "decode_mfma.hip": ["-fno-honor-nans"],
+         "prefill_bwd_mfma.hip": ["-fno-honor-nans"]}
 
 
 def build_library(verbose: bool = False, jobs: int = 4) -> str:

@@ -142,6 +142,9 @@ int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, f
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);
+bool bwd_window_mfma_supported(const NhaPrefillBwdArgs* a);
+int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta);
+int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs);
 
 }  // namespace nha
 

@@ -20,7 +20,8 @@
 // the per-token vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra
 // part of ds) -> bwd_state_kernel (reverse sweep over chunks, one workgroup per 32 state columns:
 // dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_*_kernel (reverse scan: ds, dg)
-// -> bwd_kv_window_kernel (per key: dk_swa, dv).
+// -> bwd_kv_window_kernel (per key: dk_swa, dv).  For bf16 tensors with K == V in {64,128,256} the
+// window parts (dq_swa, dk_swa, dv) run on the matrix cores instead (prefill_bwd_mfma.hip).
 #include "common.h"
 
 namespace nha {
@@ -48,6 +49,7 @@ struct BP {
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
   float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
   int T_tot, N, NT, HQ, H, K, V, M, wl, shift, nbk, nbv;
+  int win;   // 1: bwd_q_kernel also produces dq_swa (0: the matrix-core window kernels do)
   float scale;
 };
 
@@ -167,6 +169,7 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     }
     Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
   }
+  if (!p.win) return;
   // window: dq_swa[d] = scale sum_j dw[j] k_swa_j[d]   (K <= 256: one column per thread)
   const int lo = p.wl < 0 ? bos : (t - p.wl > bos ? t - p.wl : bos);
   float acc = 0.f;
@@ -689,8 +692,14 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     }
     configured = true;
   }
+  const bool wmfma = bwd_window_mfma_supported(a);
+  p.win = wmfma ? 0 : 1;
   hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
+  if (wmfma) {
+    rc = bwd_window_mfma_dq(a, p.delta);
+    if (rc != NHA_OK) return rc;
+  }
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(256), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
@@ -700,6 +709,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_final_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(gate scan)");
+  if (wmfma) return bwd_window_mfma_dkv(a, p.delta, p.dvs);
   hipLaunchKernelGGL((bwd_kv_window_kernel<T>), dim3(a->T_tot, a->H), dim3(256), lds_w, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(key pass)");
   return NHA_OK;

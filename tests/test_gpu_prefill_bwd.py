@@ -98,6 +98,16 @@ def test_bwd_head_dims_of_the_models():
     run_bwd_case("D256", d, wl=64, shift=0, dtype=BF, impl="mfma")
 
 
+@pytest.mark.parametrize("wl,shift", [(-1, 0), (5, 6), (31, 32), (45, 0), (63, 64), (64, 0), (200, 201), (1000, 0)])
+def test_bwd_window_edges_on_the_matrix_cores(wl, shift):
+    """bf16, K == V == 64: the window gradients come from the matrix-core kernels.  Packed ragged
+    sequences (1 token, mid-chunk ends, longer than several key tiles), windows shorter than a
+    32-key half tile, not a multiple of it, longer than every sequence, and unbounded."""
+    cu = [0, 1, 66, 130, 450, 519]
+    d = prefill_inputs(7400 + wl, 1, cu[-1], 4, 2, 64, 64, 16, dtype=BF, qk_scale=1.0, with_state=True, N=5)
+    run_bwd_case(f"window wl={wl}", d, wl=wl, shift=shift, dtype=BF, cu=cu, scale=0.125, with_dht=True)
+
+
 def test_bwd_rejects_unsupported_shapes():
     from nha_amd import NhaError, chunk_nha
     d = prefill_inputs(7300, 1, 64, 2, 2, 64, 64, 128, dtype=torch.float32)
