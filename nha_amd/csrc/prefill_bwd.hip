@@ -18,8 +18,8 @@
 //
 // Launches: forward state pass (chunk-start states, gate cumsums) -> bwd_q_kernel (per token: dq's and
 // the per-token vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra
-// part of ds) -> bwd_state_kernel (reverse sweep over chunks, one workgroup per 32 state columns:
-// dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_*_kernel (reverse scan: ds, dg)
+// part of ds) -> bwd_state_{direct,scan,inter}_kernel (state gradients as a linear recurrence over
+// chunks: dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_*_kernel (reverse scan: ds, dg)
 // -> bwd_kv_window_kernel (per key: dk_swa, dv).  For bf16 tensors with K == V in {64,128,256} the
 // window parts (dq_swa, dk_swa, dv) run on the matrix cores instead (prefill_bwd_mfma.hip).
 #include "common.h"
@@ -48,6 +48,8 @@ struct BP {
   float *dsp;             // [nbk+nbv][T_tot][H][M]  inter-chunk part of ds per column block
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
   float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
+  float *dks;             // [T_tot][H][K]     intra-chunk part of dk_gsa, indexed by SOURCE token
+  float *ek, *ev;         // [NT][H][K][M], [NT][H][V][M]  N_c, then E_c (see the state-gradient kernels)
   int T_tot, N, NT, HQ, H, K, V, M, wl, shift, nbk, nbv;
   int win;   // 1: bwd_q_kernel also produces dq_swa (0: the matrix-core window kernels do)
   float scale;
@@ -284,147 +286,215 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
 }
 
 // ------------------------------------------------------------------------------------------
-// reverse sweep over the chunks of one (sequence, kv-head), one workgroup per CB state columns.
-// blockIdx.z = 0: k-state (columns d of hk; rows of q_gsa / k_gsa, weights dus, matrix ck, output
-// dk_gsa); 1: v-state (columns c of hv; rows of do / v, weights p, matrix cv, output dvs).
-// E[x][m] is the gradient of the state at the end of the current chunk coming from later chunks.
+// State gradients.  E_c[x][m], the gradient of the state at the END of chunk c that comes from
+// later chunks, obeys a linear recurrence over the chunks of a sequence,
+//   E_(c-1) = e^(gl_c)[m] E_c + N_c,    N_c[x][m] = sum_i sum_a x_i^a[x] w_i^a[m] e^(gc_i[m])
+// (x = rows of q_gsa with weights scale*du for the k-state, rows of do with weights p for the
+// v-state), whose inhomogeneous term N_c does not depend on E.  Three launches, the first and
+// the last parallel over chunks:
+//   bwd_state_direct_kernel   N_c and the intra-chunk part of dk' / dv'   (per chunk, CB columns)
+//   bwd_state_scan_kernel     the recurrence, element-wise over chunks (E_c replaces N_c; dh0)
+//   bwd_state_inter_kernel    the parts of dk' / dv' / ds that involve E_c (per chunk, CB columns)
+// blockIdx.z = 0: k-state (columns d; q_gsa / k_gsa rows, weights dus, matrix ck, output dk_gsa);
+// 1: v-state (columns c; do / v rows, weights p, matrix cv, output dvs).  eg holds N then E as
+// [NT][H][X][M] per state.
 // ------------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void bwd_state_kernel(const BP p) {
+__global__ __launch_bounds__(256) void bwd_state_direct_kernel(const BP p) {
   extern __shared__ __align__(16) float lds[];
   const int M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
   const int LM = M + 1;
   const bool isv = blockIdx.z != 0;
   const int X = isv ? p.V : p.K;
-  const int nb = isv ? p.nbv : p.nbk;
-  if ((int)blockIdx.y >= nb) return;
-  const int slab = isv ? p.nbk + blockIdx.y : blockIdx.y;
-  const int x0 = blockIdx.y * CB;
-  float* E = lds;                    // [CB][LM]
-  float* En = E + CB * LM;           // [CB][LM]  update accumulated over the heads
-  float* gcl = En + CB * LM;         // [BT][LM]
-  float* dec = gcl + BT * LM;        // [BT][LM]  e^(gl - gc_r)
-  float* sE = dec + BT * LM;         // [BT][LM]  s_r e^(gl - gc_r)
-  float* Lw = sE + BT * LM;          // [BT][LM]  per head: weight_i[m] e^(gc_i[m])
+  const int nbmax = p.nbk > p.nbv ? p.nbk : p.nbv;
+  const int h = blockIdx.y / nbmax, blk = blockIdx.y % nbmax;
+  if (blk >= (isv ? p.nbv : p.nbk)) return;
+  const int x0 = blk * CB;
+  float* gcl = lds;                  // [BT][LM]
+  float* Lw = gcl + BT * LM;         // [BT][LM]  per head: weight_i[m] e^(gc_i[m])
   float* Cm = Lw + BT * LM;          // [BT][BT+1] per head
   float* xq = Cm + BT * (BT + 1);    // [BT][CB+1] per head: q_gsa / do columns
-  float* xk = xq + BT * (CB + 1);    // [BT][CB+1] k' / v' columns
-  float* acc = xk + BT * (CB + 1);   // [BT][CB+1] dk' / dv'
-  float* eg = acc + BT * (CB + 1);   // [M] e^(gl)
-  int* src = (int*)(eg + M);         // [BT]
+  int* src = (int*)(xq + BT * (CB + 1));   // [BT]
   const int tid = threadIdx.x;
-  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int chunk = blockIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
-  const int L = eos - bos;
-  const int nchunks = (L + BT - 1) / BT;
-  const T* xrow_src = isv ? (const T*)p.v : (const T*)p.k_gsa;     // [T_tot][H][X]
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
   const T* qrow_src = isv ? (const T*)p.dout : (const T*)p.q_gsa;  // [T_tot][HQ][X]
   const float* wsrc = isv ? p.pp : p.dus;
   const float* csrc = isv ? p.cv : p.ck;
-  const float* dht = isv ? p.dhvt : p.dhkt;
-  for (int e = tid; e < CB * M; e += 256) {
-    const int x = e / M, m = e - x * M;
-    float val = 0.f;
-    if (dht && x0 + x < X)
-      val = isv ? dht[(((int64_t)n * H + h) * M + m) * X + x0 + x] : dht[(((int64_t)n * H + h) * X + x0 + x) * M + m];
-    E[x * LM + m] = val;
+  if (tid < BT) {
+    const int tl = it * BT + tid - p.shift;
+    src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
   }
-  for (int it = nchunks - 1; it >= 0; --it) {
-    const int chunk = p.coff[n] + it;
-    const int c0 = bos + it * BT;
-    const int R = (L - it * BT) < BT ? (L - it * BT) : BT;
-    __syncthreads();   // previous chunk finished, E updated
-    if (tid < BT) {
-      const int tl = it * BT + tid - p.shift;
-      src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
-    }
-    for (int e = tid; e < R * M; e += 256) {
-      const int r = e / M, m = e - r * M;
-      gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
-    }
-    for (int e = tid; e < CB * M; e += 256) En[(e / M) * LM + (e % M)] = 0.f;
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
+  }
+  // this thread's outputs: 8 of the R x CB intra sums, CB*M/256 of the CB x M elements of N
+  float acc[BT * CB / 256];
+  float en[CB * 64 / 256];
+#pragma unroll
+  for (int u = 0; u < BT * CB / 256; ++u) acc[u] = 0.f;
+#pragma unroll
+  for (int u = 0; u < CB * 64 / 256; ++u) en[u] = 0.f;
+  for (int a = 0; a < NG; ++a) {
+    const int hq = h * NG + a;
     __syncthreads();
-    for (int e = tid; e < R * M; e += 256) {
-      const int r = e / M, m = e - r * M;
-      const float d = expf(gcl[(R - 1) * LM + m] - gcl[r * LM + m]);
-      const int sj = src[r];
-      dec[r * LM + m] = d;
-      sE[r * LM + m] = sj >= 0 ? d * Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m) : 0.f;
+    const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
+    for (int e = tid; e < R * R; e += 256) {
+      const int i = e / R, r = e - i * R;
+      Cm[i * (BT + 1) + r] = i >= r ? cp[i * BT + r] : 0.f;
     }
-    for (int m = tid; m < M; m += 256) eg[m] = expf(gcl[(R - 1) * LM + m]);
     for (int e = tid; e < R * CB; e += 256) {
-      const int r = e / CB, x = e - r * CB;
-      const int sj = src[r];
-      xk[r * (CB + 1) + x] = (sj >= 0 && x0 + x < X) ? Elem<T>::ld(xrow_src + ((int64_t)sj * H + h) * X + x0 + x) : 0.f;
+      const int i = e / CB, x = e - i * CB;
+      xq[i * (CB + 1) + x] = (x0 + x < X) ? Elem<T>::ld(qrow_src + ((int64_t)(c0 + i) * HQ + hq) * X + x0 + x) : 0.f;
+    }
+    for (int e = tid; e < R * M; e += 256) {
+      const int i = e / M, m = e - i * M;
+      Lw[i * LM + m] = wsrc[((int64_t)(c0 + i) * HQ + hq) * M + m] * expf(gcl[i * LM + m]);
     }
     __syncthreads();
-    // inter-chunk parts: dk'_r[x] = sum_m sE_r[m] E[x][m];  ds part = dec_r[m] sum_x k'_r[x] E[x][m]
-    for (int e = tid; e < R * CB; e += 256) {
+#pragma unroll
+    for (int u = 0; u < BT * CB / 256; ++u) {
+      const int e = tid + 256 * u;
       const int r = e / CB, x = e - r * CB;
-      float a = 0.f;
-      for (int m = 0; m < M; ++m) a += sE[r * LM + m] * E[x * LM + m];
-      acc[r * (CB + 1) + x] = a;
+      float s2 = 0.f;
+      for (int i = r; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Cm[i * (BT + 1) + r];
+      acc[u] += s2;
     }
-    for (int e = tid; e < R * M; e += 256) {
-      const int r = e / M, m = e - r * M;
-      float a = 0.f;
-      for (int x = 0; x < CB; ++x) a += xk[r * (CB + 1) + x] * E[x * LM + m];
-      p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a * dec[r * LM + m];
-    }
-    for (int a = 0; a < NG; ++a) {
-      const int hq = h * NG + a;
-      __syncthreads();
-      const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
-      for (int e = tid; e < R * R; e += 256) {
-        const int i = e / R, r = e - i * R;
-        Cm[i * (BT + 1) + r] = i >= r ? cp[i * BT + r] : 0.f;
-      }
-      for (int e = tid; e < R * CB; e += 256) {
-        const int i = e / CB, x = e - i * CB;
-        xq[i * (CB + 1) + x] = (x0 + x < X) ? Elem<T>::ld(qrow_src + ((int64_t)(c0 + i) * HQ + hq) * X + x0 + x) : 0.f;
-      }
-      for (int e = tid; e < R * M; e += 256) {
-        const int i = e / M, m = e - i * M;
-        Lw[i * LM + m] = wsrc[((int64_t)(c0 + i) * HQ + hq) * M + m] * expf(gcl[i * LM + m]);
-      }
-      __syncthreads();
-      for (int e = tid; e < R * CB; e += 256) {
-        const int r = e / CB, x = e - r * CB;
-        float s2 = 0.f;
-        for (int i = r; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Cm[i * (BT + 1) + r];
-        acc[r * (CB + 1) + x] += s2;
-      }
-      for (int e = tid; e < CB * M; e += 256) {
-        const int x = e / M, m = e - x * M;
+#pragma unroll
+    for (int u = 0; u < CB * 64 / 256; ++u) {
+      const int e = tid + 256 * u;
+      const int x = e / M, m = e - x * M;
+      if (e < CB * M) {
         float s2 = 0.f;
         for (int i = 0; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Lw[i * LM + m];
-        En[x * LM + m] += s2;
+        en[u] += s2;
       }
     }
-    __syncthreads();
-    for (int e = tid; e < R * CB; e += 256) {
-      const int r = e / CB, x = e - r * CB;
-      const int sj = src[r];
-      if (sj < 0 || x0 + x >= X) continue;
-      const float val = acc[r * (CB + 1) + x];
-      if (isv) p.dvs[((int64_t)sj * H + h) * X + x0 + x] = val;
-      else Elem<T>::st((T*)p.dk_gsa + ((int64_t)sj * H + h) * X + x0 + x, val);
-    }
-    for (int e = tid; e < CB * M; e += 256) {
-      const int x = e / M, m = e - x * M;
-      E[x * LM + m] = E[x * LM + m] * eg[m] + En[x * LM + m];
-    }
+  }
+  float* outp = isv ? p.dvs : p.dks;
+#pragma unroll
+  for (int u = 0; u < BT * CB / 256; ++u) {
+    const int e = tid + 256 * u;
+    const int r = e / CB, x = e - r * CB;
+    if (r >= R) continue;
+    const int sj = src[r];
+    if (sj >= 0 && x0 + x < X) outp[((int64_t)sj * H + h) * X + x0 + x] = acc[u];
+  }
+  float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * X * M;
+#pragma unroll
+  for (int u = 0; u < CB * 64 / 256; ++u) {
+    const int e = tid + 256 * u;
+    const int x = e / M, m = e - x * M;
+    if (e < CB * M && x0 + x < X) ep[(int64_t)(x0 + x) * M + m] = en[u];
+  }
+}
+
+// grid (N*H, ceil((K+V)*M / 256)): one thread per state element, sequential over the chunks
+__global__ __launch_bounds__(256) void bwd_state_scan_kernel(const BP p) {
+  const int K = p.K, V = p.V, M = p.M, H = p.H;
+  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  if (e >= (K + V) * M) return;
+  const bool isv = e >= K * M;
+  const int em = isv ? e - K * M : e;
+  const int X = isv ? V : K;
+  const int x = em / M, m = em % M;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int L = eos - bos;
+  const int nchunks = (L + BT - 1) / BT;
+  float* eb = isv ? p.ev : p.ek;
+  const float* dht = isv ? p.dhvt : p.dhkt;
+  float E = 0.f;
+  if (dht) E = isv ? dht[(((int64_t)n * H + h) * M + m) * X + x] : dht[(((int64_t)n * H + h) * X + x) * M + m];
+  for (int it = nchunks - 1; it >= 0; --it) {
+    const int R = (L - it * BT) < BT ? (L - it * BT) : BT;
+    const int64_t idx = (((int64_t)(p.coff[n] + it) * H + h) * X + x) * M + m;
+    const float nc = eb[idx];
+    eb[idx] = E;
+    E = E * expf(p.gc[((int64_t)(bos + it * BT + R - 1) * H + h) * M + m]) + nc;
+  }
+  float* dh0 = isv ? p.dh0v : p.dh0k;
+  if (dh0) {
+    if (isv) dh0[(((int64_t)n * H + h) * M + m) * X + x] = E;
+    else dh0[(((int64_t)n * H + h) * X + x) * M + m] = E;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_state_inter_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int M = p.M, H = p.H;
+  const int LM = M + 1;
+  const bool isv = blockIdx.z != 0;
+  const int X = isv ? p.V : p.K;
+  const int nbmax = p.nbk > p.nbv ? p.nbk : p.nbv;
+  const int h = blockIdx.y / nbmax, blk = blockIdx.y % nbmax;
+  if (blk >= (isv ? p.nbv : p.nbk)) return;
+  const int slab = isv ? p.nbk + blk : blk;
+  const int x0 = blk * CB;
+  float* E = lds;                    // [CB][LM]
+  float* gcl = E + CB * LM;          // [BT][LM]
+  float* dec = gcl + BT * LM;        // [BT][LM]  e^(gl - gc_r)
+  float* sE = dec + BT * LM;         // [BT][LM]  s_r e^(gl - gc_r)
+  float* xk = sE + BT * LM;          // [BT][CB+1] k' / v' columns
+  int* src = (int*)(xk + BT * (CB + 1));   // [BT]
+  const int tid = threadIdx.x;
+  const int chunk = blockIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const T* xrow_src = isv ? (const T*)p.v : (const T*)p.k_gsa;     // [T_tot][H][X]
+  const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * X * M;
+  if (tid < BT) {
+    const int tl = it * BT + tid - p.shift;
+    src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
+  }
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
+  }
+  for (int e = tid; e < CB * M; e += 256) {
+    const int x = e / M, m = e - x * M;
+    E[x * LM + m] = (x0 + x < X) ? ep[(int64_t)(x0 + x) * M + m] : 0.f;
   }
   __syncthreads();
-  float* dh0 = isv ? p.dh0v : p.dh0k;
-  if (dh0)
-    for (int e = tid; e < CB * M; e += 256) {
-      const int x = e / M, m = e - x * M;
-      if (x0 + x >= X) continue;
-      if (isv) dh0[(((int64_t)n * H + h) * M + m) * X + x0 + x] = E[x * LM + m];
-      else dh0[(((int64_t)n * H + h) * X + x0 + x) * M + m] = E[x * LM + m];
-    }
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    const float d = expf(gcl[(R - 1) * LM + m] - gcl[r * LM + m]);
+    const int sj = src[r];
+    dec[r * LM + m] = d;
+    sE[r * LM + m] = sj >= 0 ? d * Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m) : 0.f;
+  }
+  for (int e = tid; e < R * CB; e += 256) {
+    const int r = e / CB, x = e - r * CB;
+    const int sj = src[r];
+    xk[r * (CB + 1) + x] = (sj >= 0 && x0 + x < X) ? Elem<T>::ld(xrow_src + ((int64_t)sj * H + h) * X + x0 + x) : 0.f;
+  }
+  __syncthreads();
+  // dk'_r[x] = intra part + sum_m sE_r[m] E[x][m];  ds part = dec_r[m] sum_x k'_r[x] E[x][m]
+  float* part = isv ? p.dvs : p.dks;
+  for (int e = tid; e < R * CB; e += 256) {
+    const int r = e / CB, x = e - r * CB;
+    const int sj = src[r];
+    if (sj < 0 || x0 + x >= X) continue;
+    const int64_t oi = ((int64_t)sj * H + h) * X + x0 + x;
+    float a = part[oi];
+    for (int m = 0; m < M; ++m) a += sE[r * LM + m] * E[x * LM + m];
+    if (isv) p.dvs[oi] = a;
+    else Elem<T>::st((T*)p.dk_gsa + oi, a);
+  }
+  for (int e = tid; e < R * M; e += 256) {
+    const int r = e / M, m = e - r * M;
+    float a = 0.f;
+    for (int x = 0; x < CB; ++x) a += xk[r * (CB + 1) + x] * E[x * LM + m];
+    p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a * dec[r * LM + m];
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -585,7 +655,7 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, mfma, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, total;
+  size_t fwd, mfma, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
   bool use_mfma;
   int nbk, nbv;
 };
@@ -614,6 +684,9 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   s.dsp = off; off += aligned(thm * (s.nbk + s.nbv));
   s.dvs = off; off += aligned((size_t)a->T_tot * a->H * a->V * 4);
   s.gtot = off; off += aligned((size_t)a->NT * a->H * a->M * 4);
+  s.dks = off; off += aligned((size_t)a->T_tot * a->H * a->K * 4);
+  s.ek = off; off += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
+  s.ev = off; off += aligned((size_t)a->NT * a->H * a->V * a->M * 4);
   s.total = off;
   return s;
 }
@@ -673,6 +746,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.ck = (float*)(sc + sp.ck); p.cv = (float*)(sc + sp.cv);
   p.dsi = (float*)(sc + sp.dsi); p.dsp = (float*)(sc + sp.dsp); p.dvs = (float*)(sc + sp.dvs);
   p.gtot = (float*)(sc + sp.gtot);
+  p.dks = (float*)(sc + sp.dks); p.ek = (float*)(sc + sp.ek); p.ev = (float*)(sc + sp.ev);
   p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.K = a->K; p.V = a->V; p.M = a->M;
   p.wl = a->wl; p.shift = a->shift; p.nbk = sp.nbk; p.nbv = sp.nbv; p.scale = a->scale;
   hipStream_t st = (hipStream_t)a->stream;
@@ -680,12 +754,13 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
 
   const size_t lds_q = ((size_t)2 * K + V + 4 * M + 3 * BT + 256 + 4) * 4 + BT * 4;
   const size_t lds_i = ((size_t)5 * BT * LM + 2 * BT * (BT + 1)) * 4 + BT * 4;
-  const size_t lds_s = ((size_t)2 * CB * LM + 4 * BT * LM + BT * (BT + 1) + 3 * BT * (CB + 1) + M) * 4 + BT * 4;
+  const size_t lds_s1 = ((size_t)2 * BT * LM + BT * (BT + 1) + BT * (CB + 1)) * 4 + BT * 4;
+  const size_t lds_s3 = ((size_t)CB * LM + 3 * BT * LM + BT * (CB + 1)) * 4 + BT * 4;
   const size_t lds_w = ((size_t)K + V + 512) * 4;
   static bool configured = false;
   if (!configured) {
     hipError_t e1 = hipFuncSetAttribute((const void*)bwd_intra_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipError_t e2 = hipFuncSetAttribute((const void*)bwd_state_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e2 = hipFuncSetAttribute((const void*)bwd_state_inter_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e1 != hipSuccess || e2 != hipSuccess) {
       set_error("nha_prefill_bwd: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
       return NHA_ERR_LAUNCH;
@@ -703,8 +778,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(256), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
-  hipLaunchKernelGGL((bwd_state_kernel<T>), dim3(a->N * a->H, nbmax, 2), dim3(256), lds_s, st, p);
-  NHA_CHECK_LAUNCH("nha_prefill_bwd(state sweep)");
+  hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
+  hipLaunchKernelGGL(bwd_state_scan_kernel, dim3(a->N * a->H, ((K + V) * M + 255) / 256), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((bwd_state_inter_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s3, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(state gradients)");
   hipLaunchKernelGGL((bwd_gate_local_kernel<T>), dim3(a->NT, a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_final_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
