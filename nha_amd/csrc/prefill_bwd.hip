@@ -55,6 +55,20 @@ struct BP {
   float scale;
 };
 
+// dot product of two global rows of n elements (n a multiple of 8, rows 16-byte aligned)
+template <typename T>
+__device__ __forceinline__ float dot_rows(const T* a, const T* b, int n) {
+  float acc = 0.f;
+  for (int i = 0; i < n; i += 8) {
+    float x[8], y[8];
+    Elem<T>::ld8(a + i, x);
+    Elem<T>::ld8(b + i, y);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += x[e] * y[e];
+  }
+  return acc;
+}
+
 __device__ __forceinline__ float logaddexp_f(float a, float b) {
   const float mx = fmaxf(a, b);
   return mx + logf(expf(a - mx) + expf(b - mx));
@@ -124,52 +138,79 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   const float lt = logaddexp_f(ls, lg);
   const float dlg = p.dlse_gsa ? p.dlse_gsa[tq] : 0.f;
   const float dls = p.dlse_swa ? p.dlse_swa[tq] : 0.f;
-  for (int m = tid; m < M; m += 256) {
-    float au = 0.f, ad = 0.f;
-    for (int kk = 0; kk < K; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
-    for (int c = 0; c < V; ++c) ad += dov[c] * hv0[(int64_t)m * V + c];
-    const float e = expf(gct[m]);
-    au *= e;
-    ad *= e;
-    for (int j = 0; j <= r; ++j) {
-      const int sj = src[j];
-      if (sj >= 0) {
-        const float w = Elem<T>::ld(ss + ((int64_t)sj * H + h) * M + m) * expf(gct[m] - gcb[(int64_t)j * H * M + m]);
-        au += Aj[j] * w;
-        ad += Bj[j] * w;
+  {
+    // u[m] and dp[m] at the chunk start, then the rows of the chunk.  Every global read is
+    // coalesced: lanes run over m for hk0 [K][M] (the four waves split K), over c for hv0 [M][V]
+    // (each wave takes every fourth slot and reduces across its lanes).
+    const int m = tid & 63, part = tid >> 6;
+    float au = 0.f, adj = 0.f;
+    if (m < M) {
+      const int k0 = part * K / 4, k1 = (part + 1) * K / 4;
+      for (int kk = k0; kk < k1; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
+      au *= expf(gct[m]);
+      for (int j = part; j <= r; j += 4) {
+        const int sj = src[j];
+        if (sj >= 0) {
+          const float w = Elem<T>::ld(ss + ((int64_t)sj * H + h) * M + m) * expf(gct[m] - gcb[(int64_t)j * H * M + m]);
+          au += Aj[j] * w;
+          adj += Bj[j] * w;
+        }
       }
     }
-    const float pm = expf(au - lt);
-    const float du = pm * (ad - delta) + dlg * expf(au - lg);
-    okl[m] = au;
-    dpl[m] = ad;
-    dul[m] = p.scale * du;
-    p.dus[tq * M + m] = p.scale * du;
-    p.pp[tq * M + m] = pm;
-    p.xg[tq * M + m] = du * au + pm * ad;
+    for (int mm = part; mm < M; mm += 4) {
+      float a2 = 0.f;
+      for (int c = m; c < V; c += 64) a2 += dov[c] * hv0[(int64_t)mm * V + c];
+      a2 = wave_sum(a2);
+      if (m == 0) dpl[mm] = a2 * expf(gct[mm]);
+    }
+    pw[tid] = au;
+    __syncthreads();
+    if (part == 0 && m < M) okl[m] = (pw[m] + pw[64 + m]) + (pw[128 + m] + pw[192 + m]);
+    __syncthreads();
+    pw[tid] = adj;
+    __syncthreads();
+    if (part == 0 && m < M) {
+      const float au_t = okl[m];
+      const float ad_t = dpl[m] + (pw[m] + pw[64 + m]) + (pw[128 + m] + pw[192 + m]);
+      const float pm = expf(au_t - lt);
+      const float du = pm * (ad_t - delta) + dlg * expf(au_t - lg);
+      dul[m] = p.scale * du;
+      p.dus[tq * M + m] = p.scale * du;
+      p.pp[tq * M + m] = pm;
+      p.xg[tq * M + m] = du * au_t + pm * ad_t;
+    }
   }
   if (tid == 0) p.delta[tq] = delta;
   __syncthreads();
-  if (tid < BT) {
-    const int sj = src[tid];
+  {
+    // Wj[j] = sum_m scale du[m] s_j[m] e^(gc_r[m] - gc_j[m]): row j = tid % 64, the four waves split m
+    const int j = tid & 63, part = tid >> 6;
+    const int sj = src[j];
     float acc = 0.f;
     if (sj >= 0) {
       const T* srow = ss + ((int64_t)sj * H + h) * M;
-      const float* gj = gcb + (int64_t)tid * H * M;
-      for (int m = 0; m < M; ++m) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
+      const float* gj = gcb + (int64_t)j * H * M;
+      for (int m = part; m < M; m += 4) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
     }
-    Wj[tid] = acc;
+    pw[tid] = acc;
+    if (tid < M) dpl[tid] = dul[tid] * expf(gct[tid]);   // dp is not needed any more
+    __syncthreads();
+    if (tid < BT) Wj[tid] = (pw[tid] + pw[64 + tid]) + (pw[128 + tid] + pw[192 + tid]);
   }
   __syncthreads();
-  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]
-  for (int d = tid; d < K; d += 256) {
-    float acc = 0.f;
-    for (int m = 0; m < M; ++m) acc += dul[m] * expf(gct[m]) * hk0[(int64_t)d * M + m];
-    for (int j = 0; j <= r; ++j) {
-      const int sj = src[j];
-      if (sj >= 0) acc += Wj[j] * Elem<T>::ld(kgs + ((int64_t)sj * H + h) * K + d);
+  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]: each wave takes every fourth column, lanes run over m
+  {
+    const int lane = tid & 63, wv = tid >> 6;
+    for (int d = wv; d < K; d += 4) {
+      float acc = 0.f;
+      for (int m = lane; m < M; m += 64) acc += dpl[m] * hk0[(int64_t)d * M + m];
+      if (lane <= r) {
+        const int sj = src[lane];
+        if (sj >= 0) acc += Wj[lane] * Elem<T>::ld(kgs + ((int64_t)sj * H + h) * K + d);
+      }
+      acc = wave_sum(acc);
+      if (lane == 0) Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
     }
-    Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
   }
   if (!p.win) return;
   // window: dq_swa[d] = scale sum_j dw[j] k_swa_j[d]   (K <= 256: one column per thread)
@@ -246,10 +287,10 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
       if (sj >= 0) {
         const T* qrow = (const T*)p.q_gsa + ((int64_t)(c0 + i) * HQ + hq) * K;
         const T* krow = (const T*)p.k_gsa + ((int64_t)sj * H + h) * K;
-        for (int d = 0; d < K; ++d) av += Elem<T>::ld(qrow + d) * Elem<T>::ld(krow + d);
+        av = dot_rows<T>(qrow, krow, K);
         const T* drow = (const T*)p.dout + ((int64_t)(c0 + i) * HQ + hq) * V;
         const T* vrow = (const T*)p.v + ((int64_t)sj * H + h) * V;
-        for (int c = 0; c < V; ++c) bv += Elem<T>::ld(drow + c) * Elem<T>::ld(vrow + c);
+        bv = dot_rows<T>(drow, vrow, V);
       }
       Am[i * (BT + 1) + r] = av;
       Bm[i * (BT + 1) + r] = bv;
