@@ -160,6 +160,39 @@ def bench_prefill(torch, steps, warmup, cfg=PREFILL):
                 flops=flops, achieved_tflops=flops_out / t_out / 1e12, whole_op_tflops=flops / wall / 1e12)
 
 
+def bench_backward(torch, steps, warmup, cfg=PREFILL):
+    """Backward of the prefill op (nha_prefill_bwd behind chunk_nha's autograd node) on the same
+    synthetic inputs: milliseconds per call with HIP events on the launch stream.  Flops by the
+    usual convention for attention backwards, 2.5 x the forward's (five matrix products for two)."""
+    import numpy as np
+    from nha_amd.ops import nha_prefill, nha_prefill_bwd
+    dev = torch.device("cuda:0")
+    B, T, HQ, H, D, M, W = (cfg[k] for k in ("B", "T", "HQ", "H", "D", "M", "W"))
+    wl, shift = cfg.get("wl", W - 1), cfg.get("shift", W)
+    lens = workload_lengths(torch, cfg)
+    xs = [x.reshape(B * T, *x.shape[2:]).contiguous() for x in make_prefill_inputs(torch, cfg, dev)]
+    cu_host = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    o, ls, lg, _, _ = nha_prefill(*xs, cu_host, wl=wl, shift=shift, scale=D ** -0.5, impl="mfma")
+    gen = torch.Generator(device=dev).manual_seed(1)
+    do = torch.randn(o.shape, generator=gen, device=dev, dtype=torch.float32).to(o.dtype)
+    stream = torch.cuda.current_stream(dev)
+    run = lambda: nha_prefill_bwd(*xs, o, ls, lg, do, cu_host, wl=wl, shift=shift, scale=D ** -0.5)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    tot = 0.0
+    for _ in range(steps):
+        ev[0].record(stream)
+        run()
+        ev[1].record(stream)
+        torch.cuda.synchronize()
+        tot += ev[0].elapsed_time(ev[1])
+    ms = tot / steps
+    flops = 2.5 * sum(prefill_flops(1, L, HQ, H, D, M, wl + 1) for L in lens)
+    return dict(bwd_ms=ms, bwd_flops=flops, bwd_tflops=flops / (ms * 1e-3) / 1e12, bwd_tokens_per_s=B * T / (ms * 1e-3))
+
+
 def bench_decode(torch, warmup):
     from nha_amd import NHARingState, ring_decode_step
     cfg = DECODE
@@ -261,6 +294,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
+    ap.add_argument("--backward", action="store_true",
+                    help="with --workload: also time the backward of the prefill op")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
                     help="time the prefill of another of the reference's configurations and print its raw numbers")
     args = ap.parse_args()
@@ -283,6 +318,8 @@ def main():
         res["workload"] = {k: v for k, v in cfg.items()}
         res["min_bytes"] = 2 * cfg["B"] * cfg["T"] * (cfg["HQ"] * 3 * cfg["D"] + cfg["H"] * (3 * cfg["D"] + 2 * cfg["M"]))
         res["min_bytes_gbs"] = res["min_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9
+        if args.backward:
+            res.update(bench_backward(torch, args.steps, args.warmup, cfg))
         print(json.dumps(res))
         return
     if args.only:

@@ -51,12 +51,6 @@ def _need_cuda(*ts):
             raise RuntimeError("NHA ops run on the GPU only (tensor on %s); there is no CPU fallback" % t.device)
 
 
-def _no_grad_inputs(name, *ts):
-    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts):
-        raise NotImplementedError(f"{name}: forward only -- the backward of the reference op is not implemented; "
-                                  "call under torch.no_grad() or detach the inputs")
-
-
 # ---------------------------------------------------------------------------------------------
 # varlen tables, cached per cu_seqlens content
 # ---------------------------------------------------------------------------------------------
