@@ -138,7 +138,7 @@ int prefill_simple_impl(const NhaPrefillArgs* a);
 bool prefill_mfma_supported(const NhaPrefillArgs* a);
 size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_mfma_impl(const NhaPrefillArgs* a);
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hvc);
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);

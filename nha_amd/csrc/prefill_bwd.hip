@@ -39,6 +39,7 @@ struct BP {
   // forward recomputation (layout of the generic forward state pass)
   float *gc;          // [T_tot][H][M]      chunk-local inclusive gate cumsum, indexed by row token
   float *hkc, *hvc;   // [NT][H][K][M], [NT][H][M][V]   chunk-start states
+  float *hkct, *hvct; // [NT][H][M][K], [NT][H][V][M]   the same, transposed
   float *hkT, *hvT;   // [N][H][K][M], [N][H][M][V]     final states (for the end term of dg)
   // per-token vectors of the slot branch
   float *dus, *pp, *xg;   // [T_tot][HQ][M]   scale*du, p, du*u + p*dp
@@ -51,7 +52,6 @@ struct BP {
   float *dks;             // [T_tot][H][K]     intra-chunk part of dk_gsa, indexed by SOURCE token
   float *ek, *ev;         // [NT][H][K][M], [NT][H][V][M]  N_c, then E_c (see the state-gradient kernels)
   int T_tot, N, NT, HQ, H, K, V, M, wl, shift, nbk, nbv;
-  int win;   // 1: bwd_q_kernel also produces dq_swa (0: the matrix-core window kernels do)
   float scale;
 };
 
@@ -75,26 +75,143 @@ __device__ __forceinline__ float logaddexp_f(float a, float b) {
 }
 
 // ------------------------------------------------------------------------------------------
-// per (token, q-head): dq_swa, dq_gsa and the vectors du, p the state gradients are built from
+// per (token, q-head), ONE WAVE each (4 tokens per workgroup): dq_gsa and the vectors du, p the
+// state gradients are built from.  Lanes run over the slots m (M <= 64), over the rows j of the
+// chunk, or over columns d, so that every global read of a state is coalesced: hkc [K][M] for u,
+// hvct [V][M] for dp, hkct [M][K] for dq_gsa.
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   extern __shared__ __align__(16) float lds[];
   const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
-  float* qg = lds;             // [K] scaled slot-branch query
-  float* qs = qg + K;          // [K] scaled window query
-  float* dov = qs + K;         // [V]
-  float* gct = dov + V;        // [M]
-  float* okl = gct + M;        // [M] slot logits u
-  float* dpl = okl + M;        // [M] dp
-  float* dul = dpl + M;        // [M] scale * du
-  float* Aj = dul + M;         // [BT] q_gsa . k'_j
-  float* Bj = Aj + BT;         // [BT] do . v'_j
-  float* Wj = Bj + BT;         // [BT]
-  float* pw = Wj + BT;         // [256]
-  float* red = pw + 256;       // [4]
-  int* src = (int*)(red + 4);  // [BT]
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  float* qg = lds + wv * (K + V + 3 * BT + 3 * M);   // [K] scaled slot-branch query
+  float* dov = qg + K;        // [V]
+  float* Aj = dov + V;        // [BT] q_gsa . k'_j
+  float* Bj = Aj + BT;        // [BT] do . v'_j
+  float* Wj = Bj + BT;        // [BT]
+  float* gct = Wj + BT;       // [M]
+  float* dul = gct + M;       // [M] scale * du
+  float* due = dul + M;       // [M] scale * du * e^(gc_r)
+  const int chunk = blockIdx.x / (BT / 4), r = (blockIdx.x % (BT / 4)) * 4 + wv;
+  const int hq = blockIdx.y, h = hq / NG;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const bool valid = bos + it * BT + r < eos;   // waves past the end compute on row 0 and write nothing
+  const int rr = valid ? r : 0;
+  const int t = bos + it * BT + rr;
+  const T* kgs = (const T*)p.k_gsa;
+  const T* vv_ = (const T*)p.v;
+  const T* ss = (const T*)p.s;
+  const int64_t tq = (int64_t)t * HQ + hq;
+  float dl = 0.f;
+  for (int i = lane; i < K; i += 64) qg[i] = Elem<T>::ld((const T*)p.q_gsa + tq * K + i) * p.scale;
+  for (int i = lane; i < V; i += 64) {
+    const float d = Elem<T>::ld((const T*)p.dout + tq * V + i);
+    dov[i] = d;
+    dl += d * Elem<T>::ld((const T*)p.o + tq * V + i);
+  }
+  if (lane < M) gct[lane] = p.gc[((int64_t)t * H + h) * M + lane];
+  const float delta = wave_sum(dl);
+  __syncthreads();
+  const int tl0 = it * BT - p.shift;   // sequence-local source index of row 0 (negative: no source)
+  {
+    const int j = lane;
+    const bool has = j <= rr && tl0 + j >= 0;
+    const int64_t sj = (int64_t)bos + tl0 + j;
+    Aj[j] = has ? dot_row<T>(qg, kgs + (sj * H + h) * K, K) : 0.f;
+    Bj[j] = has ? dot_row<T>(dov, vv_ + (sj * H + h) * V, V) : 0.f;
+  }
+  __syncthreads();
+  const float* hk0 = p.hkc + ((int64_t)chunk * H + h) * K * M;
+  const float* hv0t = p.hvct + ((int64_t)chunk * H + h) * V * M;
+  const float* hk0t = p.hkct + ((int64_t)chunk * H + h) * M * K;
+  const float* gcb = p.gc + ((int64_t)(bos + it * BT) * H + h) * M;
+  const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
+  const float lt = logaddexp_f(ls, lg);
+  const float dlg = p.dlse_gsa ? p.dlse_gsa[tq] : 0.f;
+  if (lane < M) {
+    const int m = lane;
+    float au = 0.f, ad = 0.f;
+#pragma unroll 8
+    for (int kk = 0; kk < K; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
+#pragma unroll 8
+    for (int c = 0; c < V; ++c) ad += dov[c] * hv0t[(int64_t)c * M + m];
+    const float gm = gct[m];
+    const float e = expf(gm);
+    au *= e;
+    ad *= e;
+    const int jlo = tl0 < 0 ? -tl0 : 0;
+    for (int j = jlo; j <= rr; ++j) {
+      const int64_t sj = (int64_t)bos + tl0 + j;
+      const float w = Elem<T>::ld(ss + (sj * H + h) * M + m) * expf(gm - gcb[(int64_t)j * H * M + m]);
+      au += Aj[j] * w;
+      ad += Bj[j] * w;
+    }
+    const float pm = expf(au - lt);
+    const float du = pm * (ad - delta) + dlg * expf(au - lg);
+    dul[m] = p.scale * du;
+    due[m] = p.scale * du * e;
+    if (valid) {
+      p.dus[tq * M + m] = p.scale * du;
+      p.pp[tq * M + m] = pm;
+      p.xg[tq * M + m] = du * au + pm * ad;
+    }
+  }
+  if (lane == 0 && valid) p.delta[tq] = delta;
+  __syncthreads();
+  {
+    // Wj[j] = sum_m scale du[m] s_j[m] e^(gc_r[m] - gc_j[m])
+    const int j = lane;
+    float acc = 0.f;
+    if (j <= rr && tl0 + j >= 0) {
+      const T* srow = ss + (((int64_t)bos + tl0 + j) * H + h) * M;
+      const float* gj = gcb + (int64_t)j * H * M;
+      for (int m = 0; m < M; ++m) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
+    }
+    Wj[j] = acc;
+  }
+  __syncthreads();
+  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]
+  for (int d = lane; d < K; d += 64) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int m = 0; m < M; ++m) acc += due[m] * hk0t[(int64_t)m * K + d];
+    const int jlo = tl0 < 0 ? -tl0 : 0;
+    for (int j = jlo; j <= rr; ++j) acc += Wj[j] * Elem<T>::ld(kgs + (((int64_t)bos + tl0 + j) * H + h) * K + d);
+    if (valid) Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
+  }
+}
+
+// chunk-start states in the transposed layouts bwd_q_kernel reads (generic state pass only; the
+// matrix-core state pass exports them directly): hkct [NT][H][M][K], hvct [NT][H][V][M]
+__global__ __launch_bounds__(256) void bwd_transpose_states_kernel(const BP p) {
+  const int K = p.K, V = p.V, M = p.M;
+  const int64_t cg = blockIdx.x;
+  const float* hk = p.hkc + cg * K * M;
+  const float* hv = p.hvc + cg * M * V;
+  for (int e = threadIdx.x; e < K * M; e += 256) {
+    const int m = e / K, d = e - m * K;
+    p.hkct[cg * M * K + e] = hk[(int64_t)d * M + m];
+  }
+  for (int e = threadIdx.x; e < V * M; e += 256) {
+    const int c = e / M, m = e - c * M;
+    p.hvct[cg * V * M + e] = hv[(int64_t)m * V + c];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// per (token, q-head): dq_swa in fp32 VALU arithmetic (tensors the matrix-core kernels do not take)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_q_window_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int K = p.K, V = p.V, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  float* qs = lds;         // [K] scaled window query
+  float* dov = qs + K;     // [V]
+  float* pw = dov + V;     // [256]
   const int tid = threadIdx.x;
   const int chunk = blockIdx.x / BT, r = blockIdx.x % BT;
   const int hq = blockIdx.y, h = hq / NG;
@@ -103,121 +220,20 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   const int t = bos + it * BT + r;
   if (t >= eos) return;
   const T* ksw = (const T*)p.k_swa;
-  const T* kgs = (const T*)p.k_gsa;
   const T* vv_ = (const T*)p.v;
-  const T* ss = (const T*)p.s;
   const int64_t tq = (int64_t)t * HQ + hq;
-  for (int i = tid; i < K; i += 256) {
-    qg[i] = Elem<T>::ld((const T*)p.q_gsa + tq * K + i) * p.scale;
-    qs[i] = Elem<T>::ld((const T*)p.q_swa + tq * K + i) * p.scale;
-  }
-  float dl = 0.f;
-  for (int i = tid; i < V; i += 256) {
-    const float d = Elem<T>::ld((const T*)p.dout + tq * V + i);
-    dov[i] = d;
-    dl += d * Elem<T>::ld((const T*)p.o + tq * V + i);
-  }
-  for (int i = tid; i < M; i += 256) gct[i] = p.gc[((int64_t)t * H + h) * M + i];
-  if (tid < BT) {
-    const int tl = it * BT + tid - p.shift;
-    src[tid] = (tid <= r && tl >= 0) ? bos + tl : -1;
-  }
-  const float delta = block_sum(dl, red);   // includes the barrier that publishes the tables
-  if (tid < BT) {
-    const int sj = src[tid];
-    Aj[tid] = sj >= 0 ? dot_row<T>(qg, kgs + ((int64_t)sj * H + h) * K, K) : 0.f;
-  } else if (tid < 2 * BT) {
-    const int sj = src[tid - BT];
-    Bj[tid - BT] = sj >= 0 ? dot_row<T>(dov, vv_ + ((int64_t)sj * H + h) * V, V) : 0.f;
-  }
-  __syncthreads();
-  const float* hk0 = p.hkc + ((int64_t)chunk * H + h) * K * M;
-  const float* hv0 = p.hvc + ((int64_t)chunk * H + h) * M * V;
-  const float* gcb = p.gc + ((int64_t)(bos + it * BT) * H + h) * M;
-  const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
-  const float lt = logaddexp_f(ls, lg);
-  const float dlg = p.dlse_gsa ? p.dlse_gsa[tq] : 0.f;
+  for (int i = tid; i < K; i += 256) qs[i] = Elem<T>::ld((const T*)p.q_swa + tq * K + i) * p.scale;
+  for (int i = tid; i < V; i += 256) dov[i] = Elem<T>::ld((const T*)p.dout + tq * V + i);
+  const float ls = p.lse_swa[tq];
+  const float lt = logaddexp_f(ls, p.lse_gsa[tq]);
   const float dls = p.dlse_swa ? p.dlse_swa[tq] : 0.f;
-  {
-    // u[m] and dp[m] at the chunk start, then the rows of the chunk.  Every global read is
-    // coalesced: lanes run over m for hk0 [K][M] (the four waves split K), over c for hv0 [M][V]
-    // (each wave takes every fourth slot and reduces across its lanes).
-    const int m = tid & 63, part = tid >> 6;
-    float au = 0.f, adj = 0.f;
-    if (m < M) {
-      const int k0 = part * K / 4, k1 = (part + 1) * K / 4;
-      for (int kk = k0; kk < k1; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
-      au *= expf(gct[m]);
-      for (int j = part; j <= r; j += 4) {
-        const int sj = src[j];
-        if (sj >= 0) {
-          const float w = Elem<T>::ld(ss + ((int64_t)sj * H + h) * M + m) * expf(gct[m] - gcb[(int64_t)j * H * M + m]);
-          au += Aj[j] * w;
-          adj += Bj[j] * w;
-        }
-      }
-    }
-    for (int mm = part; mm < M; mm += 4) {
-      float a2 = 0.f;
-      for (int c = m; c < V; c += 64) a2 += dov[c] * hv0[(int64_t)mm * V + c];
-      a2 = wave_sum(a2);
-      if (m == 0) dpl[mm] = a2 * expf(gct[mm]);
-    }
-    pw[tid] = au;
-    __syncthreads();
-    if (part == 0 && m < M) okl[m] = (pw[m] + pw[64 + m]) + (pw[128 + m] + pw[192 + m]);
-    __syncthreads();
-    pw[tid] = adj;
-    __syncthreads();
-    if (part == 0 && m < M) {
-      const float au_t = okl[m];
-      const float ad_t = dpl[m] + (pw[m] + pw[64 + m]) + (pw[128 + m] + pw[192 + m]);
-      const float pm = expf(au_t - lt);
-      const float du = pm * (ad_t - delta) + dlg * expf(au_t - lg);
-      dul[m] = p.scale * du;
-      p.dus[tq * M + m] = p.scale * du;
-      p.pp[tq * M + m] = pm;
-      p.xg[tq * M + m] = du * au_t + pm * ad_t;
-    }
-  }
-  if (tid == 0) p.delta[tq] = delta;
-  __syncthreads();
-  {
-    // Wj[j] = sum_m scale du[m] s_j[m] e^(gc_r[m] - gc_j[m]): row j = tid % 64, the four waves split m
-    const int j = tid & 63, part = tid >> 6;
-    const int sj = src[j];
-    float acc = 0.f;
-    if (sj >= 0) {
-      const T* srow = ss + ((int64_t)sj * H + h) * M;
-      const float* gj = gcb + (int64_t)j * H * M;
-      for (int m = part; m < M; m += 4) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
-    }
-    pw[tid] = acc;
-    if (tid < M) dpl[tid] = dul[tid] * expf(gct[tid]);   // dp is not needed any more
-    __syncthreads();
-    if (tid < BT) Wj[tid] = (pw[tid] + pw[64 + tid]) + (pw[128 + tid] + pw[192 + tid]);
-  }
-  __syncthreads();
-  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]: each wave takes every fourth column, lanes run over m
-  {
-    const int lane = tid & 63, wv = tid >> 6;
-    for (int d = wv; d < K; d += 4) {
-      float acc = 0.f;
-      for (int m = lane; m < M; m += 64) acc += dpl[m] * hk0[(int64_t)d * M + m];
-      if (lane <= r) {
-        const int sj = src[lane];
-        if (sj >= 0) acc += Wj[lane] * Elem<T>::ld(kgs + ((int64_t)sj * H + h) * K + d);
-      }
-      acc = wave_sum(acc);
-      if (lane == 0) Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
-    }
-  }
-  if (!p.win) return;
-  // window: dq_swa[d] = scale sum_j dw[j] k_swa_j[d]   (K <= 256: one column per thread)
+  const float delta = p.delta[tq];
+  // dq_swa[d] = scale sum_j dw[j] k_swa_j[d]   (K <= 256: one column per thread)
   const int lo = p.wl < 0 ? bos : (t - p.wl > bos ? t - p.wl : bos);
   float acc = 0.f;
   for (int jb = lo; jb <= t; jb += 256) {
     const int j = jb + tid;
+    __syncthreads();
     float val = 0.f;
     if (j <= t) {
       const float w = dot_row<T>(qs, ksw + ((int64_t)j * H + h) * K, K);
@@ -225,7 +241,6 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
       const float dpi = dot_row<T>(dov, vv_ + ((int64_t)j * H + h) * V, V);
       val = p.scale * (pi * (dpi - delta) + dls * expf(w - ls));
     }
-    __syncthreads();
     pw[tid] = val;
     __syncthreads();
     const int cnt = (t - jb + 1) < 256 ? (t - jb + 1) : 256;
@@ -696,7 +711,7 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, mfma, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
+  size_t fwd, mfma, hkct, hvct, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
   bool use_mfma;
   int nbk, nbv;
 };
@@ -710,6 +725,8 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   s.use_mfma = prefill_mfma_supported(&f);
   s.mfma = off;
   if (s.use_mfma) off += aligned(prefill_mfma_scratch_bytes(&f));
+  s.hkct = off; off += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
+  s.hvct = off; off += aligned((size_t)a->NT * a->H * a->V * a->M * 4);
   s.hkT = off; off += aligned((size_t)a->N * a->H * a->K * a->M * 4);
   s.hvT = off; off += aligned((size_t)a->N * a->H * a->M * a->V * 4);
   const size_t tqm = aligned((size_t)a->T_tot * a->HQ * a->M * 4);
@@ -764,7 +781,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     f.scratch = sc + sp.mfma;
     f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
     rc = prefill_mfma_impl(&f);
-    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, hvc);
+    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, (float*)(sc + sp.hkct), (float*)(sc + sp.hvct));
   } else {
     f.scratch = sc + sp.fwd;
     f.scratch_bytes = prefill_simple_scratch_bytes(&f);
@@ -781,6 +798,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.dv = a->dv; p.ds = a->ds; p.dg = a->dg; p.dh0k = a->dh0k; p.dh0v = a->dh0v;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
   p.gc = gc; p.hkc = hkc; p.hvc = hvc;
+  p.hkct = (float*)(sc + sp.hkct); p.hvct = (float*)(sc + sp.hvct);
   p.hkT = (float*)(sc + sp.hkT); p.hvT = (float*)(sc + sp.hvT);
   p.dus = (float*)(sc + sp.dus); p.pp = (float*)(sc + sp.pp); p.xg = (float*)(sc + sp.xg);
   p.delta = (float*)(sc + sp.delta);
@@ -793,7 +811,8 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipStream_t st = (hipStream_t)a->stream;
   const int K = a->K, V = a->V, M = a->M, LM = M + 1;
 
-  const size_t lds_q = ((size_t)2 * K + V + 4 * M + 3 * BT + 256 + 4) * 4 + BT * 4;
+  const size_t lds_q = (size_t)4 * (K + V + 3 * BT + 3 * M) * 4;
+  const size_t lds_qw = ((size_t)K + V + 256) * 4;
   const size_t lds_i = ((size_t)5 * BT * LM + 2 * BT * (BT + 1)) * 4 + BT * 4;
   const size_t lds_s1 = ((size_t)2 * BT * LM + BT * (BT + 1) + BT * (CB + 1)) * 4 + BT * 4;
   const size_t lds_s3 = ((size_t)CB * LM + 3 * BT * LM + BT * (CB + 1)) * 4 + BT * 4;
@@ -809,12 +828,15 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     configured = true;
   }
   const bool wmfma = bwd_window_mfma_supported(a);
-  p.win = wmfma ? 0 : 1;
-  hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_q, st, p);
+  if (!sp.use_mfma) hipLaunchKernelGGL(bwd_transpose_states_kernel, dim3(a->NT * a->H), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
   if (wmfma) {
     rc = bwd_window_mfma_dq(a, p.delta);
     if (rc != NHA_OK) return rc;
+  } else {
+    hipLaunchKernelGGL((bwd_q_window_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_qw, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_bwd(window query pass)");
   }
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(256), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");

@@ -1132,12 +1132,11 @@ int launch_repair(const MP& p, hipStream_t st) {
 }
 
 // ==========================================================================================
-// fp32 copies of what the state pass left in the scratch, in the layout of the generic kernels
-// (true chunk-start states hk [K][M], hv [M][V]; gate cumsums per row token): the backward pass
-// reads those
+// fp32 copies of what the state pass left in the scratch for the backward pass: true chunk-start
+// states as hk [K][M] and transposed hk^T [M][K], hv^T [V][M]; gate cumsums per row token
 // ==========================================================================================
 template <int D>
-__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hvc) {
+__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hkct, float* hvct) {
   const int chunk = blockIdx.x, h = blockIdx.y, H = p.H;
   const int tid = threadIdx.x;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
@@ -1149,8 +1148,10 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
   for (int e = tid; e < MS * D; e += 256) {
     const int m = e / D, d = e % D;
     const float dc = p.dcum[cg * MS + m];
-    hkc[(cg * D + d) * MS + m] = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
-    hvc[(cg * MS + m) * D + d] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+    const float hk = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
+    hkc[(cg * D + d) * MS + m] = hk;
+    hkct[(cg * MS + m) * D + d] = hk;
+    hvct[(cg * D + d) * MS + m] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
   }
   for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
 }
@@ -1285,14 +1286,14 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
 }
 
 // `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
-// [NT][H][K][M], hvc [NT][H][M][V] receive fp32 copies in the layout of the generic kernels
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hvc) {
+// [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
   const dim3 grid(a->NT, a->H);
-  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
-  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
-  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hvc);
+  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
+  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
+  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state export)");
   return NHA_OK;
 }
