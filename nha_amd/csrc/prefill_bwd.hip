@@ -254,7 +254,8 @@ __global__ __launch_bounds__(256) void bwd_q_window_kernel(const BP p) {
 // per (chunk, kv-head): intra-chunk matrices ck, cv and the intra-chunk part of ds
 // ------------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
+__global__ __launch_bounds__(512) void bwd_intra_kernel(const BP p) {
+  constexpr int NTHR = 512;   // 8 waves: the tables fill most of the LDS, so one workgroup per CU
   extern __shared__ __align__(16) float lds[];
   const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
     src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
   }
   __syncthreads();
-  for (int e = tid; e < R * M; e += 256) {
+  for (int e = tid; e < R * M; e += NTHR) {
     const int r = e / M, m = e - r * M;
     gcl[r * LM + m] = p.gc[((int64_t)(c0 + r) * H + h) * M + m];
     const int sj = src[r];
@@ -289,12 +290,12 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
   for (int a = 0; a < NG; ++a) {
     const int hq = h * NG + a;
     __syncthreads();
-    for (int e = tid; e < R * M; e += 256) {
+    for (int e = tid; e < R * M; e += NTHR) {
       const int r = e / M, m = e - r * M;
       du[r * LM + m] = p.dus[((int64_t)(c0 + r) * HQ + hq) * M + m];
       pl[r * LM + m] = p.pp[((int64_t)(c0 + r) * HQ + hq) * M + m];
     }
-    for (int e = tid; e < R * R; e += 256) {
+    for (int e = tid; e < R * R; e += NTHR) {
       const int i = e / R, r = e - i * R;
       if (i < r) continue;
       const int sj = src[r];
@@ -313,7 +314,7 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
     __syncthreads();
     float* ckp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
     float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
-    for (int e = tid; e < R * R; e += 256) {
+    for (int e = tid; e < R * R; e += NTHR) {
       const int i = e / R, r = e - i * R;
       if (i < r) continue;
       float a1 = 0.f, a2 = 0.f;
@@ -325,7 +326,7 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
       ckp[i * BT + r] = a1;
       cvp[i * BT + r] = a2;
     }
-    for (int e = tid; e < R * M; e += 256) {
+    for (int e = tid; e < R * M; e += NTHR) {
       const int r = e / M, m = e - r * M;
       float acc = 0.f;
       const float gr = gcl[r * LM + m];
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(256) void bwd_intra_kernel(const BP p) {
     }
   }
   __syncthreads();
-  for (int e = tid; e < R * M; e += 256) {
+  for (int e = tid; e < R * M; e += NTHR) {
     const int r = e / M, m = e - r * M;
     p.dsi[((int64_t)(c0 + r) * H + h) * M + m] = dsl[r * LM + m];
   }
@@ -838,7 +839,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     hipLaunchKernelGGL((bwd_q_window_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_qw, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_bwd(window query pass)");
   }
-  hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(256), lds_i, st, p);
+  hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(512), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
   hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
