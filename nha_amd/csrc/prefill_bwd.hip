@@ -326,13 +326,39 @@ __global__ __launch_bounds__(512) void bwd_intra_kernel(const BP p) {
       ckp[i * BT + r] = a1;
       cvp[i * BT + r] = a2;
     }
-    for (int e = tid; e < R * M; e += NTHR) {
-      const int r = e / M, m = e - r * M;
-      float acc = 0.f;
-      const float gr = gcl[r * LM + m];
-      for (int i = r; i < R; ++i)
-        acc += (Am[i * (BT + 1) + r] * du[i * LM + m] + Bm[i * (BT + 1) + r] * pl[i * LM + m]) * expf(gcl[i * LM + m] - gr);
-      dsl[r * LM + m] += acc;
+    if (M == 64) {
+      // a thread's BT*64/NTHR outputs share the slot m (rows rb, rb + 8, ...): du_i[m], p_i[m] and
+      // gc_i[m] are read once per i
+      const int rb = tid >> 6, m = tid & 63;
+      float acc[BT * 64 / NTHR], gr[BT * 64 / NTHR];
+#pragma unroll
+      for (int u = 0; u < BT * 64 / NTHR; ++u) {
+        acc[u] = 0.f;
+        const int r = rb + (NTHR / 64) * u;
+        gr[u] = r < R ? gcl[r * LM + m] : 0.f;
+      }
+      for (int i = rb; i < R; ++i) {
+        const float dui = du[i * LM + m], pli = pl[i * LM + m], gi = gcl[i * LM + m];
+#pragma unroll
+        for (int u = 0; u < BT * 64 / NTHR; ++u) {
+          const int r = rb + (NTHR / 64) * u;
+          if (i >= r) acc[u] += (Am[i * (BT + 1) + r] * dui + Bm[i * (BT + 1) + r] * pli) * expf(gi - gr[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < BT * 64 / NTHR; ++u) {
+        const int r = rb + (NTHR / 64) * u;
+        if (r < R) dsl[r * LM + m] += acc[u];
+      }
+    } else {
+      for (int e = tid; e < R * M; e += NTHR) {
+        const int r = e / M, m = e - r * M;
+        float acc = 0.f;
+        const float gr = gcl[r * LM + m];
+        for (int i = r; i < R; ++i)
+          acc += (Am[i * (BT + 1) + r] * du[i * LM + m] + Bm[i * (BT + 1) + r] * pl[i * LM + m]) * expf(gcl[i * LM + m] - gr);
+        dsl[r * LM + m] += acc;
+      }
     }
   }
   __syncthreads();
@@ -414,22 +440,34 @@ __global__ __launch_bounds__(256) void bwd_state_direct_kernel(const BP p) {
       Lw[i * LM + m] = wsrc[((int64_t)(c0 + i) * HQ + hq) * M + m] * expf(gcl[i * LM + m]);
     }
     __syncthreads();
+    // a thread's BT*CB/256 intra sums share the column x (rows rb, rb + 256/CB, ...): one read of
+    // x_i[x] serves all of them (Cm is zero above the diagonal)
+    {
+      const int rb = tid / CB, x = tid % CB;
+      for (int i = rb; i < R; ++i) {
+        const float xv = xq[i * (CB + 1) + x];
 #pragma unroll
-    for (int u = 0; u < BT * CB / 256; ++u) {
-      const int e = tid + 256 * u;
-      const int r = e / CB, x = e - r * CB;
-      float s2 = 0.f;
-      for (int i = r; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Cm[i * (BT + 1) + r];
-      acc[u] += s2;
+        for (int u = 0; u < BT * CB / 256; ++u) acc[u] += xv * Cm[i * (BT + 1) + rb + (256 / CB) * u];
+      }
     }
+    if (M == 64) {
+      // likewise its CB*64/256 elements of N share the slot m (columns xb, xb + 4, ...)
+      const int xb = tid >> 6, m = tid & 63;
+      for (int i = 0; i < R; ++i) {
+        const float lw = Lw[i * LM + m];
 #pragma unroll
-    for (int u = 0; u < CB * 64 / 256; ++u) {
-      const int e = tid + 256 * u;
-      const int x = e / M, m = e - x * M;
-      if (e < CB * M) {
-        float s2 = 0.f;
-        for (int i = 0; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Lw[i * LM + m];
-        en[u] += s2;
+        for (int u = 0; u < CB * 64 / 256; ++u) en[u] += xq[i * (CB + 1) + xb + 4 * u] * lw;
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < CB * 64 / 256; ++u) {
+        const int e = tid + 256 * u;
+        const int x = e / M, m = e - x * M;
+        if (e < CB * M) {
+          float s2 = 0.f;
+          for (int i = 0; i < R; ++i) s2 += xq[i * (CB + 1) + x] * Lw[i * LM + m];
+          en[u] += s2;
+        }
       }
     }
   }
@@ -534,23 +572,53 @@ __global__ __launch_bounds__(256) void bwd_state_inter_kernel(const BP p) {
     xk[r * (CB + 1) + x] = (sj >= 0 && x0 + x < X) ? Elem<T>::ld(xrow_src + ((int64_t)sj * H + h) * X + x0 + x) : 0.f;
   }
   __syncthreads();
-  // dk'_r[x] = intra part + sum_m sE_r[m] E[x][m];  ds part = dec_r[m] sum_x k'_r[x] E[x][m]
+  // dk'_r[x] = intra part + sum_m sE_r[m] E[x][m];  ds part = dec_r[m] sum_x k'_r[x] E[x][m].
+  // A thread's outputs share x (resp. m), so every E element it reads serves all of them.
   float* part = isv ? p.dvs : p.dks;
-  for (int e = tid; e < R * CB; e += 256) {
-    const int r = e / CB, x = e - r * CB;
-    const int sj = src[r];
-    if (sj < 0 || x0 + x >= X) continue;
-    const int64_t oi = ((int64_t)sj * H + h) * X + x0 + x;
-    float a = part[oi];
-    for (int m = 0; m < M; ++m) a += sE[r * LM + m] * E[x * LM + m];
-    if (isv) p.dvs[oi] = a;
-    else Elem<T>::st((T*)p.dk_gsa + oi, a);
+  {
+    const int rb = tid / CB, x = tid % CB;
+    float a[BT * CB / 256];
+#pragma unroll
+    for (int u = 0; u < BT * CB / 256; ++u) a[u] = 0.f;
+    for (int m = 0; m < M; ++m) {
+      const float ev = E[x * LM + m];
+#pragma unroll
+      for (int u = 0; u < BT * CB / 256; ++u) a[u] += sE[(rb + (256 / CB) * u) * LM + m] * ev;
+    }
+#pragma unroll
+    for (int u = 0; u < BT * CB / 256; ++u) {
+      const int r = rb + (256 / CB) * u;
+      if (r >= R) continue;
+      const int sj = src[r];
+      if (sj < 0 || x0 + x >= X) continue;
+      const int64_t oi = ((int64_t)sj * H + h) * X + x0 + x;
+      const float val = part[oi] + a[u];
+      if (isv) p.dvs[oi] = val;
+      else Elem<T>::st((T*)p.dk_gsa + oi, val);
+    }
   }
-  for (int e = tid; e < R * M; e += 256) {
-    const int r = e / M, m = e - r * M;
-    float a = 0.f;
-    for (int x = 0; x < CB; ++x) a += xk[r * (CB + 1) + x] * E[x * LM + m];
-    p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a * dec[r * LM + m];
+  if (M == 64) {
+    const int rb = tid >> 6, m = tid & 63;
+    float a[BT * 64 / 256];
+#pragma unroll
+    for (int u = 0; u < BT * 64 / 256; ++u) a[u] = 0.f;
+    for (int x = 0; x < CB; ++x) {
+      const float ev = E[x * LM + m];
+#pragma unroll
+      for (int u = 0; u < BT * 64 / 256; ++u) a[u] += xk[(rb + 4 * u) * (CB + 1) + x] * ev;
+    }
+#pragma unroll
+    for (int u = 0; u < BT * 64 / 256; ++u) {
+      const int r = rb + 4 * u;
+      if (r < R) p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a[u] * dec[r * LM + m];
+    }
+  } else {
+    for (int e = tid; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      float a = 0.f;
+      for (int x = 0; x < CB; ++x) a += xk[r * (CB + 1) + x] * E[x * LM + m];
+      p.dsp[(((int64_t)slab * p.T_tot + c0 + r) * H + h) * M + m] = a * dec[r * LM + m];
+    }
   }
 }
 
