@@ -108,6 +108,25 @@ def test_bwd_window_edges_on_the_matrix_cores(wl, shift):
     run_bwd_case(f"window wl={wl}", d, wl=wl, shift=shift, dtype=BF, cu=cu, scale=0.125, with_dht=True)
 
 
+def test_bwd_matrix_core_path_matches_fp32_path_at_size():
+    """A size the CPU recurrence cannot differentiate in seconds (B=2, T=1536, 8/2 heads, D=128,
+    W=512, both conventions): the bf16 call (matrix-core state recomputation and window kernels)
+    against the fp32 call (generic kernels only) on the same bf16-rounded inputs and cotangent."""
+    from nha_amd import chunk_nha
+    B, T, HQ, H, D, M, W = 2, 1536, 8, 2, 128, 64, 512
+    d = prefill_inputs(7500, B, T, HQ, H, D, D, M, dtype=BF, qk_scale=D ** -0.5, gate_div=1.0, gate_mean=-1.0)
+    do = torch.randn(B, T, HQ, D, generator=torch.Generator().manual_seed(3)).to(BF)
+    for wl, shift in ((W - 1, W), (W, 0)):
+        grads = []
+        for dt in (BF, torch.float32):
+            x = [d[k].cuda().to(dt).requires_grad_(True) for k in KEYS]
+            o = chunk_nha(*x, window_size_left=wl, gsa_kv_shift=shift)[0]
+            o.backward(do.cuda().to(dt))
+            grads.append([t.grad for t in x])
+        for k, gb, gf in zip(KEYS, *grads):
+            check_grad(f"size wl={wl} d{k}", gb, gf.double().cpu(), BF)
+
+
 def test_bwd_rejects_unsupported_shapes():
     from nha_amd import NhaError, chunk_nha
     d = prefill_inputs(7300, 1, 64, 2, 2, 64, 64, 128, dtype=torch.float32)
