@@ -138,7 +138,8 @@ int prefill_simple_impl(const NhaPrefillArgs* a);
 bool prefill_mfma_supported(const NhaPrefillArgs* a);
 size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_mfma_impl(const NhaPrefillArgs* a);
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct);
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb);
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, float* ap, float* bp, float* ust, float* dpst);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);

@@ -48,6 +48,8 @@ struct BP {
   float *dsi;             // [T_tot][H][M]     intra-chunk part of ds, indexed by row token
   float *dsp;             // [nbk+nbv][T_tot][H][M]  inter-chunk part of ds per column block
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
+  const float *ap, *bp;   // [NT][HQ][BT][BT]  q_gsa_i . k'_j and do_i . v'_j from the matrix cores, or NULL
+  const float *ust, *dpst; // [T_tot][HQ][M]    q_gsa_t . hk0[:,m] and do_t . hv0[m,:] (chunk-start states), or NULL
   float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
   float *dks;             // [T_tot][H][K]     intra-chunk part of dk_gsa, indexed by SOURCE token
   float *ek, *ev;         // [NT][H][K][M], [NT][H][V][M]  N_c, then E_c (see the state-gradient kernels)
@@ -120,8 +122,14 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     const int j = lane;
     const bool has = j <= rr && tl0 + j >= 0;
     const int64_t sj = (int64_t)bos + tl0 + j;
-    Aj[j] = has ? dot_row<T>(qg, kgs + (sj * H + h) * K, K) : 0.f;
-    Bj[j] = has ? dot_row<T>(dov, vv_ + (sj * H + h) * V, V) : 0.f;
+    if (p.ap) {
+      const int64_t pi = (((int64_t)chunk * HQ + hq) * BT + rr) * BT + j;
+      Aj[j] = has ? p.ap[pi] * p.scale : 0.f;
+      Bj[j] = has ? p.bp[pi] : 0.f;
+    } else {
+      Aj[j] = has ? dot_row<T>(qg, kgs + (sj * H + h) * K, K) : 0.f;
+      Bj[j] = has ? dot_row<T>(dov, vv_ + (sj * H + h) * V, V) : 0.f;
+    }
   }
   __syncthreads();
   const float* hk0 = p.hkc + ((int64_t)chunk * H + h) * K * M;
@@ -134,10 +142,15 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   if (lane < M) {
     const int m = lane;
     float au = 0.f, ad = 0.f;
+    if (p.ust) {
+      au = p.ust[tq * M + m] * p.scale;
+      ad = p.dpst[tq * M + m];
+    } else {
 #pragma unroll 8
-    for (int kk = 0; kk < K; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
+      for (int kk = 0; kk < K; ++kk) au += qg[kk] * hk0[(int64_t)kk * M + m];
 #pragma unroll 8
-    for (int c = 0; c < V; ++c) ad += dov[c] * hv0t[(int64_t)c * M + m];
+      for (int c = 0; c < V; ++c) ad += dov[c] * hv0t[(int64_t)c * M + m];
+    }
     const float gm = gct[m];
     const float e = expf(gm);
     au *= e;
@@ -300,7 +313,10 @@ __global__ __launch_bounds__(512) void bwd_intra_kernel(const BP p) {
       if (i < r) continue;
       const int sj = src[r];
       float av = 0.f, bv = 0.f;
-      if (sj >= 0) {
+      if (sj >= 0 && p.ap) {
+        av = p.ap[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r];
+        bv = p.bp[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r];
+      } else if (sj >= 0) {
         const T* qrow = (const T*)p.q_gsa + ((int64_t)(c0 + i) * HQ + hq) * K;
         const T* krow = (const T*)p.k_gsa + ((int64_t)sj * H + h) * K;
         av = dot_rows<T>(qrow, krow, K);
@@ -780,7 +796,7 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, mfma, hkct, hvct, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
+  size_t fwd, mfma, hkct, hvct, hkb, hvb, ap, bp, ust, dpst, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
   bool use_mfma;
   int nbk, nbv;
 };
@@ -796,6 +812,15 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   if (s.use_mfma) off += aligned(prefill_mfma_scratch_bytes(&f));
   s.hkct = off; off += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
   s.hvct = off; off += aligned((size_t)a->NT * a->H * a->V * a->M * 4);
+  s.hkb = s.hvb = s.ap = s.bp = s.ust = s.dpst = off;
+  if (s.use_mfma) {
+    s.hkb = off; off += aligned((size_t)a->NT * a->H * a->M * a->K * 2);
+    s.hvb = off; off += aligned((size_t)a->NT * a->H * a->M * a->V * 2);
+    s.ap = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
+    s.bp = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
+    s.ust = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
+    s.dpst = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
+  }
   s.hkT = off; off += aligned((size_t)a->N * a->H * a->K * a->M * 4);
   s.hvT = off; off += aligned((size_t)a->N * a->H * a->M * a->V * 4);
   const size_t tqm = aligned((size_t)a->T_tot * a->HQ * a->M * 4);
@@ -850,7 +875,9 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     f.scratch = sc + sp.mfma;
     f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
     rc = prefill_mfma_impl(&f);
-    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, (float*)(sc + sp.hkct), (float*)(sc + sp.hvct));
+    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, (float*)(sc + sp.hkct), (float*)(sc + sp.hvct), sc + sp.hkb, sc + sp.hvb);
+    // the decay-free products of the slot branch on the matrix cores
+    if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst));
   } else {
     f.scratch = sc + sp.fwd;
     f.scratch_bytes = prefill_simple_scratch_bytes(&f);
@@ -868,6 +895,11 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
   p.gc = gc; p.hkc = hkc; p.hvc = hvc;
   p.hkct = (float*)(sc + sp.hkct); p.hvct = (float*)(sc + sp.hvct);
+  p.ap = p.bp = p.ust = p.dpst = nullptr;
+  if (sp.use_mfma) {
+    p.ap = (float*)(sc + sp.ap); p.bp = (float*)(sc + sp.bp);
+    p.ust = (float*)(sc + sp.ust); p.dpst = (float*)(sc + sp.dpst);
+  }
   p.hkT = (float*)(sc + sp.hkT); p.hvT = (float*)(sc + sp.hvT);
   p.dus = (float*)(sc + sp.dus); p.pp = (float*)(sc + sp.pp); p.xg = (float*)(sc + sp.xg);
   p.delta = (float*)(sc + sp.delta);

@@ -359,6 +359,94 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
   }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Slot branch, products that do not involve the decay: per (chunk, q-head)
+//   A[i][j] = q_gsa_i . k'_j      B[i][j] = do_i . v'_j          (rows i, j of the chunk; k', v' read at
+//   U0[i][m] = q_gsa_i . hk0[:,m]  P0[i][m] = do_i . hv0[m,:]      the source token of row j)
+// all of the form X Y^T with X in {q_gsa, do} (64 rows through LDS) and Y in {k', hk0^T, v', hv0}
+// (64 rows as register fragments, 16 per wave).  grid (HQ, NT), 4 waves.
+// ------------------------------------------------------------------------------------------
+struct SP1 {
+  const bf16_t *q, *dout, *kg, *v;   // q_gsa [T,HQ,D], dout [T,HQ,D], k_gsa [T,H,D], v [T,H,D]
+  const bf16_t *hkb, *hvb;           // [NT][H][64][D] chunk-start states, hk transposed
+  float *ap, *bp;                    // [NT][HQ][64][64]
+  float *ust, *dpst;                 // [T][HQ][64]
+  const int32_t *cu, *cidx;
+  int HQ, H, NG, shift;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
+  constexpr int KS = D / 32, LDT = D + 16, TILE = BT * LDT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* const Qt = (lbf16*)smem;
+  lbf16* const Ot = Qt + TILE;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ;
+  const int hq = blockIdx.x, h = hq / p.NG;
+  const int chunk = blockIdx.y;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  {
+    Tile<BT, D> rq, ro;
+    rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    rq.store(Qt, tid);
+    ro.store(Ot, tid);
+  }
+  // this lane's Y rows: row j = 16 wave + l16 of the chunk (source token c0 + j - shift), slot m = j
+  const int j = 16 * wave + l16;
+  const int tl = it * BT + j - p.shift;
+  const bool has = j < R && tl >= 0;
+  const int64_t sj = ((int64_t)bos + (has ? tl : 0)) * H + h;
+  const int64_t cg = ((int64_t)chunk * H + h) * BT + j;
+  bf16x8 yk[KS], yv[KS], yhk[KS], yhv[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    uint4 a = make_uint4(0, 0, 0, 0), b = a;
+    if (has) {
+      a = *reinterpret_cast<const uint4*>(p.kg + sj * D + 32 * ks + 8 * kb);
+      b = *reinterpret_cast<const uint4*>(p.v + sj * D + 32 * ks + 8 * kb);
+    }
+    yk[ks] = __builtin_bit_cast(bf16x8, a);
+    yv[ks] = __builtin_bit_cast(bf16x8, b);
+    yhk[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkb + cg * D + 32 * ks + 8 * kb));
+    yhv[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvb + cg * D + 32 * ks + 8 * kb));
+  }
+  lds_barrier();
+  float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+  float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+#pragma unroll
+  for (int blk = 0; blk < 4; ++blk) {
+    f32x4 cA = {0.f, 0.f, 0.f, 0.f}, cB = cA, cU = cA, cP = cA;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 xq = lds_frag(Qt, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
+      const bf16x8 xo = lds_frag(Ot, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
+      cA = mfma16(xq, yk[ks], cA);
+      cU = mfma16(xq, yhk[ks], cU);
+      cB = mfma16(xo, yv[ks], cB);
+      cP = mfma16(xo, yhv[ks], cP);
+    }
+    // C[i = 16 blk + 4 kb + r][j = 16 wave + l16]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = 16 * blk + 4 * kb + r;
+      ap[i * BT + j] = cA[r];
+      bp[i * BT + j] = cB[r];
+      if (i < R) {
+        const int64_t tq = ((int64_t)(c0 + i) * HQ + hq) * BT + j;
+        p.ust[tq] = cU[r];
+        p.dpst[tq] = cP[r];
+      }
+    }
+  }
+}
+
 template <int D, int TK>
 int launch_dq(const WP& p, int NT, hipStream_t st) {
   const size_t lds = (size_t)4 * TK * (D + 16) * 2;
@@ -427,6 +515,37 @@ int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const fl
   int rc = launch_dkv<256, 32, 1>(p, a->NT, st);
   if (rc != NHA_OK) return rc;
   return launch_dkv<256, 32, 2>(p, a->NT, st);
+}
+
+template <int D>
+static int launch_slot_products(const SP1& p, int NT, hipStream_t st) {
+  const size_t lds = (size_t)2 * BT * (D + 16) * 2;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_products_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) {
+      set_error("nha_prefill_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+      return NHA_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL((bwd_slot_products_kernel<D>), dim3(p.HQ, NT), dim3(256), lds, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products)");
+  return NHA_OK;
+}
+
+// bf16, K == V in {64,128,256}, M == 64 (the shapes of the matrix-core state pass)
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, float* ap, float* bp, float* ust, float* dpst) {
+  SP1 p;
+  p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.v = (const bf16_t*)a->v;
+  p.hkb = (const bf16_t*)hkb; p.hvb = (const bf16_t*)hvb;
+  p.ap = ap; p.bp = bp; p.ust = ust; p.dpst = dpst;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
+  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->K == 64) return launch_slot_products<64>(p, a->NT, st);
+  if (a->K == 128) return launch_slot_products<128>(p, a->NT, st);
+  return launch_slot_products<256>(p, a->NT, st);
 }
 
 }  // namespace nha

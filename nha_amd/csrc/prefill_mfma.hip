@@ -1133,10 +1133,11 @@ int launch_repair(const MP& p, hipStream_t st) {
 
 // ==========================================================================================
 // fp32 copies of what the state pass left in the scratch for the backward pass: true chunk-start
-// states as hk [K][M] and transposed hk^T [M][K], hv^T [V][M]; gate cumsums per row token
+// states as hk [K][M] and transposed hk^T [M][K], hv^T [V][M], plus bf16 copies hk^T [M][K] and
+// hv [M][V] as matrix-core operands; gate cumsums per row token
 // ==========================================================================================
 template <int D>
-__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hkct, float* hvct) {
+__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hkct, float* hvct, bf16_t* hkb, bf16_t* hvb) {
   const int chunk = blockIdx.x, h = blockIdx.y, H = p.H;
   const int tid = threadIdx.x;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
@@ -1151,7 +1152,10 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
     const float hk = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
     hkc[(cg * D + d) * MS + m] = hk;
     hkct[(cg * MS + m) * D + d] = hk;
-    hvct[(cg * D + d) * MS + m] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+    const float hv = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+    hvct[(cg * D + d) * MS + m] = hv;
+    hkb[(cg * MS + m) * D + d] = f32_to_bf16(hk);
+    hvb[(cg * MS + m) * D + d] = f32_to_bf16(hv);
   }
   for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
 }
@@ -1286,14 +1290,15 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
 }
 
 // `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
-// [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct) {
+// [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies, hkb [NT][H][M][K] and
+// hvb [NT][H][M][V] bf16 copies
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
   const dim3 grid(a->NT, a->H);
-  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
-  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
-  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct);
+  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
+  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
+  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state export)");
   return NHA_OK;
 }
