@@ -16,9 +16,9 @@
 //   dg_r  = dg_(r+1) + sum_a (du u + p dp)_r - s_r ds_r        (dg past the end = <dh_T, h_T>)
 // (the last line is the usual reverse cumulative sum of gated linear attention: <Dh_r, h_r> telescopes).
 //
-// Launches: forward state pass (chunk-start states, gate cumsums) -> bwd_q_kernel (per token: dq's and
-// the per-token vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra
-// part of ds) -> bwd_state_{direct,scan,inter}_kernel (state gradients as a linear recurrence over
+// Launches: forward state pass (chunk-start states, gate cumsums) -> bwd_q_kernel (per token: the
+// vectors du, p) -> bwd_intra_kernel (per chunk: intra-chunk matrices and the intra part of ds)
+// -> bwd_dqg_kernel (per token: dq_gsa) -> bwd_state_{direct,scan,inter}_kernel (state gradients as a linear recurrence over
 // chunks: dk_gsa, slot-branch dv, inter-chunk part of ds, dh0) -> bwd_gate_*_kernel (reverse scan: ds, dg)
 // -> bwd_kv_window_kernel (per key: dk_swa, dv).  For bf16 tensors with K == V in {64,128,256} the
 // window parts (dq_swa, dk_swa, dv) run on the matrix cores instead (prefill_bwd_mfma.hip).
@@ -77,10 +77,10 @@ __device__ __forceinline__ float logaddexp_f(float a, float b) {
 }
 
 // ------------------------------------------------------------------------------------------
-// per (token, q-head), ONE WAVE each (4 tokens per workgroup): dq_gsa and the vectors du, p the
-// state gradients are built from.  Lanes run over the slots m (M <= 64), over the rows j of the
-// chunk, or over columns d, so that every global read of a state is coalesced: hkc [K][M] for u,
-// hvct [V][M] for dp, hkct [M][K] for dq_gsa.
+// per (token, q-head), ONE WAVE each (4 tokens per workgroup): the vectors du, p (and du u + p dp)
+// the other passes are built from.  Lanes run over the slots m (M <= 64) or over the rows j of
+// the chunk, so that every global read of a state is coalesced: hkc [K][M] for u, hvct [V][M] for
+// dp (bwd_dqg_kernel reads hkct [M][K]).
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
@@ -88,14 +88,11 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   const int K = p.K, V = p.V, M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  float* qg = lds + wv * (K + V + 3 * BT + 3 * M);   // [K] scaled slot-branch query
+  float* qg = lds + wv * (K + V + 2 * BT + M);   // [K] scaled slot-branch query
   float* dov = qg + K;        // [V]
   float* Aj = dov + V;        // [BT] q_gsa . k'_j
   float* Bj = Aj + BT;        // [BT] do . v'_j
-  float* Wj = Bj + BT;        // [BT]
-  float* gct = Wj + BT;       // [M]
-  float* dul = gct + M;       // [M] scale * du
-  float* due = dul + M;       // [M] scale * du * e^(gc_r)
+  float* gct = Bj + BT;       // [M]
   const int chunk = blockIdx.x / (BT / 4), r = (blockIdx.x % (BT / 4)) * 4 + wv;
   const int hq = blockIdx.y, h = hq / NG;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
@@ -134,7 +131,6 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   __syncthreads();
   const float* hk0 = p.hkc + ((int64_t)chunk * H + h) * K * M;
   const float* hv0t = p.hvct + ((int64_t)chunk * H + h) * V * M;
-  const float* hk0t = p.hkct + ((int64_t)chunk * H + h) * M * K;
   const float* gcb = p.gc + ((int64_t)(bos + it * BT) * H + h) * M;
   const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
   const float lt = logaddexp_f(ls, lg);
@@ -164,8 +160,6 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     }
     const float pm = expf(au - lt);
     const float du = pm * (ad - delta) + dlg * expf(au - lg);
-    dul[m] = p.scale * du;
-    due[m] = p.scale * du * e;
     if (valid) {
       p.dus[tq * M + m] = p.scale * du;
       p.pp[tq * M + m] = pm;
@@ -173,25 +167,40 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     }
   }
   if (lane == 0 && valid) p.delta[tq] = delta;
+}
+
+// ------------------------------------------------------------------------------------------
+// per (token, q-head), one wave each, after bwd_intra_kernel:
+//   dq_gsa[d] = sum_m scale du[m] hk_t[d][m]
+//             = sum_m (scale du[m] e^(gc_r[m])) hk0[d][m] + sum_(j<=r) ck[r][j] k'_j[d]
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_dqg_kernel(const BP p) {
+  extern __shared__ __align__(16) float lds[];
+  const int K = p.K, M = p.M, H = p.H, HQ = p.HQ;
+  const int NG = HQ / H;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  float* due = lds + wv * (M + BT);   // [M] scale * du * e^(gc_r)
+  float* Wj = due + M;                // [BT] row r of ck
+  const int chunk = blockIdx.x / (BT / 4), r = (blockIdx.x % (BT / 4)) * 4 + wv;
+  const int hq = blockIdx.y, h = hq / NG;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const bool valid = bos + it * BT + r < eos;
+  const int rr = valid ? r : 0;
+  const int t = bos + it * BT + rr;
+  const int64_t tq = (int64_t)t * HQ + hq;
+  if (lane < M) due[lane] = p.dus[tq * M + lane] * expf(p.gc[((int64_t)t * H + h) * M + lane]);
+  Wj[lane] = lane <= rr ? p.ck[(((int64_t)chunk * HQ + hq) * BT + rr) * BT + lane] : 0.f;
   __syncthreads();
-  {
-    // Wj[j] = sum_m scale du[m] s_j[m] e^(gc_r[m] - gc_j[m])
-    const int j = lane;
-    float acc = 0.f;
-    if (j <= rr && tl0 + j >= 0) {
-      const T* srow = ss + (((int64_t)bos + tl0 + j) * H + h) * M;
-      const float* gj = gcb + (int64_t)j * H * M;
-      for (int m = 0; m < M; ++m) acc += dul[m] * Elem<T>::ld(srow + m) * expf(gct[m] - gj[m]);
-    }
-    Wj[j] = acc;
-  }
-  __syncthreads();
-  // dq_gsa[d] = sum_m scale du[m] hk_t[d][m]
+  const float* hk0t = p.hkct + ((int64_t)chunk * H + h) * M * K;
+  const T* kgs = (const T*)p.k_gsa;
+  const int tl0 = it * BT - p.shift;
+  const int jlo = tl0 < 0 ? -tl0 : 0;
   for (int d = lane; d < K; d += 64) {
     float acc = 0.f;
 #pragma unroll 8
     for (int m = 0; m < M; ++m) acc += due[m] * hk0t[(int64_t)m * K + d];
-    const int jlo = tl0 < 0 ? -tl0 : 0;
     for (int j = jlo; j <= rr; ++j) acc += Wj[j] * Elem<T>::ld(kgs + (((int64_t)bos + tl0 + j) * H + h) * K + d);
     if (valid) Elem<T>::st((T*)p.dq_gsa + tq * K + d, acc);
   }
@@ -912,7 +921,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipStream_t st = (hipStream_t)a->stream;
   const int K = a->K, V = a->V, M = a->M, LM = M + 1;
 
-  const size_t lds_q = (size_t)4 * (K + V + 3 * BT + 3 * M) * 4;
+  const size_t lds_q = (size_t)4 * (K + V + 2 * BT + M) * 4;
   const size_t lds_qw = ((size_t)K + V + 256) * 4;
   const size_t lds_i = ((size_t)5 * BT * LM + 2 * BT * (BT + 1)) * 4 + BT * 4;
   const size_t lds_s1 = ((size_t)2 * BT * LM + BT * (BT + 1) + BT * (CB + 1)) * 4 + BT * 4;
@@ -941,6 +950,8 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(512), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
+  hipLaunchKernelGGL((bwd_dqg_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), (size_t)4 * (M + BT) * 4, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(dq_gsa pass)");
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
   hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
   hipLaunchKernelGGL(bwd_state_scan_kernel, dim3(a->N * a->H, ((K + V) * M + 255) / 256), dim3(256), 0, st, p);
