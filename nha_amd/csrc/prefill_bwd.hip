@@ -950,10 +950,20 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(512), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
-  hipLaunchKernelGGL((bwd_dqg_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), (size_t)4 * (M + BT) * 4, st, p);
-  NHA_CHECK_LAUNCH("nha_prefill_bwd(dq_gsa pass)");
+  if (sp.use_mfma) {
+    rc = bwd_slot_products2(a, 0, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs);
+    if (rc != NHA_OK) return rc;
+  } else {
+    hipLaunchKernelGGL((bwd_dqg_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), (size_t)4 * (M + BT) * 4, st, p);
+    NHA_CHECK_LAUNCH("nha_prefill_bwd(dq_gsa pass)");
+  }
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
-  hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
+  if (sp.use_mfma) {
+    rc = bwd_slot_products2(a, 1, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs);
+    if (rc != NHA_OK) return rc;
+  } else {
+    hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
+  }
   hipLaunchKernelGGL(bwd_state_scan_kernel, dim3(a->N * a->H, ((K + V) * M + 255) / 256), dim3(256), 0, st, p);
   hipLaunchKernelGGL((bwd_state_inter_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s3, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state gradients)");

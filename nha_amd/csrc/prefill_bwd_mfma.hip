@@ -447,6 +447,186 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Slot branch, products over the rows of a chunk (bf16 operands, fp32 accumulation).
+//
+// bwd_slot_state_kernel, grid (H, NT, 2): per (chunk, kv-head) and state (z = 0: k-state with
+// X = q_gsa, weights scale*du, matrix ck; z = 1: v-state with X = do, weights p, matrix cv), summed
+// over the q-heads of the group:
+//   N[x][m]  = sum_i X_i[x] w_i[m] e^(gc_i[m])        inhomogeneous term of the state-gradient recurrence
+//   out[r][x] = sum_(i>=r) c[i][r] X_i[x]              intra-chunk part of dk' / dv'
+// Both are X^T times a 64-row table, so they share the transposed X fragments (A operand); the
+// tables are staged transposed ([column][row i], bf16) so that a B fragment is two 8-byte reads.
+//
+// bwd_slot_dq_kernel, grid (HQ, NT): per (chunk, q-head)
+//   dq_gsa[i][d] = sum_m (scale du_i[m] e^(gc_i[m])) hk0[d][m] + sum_(j<=i) ck[i][j] k'_j[d]
+// as dQ^T = hk0 W^T + K'^T C^T with the state and the k' rows as transposed A fragments.
+// ------------------------------------------------------------------------------------------
+constexpr int TLD = 72;   // bf16 row stride of the 64 x 64 tables in LDS
+
+struct SP2 {
+  const bf16_t *q, *dout, *kg, *s;   // q_gsa, dout [T,HQ,D]; k_gsa [T,H,D]
+  const bf16_t* hkb;                 // [NT][H][64][D]
+  const float *dus, *pp, *ck, *cv;   // [T][HQ][64] x2, [NT][HQ][64][64] x2
+  const float* gc;                   // [T][H][64]
+  float *ek, *ev;                    // [NT][H][D][64] x2
+  float *dks, *dvs;                  // [T][H][D] x2 (source-token index)
+  bf16_t* dq;                        // dq_gsa [T,HQ,D]
+  const int32_t *cu, *cidx;
+  int HQ, H, NG, shift;
+};
+
+// B fragment from a transposed table tab[n][i] (row stride TLD): rows of the contraction
+// i = 32 hf + 4 kb + e (e < 4) and 32 hf + 16 + 4 kb + (e - 4), column n
+__device__ __forceinline__ bf16x8 table_frag(const lbf16* tab, int n, int hf, int kb) {
+  struct { bf16x4 a, b; } t;
+  t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(tab + n * TLD + 32 * hf + 4 * kb);
+  t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(tab + n * TLD + 32 * hf + 16 + 4 * kb);
+  return __builtin_bit_cast(bf16x8, t);
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
+  constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* const Xt = (lbf16*)smem;        // [64 rows i][D]
+  lbf16* const Wt = Xt + TILE;           // [64 m][TLD]  (w_i[m] e^(gc_i[m]))^T
+  lbf16* const Ct = Wt + BT * TLD;       // [64 r][TLD]  c[i][r]^T, zero for i < r
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ, NG = p.NG;
+  const int h = blockIdx.x, chunk = blockIdx.y;
+  const bool isv = blockIdx.z != 0;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const bf16_t* xsrc = isv ? p.dout : p.q;
+  const float* wsrc = isv ? p.pp : p.dus;
+  const float* csrc = isv ? p.cv : p.ck;
+  f32x4 accN[DB], accO[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    accN[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    accO[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  const int col = 16 * wave + l16;   // this lane's column: slot m of N, row r of out
+  for (int a = 0; a < NG; ++a) {
+    const int hq = h * NG + a;
+    if (a > 0) lds_barrier();   // everyone is done with the previous head's tiles
+    {
+      Tile<BT, D> rx;
+      rx.load(xsrc + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+      rx.store(Xt, tid);
+    }
+    const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
+    for (int e = tid; e < BT * BT; e += 256) {
+      const int i = e >> 6, c = e & 63;   // coalesced reads over c, transposed writes
+      float w = 0.f, cc = 0.f;
+      if (i < R) {
+        w = wsrc[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
+        if (c <= i) cc = cp[i * BT + c];
+      }
+      Wt[c * TLD + i] = f32_to_bf16(w);
+      Ct[c * TLD + i] = f32_to_bf16(cc);
+    }
+    lds_barrier();
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const bf16x8 bw = table_frag(Wt, col, hf, kb);
+      const bf16x8 bc = table_frag(Ct, col, hf, kb);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const bf16x8 xa = lds_frag_tr(Xt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // X^T[x][i]
+        accN[db] = mfma16(xa, bw, accN[db]);
+        accO[db] = mfma16(xa, bc, accO[db]);
+      }
+    }
+  }
+  // N[x = 16 db + 4 kb + r][m = col];  out^T[x][row = col]
+  float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
+  const int tl = it * BT + col - p.shift;
+  const bool has = col < R && tl >= 0;
+  float* op = (isv ? p.dvs : p.dks) + (((int64_t)bos + (has ? tl : 0)) * H + h) * D;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ep[(16 * db + 4 * kb + r) * BT + col] = accN[db][r];
+    if (has) *reinterpret_cast<float4*>(op + 16 * db + 4 * kb) = make_float4(accO[db][0], accO[db][1], accO[db][2], accO[db][3]);
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
+  constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* const Ht = (lbf16*)smem;        // [64 m][D]  hk0^T
+  lbf16* const Kt = Ht + TILE;           // [64 j][D]  k' rows
+  lbf16* const Wt = Kt + TILE;           // [64 i][TLD]  scale du_i[m] e^(gc_i[m])
+  lbf16* const Ct = Wt + BT * TLD;       // [64 i][TLD]  ck[i][j], zero for j > i
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ;
+  const int hq = blockIdx.x, h = hq / p.NG, chunk = blockIdx.y;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  {
+    Tile<BT, D> rh, rk;
+    rh.load(p.hkb + ((int64_t)chunk * H + h) * BT * D, D, 0, BT, tid);
+    // k' row j is the k_gsa row of source token c0 + j - shift: rows before the sequence are zero
+    int vlo = p.shift - it * BT;
+    vlo = vlo < 0 ? 0 : vlo;
+#pragma unroll
+    for (int u = 0; u < Tile<BT, D>::NPC; ++u) {
+      const int c = tid + 256 * u;
+      const int row = c / (D / 8), cc = (c % (D / 8)) * 8;
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(p.kg + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
+      rk.r[u] = x;
+    }
+    rh.store(Ht, tid);
+    rk.store(Kt, tid);
+  }
+  const float* cp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
+  for (int e = tid; e < BT * BT; e += 256) {
+    const int i = e >> 6, c = e & 63;
+    float w = 0.f, cc = 0.f;
+    if (i < R) {
+      w = p.dus[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
+      if (c <= i) cc = cp[i * BT + c];
+    }
+    Wt[i * TLD + c] = f32_to_bf16(w);
+    Ct[i * TLD + c] = f32_to_bf16(cc);
+  }
+  lds_barrier();
+  const int i = 16 * wave + l16;   // this lane's row of the chunk
+  f32x4 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    const bf16x8 bw = table_frag(Wt, i, hf, kb);   // contraction over m
+    const bf16x8 bc = table_frag(Ct, i, hf, kb);   // contraction over j
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      acc[db] = mfma16(lds_frag_tr(Ht, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane), bw, acc[db]);   // hk0[d][m]
+      acc[db] = mfma16(lds_frag_tr(Kt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane), bc, acc[db]);   // k'_j[d]
+    }
+  }
+  if (i < R) {
+    bf16_t* op = p.dq + ((int64_t)(c0 + i) * HQ + hq) * D + 4 * kb;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      bf16x4 pk;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pk[r] = (__bf16)acc[db][r];
+      *reinterpret_cast<bf16x4*>(op + 16 * db) = pk;
+    }
+  }
+}
+
 template <int D, int TK>
 int launch_dq(const WP& p, int NT, hipStream_t st) {
   const size_t lds = (size_t)4 * TK * (D + 16) * 2;
@@ -546,6 +726,44 @@ int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* h
   if (a->K == 64) return launch_slot_products<64>(p, a->NT, st);
   if (a->K == 128) return launch_slot_products<128>(p, a->NT, st);
   return launch_slot_products<256>(p, a->NT, st);
+}
+
+template <int D>
+static int launch_slot_stage2(const SP2& p, int NT, bool state, hipStream_t st) {
+  const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
+  const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
+    hipError_t e2 = hipFuncSetAttribute((const void*)bwd_slot_dq_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("nha_prefill_bwd: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+      return NHA_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  if (state) hipLaunchKernelGGL((bwd_slot_state_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_s, st, p);
+  else hipLaunchKernelGGL((bwd_slot_dq_kernel<D>), dim3(p.HQ, NT), dim3(256), lds_q, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products, second stage)");
+  return NHA_OK;
+}
+
+// which = 0: dq_gsa (bwd_slot_dq_kernel); 1: N_c and the intra-chunk parts of dk' / dv'
+// (bwd_slot_state_kernel).  Same shapes as bwd_slot_products.
+int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
+                       const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs) {
+  SP2 p;
+  p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.s = (const bf16_t*)a->s;
+  p.hkb = (const bf16_t*)hkb;
+  p.dus = dus; p.pp = pp; p.ck = ck; p.cv = cv; p.gc = gc;
+  p.ek = ek; p.ev = ev; p.dks = dks; p.dvs = dvs;
+  p.dq = (bf16_t*)a->dq_gsa;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
+  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->K == 64) return launch_slot_stage2<64>(p, a->NT, which != 0, st);
+  if (a->K == 128) return launch_slot_stage2<128>(p, a->NT, which != 0, st);
+  return launch_slot_stage2<256>(p, a->NT, which != 0, st);
 }
 
 }  // namespace nha
