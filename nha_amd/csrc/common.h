@@ -140,7 +140,7 @@ size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_mfma_impl(const NhaPrefillArgs* a);
 int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb);
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
-                       const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs);
+                       const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs, float* dsp);
 int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, float* ap, float* bp, float* ust, float* dpst);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);

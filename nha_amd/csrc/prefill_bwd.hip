@@ -712,11 +712,25 @@ __global__ void bwd_gate_scan_kernel(const BP p) {
     const float* b = p.hvT + (((int64_t)n * H + h) * M + m) * V;
     for (int c = 0; c < V; ++c) run += a[c] * b[c];
   }
+  // four chunk sums are fetched before the first is consumed, so the loads overlap
   const int nchunks = (eos - bos + BT - 1) / BT;
-  for (int it = nchunks - 1; it >= 0; --it) {
-    const int64_t idx = ((int64_t)(p.coff[n] + it) * H + h) * M + m;
-    const float tot = p.gtot[idx];
-    p.gtot[idx] = run;
+  float* gt = p.gtot + ((int64_t)p.coff[n] * H + h) * M + m;
+  const int64_t cs = (int64_t)H * M;
+  int it = nchunks - 1;
+  for (; it >= 3; it -= 4) {
+    const float t0 = gt[it * cs], t1 = gt[(it - 1) * cs], t2 = gt[(it - 2) * cs], t3 = gt[(it - 3) * cs];
+    gt[it * cs] = run;
+    run += t0;
+    gt[(it - 1) * cs] = run;
+    run += t1;
+    gt[(it - 2) * cs] = run;
+    run += t2;
+    gt[(it - 3) * cs] = run;
+    run += t3;
+  }
+  for (; it >= 0; --it) {
+    const float tot = gt[it * cs];
+    gt[it * cs] = run;
     run += tot;
   }
 }
@@ -951,7 +965,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(512), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");
   if (sp.use_mfma) {
-    rc = bwd_slot_products2(a, 0, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs);
+    rc = bwd_slot_products2(a, 0, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs, p.dsp);
     if (rc != NHA_OK) return rc;
   } else {
     hipLaunchKernelGGL((bwd_dqg_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), (size_t)4 * (M + BT) * 4, st, p);
@@ -959,13 +973,20 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   const int nbmax = sp.nbk > sp.nbv ? sp.nbk : sp.nbv;
   if (sp.use_mfma) {
-    rc = bwd_slot_products2(a, 1, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs);
+    rc = bwd_slot_products2(a, 1, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs, p.dsp);
     if (rc != NHA_OK) return rc;
   } else {
     hipLaunchKernelGGL((bwd_state_direct_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s1, st, p);
   }
   hipLaunchKernelGGL(bwd_state_scan_kernel, dim3(a->N * a->H, ((K + V) * M + 255) / 256), dim3(256), 0, st, p);
-  hipLaunchKernelGGL((bwd_state_inter_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s3, st, p);
+  if (sp.use_mfma) {
+    // one partial-ds slab per state instead of one per 32-column block
+    p.nbk = p.nbv = 1;
+    rc = bwd_slot_products2(a, 2, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs, p.dsp);
+    if (rc != NHA_OK) return rc;
+  } else {
+    hipLaunchKernelGGL((bwd_state_inter_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s3, st, p);
+  }
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state gradients)");
   hipLaunchKernelGGL((bwd_gate_local_kernel<T>), dim3(a->NT, a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);

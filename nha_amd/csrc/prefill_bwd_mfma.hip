@@ -471,6 +471,10 @@ struct SP2 {
   const float* gc;                   // [T][H][64]
   float *ek, *ev;                    // [NT][H][D][64] x2
   float *dks, *dvs;                  // [T][H][D] x2 (source-token index)
+  float* dsp;                        // [2][T][H][64] inter-chunk part of ds per state
+  const bf16_t* v;                   // [T,H,D]
+  bf16_t* dkg;                       // dk_gsa [T,H,D]
+  int T_tot;
   bf16_t* dq;                        // dq_gsa [T,HQ,D]
   const int32_t *cu, *cidx;
   int HQ, H, NG, shift;
@@ -627,6 +631,106 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   }
 }
 
+// bwd_slot_inter_kernel, grid (H, NT, 2): the parts that involve E_c, the state gradient carried
+// into the END of chunk c (z = 0: k-state, rows k', output dk_gsa; z = 1: v-state, rows v', output
+// dvs), with dec_r[m] = e^(gl[m] - gc_r[m]):
+//   out[r][x] = intra part + sum_m (s_r[m] dec_r[m]) E[x][m]         as out^T = E sE^T
+//   dsp[r][m] = dec_r[m] sum_x y_r[x] E[x][m]                         as Y E
+template <int D>
+__global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
+  constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT, ELD = BT + 8;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* const Yt = (lbf16*)smem;        // [64 rows r][D]   k' / v'
+  lbf16* const Et = Yt + TILE;           // [D x][ELD]       E[x][m]
+  lbf16* const St = Et + D * ELD;        // [64 r][TLD]      s_r[m] dec_r[m]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H;
+  const int h = blockIdx.x, chunk = blockIdx.y;
+  const bool isv = blockIdx.z != 0;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  const bf16_t* ysrc = isv ? p.v : p.kg;
+  int vlo = p.shift - it * BT;
+  vlo = vlo < 0 ? 0 : vlo;
+  {
+    Tile<BT, D> ry;
+#pragma unroll
+    for (int u = 0; u < Tile<BT, D>::NPC; ++u) {
+      const int c = tid + 256 * u;
+      const int row = c / (D / 8), cc = (c % (D / 8)) * 8;
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(ysrc + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
+      ry.r[u] = x;
+    }
+    ry.store(Yt, tid);
+  }
+  const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
+  for (int e = tid; e < D * BT; e += 256) Et[(e >> 6) * ELD + (e & 63)] = f32_to_bf16(ep[e]);
+  const float* gcb = p.gc + ((int64_t)c0 * H + h) * BT;
+  for (int e = tid; e < BT * BT; e += 256) {
+    const int r = e >> 6, m = e & 63;
+    float v = 0.f;
+    if (r >= vlo && r < R)
+      v = bf16_to_f32(p.s[(((int64_t)c0 + r - p.shift) * H + h) * BT + m]) *
+          __expf(gcb[(int64_t)(R - 1) * H * BT + m] - gcb[(int64_t)r * H * BT + m]);
+    St[r * TLD + m] = f32_to_bf16(v);
+  }
+  lds_barrier();
+  const int col = 16 * wave + l16;
+  // out^T[x][r = col] = sum_m E[x][m] sE[r][m]: A = E rows (plain), B = sE rows (plain), contraction m in 2 steps
+  f32x4 accO[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) accO[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    const bf16x8 bs = lds_frag(St, TLD, col, 32 * ks + 8 * kb);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) accO[db] = mfma16(lds_frag(Et, ELD, 16 * db + l16, 32 * ks + 8 * kb), bs, accO[db]);
+  }
+  const bool has = col >= vlo && col < R;
+  if (has) {
+    const int64_t oi = (((int64_t)c0 + col - p.shift) * H + h) * D;
+    float* part = isv ? p.dvs : p.dks;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const float4 pv = *reinterpret_cast<const float4*>(part + oi + 16 * db + 4 * kb);
+      const float o0 = accO[db][0] + pv.x, o1 = accO[db][1] + pv.y, o2 = accO[db][2] + pv.z, o3 = accO[db][3] + pv.w;
+      if (isv) {
+        *reinterpret_cast<float4*>(p.dvs + oi + 16 * db + 4 * kb) = make_float4(o0, o1, o2, o3);
+      } else {
+        bf16x4 pk;
+        pk[0] = (__bf16)o0; pk[1] = (__bf16)o1; pk[2] = (__bf16)o2; pk[3] = (__bf16)o3;
+        *reinterpret_cast<bf16x4*>(p.dkg + oi + 16 * db + 4 * kb) = pk;
+      }
+    }
+  }
+  // dsp[r][m = col] = dec_r[m] sum_x y_r[x] E[x][m]: A = y rows (two 8-byte reads, contraction index
+  // permuted like the transposing read), B = E via the transposing read
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int xs = 0; xs < D / 32; ++xs) {
+      struct { bf16x4 a, b; } t;
+      t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 4 * kb);
+      t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 16 + 4 * kb);
+      acc = mfma16(__builtin_bit_cast(bf16x8, t), lds_frag_tr(Et, ELD, 32 * xs, 32 * xs + 16, 16 * wave, lane), acc);
+    }
+    // C[r = 16 rb + 4 kb + q][m = col]
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = 16 * rb + 4 * kb + q;
+      if (r < R) {
+        const float dec = __expf(gcb[(int64_t)(R - 1) * H * BT + col] - gcb[(int64_t)r * H * BT + col]);
+        p.dsp[(((int64_t)(isv ? 1 : 0) * p.T_tot + c0 + r) * H + h) * BT + col] = acc[q] * dec;
+      }
+    }
+  }
+}
+
 template <int D, int TK>
 int launch_dq(const WP& p, int NT, hipStream_t st) {
   const size_t lds = (size_t)4 * TK * (D + 16) * 2;
@@ -729,41 +833,48 @@ int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* h
 }
 
 template <int D>
-static int launch_slot_stage2(const SP2& p, int NT, bool state, hipStream_t st) {
+static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
   const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
   const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
+  const size_t lds_i = (size_t)BT * (D + 16) * 2 + (size_t)D * (BT + 8) * 2 + (size_t)BT * TLD * 2;
   static bool configured = false;
   if (!configured) {
     hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
     hipError_t e2 = hipFuncSetAttribute((const void*)bwd_slot_dq_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
+    hipError_t e3 = hipFuncSetAttribute((const void*)bwd_slot_inter_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_i);
+    if (e1 == hipSuccess) e1 = e3;
     if (e1 != hipSuccess || e2 != hipSuccess) {
       set_error("nha_prefill_bwd: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
       return NHA_ERR_LAUNCH;
     }
     configured = true;
   }
-  if (state) hipLaunchKernelGGL((bwd_slot_state_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_s, st, p);
+  if (which == 1) hipLaunchKernelGGL((bwd_slot_state_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_s, st, p);
+  else if (which == 2) hipLaunchKernelGGL((bwd_slot_inter_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_i, st, p);
   else hipLaunchKernelGGL((bwd_slot_dq_kernel<D>), dim3(p.HQ, NT), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products, second stage)");
   return NHA_OK;
 }
 
 // which = 0: dq_gsa (bwd_slot_dq_kernel); 1: N_c and the intra-chunk parts of dk' / dv'
-// (bwd_slot_state_kernel).  Same shapes as bwd_slot_products.
+// (bwd_slot_state_kernel); 2: the parts that involve the scanned E_c (bwd_slot_inter_kernel).
+// Same shapes as bwd_slot_products.
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
-                       const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs) {
+                       const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs,
+                       float* dsp) {
   SP2 p;
   p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.s = (const bf16_t*)a->s;
   p.hkb = (const bf16_t*)hkb;
   p.dus = dus; p.pp = pp; p.ck = ck; p.cv = cv; p.gc = gc;
-  p.ek = ek; p.ev = ev; p.dks = dks; p.dvs = dvs;
+  p.ek = ek; p.ev = ev; p.dks = dks; p.dvs = dvs; p.dsp = dsp;
+  p.v = (const bf16_t*)a->v; p.dkg = (bf16_t*)a->dk_gsa; p.T_tot = a->T_tot;
   p.dq = (bf16_t*)a->dq_gsa;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
   p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift;
   hipStream_t st = (hipStream_t)a->stream;
-  if (a->K == 64) return launch_slot_stage2<64>(p, a->NT, which != 0, st);
-  if (a->K == 128) return launch_slot_stage2<128>(p, a->NT, which != 0, st);
-  return launch_slot_stage2<256>(p, a->NT, which != 0, st);
+  if (a->K == 64) return launch_slot_stage2<64>(p, a->NT, which, st);
+  if (a->K == 128) return launch_slot_stage2<128>(p, a->NT, which, st);
+  return launch_slot_stage2<256>(p, a->NT, which, st);
 }
 
 }  // namespace nha
