@@ -650,9 +650,9 @@ __global__ __launch_bounds__(256) void bwd_state_inter_kernel(const BP p) {
 // ------------------------------------------------------------------------------------------
 // ds and dg.  dg is a reverse cumulative sum over the rows of a sequence; three small launches:
 // per chunk the summand, ds and the chunk-local sums (bwd_gate_local_kernel), per sequence the
-// sums of all later chunks plus the end term (bwd_gate_scan_kernel, which also zeroes the
-// gradients of the tokens that never reach the slots: the last `shift` of a sequence), per chunk
-// the final values (bwd_gate_final_kernel).  One thread per slot.
+// sums of all later chunks plus the end term (bwd_gate_scan_kernel), per chunk the final values
+// (bwd_gate_final_kernel, which also zeroes the gradients of the tokens that never reach the
+// slots: the last `shift` of a sequence).  One thread per slot.
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void bwd_gate_local_kernel(const BP p) {
@@ -689,16 +689,6 @@ __global__ void bwd_gate_scan_kernel(const BP p) {
   const int n = blockIdx.x / H, h = blockIdx.x % H;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int tid = threadIdx.x;
-  int z0 = eos - p.shift;
-  z0 = z0 < bos ? bos : z0;
-  for (int j = z0; j < eos; ++j) {
-    for (int m = tid; m < M; m += blockDim.x) {
-      Elem<T>::st((T*)p.ds + ((int64_t)j * H + h) * M + m, 0.f);
-      Elem<T>::st((T*)p.dg + ((int64_t)j * H + h) * M + m, 0.f);
-    }
-    for (int d = tid; d < K; d += blockDim.x) Elem<T>::st((T*)p.dk_gsa + ((int64_t)j * H + h) * K + d, 0.f);
-    for (int c = tid; c < V; c += blockDim.x) p.dvs[((int64_t)j * H + h) * V + c] = 0.f;
-  }
   const int m = tid;
   if (m >= M) return;
   float run = 0.f;   // <dh_T, h_T>: what the gates past the end of the sequence would receive
@@ -749,6 +739,19 @@ __global__ __launch_bounds__(256) void bwd_gate_final_kernel(const BP p) {
     if (sj < bos) continue;
     const float val = p.dsi[((int64_t)t * H + h) * M + m] + p.gtot[((int64_t)chunk * H + h) * M + m];
     Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, val);
+  }
+  // tokens of this chunk that never reach the slots (the last `shift` of the sequence): zero gradients
+  const int K = p.K, V = p.V;
+  int r0 = eos - p.shift - c0;
+  r0 = r0 < 0 ? 0 : r0;
+  for (int r = r0; r < R; ++r) {
+    const int64_t jh = (int64_t)(c0 + r) * H + h;
+    for (int e = threadIdx.x; e < M; e += 256) {
+      Elem<T>::st((T*)p.ds + jh * M + e, 0.f);
+      Elem<T>::st((T*)p.dg + jh * M + e, 0.f);
+    }
+    for (int e = threadIdx.x; e < K; e += 256) Elem<T>::st((T*)p.dk_gsa + jh * K + e, 0.f);
+    for (int e = threadIdx.x; e < V; e += 256) p.dvs[jh * V + e] = 0.f;
   }
 }
 
@@ -898,7 +901,8 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     f.scratch = sc + sp.mfma;
     f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
     rc = prefill_mfma_impl(&f);
-    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, hkc, (float*)(sc + sp.hkct), (float*)(sc + sp.hvct), sc + sp.hkb, sc + sp.hvb);
+    // every consumer of the states on this path reads the bf16 copies
+    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb);
     // the decay-free products of the slot branch on the matrix cores
     if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst));
   } else {

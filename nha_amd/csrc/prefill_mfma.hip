@@ -1150,10 +1150,12 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
     const int m = e / D, d = e % D;
     const float dc = p.dcum[cg * MS + m];
     const float hk = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
-    hkc[(cg * D + d) * MS + m] = hk;
-    hkct[(cg * MS + m) * D + d] = hk;
     const float hv = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
-    hvct[(cg * D + d) * MS + m] = hv;
+    if (hkc) {   // fp32 copies: only the VALU kernels of the backward read them
+      hkc[(cg * D + d) * MS + m] = hk;
+      hkct[(cg * MS + m) * D + d] = hk;
+      hvct[(cg * D + d) * MS + m] = hv;
+    }
     hkb[(cg * MS + m) * D + d] = f32_to_bf16(hk);
     hvb[(cg * MS + m) * D + d] = f32_to_bf16(hv);
   }
@@ -1291,7 +1293,7 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
 
 // `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
 // [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies, hkb [NT][H][M][K] and
-// hvb [NT][H][M][V] bf16 copies
+// hvb [NT][H][M][V] bf16 copies (hkc, hkct, hvct may be NULL together)
 int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
