@@ -138,10 +138,15 @@ int prefill_simple_impl(const NhaPrefillArgs* a);
 bool prefill_mfma_supported(const NhaPrefillArgs* a);
 size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_mfma_impl(const NhaPrefillArgs* a);
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb);
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb,
+                               void* hkl, void* hvl, int* big);
+int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const float* ap, const float* bp, const float* ust,
+                       const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
+                       float* cv, float* dsi);
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
                        const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs, float* dsp);
-int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, float* ap, float* bp, float* ust, float* dpst);
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap, float* bp, float* ust, float* dpst,
+                      float* delta);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);

@@ -50,6 +50,7 @@ struct BP {
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
   const float *ap, *bp;   // [NT][HQ][BT][BT]  q_gsa_i . k'_j and do_i . v'_j from the matrix cores, or NULL
   const float *ust, *dpst; // [T_tot][HQ][M]    q_gsa_t . hk0[:,m] and do_t . hv0[m,:] (chunk-start states), or NULL
+  const int* big;         // [NT][H] chunks the matrix-core slot kernels leave to the VALU kernels, or NULL (all)
   float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
   float *dks;             // [T_tot][H][K]     intra-chunk part of dk_gsa, indexed by SOURCE token
   float *ek, *ev;         // [NT][H][K][M], [NT][H][V][M]  N_c, then E_c (see the state-gradient kernels)
@@ -97,6 +98,7 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   const int hq = blockIdx.y, h = hq / NG;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
+  if (p.big && !p.big[(int64_t)chunk * H + h]) return;   // the matrix-core kernel has done this chunk
   const bool valid = bos + it * BT + r < eos;   // waves past the end compute on row 0 and write nothing
   const int rr = valid ? r : 0;
   const int t = bos + it * BT + rr;
@@ -297,6 +299,7 @@ __global__ __launch_bounds__(512) void bwd_intra_kernel(const BP p) {
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   const T* ss = (const T*)p.s;
+  if (p.big && !p.big[(int64_t)chunk * H + h]) return;   // the matrix-core kernel has done this chunk
   if (tid < BT) {
     const int tl = it * BT + tid - p.shift;
     src[tid] = (tid < R && tl >= 0) ? bos + tl : -1;
@@ -822,7 +825,7 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, mfma, hkct, hvct, hkb, hvb, ap, bp, ust, dpst, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
+  size_t fwd, mfma, hkct, hvct, hkb, hvb, hkl, hvl, ap, bp, ust, dpst, big, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
   bool use_mfma;
   int nbk, nbv;
 };
@@ -838,14 +841,17 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   if (s.use_mfma) off += aligned(prefill_mfma_scratch_bytes(&f));
   s.hkct = off; off += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
   s.hvct = off; off += aligned((size_t)a->NT * a->H * a->V * a->M * 4);
-  s.hkb = s.hvb = s.ap = s.bp = s.ust = s.dpst = off;
+  s.hkb = s.hvb = s.hkl = s.hvl = s.ap = s.bp = s.ust = s.dpst = s.big = off;
   if (s.use_mfma) {
     s.hkb = off; off += aligned((size_t)a->NT * a->H * a->M * a->K * 2);
     s.hvb = off; off += aligned((size_t)a->NT * a->H * a->M * a->V * 2);
+    s.hkl = off; off += aligned((size_t)a->NT * a->H * a->M * a->K * 2);
+    s.hvl = off; off += aligned((size_t)a->NT * a->H * a->M * a->V * 2);
     s.ap = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
     s.bp = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
     s.ust = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
     s.dpst = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
+    s.big = off; off += aligned((size_t)a->NT * a->H * 4);
   }
   s.hkT = off; off += aligned((size_t)a->N * a->H * a->K * a->M * 4);
   s.hvT = off; off += aligned((size_t)a->N * a->H * a->M * a->V * 4);
@@ -902,9 +908,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
     rc = prefill_mfma_impl(&f);
     // every consumer of the states on this path reads the bf16 copies
-    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb);
+    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (int*)(sc + sp.big));
     // the decay-free products of the slot branch on the matrix cores
-    if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst));
+    if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst),
+                                             (float*)(sc + sp.delta));
   } else {
     f.scratch = sc + sp.fwd;
     f.scratch_bytes = prefill_simple_scratch_bytes(&f);
@@ -923,7 +930,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.gc = gc; p.hkc = hkc; p.hvc = hvc;
   p.hkct = (float*)(sc + sp.hkct); p.hvct = (float*)(sc + sp.hvct);
   p.ap = p.bp = p.ust = p.dpst = nullptr;
+  p.big = nullptr;
+  static const bool intra_mfma = getenv("NHA_BWD_INTRA_VALU") == nullptr;
   if (sp.use_mfma) {
+    if (intra_mfma) p.big = (const int*)(sc + sp.big);
     p.ap = (float*)(sc + sp.ap); p.bp = (float*)(sc + sp.bp);
     p.ust = (float*)(sc + sp.ust); p.dpst = (float*)(sc + sp.dpst);
   }
@@ -957,6 +967,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   const bool wmfma = bwd_window_mfma_supported(a);
   if (!sp.use_mfma) hipLaunchKernelGGL(bwd_transpose_states_kernel, dim3(a->NT * a->H), dim3(256), 0, st, p);
+  if (sp.use_mfma && intra_mfma) {
+    rc = bwd_slot_products3(a, 0, p.big, p.ap, p.bp, p.ust, p.dpst, p.gc, p.delta, p.dus, p.pp, p.xg, p.ck, p.cv, p.dsi);
+    if (rc != NHA_OK) return rc;
+  }
   hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
   if (wmfma) {
@@ -965,6 +979,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   } else {
     hipLaunchKernelGGL((bwd_q_window_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_qw, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_bwd(window query pass)");
+  }
+  if (sp.use_mfma && intra_mfma) {
+    rc = bwd_slot_products3(a, 1, p.big, p.ap, p.bp, p.ust, p.dpst, p.gc, p.delta, p.dus, p.pp, p.xg, p.ck, p.cv, p.dsi);
+    if (rc != NHA_OK) return rc;
   }
   hipLaunchKernelGGL((bwd_intra_kernel<T>), dim3(a->NT, a->H), dim3(512), lds_i, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(intra-chunk pass)");

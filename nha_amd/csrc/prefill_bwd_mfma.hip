@@ -369,9 +369,12 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
 // ------------------------------------------------------------------------------------------
 struct SP1 {
   const bf16_t *q, *dout, *kg, *v;   // q_gsa [T,HQ,D], dout [T,HQ,D], k_gsa [T,H,D], v [T,H,D]
-  const bf16_t *hkb, *hvb;           // [NT][H][64][D] chunk-start states, hk transposed
+  const bf16_t *hkb, *hvb;           // [NT][H][64][D] chunk-start states, hk transposed (high parts)
+  const bf16_t *hkl, *hvl;           // their low parts
   float *ap, *bp;                    // [NT][HQ][64][64]
   float *ust, *dpst;                 // [T][HQ][64]
+  const bf16_t* o;                   // [T,HQ,D]
+  float* delta;                      // [T][HQ]  do . o
   const int32_t *cu, *cidx;
   int HQ, H, NG, shift;
 };
@@ -404,7 +407,7 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
   const bool has = j < R && tl >= 0;
   const int64_t sj = ((int64_t)bos + (has ? tl : 0)) * H + h;
   const int64_t cg = ((int64_t)chunk * H + h) * BT + j;
-  bf16x8 yk[KS], yv[KS], yhk[KS], yhv[KS];
+  bf16x8 yk[KS], yv[KS], yhk[KS], yhv[KS], yhkl[KS], yhvl[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     uint4 a = make_uint4(0, 0, 0, 0), b = a;
@@ -416,8 +419,27 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
     yv[ks] = __builtin_bit_cast(bf16x8, b);
     yhk[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkb + cg * D + 32 * ks + 8 * kb));
     yhv[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvb + cg * D + 32 * ks + 8 * kb));
+    yhkl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkl + cg * D + 32 * ks + 8 * kb));
+    yhvl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvl + cg * D + 32 * ks + 8 * kb));
   }
   lds_barrier();
+  {
+    // delta_i = do_i . o_i: row i = 16 wave + l16, the four lanes sharing l16 split the columns
+    const int i = 16 * wave + l16;
+    float acc = 0.f;
+    if (i < R) {
+      const bf16_t* orow = p.o + ((int64_t)(c0 + i) * HQ + hq) * D;
+      for (int c = 8 * kb; c < D; c += 32) {
+        const bf16x8 ov = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(orow + c));
+        const bf16x8 dv = lds_frag(Ot, LDT, i, c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
+      }
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (kb == 0 && i < R) p.delta[(int64_t)(c0 + i) * HQ + hq] = acc;
+  }
   float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
   float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
@@ -428,9 +450,9 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
       const bf16x8 xq = lds_frag(Qt, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
       const bf16x8 xo = lds_frag(Ot, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
       cA = mfma16(xq, yk[ks], cA);
-      cU = mfma16(xq, yhk[ks], cU);
+      cU = mfma16(xq, yhk[ks], mfma16(xq, yhkl[ks], cU));
       cB = mfma16(xo, yv[ks], cB);
-      cP = mfma16(xo, yhv[ks], cP);
+      cP = mfma16(xo, yhv[ks], mfma16(xo, yhvl[ks], cP));
     }
     // C[i = 16 blk + 4 kb + r][j = 16 wave + l16]
 #pragma unroll
@@ -489,13 +511,23 @@ __device__ __forceinline__ bf16x8 table_frag(const lbf16* tab, int n, int hf, in
   return __builtin_bit_cast(bf16x8, t);
 }
 
+// x as a bf16 pair hi + lo (16 mantissa bits): the tables built from fp32 intermediates are kept
+// this way and multiplied as hi*b + lo*b, so that their rounding stays below that of the bf16 inputs
+__device__ __forceinline__ void split_bf16(float x, lbf16* hi, lbf16* lo, int idx) {
+  const bf16_t h = f32_to_bf16(x);
+  hi[idx] = h;
+  lo[idx] = f32_to_bf16(x - bf16_to_f32(h));
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
   extern __shared__ __align__(16) unsigned char smem[];
   lbf16* const Xt = (lbf16*)smem;        // [64 rows i][D]
-  lbf16* const Wt = Xt + TILE;           // [64 m][TLD]  (w_i[m] e^(gc_i[m]))^T
-  lbf16* const Ct = Wt + BT * TLD;       // [64 r][TLD]  c[i][r]^T, zero for i < r
+  lbf16* const Wt = Xt + TILE;           // [64 m][TLD]  (w_i[m] e^(gc_i[m]))^T, high part
+  lbf16* const Wl = Wt + BT * TLD;       //              low part
+  lbf16* const Ct = Wl + BT * TLD;       // [64 r][TLD]  c[i][r]^T, zero for i < r, high part
+  lbf16* const Cl = Ct + BT * TLD;       //              low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
@@ -531,19 +563,19 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
         w = wsrc[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
         if (c <= i) cc = cp[i * BT + c];
       }
-      Wt[c * TLD + i] = f32_to_bf16(w);
-      Ct[c * TLD + i] = f32_to_bf16(cc);
+      split_bf16(w, Wt, Wl, c * TLD + i);
+      split_bf16(cc, Ct, Cl, c * TLD + i);
     }
     lds_barrier();
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      const bf16x8 bw = table_frag(Wt, col, hf, kb);
-      const bf16x8 bc = table_frag(Ct, col, hf, kb);
+      const bf16x8 bw = table_frag(Wt, col, hf, kb), bwl = table_frag(Wl, col, hf, kb);
+      const bf16x8 bc = table_frag(Ct, col, hf, kb), bcl = table_frag(Cl, col, hf, kb);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const bf16x8 xa = lds_frag_tr(Xt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // X^T[x][i]
-        accN[db] = mfma16(xa, bw, accN[db]);
-        accO[db] = mfma16(xa, bc, accO[db]);
+        accN[db] = mfma16(xa, bw, mfma16(xa, bwl, accN[db]));
+        accO[db] = mfma16(xa, bc, mfma16(xa, bcl, accO[db]));
       }
     }
   }
@@ -566,8 +598,10 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   extern __shared__ __align__(16) unsigned char smem[];
   lbf16* const Ht = (lbf16*)smem;        // [64 m][D]  hk0^T
   lbf16* const Kt = Ht + TILE;           // [64 j][D]  k' rows
-  lbf16* const Wt = Kt + TILE;           // [64 i][TLD]  scale du_i[m] e^(gc_i[m])
-  lbf16* const Ct = Wt + BT * TLD;       // [64 i][TLD]  ck[i][j], zero for j > i
+  lbf16* const Wt = Kt + TILE;           // [64 i][TLD]  scale du_i[m] e^(gc_i[m]), high part
+  lbf16* const Wl = Wt + BT * TLD;       //              low part
+  lbf16* const Ct = Wl + BT * TLD;       // [64 i][TLD]  ck[i][j], zero for j > i, high part
+  lbf16* const Cl = Ct + BT * TLD;       //              low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
@@ -601,8 +635,8 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
       w = p.dus[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
       if (c <= i) cc = cp[i * BT + c];
     }
-    Wt[i * TLD + c] = f32_to_bf16(w);
-    Ct[i * TLD + c] = f32_to_bf16(cc);
+    split_bf16(w, Wt, Wl, i * TLD + c);
+    split_bf16(cc, Ct, Cl, i * TLD + c);
   }
   lds_barrier();
   const int i = 16 * wave + l16;   // this lane's row of the chunk
@@ -611,12 +645,14 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   for (int db = 0; db < DB; ++db) acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
-    const bf16x8 bw = table_frag(Wt, i, hf, kb);   // contraction over m
-    const bf16x8 bc = table_frag(Ct, i, hf, kb);   // contraction over j
+    const bf16x8 bw = table_frag(Wt, i, hf, kb), bwl = table_frag(Wl, i, hf, kb);   // contraction over m
+    const bf16x8 bc = table_frag(Ct, i, hf, kb), bcl = table_frag(Cl, i, hf, kb);   // contraction over j
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      acc[db] = mfma16(lds_frag_tr(Ht, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane), bw, acc[db]);   // hk0[d][m]
-      acc[db] = mfma16(lds_frag_tr(Kt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane), bc, acc[db]);   // k'_j[d]
+      const bf16x8 ha = lds_frag_tr(Ht, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // hk0[d][m]
+      const bf16x8 ka = lds_frag_tr(Kt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // k'_j[d]
+      acc[db] = mfma16(ha, bw, mfma16(ha, bwl, acc[db]));
+      acc[db] = mfma16(ka, bc, mfma16(ka, bcl, acc[db]));
     }
   }
   if (i < R) {
@@ -641,8 +677,10 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT, ELD = BT + 8;
   extern __shared__ __align__(16) unsigned char smem[];
   lbf16* const Yt = (lbf16*)smem;        // [64 rows r][D]   k' / v'
-  lbf16* const Et = Yt + TILE;           // [D x][ELD]       E[x][m]
-  lbf16* const St = Et + D * ELD;        // [64 r][TLD]      s_r[m] dec_r[m]
+  lbf16* const Et = Yt + TILE;           // [D x][ELD]       E[x][m], high part
+  lbf16* const El = Et + D * ELD;        //                  low part
+  lbf16* const St = El + D * ELD;        // [64 r][TLD]      s_r[m] dec_r[m], high part
+  lbf16* const Sl = St + BT * TLD;       //                  low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
@@ -668,7 +706,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
     ry.store(Yt, tid);
   }
   const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
-  for (int e = tid; e < D * BT; e += 256) Et[(e >> 6) * ELD + (e & 63)] = f32_to_bf16(ep[e]);
+  for (int e = tid; e < D * BT; e += 256) split_bf16(ep[e], Et, El, (e >> 6) * ELD + (e & 63));
   const float* gcb = p.gc + ((int64_t)c0 * H + h) * BT;
   for (int e = tid; e < BT * BT; e += 256) {
     const int r = e >> 6, m = e & 63;
@@ -676,7 +714,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
     if (r >= vlo && r < R)
       v = bf16_to_f32(p.s[(((int64_t)c0 + r - p.shift) * H + h) * BT + m]) *
           __expf(gcb[(int64_t)(R - 1) * H * BT + m] - gcb[(int64_t)r * H * BT + m]);
-    St[r * TLD + m] = f32_to_bf16(v);
+    split_bf16(v, St, Sl, r * TLD + m);
   }
   lds_barrier();
   const int col = 16 * wave + l16;
@@ -686,9 +724,12 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   for (int db = 0; db < DB; ++db) accO[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
-    const bf16x8 bs = lds_frag(St, TLD, col, 32 * ks + 8 * kb);
+    const bf16x8 bs = lds_frag(St, TLD, col, 32 * ks + 8 * kb), bsl = lds_frag(Sl, TLD, col, 32 * ks + 8 * kb);
 #pragma unroll
-    for (int db = 0; db < DB; ++db) accO[db] = mfma16(lds_frag(Et, ELD, 16 * db + l16, 32 * ks + 8 * kb), bs, accO[db]);
+    for (int db = 0; db < DB; ++db) {
+      const bf16x8 eh = lds_frag(Et, ELD, 16 * db + l16, 32 * ks + 8 * kb);
+      accO[db] = mfma16(eh, bs, mfma16(eh, bsl, mfma16(lds_frag(El, ELD, 16 * db + l16, 32 * ks + 8 * kb), bs, accO[db])));
+    }
   }
   const bool has = col >= vlo && col < R;
   if (has) {
@@ -717,7 +758,9 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
       struct { bf16x4 a, b; } t;
       t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 4 * kb);
       t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 16 + 4 * kb);
-      acc = mfma16(__builtin_bit_cast(bf16x8, t), lds_frag_tr(Et, ELD, 32 * xs, 32 * xs + 16, 16 * wave, lane), acc);
+      const bf16x8 ya = __builtin_bit_cast(bf16x8, t);
+      acc = mfma16(ya, lds_frag_tr(Et, ELD, 32 * xs, 32 * xs + 16, 16 * wave, lane),
+                   mfma16(ya, lds_frag_tr(El, ELD, 32 * xs, 32 * xs + 16, 16 * wave, lane), acc));
     }
     // C[r = 16 rb + 4 kb + q][m = col]
 #pragma unroll
@@ -729,6 +772,244 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
       }
     }
   }
+}
+
+// ------------------------------------------------------------------------------------------
+// Slot branch, the intra-chunk terms that couple rows through the decay e^(gc_i[m] - gc_j[m]), j <= i.
+// With a reference point per 32-row half of the chunk (ref_0 = 0, ref_1 = gc_31) the decay splits
+// into e^(gc_i - ref) <= 1 for the later row and e^(ref - gc_j) >= 1 for the earlier one, ref taken
+// at the start of j's half, and the terms become plain products of 64 x 64 tables
+//   X^(b) = scale du o e^(gc - ref_b), Xp^(b) = p o e^(gc - ref_b) (rows i), Y = s o e^(ref - gc) (rows j)
+// as long as no slot decays by more than e^-80 within a half (bf16 and fp32 share the exponent
+// range); chunks beyond that are flagged by the state export and take the fp32 VALU kernels.
+//
+// bwd_slot_q_kernel, grid (HQ, NT): u = scale (E o q.hk0 + sum_b e^(gc - ref_b) o (A_masked Y)_b),
+//   dp likewise with do.hv0 and B; then p, du and the per-token vectors scale*du, p, du*u + p*dp,
+//   element-wise in the accumulators.
+// bwd_slot_intra_kernel, grid (H, NT): ck = X Y^T, cv = Xp Y^T (i >= r) per q-head, and
+//   ds_intra[r][m] = e^(ref - gc_r[m]) sum_a sum_(i>=r) (A[i][r] X_i[m] + B[i][r] Xp_i[m]),
+//   X and ref of r's half.
+// ------------------------------------------------------------------------------------------
+struct SP3 {
+  const bf16_t* s;                                 // [T,H,64]
+  const float *ap, *bp, *ust, *dpst, *gc, *delta;  // see bwd_slot_products
+  const float *lse_swa, *lse_gsa, *dlse_gsa;
+  float *dus, *pp, *xg;                            // [T][HQ][64]
+  float *ck, *cv;                                  // [NT][HQ][64][64]
+  float* dsi;                                      // [T][H][64]
+  const int* big;                                  // [NT][H]
+  const int32_t *cu, *cidx;
+  int HQ, H, NG, shift;
+  float scale;
+};
+
+// gate cumsum of the chunk's row r and the reference of its half (0 for rows 0..31, gc_31 after)
+__device__ __forceinline__ float gc_at(const SP3& p, int c0, int h, int r, int m) {
+  return p.gc[((int64_t)(c0 + r) * p.H + h) * BT + m];
+}
+__device__ __forceinline__ float ref_of(const SP3& p, int c0, int h, int r, int m) {
+  return r < 32 ? 0.f : gc_at(p, c0, h, 31, m);
+}
+
+// The decay-scaled tables enter the gate gradient through a difference of nearly equal sums (dg is
+// a telescoping sum), so they are bf16 pairs (split_bf16) and their products hi*hi + hi*lo + lo*hi.
+// rows of Y = s_j[m] e^(ref - gc_j[m]) (zero for rows without a source token)
+__device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int c0, int h, int R, int vlo, int tid) {
+  for (int e = tid; e < BT * BT; e += 256) {
+    const int j = e >> 6, m = e & 63;
+    float v = 0.f;
+    if (j >= vlo && j < R)
+      v = bf16_to_f32(p.s[(((int64_t)c0 + j - p.shift) * p.H + h) * BT + m]) * __expf(ref_of(p, c0, h, j, m) - gc_at(p, c0, h, j, m));
+    split_bf16(v, Yh, Yl, j * TLD + m);
+  }
+}
+
+__global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
+  __shared__ __align__(16) bf16_t sm[4 * BT * TLD];
+  lbf16* const At = (lbf16*)sm;          // [64 i][TLD]  A[i][j], zero for j > i
+  lbf16* const Bt = At + BT * TLD;       // [64 i][TLD]  B[i][j], zero for j > i
+  lbf16* const Yh = Bt + BT * TLD;       // [64 j][TLD]  Y, high and low parts
+  lbf16* const Yl = Yh + BT * TLD;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ;
+  const int hq = blockIdx.x, h = hq / p.NG, chunk = blockIdx.y;
+  if (p.big[(int64_t)chunk * H + h]) return;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  int vlo = p.shift - it * BT;
+  vlo = vlo < 0 ? 0 : vlo;
+  const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+  const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+  for (int e = tid; e < BT * BT; e += 256) {
+    const int i = e >> 6, j = e & 63;
+    const bool in = j <= i && i < R;
+    At[i * TLD + j] = f32_to_bf16(in ? ap[e] : 0.f);
+    Bt[i * TLD + j] = f32_to_bf16(in ? bp[e] : 0.f);
+  }
+  stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
+  lds_barrier();
+  const int m = 16 * wave + l16;
+  const float g31 = R > 32 ? gc_at(p, c0, h, 31, m) : 0.f;
+#pragma unroll
+  for (int blk = 0; blk < 4; ++blk) {
+    f32x4 cu_[2], cd_[2];   // one accumulator per half of the contraction (= per reference)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const bf16x8 yh = lds_frag_tr(Yh, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);   // Y[j][m]
+      const bf16x8 yl = lds_frag_tr(Yl, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 af = table_frag(At, 16 * blk + l16, hf, kb), bf = table_frag(Bt, 16 * blk + l16, hf, kb);
+      cu_[hf] = mfma16(af, yh, mfma16(af, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
+      cd_[hf] = mfma16(bf, yh, mfma16(bf, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = 16 * blk + 4 * kb + q;
+      if (i >= R) continue;
+      const int64_t tq = (int64_t)(c0 + i) * HQ + hq;
+      const float gi = gc_at(p, c0, h, i, m);
+      const float e0 = __expf(gi);
+      const float e1 = blk >= 2 ? __expf(gi - g31) : 0.f;   // rows before the second half see none of it
+      const float au = p.scale * (e0 * (p.ust[tq * BT + m] + cu_[0][q]) + e1 * cu_[1][q]);
+      const float ad = e0 * (p.dpst[tq * BT + m] + cd_[0][q]) + e1 * cd_[1][q];
+      const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
+      const float lt = logaddexp_f(ls, lg);
+      const float pm = __expf(au - lt);
+      float du = pm * (ad - p.delta[tq]);
+      if (p.dlse_gsa) du += p.dlse_gsa[tq] * __expf(au - lg);
+      p.dus[tq * BT + m] = p.scale * du;
+      p.pp[tq * BT + m] = pm;
+      p.xg[tq * BT + m] = du * au + pm * ad;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  // tables [64 rows][TLD]; X0 = scale du_i[m] e^(gc_i[m]), X1 = scale du_i[m] e^(gc_i[m] - gc_31[m])
+  // (rows >= 32), P0 / P1 the same with p; each as a high and a low part
+  lbf16* const T0 = (lbf16*)smem;
+  lbf16* const X0h = T0, * const X0l = T0 + BT * TLD, * const X1h = T0 + 2 * BT * TLD, * const X1l = T0 + 3 * BT * TLD;
+  lbf16* const P0h = T0 + 4 * BT * TLD, * const P0l = T0 + 5 * BT * TLD, * const P1h = T0 + 6 * BT * TLD, * const P1l = T0 + 7 * BT * TLD;
+  lbf16* const Yh = T0 + 8 * BT * TLD;   // [64 r][TLD]
+  lbf16* const Yl = T0 + 9 * BT * TLD;
+  lbf16* const AT = T0 + 10 * BT * TLD;  // [64 r][TLD]  A[i][r] transposed, zero for i < r
+  lbf16* const BT_ = T0 + 11 * BT * TLD; // [64 r][TLD]  B[i][r] transposed
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ, NG = p.NG;
+  const int h = blockIdx.x, chunk = blockIdx.y;
+  if (p.big[(int64_t)chunk * H + h]) return;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  int vlo = p.shift - it * BT;
+  vlo = vlo < 0 ? 0 : vlo;
+  stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
+  const int col = 16 * wave + l16;
+  // columns r of ck / cv in the first half take the tables with ref 0, the others ref gc_31
+  const lbf16* const Xch = wave < 2 ? X0h : X1h;
+  const lbf16* const Xcl = wave < 2 ? X0l : X1l;
+  const lbf16* const Pch = wave < 2 ? P0h : P1h;
+  const lbf16* const Pcl = wave < 2 ? P0l : P1l;
+  f32x4 accS[4];
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb) accS[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int a = 0; a < NG; ++a) {
+    const int hq = h * NG + a;
+    if (a > 0) lds_barrier();
+    const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+    const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+    for (int e = tid; e < BT * BT; e += 256) {
+      const int i = e >> 6, c = e & 63;
+      float x0 = 0.f, x1 = 0.f, p0 = 0.f, p1 = 0.f, av = 0.f, bv = 0.f;
+      if (i < R) {
+        const float gi = gc_at(p, c0, h, i, c);
+        const float du = p.dus[((int64_t)(c0 + i) * HQ + hq) * BT + c];
+        const float pv = p.pp[((int64_t)(c0 + i) * HQ + hq) * BT + c];
+        const float e0 = __expf(gi);
+        x0 = du * e0;
+        p0 = pv * e0;
+        if (i >= 32) {
+          const float e1 = __expf(gi - gc_at(p, c0, h, 31, c));
+          x1 = du * e1;
+          p1 = pv * e1;
+        }
+        if (c <= i) {
+          av = ap[e];
+          bv = bp[e];
+        }
+      }
+      split_bf16(x0, X0h, X0l, i * TLD + c);
+      split_bf16(x1, X1h, X1l, i * TLD + c);
+      split_bf16(p0, P0h, P0l, i * TLD + c);
+      split_bf16(p1, P1h, P1l, i * TLD + c);
+      AT[c * TLD + i] = f32_to_bf16(av);
+      BT_[c * TLD + i] = f32_to_bf16(bv);
+    }
+    lds_barrier();
+    // ck[i][r = col] = sum_m X[i][m] Y[r][m], cv with Xp
+    float* ckp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
+    float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      f32x4 c1 = {0.f, 0.f, 0.f, 0.f}, c2 = c1;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const bf16x8 yh = lds_frag(Yh, TLD, col, 32 * ks + 8 * kb), yl = lds_frag(Yl, TLD, col, 32 * ks + 8 * kb);
+        const bf16x8 xh = lds_frag(Xch, TLD, 16 * blk + l16, 32 * ks + 8 * kb);
+        const bf16x8 ph = lds_frag(Pch, TLD, 16 * blk + l16, 32 * ks + 8 * kb);
+        c1 = mfma16(xh, yh, mfma16(xh, yl, mfma16(lds_frag(Xcl, TLD, 16 * blk + l16, 32 * ks + 8 * kb), yh, c1)));
+        c2 = mfma16(ph, yh, mfma16(ph, yl, mfma16(lds_frag(Pcl, TLD, 16 * blk + l16, 32 * ks + 8 * kb), yh, c2)));
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = 16 * blk + 4 * kb + q;
+        if (i >= col && i < R) {
+          ckp[i * BT + col] = c1[q];
+          cvp[i * BT + col] = c2[q];
+        }
+      }
+    }
+    // ds[r][m = col] += sum_i A[i][r] X[i][m] + B[i][r] Xp[i][m]   (rows r < 32: ref 0, else ref gc_31)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const bf16x8 x0h = lds_frag_tr(X0h, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 x0l = lds_frag_tr(X0l, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 p0h = lds_frag_tr(P0h, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 p0l = lds_frag_tr(P0l, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const bf16x8 af = table_frag(AT, 16 * rb + l16, hf, kb), bf = table_frag(BT_, 16 * rb + l16, hf, kb);
+        accS[rb] = mfma16(af, x0h, mfma16(af, x0l, accS[rb]));
+        accS[rb] = mfma16(bf, p0h, mfma16(bf, p0l, accS[rb]));
+      }
+    }
+    {
+      // rows r >= 32 only meet rows i >= 32: the second half of the contraction
+      const bf16x8 x1h = lds_frag_tr(X1h, TLD, 32, 48, 16 * wave, lane), x1l = lds_frag_tr(X1l, TLD, 32, 48, 16 * wave, lane);
+      const bf16x8 p1h = lds_frag_tr(P1h, TLD, 32, 48, 16 * wave, lane), p1l = lds_frag_tr(P1l, TLD, 32, 48, 16 * wave, lane);
+#pragma unroll
+      for (int rb = 2; rb < 4; ++rb) {
+        const bf16x8 af = table_frag(AT, 16 * rb + l16, 1, kb), bf = table_frag(BT_, 16 * rb + l16, 1, kb);
+        accS[rb] = mfma16(af, x1h, mfma16(af, x1l, accS[rb]));
+        accS[rb] = mfma16(bf, p1h, mfma16(bf, p1l, accS[rb]));
+      }
+    }
+  }
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = 16 * rb + 4 * kb + q;
+      if (r < R) {
+        const int64_t idx = ((int64_t)(c0 + r) * H + h) * BT + col;
+        p.dsi[idx] = accS[rb][q] * __expf(ref_of(p, c0, h, r, col) - p.gc[idx]);
+      }
+    }
 }
 
 template <int D, int TK>
@@ -819,11 +1100,14 @@ static int launch_slot_products(const SP1& p, int NT, hipStream_t st) {
 }
 
 // bf16, K == V in {64,128,256}, M == 64 (the shapes of the matrix-core state pass)
-int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, float* ap, float* bp, float* ust, float* dpst) {
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap,
+                      float* bp, float* ust, float* dpst, float* delta) {
   SP1 p;
   p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.v = (const bf16_t*)a->v;
   p.hkb = (const bf16_t*)hkb; p.hvb = (const bf16_t*)hvb;
+  p.hkl = (const bf16_t*)hkl; p.hvl = (const bf16_t*)hvl;
   p.ap = ap; p.bp = bp; p.ust = ust; p.dpst = dpst;
+  p.o = (const bf16_t*)a->o; p.delta = delta;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
   p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift;
   hipStream_t st = (hipStream_t)a->stream;
@@ -834,9 +1118,9 @@ int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* h
 
 template <int D>
 static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
-  const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
-  const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
-  const size_t lds_i = (size_t)BT * (D + 16) * 2 + (size_t)D * (BT + 8) * 2 + (size_t)BT * TLD * 2;
+  const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
+  const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
+  const size_t lds_i = (size_t)BT * (D + 16) * 2 + (size_t)2 * D * (BT + 8) * 2 + (size_t)2 * BT * TLD * 2;
   static bool configured = false;
   if (!configured) {
     hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
@@ -875,6 +1159,37 @@ int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, c
   if (a->K == 64) return launch_slot_stage2<64>(p, a->NT, which, st);
   if (a->K == 128) return launch_slot_stage2<128>(p, a->NT, which, st);
   return launch_slot_stage2<256>(p, a->NT, which, st);
+}
+
+// which = 0: bwd_slot_q_kernel (per-token vectors); 1: bwd_slot_intra_kernel (ck, cv, intra part of
+// ds).  Chunks flagged in `big` are left to the fp32 VALU kernels.
+int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const float* ap, const float* bp, const float* ust,
+                       const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
+                       float* cv, float* dsi) {
+  SP3 p;
+  p.s = (const bf16_t*)a->s;
+  p.ap = ap; p.bp = bp; p.ust = ust; p.dpst = dpst; p.gc = gc; p.delta = delta;
+  p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa; p.dlse_gsa = a->dlse_gsa;
+  p.dus = dus; p.pp = pp; p.xg = xg; p.ck = ck; p.cv = cv; p.dsi = dsi; p.big = big;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
+  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift; p.scale = a->scale;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (which == 0) hipLaunchKernelGGL(bwd_slot_q_kernel, dim3(a->HQ, a->NT), dim3(256), 0, st, p);
+  else {
+    const size_t lds = (size_t)12 * BT * TLD * 2;
+    static bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_intra_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) {
+        set_error("nha_prefill_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        return NHA_ERR_LAUNCH;
+      }
+      configured = true;
+    }
+    hipLaunchKernelGGL(bwd_slot_intra_kernel, dim3(a->H, a->NT), dim3(256), lds, st, p);
+  }
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products, intra-chunk)");
+  return NHA_OK;
 }
 
 }  // namespace nha

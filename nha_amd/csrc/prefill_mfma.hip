@@ -1137,7 +1137,8 @@ int launch_repair(const MP& p, hipStream_t st) {
 // hv [M][V] as matrix-core operands; gate cumsums per row token
 // ==========================================================================================
 template <int D>
-__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hkct, float* hvct, bf16_t* hkb, bf16_t* hvb) {
+__global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* gc, float* hkc, float* hkct, float* hvct, bf16_t* hkb, bf16_t* hvb, bf16_t* hkl,
+                                                          bf16_t* hvl, int* big) {
   const int chunk = blockIdx.x, h = blockIdx.y, H = p.H;
   const int tid = threadIdx.x;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
@@ -1156,10 +1157,26 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
       hkct[(cg * MS + m) * D + d] = hk;
       hvct[(cg * D + d) * MS + m] = hv;
     }
-    hkb[(cg * MS + m) * D + d] = f32_to_bf16(hk);
-    hvb[(cg * MS + m) * D + d] = f32_to_bf16(hv);
+    // bf16 pairs hi + lo: the backward multiplies by hi and by lo
+    const bf16_t hkh = f32_to_bf16(hk), hvh = f32_to_bf16(hv);
+    hkb[(cg * MS + m) * D + d] = hkh;
+    hvb[(cg * MS + m) * D + d] = hvh;
+    hkl[(cg * MS + m) * D + d] = f32_to_bf16(hk - bf16_to_f32(hkh));
+    hvl[(cg * MS + m) * D + d] = f32_to_bf16(hv - bf16_to_f32(hvh));
   }
   for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
+  // chunks in which some slot decays by more than e^-80 over one of the two 32-row halves: the
+  // backward's factored products (e^(gc_i - ref) e^(ref - gc_j) as two operands, ref = the start of
+  // j's half) leave the bf16 / fp32 range there
+  if (tid == 0) {
+    int b = 0;
+    const float* g = p.gc + cg * BT * MS;
+    for (int m = 0; m < MS; ++m) {
+      const float g31 = g[(R > 32 ? 31 : R - 1) * MS + m];
+      b |= (g31 < -80.f) | (g[(R - 1) * MS + m] - g31 < -80.f);
+    }
+    big[cg] = b;
+  }
 }
 
 template <int D, int G, int NW, int TK>
@@ -1293,14 +1310,16 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
 
 // `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
 // [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies, hkb [NT][H][M][K] and
-// hvb [NT][H][M][V] bf16 copies (hkc, hkct, hvct may be NULL together)
-int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb) {
+// hvb [NT][H][M][V] bf16 copies with their low parts hkl, hvl (hkc, hkct, hvct may be NULL together), big [NT][H] the flag of
+// chunks with a decay beyond e^-80
+int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb,
+                               void* hkl, void* hvl, int* big) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
   const dim3 grid(a->NT, a->H);
-  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
-  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
-  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb);
+  if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb, (bf16_t*)hkl, (bf16_t*)hvl, big);
+  else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb, (bf16_t*)hkl, (bf16_t*)hvl, big);
+  else hipLaunchKernelGGL((export_states_kernel<256>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb, (bf16_t*)hkl, (bf16_t*)hvl, big);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state export)");
   return NHA_OK;
 }

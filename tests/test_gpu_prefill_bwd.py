@@ -18,7 +18,7 @@ KEYS = ["q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g"]
 BF = torch.bfloat16
 
 
-def check_grad(name, got, ref, dtype):
+def check_grad(name, got, ref, dtype, rel_bar=1e-2):
     got = got.detach().double().cpu()
     ref = ref.detach().double()
     assert got.shape == ref.shape, (name, got.shape, ref.shape)
@@ -27,13 +27,14 @@ def check_grad(name, got, ref, dtype):
     err = (got - ref).abs().max().item()
     if dtype == BF:
         rel = ((got - ref).norm() / max(ref.norm().item(), 1e-30)).item()
-        assert rel <= 1e-2, f"{name}: relative L2 error {rel:.3e}"
+        assert rel <= rel_bar, f"{name}: relative L2 error {rel:.3e}"
         assert err <= 3e-2 * scale, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
     else:
         assert err <= 1e-4 * scale, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
 
 
-def run_bwd_case(tag, d, *, wl, shift, dtype, cu=None, scale=None, with_lse=False, with_dht=False, impl=None, seed=0):
+def run_bwd_case(tag, d, *, wl, shift, dtype, cu=None, scale=None, with_lse=False, with_dht=False, impl=None, seed=0,
+                 dg_bar=1e-2):
     from nha_amd import chunk_nha
     print("case", tag, dtype, flush=True)
     gen = torch.Generator().manual_seed(seed)
@@ -60,7 +61,7 @@ def run_bwd_case(tag, d, *, wl, shift, dtype, cu=None, scale=None, with_lse=Fals
                            initial_state=h0, scale=scale, dlse_swa=dl1, dlse_gsa=dl2, dht=dht)
     for k, t in zip(KEYS, x):
         assert t.grad is not None and t.grad.dtype == dtype, k
-        check_grad(f"{tag} d{k}", t.grad, G["d" + k], dtype)
+        check_grad(f"{tag} d{k}", t.grad, G["d" + k], dtype, dg_bar if k == "g" else 1e-2)
     if h0 is not None:
         # fp32 tensors, but computed from the same rounded o / do as the other gradients
         check_grad(f"{tag} dh0k", h0c[0].grad, G["dh0k"], dtype)
@@ -106,6 +107,23 @@ def test_bwd_window_edges_on_the_matrix_cores(wl, shift):
     cu = [0, 1, 66, 130, 450, 519]
     d = prefill_inputs(7400 + wl, 1, cu[-1], 4, 2, 64, 64, 16, dtype=BF, qk_scale=1.0, with_state=True, N=5)
     run_bwd_case(f"window wl={wl}", d, wl=wl, shift=shift, dtype=BF, cu=cu, scale=0.125, with_dht=True)
+
+
+@pytest.mark.parametrize("gate_mean", [-1.0, -2.0, -4.0])
+def test_bwd_strong_gates(gate_mean):
+    """Gate logits N(gate_mean, 1) -> logsigmoid without the /8: a 32-row half of a chunk decays by
+    about e^-45 / e^-70 / e^-130.  Up to e^-80 the matrix-core slot kernels factor the decay
+    around the half's start; beyond, the state export flags the chunk and the fp32 VALU kernels
+    take it.  Mixed within one call for gate_mean = -2 (some slots cross the bound, most do not).
+    dg is a telescoping sum (large per-row terms that cancel against the final-state term); with a
+    cotangent on the final states and gates this strong its relative L2 error in bf16 reaches
+    1.4e-2, so that one gradient is held to the reference's own 2e-2 bar
+    (scripts/verify_opt_parity.py:753) in the first case; everything else stays at 1e-2."""
+    cu = [0, 130, 300]
+    d = prefill_inputs(7600, 1, cu[-1], 4, 2, 64, 64, 64, dtype=BF, qk_scale=64 ** -0.5, gate_div=1.0, gate_mean=gate_mean,
+                       with_state=True, N=2)
+    run_bwd_case(f"strong gates {gate_mean} shifted", d, wl=31, shift=32, dtype=BF, cu=cu, with_dht=True, dg_bar=2e-2)
+    run_bwd_case(f"strong gates {gate_mean} layer", d, wl=40, shift=0, dtype=BF, cu=cu, with_lse=False)
 
 
 def test_bwd_matrix_core_path_matches_fp32_path_at_size():
