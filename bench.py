@@ -327,6 +327,7 @@ def main():
         print(json.dumps(res))
         return
     pf = bench_prefill(torch, args.steps, args.warmup)
+    bw = bench_backward(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     dc = bench_decode(torch, args.warmup)
     cpu = None if args.no_cpu_baseline else cpu_baseline(torch)
     out = {
@@ -355,6 +356,9 @@ def main():
                    "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel<128,4,2>", "achieved": dc["achieved_gbs"],
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
                                 "traffic": TRAFFIC_BYTES["decode_mfma_kernel<128,4,2>"], "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
+        "backward": {"metric": "backward of the same prefill call", "ms_per_call": bw["bwd_ms"], "unit": "ms",
+                     "tokens_per_s": bw["bwd_tokens_per_s"], "tflops": bw["bwd_tflops"],
+                     "flop": bw["bwd_flops"], "note": "2.5 x the forward's algorithmic flop"},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -981,8 +981,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
 // that sub-block are recomputed here token by token with the unfactored decay (<= 1), in fp32
 // VALU arithmetic, from the same chunk-start states and gate table: slot logits
 // (nha_fla/ops/nha/chunk_fused.py:186-222), window logits, one softmax (:233-240), both reads
-// (:242-283) and the branch LSEs (nha_fla/ops/nha/chunk.py:459-470).  grid (chunk, q-head);
-// workgroups of unflagged chunks leave at once.
+// (:242-283) and the branch LSEs (nha_fla/ops/nha/chunk.py:459-470).  grid (chunk, kv-head), the
+// q-heads of the group in turn; workgroups of unflagged chunks leave at once.
 template <int D>
 struct RepairSmem {
   static constexpr int LDH = D + 1;
@@ -992,8 +992,8 @@ struct RepairSmem {
 template <int D>
 __global__ __launch_bounds__(256) void mfma_repair_kernel(const MP p) {
   constexpr int LDH = RepairSmem<D>::LDH;
-  const int chunk = blockIdx.x, hq = blockIdx.y;
-  const int H = p.H, HQ = p.HQ, h = hq / p.NG;
+  const int chunk = blockIdx.x, h = blockIdx.y;
+  const int H = p.H, HQ = p.HQ;
   const int64_t cg = (int64_t)chunk * H + h;
   const int* fl = p.flags + cg * 4;
   const int bits = fl[0] | fl[1] | fl[2] | fl[3];
@@ -1025,6 +1025,7 @@ __global__ __launch_bounds__(256) void mfma_repair_kernel(const MP p) {
   }
   for (int e = tid; e < BT * MS; e += 256) gcl[e] = p.gc[cg * BT * MS + e];
 
+  for (int hq = h * p.NG; hq < (h + 1) * p.NG; ++hq)
   for (int r = 0; r < rows; ++r) {
     if (!((bits >> (r >> 4)) & 1)) continue;
     const int t = c0 + r;
@@ -1126,7 +1127,7 @@ int launch_repair(const MP& p, hipStream_t st) {
     }
     configured = true;
   }
-  hipLaunchKernelGGL((mfma_repair_kernel<D>), dim3(p.NT, p.HQ), dim3(256), lds, st, p);
+  hipLaunchKernelGGL((mfma_repair_kernel<D>), dim3(p.NT, p.H), dim3(256), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma repair pass)");
   return NHA_OK;
 }
