@@ -193,6 +193,40 @@ def bench_backward(torch, steps, warmup, cfg=PREFILL):
     return dict(bwd_ms=ms, bwd_flops=flops, bwd_tflops=flops / (ms * 1e-3) / 1e12, bwd_tokens_per_s=B * T / (ms * 1e-3))
 
 
+def bench_glue(torch, steps, warmup, cfg=PREFILL):
+    """The two fused glue launches of the layer at the prefill workload's shape (raw projections ->
+    op operands, op output -> input of the output projection): microseconds per launch with HIP
+    events on the launch stream, and the algorithmic bytes (every element read / written once)."""
+    from nha_amd.ops import nha_layer_epilogue, nha_layer_prologue
+    dev = torch.device("cuda:0")
+    B, T, HQ, H, D, M = (cfg[k] for k in ("B", "T", "HQ", "H", "D", "M"))
+    gen = torch.Generator(device=dev).manual_seed(2)
+    r = lambda *s: torch.randn(*s, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v, f = r(B, T, HQ, D), r(B, T, H, D), r(B, T, H, D), r(B, T, H, M)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32, device=dev) / D))
+    o, w = r(B * T, HQ * D), torch.ones(HQ * D, device=dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record(stream)
+        for _ in range(steps):
+            fn()
+        ev[1].record(stream)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / steps * 1e3
+
+    us_p = timed(lambda: nha_layer_prologue(q, k, v, f, inv, feature_map="swish", gate_logit_normalizer=8))
+    us_e = timed(lambda: nha_layer_epilogue(o, w, None, 1e-5))
+    by_p = 2 * (3 * q.numel() + 3 * k.numel() + 2 * v.numel() + 3 * f.numel())
+    by_e = 2 * 2 * o.numel()
+    return dict(prologue_us=us_p, prologue_bytes=by_p, prologue_gbs=by_p / us_p / 1e3,
+                epilogue_us=us_e, epilogue_bytes=by_e, epilogue_gbs=by_e / us_e / 1e3)
+
+
 def bench_decode(torch, warmup):
     from nha_amd import NHARingState, ring_decode_step
     cfg = DECODE
@@ -292,7 +326,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "glue"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
     ap.add_argument("--backward", action="store_true",
                     help="with --workload: also time the backward of the prefill op")
@@ -323,12 +357,14 @@ def main():
         print(json.dumps(res))
         return
     if args.only:
-        res = bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else bench_decode(torch, args.warmup)
+        res = (bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else
+               bench_glue(torch, args.steps, args.warmup) if args.only == "glue" else bench_decode(torch, args.warmup))
         print(json.dumps(res))
         return
     pf = bench_prefill(torch, args.steps, args.warmup)
     bw = bench_backward(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     dc = bench_decode(torch, args.warmup)
+    gl = bench_glue(torch, args.steps, args.warmup)
     cpu = None if args.no_cpu_baseline else cpu_baseline(torch)
     out = {
         "metric": "NHA prefill tokens/s @T=8K bf16",
@@ -359,6 +395,13 @@ def main():
         "backward": {"metric": "backward of the same prefill call", "ms_per_call": bw["bwd_ms"], "unit": "ms",
                      "tokens_per_s": bw["bwd_tokens_per_s"], "tflops": bw["bwd_tflops"],
                      "flop": bw["bwd_flops"], "note": "2.5 x the forward's algorithmic flop"},
+        "layer_glue": {"metric": "fused layer prologue / epilogue at the prefill shape", "unit": "us/launch",
+                       "prologue_us": gl["prologue_us"], "epilogue_us": gl["epilogue_us"],
+                       "roofline": {"bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                    "prologue": {"achieved": gl["prologue_gbs"], "frac": gl["prologue_gbs"] / PEAK_HBM_GBS,
+                                                 "algorithmic_bytes": gl["prologue_bytes"]},
+                                    "epilogue": {"achieved": gl["epilogue_gbs"], "frac": gl["epilogue_gbs"] / PEAK_HBM_GBS,
+                                                 "algorithmic_bytes": gl["epilogue_bytes"]}}},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 3
+#define NHA_ABI_VERSION 4
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -228,6 +228,68 @@ int nha_decode_advance(int32_t* count, int32_t B, void* stream);
 int32_t nha_varlen_num_chunks(const int32_t* cu_seqlens_host, int32_t N, int32_t BT);
 int nha_varlen_indices(const int32_t* cu_seqlens_host, int32_t N, int32_t BT,
                        int32_t* chunk_idx_host /* [NT,2] */, int32_t* chunk_off_host /* [N+1] */);
+
+/* ------------------------------------------------------------------------------------------
+ * Layer glue on either side of the fused op, one launch each (device pointers, contiguous,
+ * 16-byte aligned, all tensors in `dtype`).
+ *
+ * nha_layer_prologue replaces the chain of elementwise tensor ops at
+ * nha_fla/layers/nha.py:214-237: from the raw projections q [T_tot,HQ,K], k [T_tot,H,K],
+ * v [T_tot,H,V], f [T_tot,H,M] it writes
+ *   q_swa, k_swa  rotate-half RoPE over the whole head dim (:237); the position of token t is
+ *                 t - cu_seqlens[n] + seqlen_offset inside its sequence n, or (t mod T_tot/N) +
+ *                 seqlen_offset when cu_seqlens is NULL; angle = position * inv_freq[i], i < K/2;
+ *   q_gsa, k_gsa  the feature map of q, k (:219-222): NHA_FMAP_SWISH x*sigmoid(x), NHA_FMAP_RELU;
+ *                 with NHA_FMAP_NONE they are not written (the caller passes q, k themselves);
+ *   v_out         silu(v) (:223);
+ *   g             logsigmoid(f) / gate_logit_normalizer, s = 1 - exp(g) (:225-227), each step
+ *                 rounded to `dtype` as the reference's tensor ops round it.
+ * k, v, s, g stay at the kv-head count H: the op reads them per group, the reference's repeat
+ * (:229-230) is not materialised.
+ *
+ * nha_layer_epilogue replaces the normalisation half of rms_norm_linear(silu(o), ...) at
+ * nha_fla/layers/nha.py:278: y[r,:] = silu(o[r,:]) * rsqrt(mean(silu(o[r,:])^2) + eps) * weight
+ * (+ bias), rows of `dim` = HQ*V elements; weight and bias are fp32 [dim] or NULL.  The output
+ * projection itself stays a library GEMM on the caller's side.
+ * ------------------------------------------------------------------------------------------ */
+#define NHA_FMAP_NONE 0
+#define NHA_FMAP_SWISH 1
+#define NHA_FMAP_RELU 2
+
+typedef struct NhaLayerPrologueArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* f;
+  void* q_swa;
+  void* k_swa;
+  void* q_gsa;
+  void* k_gsa;
+  void* v_out;
+  void* s;
+  void* g;
+  const float* inv_freq;     /* [K/2] fp32 */
+  const int32_t* cu_seqlens; /* device [N+1], or NULL */
+  int32_t T_tot, N, HQ, H, K, V, M;
+  int32_t feature_map;
+  int32_t seqlen_offset;
+  int32_t dtype;
+  float gate_logit_normalizer;
+  void* stream;
+} NhaLayerPrologueArgs;
+
+typedef struct NhaLayerEpilogueArgs {
+  const void* o;
+  void* y;
+  const float* weight;
+  const float* bias;
+  int32_t rows, dim, dtype;
+  float eps;
+  void* stream;
+} NhaLayerEpilogueArgs;
+
+int nha_layer_prologue(const NhaLayerPrologueArgs* a);
+int nha_layer_epilogue(const NhaLayerEpilogueArgs* a);
 
 const char* nha_last_error(void);
 int nha_abi_version(void);

@@ -116,6 +116,37 @@ int nha_decode_step(const NhaDecodeArgs* a) { return decode_step_impl(a); }
 
 int nha_decode_advance(int32_t* count, int32_t B, void* stream) { return decode_advance_impl(count, B, stream); }
 
+int nha_layer_prologue(const NhaLayerPrologueArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_layer_prologue: null args");
+  NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->HQ > 0 && a->H > 0 && a->K > 0 && a->V > 0 && a->M > 0,
+                "nha_layer_prologue: non-positive dimension");
+  NHA_CHECK_ARG(a->K % 2 == 0 && a->K <= 1024, "nha_layer_prologue: K must be even and <= 1024, got %d", a->K);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_layer_prologue: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->feature_map >= NHA_FMAP_NONE && a->feature_map <= NHA_FMAP_RELU,
+                "nha_layer_prologue: bad feature_map %d", a->feature_map);
+  NHA_CHECK_ARG(a->q && a->k && a->v && a->f && a->q_swa && a->k_swa && a->v_out && a->s && a->g && a->inv_freq,
+                "nha_layer_prologue: q, k, v, f, q_swa, k_swa, v_out, s, g, inv_freq are required");
+  NHA_CHECK_ARG(a->feature_map == NHA_FMAP_NONE || (a->q_gsa && a->k_gsa),
+                "nha_layer_prologue: q_gsa and k_gsa are required with a feature map");
+  NHA_CHECK_ARG(a->cu_seqlens != nullptr || a->T_tot % a->N == 0,
+                "nha_layer_prologue: T_tot (%d) must be a multiple of N (%d) without cu_seqlens", a->T_tot, a->N);
+  NHA_CHECK_ARG(a->gate_logit_normalizer != 0.f, "nha_layer_prologue: gate_logit_normalizer must not be 0");
+  const void* ptrs[] = {a->q, a->k, a->v, a->f, a->q_swa, a->k_swa, a->q_gsa, a->k_gsa, a->v_out, a->s, a->g};
+  for (const void* p : ptrs)
+    NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(p) & 15) == 0, "nha_layer_prologue: tensors must be 16-byte aligned");
+  return layer_prologue_impl(a);
+}
+
+int nha_layer_epilogue(const NhaLayerEpilogueArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_layer_epilogue: null args");
+  NHA_CHECK_ARG(a->rows > 0 && a->dim > 0, "nha_layer_epilogue: non-positive dimension");
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_layer_epilogue: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->o && a->y, "nha_layer_epilogue: o and y are required");
+  NHA_CHECK_ARG(((reinterpret_cast<uintptr_t>(a->o) | reinterpret_cast<uintptr_t>(a->y)) & 15) == 0,
+                "nha_layer_epilogue: tensors must be 16-byte aligned");
+  return layer_epilogue_impl(a);
+}
+
 int32_t nha_varlen_num_chunks(const int32_t* cu, int32_t N, int32_t BT) {
   if (!cu || N <= 0 || BT <= 0) {
     set_error("nha_varlen_num_chunks: bad arguments");

@@ -14,12 +14,10 @@ typedef uint16_t bf16_t;  // raw bf16 bit pattern
 __device__ __forceinline__ float bf16_to_f32(bf16_t x) {
   return __uint_as_float(((uint32_t)x) << 16);
 }
-// round-to-nearest-even, NaN preserved
+// round-to-nearest-even, NaN stays NaN: the hardware conversion of gfx950 (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
 }
 
 typedef unsigned int nha_u32x4 __attribute__((ext_vector_type(4)));
@@ -64,12 +62,11 @@ template <> struct Elem<bf16_t> {
     o[6] = __uint_as_float(a[3] << 16); o[7] = __uint_as_float(a[3] & 0xffff0000u);
   }
   static __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
-    uint4 a;
-    a.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-    a.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
-    a.z = (uint32_t)f32_to_bf16(v[4]) | ((uint32_t)f32_to_bf16(v[5]) << 16);
-    a.w = (uint32_t)f32_to_bf16(v[6]) | ((uint32_t)f32_to_bf16(v[7]) << 16);
-    *reinterpret_cast<uint4*>(p) = a;
+    typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+    bf16x8_t a;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = (__bf16)v[e];  // pairs convert in one packed instruction
+    *reinterpret_cast<bf16x8_t*>(p) = a;
   }
 };
 
@@ -129,6 +126,8 @@ static inline int next_pow2_i(int x) {
 // host-side error plumbing (thread-local message)
 void set_error(const char* fmt, ...);
 
+int layer_prologue_impl(const NhaLayerPrologueArgs* a);
+int layer_epilogue_impl(const NhaLayerEpilogueArgs* a);
 int decode_step_impl(const NhaDecodeArgs* a);
 int decode_advance_impl(int32_t* count, int32_t B, void* stream);
 bool decode_mfma_supported(const NhaDecodeArgs* a);

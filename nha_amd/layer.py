@@ -9,6 +9,8 @@ The reference takes RMSNorm, RotaryEmbedding, ShortConvolution, the feature maps
 and the unpad helpers from flash-linear-attention, which is not vendored; they are restated here in
 plain PyTorch from their published behaviour (elementwise / projection glue around the hot path).
 The layer is trainable: chunk_nha carries its own backward, the glue around it is plain autograd.
+With autograd off (inference) the elementwise glue on either side of the op runs as two fused HIP
+launches instead (nha_layer_prologue / nha_layer_epilogue); `fuse_glue = False` keeps the tensor-op chain.
 """
 from __future__ import annotations
 
@@ -19,7 +21,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .ops import chunk_nha
+from .ops import chunk_nha, nha_layer_epilogue, nha_layer_prologue
 
 
 class RMSNorm(nn.Module):
@@ -72,8 +74,11 @@ class RotaryEmbedding(nn.Module):
         super().__init__()
         self.dim, self.base = dim, base
 
+    def inv_freq(self, device) -> torch.Tensor:
+        return 1.0 / (self.base ** (torch.arange(0, self.dim, 2, device=device, dtype=torch.float32) / self.dim))
+
     def _tables(self, pos: torch.Tensor, dtype):
-        inv = 1.0 / (self.base ** (torch.arange(0, self.dim, 2, device=pos.device, dtype=torch.float32) / self.dim))
+        inv = self.inv_freq(pos.device)
         fr = pos.float()[:, None] * inv[None, :]
         return fr.cos().to(dtype), fr.sin().to(dtype)
 
@@ -232,6 +237,16 @@ class NativeHybridAttention(nn.Module):
         self.g_norm = RMSNorm(self.hidden_size, elementwise_affine, eps=norm_eps, dtype=torch.float32)
         self.o_proj = nn.Linear(self.value_dim, self.hidden_size, bias=False)
         self.rotary = RotaryEmbedding(dim=self.head_k_dim, base=self.rope_theta)
+        self.fuse_glue = True
+        self._inv_freq = None
+
+    def _fused_glue(self, x: torch.Tensor) -> bool:
+        """The fused prologue/epilogue kernels record no autograd graph and cover the swish, relu and
+        identity feature maps in bf16 / fp32 on the GPU."""
+        return (self.fuse_glue and not torch.is_grad_enabled() and x.is_cuda
+                and x.dtype in (torch.bfloat16, torch.float32)
+                and isinstance(self.feature_map, (SwishFeatureMap, ReLUFeatureMap, type(None)))
+                and self.o_proj.weight.dtype == x.dtype and self.head_k_dim % 2 == 0)
 
     def forward(
         self,
@@ -280,20 +295,29 @@ class NativeHybridAttention(nn.Module):
         k = k.unflatten(-1, (-1, self.head_k_dim))
         v = v.unflatten(-1, (-1, self.head_v_dim))
         f = f.unflatten(-1, (-1, self.num_slots))
-        if self.feature_map is not None:
-            q_gsa, k_gsa = self.feature_map(q), self.feature_map(k)
-        else:
-            q_gsa, k_gsa = q, k
-        v = F.silu(v)
-        f = F.logsigmoid(f) / self.gate_logit_normalizer
-        s = (1 - f.exp()).to(f.dtype)
-        g = f
         seqlen_offset = 0
         if last_state is not None and 'seqlen_offset' in last_state:
             seqlen_offset = last_state['seqlen_offset']
-        # rotary on the kv-head keys: identical across the heads of a group, so rotating before the
-        # (implicit, in-kernel) group expansion equals the reference's repeat-then-rotate
-        q_swa, k_swa = self.rotary(q, k, seqlen_offset=seqlen_offset, cu_seqlens=cu_seqlens)
+        fused = self._fused_glue(q) and f.dtype == q.dtype
+        if fused:
+            if self._inv_freq is None or self._inv_freq.device != q.device:
+                self._inv_freq = self.rotary.inv_freq(q.device)
+            fm = None if self.feature_map is None else ('swish' if isinstance(self.feature_map, SwishFeatureMap) else 'relu')
+            q_swa, k_swa, q_gsa, k_gsa, v, s, g = nha_layer_prologue(
+                q, k, v, f, self._inv_freq, feature_map=fm, gate_logit_normalizer=self.gate_logit_normalizer,
+                seqlen_offset=seqlen_offset, cu_seqlens=cu_seqlens)
+        else:
+            if self.feature_map is not None:
+                q_gsa, k_gsa = self.feature_map(q), self.feature_map(k)
+            else:
+                q_gsa, k_gsa = q, k
+            v = F.silu(v)
+            f = F.logsigmoid(f) / self.gate_logit_normalizer
+            s = (1 - f.exp()).to(f.dtype)
+            g = f
+            # rotary on the kv-head keys: identical across the heads of a group, so rotating before the
+            # (implicit, in-kernel) group expansion equals the reference's repeat-then-rotate
+            q_swa, k_swa = self.rotary(q, k, seqlen_offset=seqlen_offset, cu_seqlens=cu_seqlens)
         if mode == 'chunk':
             output, lse_swa, lse_gsa = chunk_nha(
                 q_swa=q_swa, k_swa=k_swa, q_gsa=q_gsa, k_gsa=k_gsa, v=v, s=s, g=g,
@@ -319,8 +343,12 @@ class NativeHybridAttention(nn.Module):
                 offset=q_len,
             )
         o = output[:, :, :, :self.head_v_dim].flatten(-2)
-        o = rms_norm_linear(F.silu(o), self.g_norm.weight, self.g_norm.bias, self.o_proj.weight, self.o_proj.bias,
-                            eps=self.norm_eps)
+        if fused:
+            o = F.linear(nha_layer_epilogue(o, self.g_norm.weight, self.g_norm.bias, self.norm_eps),
+                         self.o_proj.weight, self.o_proj.bias)
+        else:
+            o = rms_norm_linear(F.silu(o), self.g_norm.weight, self.g_norm.bias, self.o_proj.weight, self.o_proj.bias,
+                                eps=self.norm_eps)
         if attention_mask is not None:
             o = pad_input(o.squeeze(0), indices, batch_size, q_len)
         return o, None, past_key_values

@@ -24,7 +24,7 @@ from . import _lib
 from .varlen import CHUNK, chunk_tables
 
 __all__ = ["chunk_nha", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
-           "prefill_tables", "nha_prefill", "nha_prefill_bwd"]
+           "prefill_tables", "nha_prefill", "nha_prefill_bwd", "nha_layer_prologue", "nha_layer_epilogue"]
 
 _DT = {torch.float32: _lib.NHA_DTYPE_F32, torch.bfloat16: _lib.NHA_DTYPE_BF16}
 _IMPL = {None: _lib.NHA_IMPL_AUTO, "auto": _lib.NHA_IMPL_AUTO, "simple": _lib.NHA_IMPL_SIMPLE,
@@ -158,6 +158,64 @@ def nha_prefill_bwd(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, do
     a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
     _lib.check(lib.nha_prefill_bwd(C.byref(a)))
     return (*outs, dh0k, dh0v)
+
+
+_FMAP = {None: _lib.NHA_FMAP_NONE, "none": _lib.NHA_FMAP_NONE, "swish": _lib.NHA_FMAP_SWISH, "relu": _lib.NHA_FMAP_RELU}
+
+
+def nha_layer_prologue(q, k, v, f, inv_freq, *, feature_map: Optional[str], gate_logit_normalizer: float,
+                       seqlen_offset: int = 0, cu_seqlens: Optional[torch.Tensor] = None):
+    """One launch for the elementwise chain of nha_fla/layers/nha.py:214-237 on the raw projections
+    q [B,T,HQ,K], k [B,T,H,K], v [B,T,H,V], f [B,T,H,M] (B = 1 with cu_seqlens, an int32 device
+    tensor).  Returns (q_swa, k_swa, q_gsa, k_gsa, v, s, g); without a feature map q_gsa / k_gsa
+    are q / k themselves.  Inference only: no autograd graph is recorded."""
+    lib = _lib.load()
+    _need_cuda(q, k, v, f, inv_freq, cu_seqlens)
+    if feature_map not in _FMAP:
+        raise NotImplementedError(f"Feature map `{feature_map}` has no fused prologue.")
+    B, T, HQ, K = q.shape
+    H, V, M = k.shape[2], v.shape[3], f.shape[3]
+    if cu_seqlens is not None and B != 1:
+        raise ValueError("cu_seqlens needs the packed layout [1, T_tot, ...]")
+    dt = _dtype_code(q)
+    q, k, v, f = (x.contiguous() for x in (q, k, v, f))
+    for x in (k, v, f):
+        if x.dtype != q.dtype:
+            raise TypeError("q, k, v, f must share one dtype")
+    inv_freq = inv_freq.to(torch.float32).contiguous()
+    if inv_freq.numel() != K // 2:
+        raise ValueError(f"inv_freq must hold K/2 = {K // 2} entries, got {inv_freq.numel()}")
+    fm = _FMAP[feature_map]
+    q_swa, k_swa, v_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    s, g = torch.empty_like(f), torch.empty_like(f)
+    q_gsa = torch.empty_like(q) if fm else None
+    k_gsa = torch.empty_like(k) if fm else None
+    cu = None if cu_seqlens is None else cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()
+    a = _lib.NhaLayerPrologueArgs(
+        q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), q_swa=_ptr(q_swa), k_swa=_ptr(k_swa), q_gsa=_ptr(q_gsa),
+        k_gsa=_ptr(k_gsa), v_out=_ptr(v_out), s=_ptr(s), g=_ptr(g), inv_freq=_ptr(inv_freq), cu_seqlens=_ptr(cu),
+        T_tot=B * T, N=(cu.numel() - 1) if cu is not None else B, HQ=HQ, H=H, K=K, V=V, M=M, feature_map=fm,
+        seqlen_offset=int(seqlen_offset), dtype=dt, gate_logit_normalizer=float(gate_logit_normalizer),
+        stream=_stream(q.device))
+    _lib.check(lib.nha_layer_prologue(C.byref(a)))
+    return q_swa, k_swa, (q_gsa if fm else q), (k_gsa if fm else k), v_out, s, g
+
+
+def nha_layer_epilogue(o, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float):
+    """rms_norm(silu(o)) * weight (+ bias) over the last dimension in one launch: the normalisation
+    half of nha_fla/layers/nha.py:278.  Inference only."""
+    lib = _lib.load()
+    _need_cuda(o, weight, bias)
+    dt = _dtype_code(o)
+    o = o.contiguous()
+    dim = o.shape[-1]
+    w = None if weight is None else weight.detach().to(torch.float32).contiguous()
+    b = None if bias is None else bias.detach().to(torch.float32).contiguous()
+    y = torch.empty_like(o)
+    a = _lib.NhaLayerEpilogueArgs(o=_ptr(o), y=_ptr(y), weight=_ptr(w), bias=_ptr(b), rows=o.numel() // dim, dim=dim,
+                                  dtype=dt, eps=float(eps), stream=_stream(o.device))
+    _lib.check(lib.nha_layer_epilogue(C.byref(a)))
+    return y
 
 
 class _ChunkNHAFunction(torch.autograd.Function):

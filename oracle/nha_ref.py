@@ -21,7 +21,9 @@ something that is *not* a retyping of its own formula -- torch's
 scaled_dot_product_attention (slots degenerate to zero sinks), the explicit
 double-sum closed form of the gated recurrence, the two-branch LSE merge of
 chunk.py:459-470, an independent chunk-form evaluation, complex-number RoPE,
-decode == last row of prefill, packed == per-sequence.  What nothing in this
+decode == last row of prefill, packed == per-sequence; the layer glue against
+torch's sigmoid / rms_norm library routines, RoPE's norm and relative-position
+invariants and s + exp(g) = 1.  What nothing in this
 container pins: the exact bf16 rounding sequence of the Triton/fla chain and
 flash-attn's window inclusivity for ``window_size_left`` (third-party documented
 semantics: key j visible to query i iff i - wl <= j <= i).
@@ -34,6 +36,8 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 __all__ = [
+    "layer_prologue_ref",
+    "layer_epilogue_ref",
     "rope_rotate_half",
     "gsa_step",
     "prefill_ref",
@@ -51,6 +55,34 @@ def rope_rotate_half(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> t
     half = x.shape[-1] // 2
     rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
     return x * cos.unsqueeze(-2) + rot * sin.unsqueeze(-2)
+
+
+def layer_prologue_ref(q, k, v, f, *, feature_map, gate_logit_normalizer, positions, rope_theta=10000.0):
+    """The elementwise chain of nha_fla/layers/nha.py:214-237 in the dtype of the inputs (pass
+    float64 for the checker): q [B,T,HQ,K], k [B,T,H,K], v [B,T,H,V], f [B,T,H,M],
+    positions [B,T] or [T] (token index inside its sequence + seqlen_offset).
+    Returns (q_swa, k_swa, q_gsa, k_gsa, v, s, g).  The rotary angle is formed in float32
+    (position * inv_freq, as the rotary module's cos/sin cache is) and then widened."""
+    K = q.shape[-1]
+    fmap = {"swish": torch.nn.functional.silu, "relu": torch.relu, None: (lambda x: x)}[feature_map]
+    inv = 1.0 / (rope_theta ** (torch.arange(0, K, 2, dtype=torch.float32) / K))
+    ang = (positions.to(torch.float32)[..., None] * inv).to(q.dtype)          # [..., T, K/2]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1), torch.cat([ang.sin(), ang.sin()], -1)
+    g = torch.nn.functional.logsigmoid(f) / gate_logit_normalizer
+    return (rope_rotate_half(q, cos, sin), rope_rotate_half(k, cos, sin), fmap(q), fmap(k),
+            torch.nn.functional.silu(v), 1 - g.exp(), g)
+
+
+def layer_epilogue_ref(o, weight, bias, eps):
+    """rms_norm(silu(o)) * weight (+ bias) over the last dim: the normalisation half of
+    rms_norm_linear(F.silu(o), ...) at nha_fla/layers/nha.py:278."""
+    y = torch.nn.functional.silu(o)
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * weight
+    if bias is not None:
+        y = y + bias
+    return y
 
 
 def gsa_step(hk, hv, k, v, s, g):

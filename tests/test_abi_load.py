@@ -33,8 +33,12 @@ def test_struct_sizes_match_the_header(tmp_path):
     probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream", "count_next")]
     probes += [("NhaPrefillBwdArgs", f) for f in ("q_swa", "o", "dout", "dhvt", "dq_swa", "dg", "dh0v", "cu_seqlens",
                                                   "scratch_bytes", "T_tot", "dtype", "scale", "stream")]
+    probes += [("NhaLayerPrologueArgs", f) for f in ("q", "q_swa", "g", "inv_freq", "cu_seqlens", "T_tot", "M", "feature_map",
+                                                     "seqlen_offset", "dtype", "gate_logit_normalizer", "stream")]
+    probes += [("NhaLayerEpilogueArgs", f) for f in ("o", "y", "weight", "bias", "rows", "dim", "dtype", "eps", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
-           'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));']
+           'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));',
+           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueArgs), sizeof(NhaLayerEpilogueArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
     src += ['return 0; }']
     cfile = tmp_path / "probe.c"
@@ -44,7 +48,8 @@ def test_struct_sizes_match_the_header(tmp_path):
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert int(out[0]) == C.sizeof(_lib.NhaPrefillArgs) and int(out[1]) == C.sizeof(_lib.NhaDecodeArgs)
     assert int(out[2]) == C.sizeof(_lib.NhaPrefillBwdArgs)
-    for (t, f), off in zip(probes, out[3:]):
+    assert int(out[3]) == C.sizeof(_lib.NhaLayerPrologueArgs) and int(out[4]) == C.sizeof(_lib.NhaLayerEpilogueArgs)
+    for (t, f), off in zip(probes, out[5:]):
         assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 
@@ -66,6 +71,18 @@ def test_argument_validation_without_gpu():
     d.B = d.H = d.K = d.V = d.M = d.W = 8
     d.HQ = 12
     assert lib.nha_decode_step(C.byref(d)) == _lib.NHA_ERR_INVALID and b"multiple" in lib.nha_last_error()
+    lp = _lib.NhaLayerPrologueArgs()
+    assert lib.nha_layer_prologue(C.byref(lp)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
+    lp.T_tot, lp.N, lp.HQ, lp.H, lp.K, lp.V, lp.M = 10, 1, 2, 1, 7, 8, 8
+    assert lib.nha_layer_prologue(C.byref(lp)) == _lib.NHA_ERR_INVALID and b"even" in lib.nha_last_error()
+    lp.K, lp.feature_map = 8, 3
+    assert lib.nha_layer_prologue(C.byref(lp)) == _lib.NHA_ERR_INVALID and b"feature_map" in lib.nha_last_error()
+    lp.feature_map = 1
+    assert lib.nha_layer_prologue(C.byref(lp)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    le = _lib.NhaLayerEpilogueArgs()
+    assert lib.nha_layer_epilogue(C.byref(le)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
+    le.rows, le.dim = 4, 64
+    assert lib.nha_layer_epilogue(C.byref(le)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
     with pytest.raises(_lib.NhaError):
         chunk_tables([0, 5, 5])          # zero-length sequence
     with pytest.raises(_lib.NhaError):

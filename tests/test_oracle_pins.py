@@ -322,3 +322,38 @@ def test_gradients_match_finite_differences(wl, shift, varlen):
     if varlen and shift >= 1:
         # tokens of a sequence no longer than the shift never reach the slots: no slot-branch gradient
         assert G["dk_gsa"][0, 5:6].abs().max() == 0 and G["dg"][0, 5:6].abs().max() == 0
+
+
+def test_layer_glue_against_library_routines_and_invariants():
+    """Pins layer_prologue_ref / layer_epilogue_ref without retyping them: torch's sigmoid and
+    rms_norm routines, the complex-number form of RoPE, its norm and relative-position invariants."""
+    torch.manual_seed(11)
+    B, T, HQ, H, K, V, M = 2, 9, 4, 2, 8, 6, 5
+    r = lambda *s: torch.randn(*s, dtype=DT)
+    q, k, v, f = r(B, T, HQ, K), r(B, T, H, K), r(B, T, H, V), 3 * r(B, T, H, M)
+    pos = torch.arange(T) + 7
+    q_swa, k_swa, q_gsa, k_gsa, vo, s, g = R.layer_prologue_ref(q, k, v, f, feature_map="swish", gate_logit_normalizer=8,
+                                                                positions=pos, rope_theta=10000.0)
+    # gates: exp(normalizer * g) is the library sigmoid, s + exp(g) = 1, g <= 0
+    assert torch.allclose((8 * g).exp(), torch.sigmoid(f), atol=1e-12)
+    assert torch.allclose(s + g.exp(), torch.ones_like(s), atol=1e-14) and (g <= 0).all() and (s >= 0).all()
+    assert torch.allclose(vo, v * torch.sigmoid(v), atol=1e-12) and torch.allclose(q_gsa, q * torch.sigmoid(q), atol=1e-12)
+    assert torch.equal(R.layer_prologue_ref(q, k, v, f, feature_map="relu", gate_logit_normalizer=8, positions=pos)[3],
+                       k.clamp_min(0))
+    assert R.layer_prologue_ref(q, k, v, f, feature_map=None, gate_logit_normalizer=8, positions=pos)[2] is q
+    # RoPE: (x1 + i x2) * exp(i * pos * theta^(-2j/K)), norms kept, scores depend on pos differences only
+    inv = 10000.0 ** (-torch.arange(0, K, 2, dtype=DT) / K)
+    z = torch.complex(q[..., : K // 2], q[..., K // 2:]) * torch.polar(torch.ones(T, K // 2, dtype=DT),
+                                                                        (pos[:, None].float() * inv.float()).double())[None, :, None, :]
+    assert torch.allclose(torch.cat([z.real, z.imag], -1), q_swa, atol=1e-12)
+    assert torch.allclose(q_swa.norm(dim=-1), q.norm(dim=-1), atol=1e-12)
+    q2, k2 = R.layer_prologue_ref(q, k, v, f, feature_map=None, gate_logit_normalizer=8, positions=pos + 100)[:2]
+    sc1 = torch.einsum("bihk,bjhk->bhij", q_swa[:, :, :H], k_swa)
+    sc2 = torch.einsum("bihk,bjhk->bhij", q2[:, :, :H], k2)
+    assert torch.allclose(sc1, sc2, atol=1e-4)             # the angle is formed in float32: 1e-5-level drift at pos ~100
+    # epilogue: torch's rms_norm on silu(o)
+    o, w, b = r(B, T, HQ * V), r(HQ * V), r(HQ * V)
+    ref = F.rms_norm(F.silu(o), (HQ * V,), weight=w, eps=1e-5) + b
+    assert torch.allclose(R.layer_epilogue_ref(o, w, b, 1e-5), ref, atol=1e-12)
+    y = R.layer_epilogue_ref(o, None, None, 0.0)
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(B, T, dtype=DT), atol=1e-12)
