@@ -36,6 +36,44 @@ class NHARingState:
         return cls(z(B, H, K, M, dt=torch.float32), z(B, H, M, V, dt=torch.float32), z(B, W, H, K), z(B, W, H, K),
                    z(B, W, H, V), z(B, W, H, M), z(B, dt=torch.int32))
 
+    @classmethod
+    def from_prefill(cls, k_swa, k_gsa, v, g, final_state, window: int, cu_seqlens=None) -> "NHARingState":
+        """The decode state that continues a prefill with ``(window_size_left, gsa_kv_shift) =
+        (window - 1, window)``: the slot state is the prefill's final state (it has absorbed the
+        tokens that left the window), ring slot ``j % window`` holds token ``j`` for the last
+        ``min(L, window)`` tokens of each sequence and ``count = L``.  Takes the prefill's own
+        operands: k_swa (rotated), k_gsa, v ``[B,T,H,*]``, g ``[B,T,H,M]`` (``[1,T_tot,...]`` with
+        cu_seqlens) and ``final_state = (hk [N,H,K,M], hv [N,H,M,V])``.  The hand-over the reference
+        does by slicing the last ``window`` rows into its cache (nha_fla/models/nha_cache.py:87-91)."""
+        _need_cuda(k_swa, k_gsa, v, g, final_state[0], final_state[1])
+        dev, W = k_swa.device, int(window)
+        B, T, H, K = k_swa.shape
+        V, M = v.shape[-1], g.shape[-1]
+        if cu_seqlens is None:
+            starts = torch.arange(B, device=dev, dtype=torch.long) * T
+            lens = torch.full((B,), T, device=dev, dtype=torch.long)
+        else:
+            if B != 1:
+                raise ValueError("cu_seqlens needs the packed layout [1, T_tot, ...]")
+            cu = cu_seqlens.to(device=dev, dtype=torch.long)
+            starts, lens = cu[:-1], cu[1:] - cu[:-1]
+        N = starts.numel()
+        hk, hv = final_state
+        if tuple(hk.shape) != (N, H, K, M) or tuple(hv.shape) != (N, H, M, V):
+            raise ValueError(f"final_state must be ([{N},{H},{K},{M}], [{N},{H},{M},{V}]), got {tuple(hk.shape)}, {tuple(hv.shape)}")
+        r = torch.arange(W, device=dev, dtype=torch.long)
+        last = (lens - 1)[:, None]
+        tok = last - torch.remainder(last - r[None, :], W)            # newest token j <= L-1 with j % W == r
+        valid = tok >= 0
+        src = (starts[:, None] + tok.clamp_min(0)).reshape(-1)
+
+        def gather(x):
+            rows = x.reshape(B * T, *x.shape[2:]).index_select(0, src).reshape(N, W, *x.shape[2:])
+            return rows * valid[:, :, None, None].to(rows.dtype)
+
+        return cls(hk.to(torch.float32).clone(), hv.to(torch.float32).clone(), gather(k_swa), gather(k_gsa), gather(v),
+                   gather(g), lens.to(torch.int32))
+
     @property
     def window(self) -> int:
         return self.ring_k.shape[1]

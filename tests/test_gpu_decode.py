@@ -152,3 +152,31 @@ def test_ring_decode_steps(NG, K, M, W):
     assert_close("ring hv", st.hv, ref["hv"], dtype)
     assert torch.equal(st.ring_k.cpu().double(), ref["rings"][0])
     assert torch.equal(st.ring_g.cpu().double(), ref["rings"][3])
+
+
+@pytest.mark.parametrize("W,lens,NG,K", [(32, (70, 20, 32), 4, 128), (64, (130, 64, 1), 1, 64), (48, (200,), 8, 64)])
+def test_prefill_hands_over_to_ring_decode(W, lens, NG, K):
+    """Packed prefill of the prompts -> NHARingState.from_prefill -> decode steps == the oracle's
+    prefill of the extended sequences, row by row (prompts shorter than, equal to and longer than
+    the window)."""
+    import nha_amd
+    from nha_amd import NHARingState, ring_decode_step
+    from tests.util import prefill_inputs
+    dtype, H, M, steps = torch.bfloat16, 2, 64, 5
+    HQ, V = H * NG, K
+    names = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+    full = [prefill_inputs(40 + n, 1, L + steps, HQ, H, K, V, M, dtype=dtype) for n, L in enumerate(lens)]
+    refs = [R.prefill_ref(*[d[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W)[0] for d in full]
+    packed = {k: torch.cat([d[k][:, :L] for d, L in zip(full, lens)], 1).cuda() for k in names}
+    cu = torch.tensor([0] + list(itertools.accumulate(lens)), dtype=torch.int32)
+    o, _, _, (hk, hv) = nha_amd.chunk_nha(*[packed[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W,
+                                           cu_seqlens=cu.cuda(), output_final_state=True)
+    assert_close("prompt o", o, torch.cat([r[:, :L] for r, L in zip(refs, lens)], 1), dtype)
+    st = NHARingState.from_prefill(packed["k_swa"], packed["k_gsa"], packed["v"], packed["g"], (hk, hv), W,
+                                   cu_seqlens=cu.cuda())
+    assert st.count.tolist() == list(lens) and st.ring_k.shape == (len(lens), W, H, K)
+    for i in range(steps):
+        row = lambda k: torch.stack([d[k][0, L + i] for d, L in zip(full, lens)]).cuda().contiguous()
+        oi = ring_decode_step(st, row("q_gsa"), row("q_swa"), row("k_swa"), row("k_gsa"), row("v"), row("g"))
+        assert_close(f"decode step {i}", oi, torch.stack([r[0, L + i] for r, L in zip(refs, lens)]), dtype)
+    assert st.count.tolist() == [L + steps for L in lens]
