@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 4
+#define NHA_ABI_VERSION 5
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -290,6 +290,61 @@ typedef struct NhaLayerEpilogueArgs {
 
 int nha_layer_prologue(const NhaLayerPrologueArgs* a);
 int nha_layer_epilogue(const NhaLayerEpilogueArgs* a);
+
+/* Backward of the two launches above (what autograd derives from the tensor-op chain of
+ * nha_fla/layers/nha.py:214-237, :278; the reference has no hand-written counterpart).
+ *
+ * nha_layer_prologue_bwd: from the raw projections and the cotangents of the seven outputs it
+ * writes dq, dk, dv, df: the rotation by the opposite angle of dq_swa / dk_swa plus the feature
+ * map's derivative times dq_gsa / dk_gsa (not read with NHA_FMAP_NONE: the caller adds the slot
+ * cotangent itself, q_gsa being q), dv_out * silu'(v), and
+ * df = (dg - ds * exp(g)) / normalizer * sigmoid(-f).
+ *
+ * nha_layer_epilogue_bwd: dout = d silu(o) of the RMS-norm backward; the weight and bias
+ * gradients leave as partial sums dweight_partial / dbias_partial [parts, dim] fp32 with
+ * parts = nha_layer_epilogue_bwd_parts(rows), which the caller adds up over the first axis
+ * (fixed order: run-to-run identical).  Either may be NULL.  dim: multiple of 8, <= 8192. */
+typedef struct NhaLayerPrologueBwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* f;
+  const void* dq_swa;
+  const void* dk_swa;
+  const void* dq_gsa;
+  const void* dk_gsa;
+  const void* dv_out;
+  const void* ds;
+  const void* dg;
+  void* dq;
+  void* dk;
+  void* dv;
+  void* df;
+  const float* inv_freq;
+  const int32_t* cu_seqlens;
+  int32_t T_tot, N, HQ, H, K, V, M;
+  int32_t feature_map;
+  int32_t seqlen_offset;
+  int32_t dtype;
+  float gate_logit_normalizer;
+  void* stream;
+} NhaLayerPrologueBwdArgs;
+
+typedef struct NhaLayerEpilogueBwdArgs {
+  const void* o;
+  const void* dy;
+  void* dout;
+  const float* weight;
+  float* dweight_partial;
+  float* dbias_partial;
+  int32_t rows, dim, dtype;
+  float eps;
+  void* stream;
+} NhaLayerEpilogueBwdArgs;
+
+int nha_layer_prologue_bwd(const NhaLayerPrologueBwdArgs* a);
+int32_t nha_layer_epilogue_bwd_parts(int32_t rows);
+int nha_layer_epilogue_bwd(const NhaLayerEpilogueBwdArgs* a);
 
 const char* nha_last_error(void);
 int nha_abi_version(void);

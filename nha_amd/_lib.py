@@ -14,12 +14,13 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 4
+ABI_VERSION = 5
 NHA_FMAP_NONE, NHA_FMAP_SWISH, NHA_FMAP_RELU = 0, 1, 2
 
 EXPORTS = (
     "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
     "nha_decode_step", "nha_decode_advance", "nha_layer_prologue", "nha_layer_epilogue",
+    "nha_layer_prologue_bwd", "nha_layer_epilogue_bwd", "nha_layer_epilogue_bwd_parts",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
 )
 
@@ -97,6 +98,28 @@ class NhaLayerEpilogueArgs(C.Structure):
     ]
 
 
+class NhaLayerPrologueBwdArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("f", C.c_void_p),
+        ("dq_swa", C.c_void_p), ("dk_swa", C.c_void_p), ("dq_gsa", C.c_void_p), ("dk_gsa", C.c_void_p),
+        ("dv_out", C.c_void_p), ("ds", C.c_void_p), ("dg", C.c_void_p),
+        ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p), ("df", C.c_void_p),
+        ("inv_freq", C.c_void_p), ("cu_seqlens", C.c_void_p),
+        ("T_tot", C.c_int32), ("N", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32),
+        ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
+        ("feature_map", C.c_int32), ("seqlen_offset", C.c_int32), ("dtype", C.c_int32),
+        ("gate_logit_normalizer", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
+class NhaLayerEpilogueBwdArgs(C.Structure):
+    _fields_ = [
+        ("o", C.c_void_p), ("dy", C.c_void_p), ("dout", C.c_void_p), ("weight", C.c_void_p),
+        ("dweight_partial", C.c_void_p), ("dbias_partial", C.c_void_p),
+        ("rows", C.c_int32), ("dim", C.c_int32), ("dtype", C.c_int32), ("eps", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
 class NhaError(RuntimeError):
     def __init__(self, code: int, msg: str):
         super().__init__(f"libnha_hip error {code}: {msg}")
@@ -131,6 +154,12 @@ def load() -> C.CDLL:
     lib.nha_layer_prologue.argtypes = [C.POINTER(NhaLayerPrologueArgs)]
     lib.nha_layer_epilogue.restype = C.c_int
     lib.nha_layer_epilogue.argtypes = [C.POINTER(NhaLayerEpilogueArgs)]
+    lib.nha_layer_prologue_bwd.restype = C.c_int
+    lib.nha_layer_prologue_bwd.argtypes = [C.POINTER(NhaLayerPrologueBwdArgs)]
+    lib.nha_layer_epilogue_bwd.restype = C.c_int
+    lib.nha_layer_epilogue_bwd.argtypes = [C.POINTER(NhaLayerEpilogueBwdArgs)]
+    lib.nha_layer_epilogue_bwd_parts.restype = C.c_int32
+    lib.nha_layer_epilogue_bwd_parts.argtypes = [C.c_int32]
     lib.nha_varlen_num_chunks.restype = C.c_int32
     lib.nha_varlen_num_chunks.argtypes = [C.c_void_p, C.c_int32, C.c_int32]
     lib.nha_varlen_indices.restype = C.c_int

@@ -147,6 +147,42 @@ int nha_layer_epilogue(const NhaLayerEpilogueArgs* a) {
   return layer_epilogue_impl(a);
 }
 
+int nha_layer_prologue_bwd(const NhaLayerPrologueBwdArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_layer_prologue_bwd: null args");
+  NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->HQ > 0 && a->H > 0 && a->K > 0 && a->V > 0 && a->M > 0,
+                "nha_layer_prologue_bwd: non-positive dimension");
+  NHA_CHECK_ARG(a->K % 2 == 0 && a->K <= 1024, "nha_layer_prologue_bwd: K must be even and <= 1024, got %d", a->K);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_layer_prologue_bwd: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->feature_map >= NHA_FMAP_NONE && a->feature_map <= NHA_FMAP_RELU,
+                "nha_layer_prologue_bwd: bad feature_map %d", a->feature_map);
+  NHA_CHECK_ARG(a->q && a->k && a->v && a->f && a->dq_swa && a->dk_swa && a->dv_out && a->ds && a->dg && a->dq && a->dk &&
+                    a->dv && a->df && a->inv_freq,
+                "nha_layer_prologue_bwd: q, k, v, f, dq_swa, dk_swa, dv_out, ds, dg, dq, dk, dv, df, inv_freq are required");
+  NHA_CHECK_ARG(a->feature_map == NHA_FMAP_NONE || (a->dq_gsa && a->dk_gsa),
+                "nha_layer_prologue_bwd: dq_gsa and dk_gsa are required with a feature map");
+  NHA_CHECK_ARG(a->cu_seqlens != nullptr || a->T_tot % a->N == 0,
+                "nha_layer_prologue_bwd: T_tot (%d) must be a multiple of N (%d) without cu_seqlens", a->T_tot, a->N);
+  NHA_CHECK_ARG(a->gate_logit_normalizer != 0.f, "nha_layer_prologue_bwd: gate_logit_normalizer must not be 0");
+  const void* ptrs[] = {a->q, a->k, a->v, a->f, a->dq_swa, a->dk_swa, a->dq_gsa, a->dk_gsa, a->dv_out, a->ds, a->dg,
+                        a->dq, a->dk, a->dv, a->df};
+  for (const void* p : ptrs)
+    NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(p) & 15) == 0, "nha_layer_prologue_bwd: tensors must be 16-byte aligned");
+  return layer_prologue_bwd_impl(a);
+}
+
+int32_t nha_layer_epilogue_bwd_parts(int32_t rows) { return rows > 0 ? layer_epilogue_bwd_parts(rows) : 0; }
+
+int nha_layer_epilogue_bwd(const NhaLayerEpilogueBwdArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_layer_epilogue_bwd: null args");
+  NHA_CHECK_ARG(a->rows > 0 && a->dim > 0, "nha_layer_epilogue_bwd: non-positive dimension");
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_layer_epilogue_bwd: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->o && a->dy && a->dout, "nha_layer_epilogue_bwd: o, dy and dout are required");
+  const void* ptrs[] = {a->o, a->dy, a->dout, a->weight, a->dweight_partial, a->dbias_partial};
+  for (const void* p : ptrs)
+    NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(p) & 15) == 0, "nha_layer_epilogue_bwd: tensors must be 16-byte aligned");
+  return layer_epilogue_bwd_impl(a);
+}
+
 int32_t nha_varlen_num_chunks(const int32_t* cu, int32_t N, int32_t BT) {
   if (!cu || N <= 0 || BT <= 0) {
     set_error("nha_varlen_num_chunks: bad arguments");

@@ -128,6 +128,9 @@ void set_error(const char* fmt, ...);
 
 int layer_prologue_impl(const NhaLayerPrologueArgs* a);
 int layer_epilogue_impl(const NhaLayerEpilogueArgs* a);
+int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a);
+int layer_epilogue_bwd_parts(int rows);
+int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a);
 int decode_step_impl(const NhaDecodeArgs* a);
 int decode_advance_impl(int32_t* count, int32_t B, void* stream);
 bool decode_mfma_supported(const NhaDecodeArgs* a);

@@ -19,7 +19,14 @@ struct LP {
   const int32_t* cu;
   int T_tot, N, T, HQ, H, K, V, M, fm, off;
   float inv_norm;
+  // backward only: cotangents of the seven outputs, gradients of the four inputs
+  const void *dq_swa, *dk_swa, *dq_gsa, *dk_gsa, *dv_out, *ds, *dg;
+  void *dq, *dk, *dv, *df;
 };
+
+constexpr int TOK_PER_WG = 4;     // one wave per token
+constexpr int ROWS_PER_WAVE = 4;  // epilogue rows a wave walks with its weight slice in registers
+constexpr int BWD_ROWS = 32;      // epilogue backward: rows per workgroup (one partial weight gradient each)
 
 template <typename T> __device__ __forceinline__ float rnd(float x);
 template <> __device__ __forceinline__ float rnd<float>(float x) { return x; }
@@ -37,6 +44,34 @@ template <typename T, int VEC> __device__ __forceinline__ void stv(T* p, const f
   if constexpr (VEC == 8) Elem<T>::st8(p, v);
   else Elem<T>::st(p, v[0]);
 }
+
+// VEC elements as loaded (conversion deferred, so a prefetched row costs half the registers in bf16)
+template <typename T, int VEC> struct Raw;
+template <> struct Raw<bf16_t, 8> {
+  uint4 r;
+  __device__ __forceinline__ void load(const bf16_t* p) { r = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void unpack(float* o) const {
+    o[0] = __uint_as_float(r.x << 16); o[1] = __uint_as_float(r.x & 0xffff0000u);
+    o[2] = __uint_as_float(r.y << 16); o[3] = __uint_as_float(r.y & 0xffff0000u);
+    o[4] = __uint_as_float(r.z << 16); o[5] = __uint_as_float(r.z & 0xffff0000u);
+    o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
+  }
+};
+template <> struct Raw<float, 8> {
+  float4 a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
+  }
+  __device__ __forceinline__ void unpack(float* o) const {
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+};
+template <typename T> struct Raw<T, 1> {
+  T r;
+  __device__ __forceinline__ void load(const T* p) { r = *p; }
+  __device__ __forceinline__ void unpack(float* o) const { o[0] = Elem<T>::ld(&r); }
+};
 
 // rotate-half RoPE of `heads` rows of K elements + the feature map of the same rows
 template <typename T, int VEC>
@@ -68,17 +103,12 @@ __device__ __forceinline__ void rope_rows(const T* src, T* swa, T* gsa, int head
   }
 }
 
-constexpr int TOK_PER_WG = 4;     // one wave per token
-constexpr int ROWS_PER_WAVE = 4;  // epilogue rows a wave walks with its weight slice in registers
-
-template <typename T, int VEC>
-__global__ __launch_bounds__(256) void layer_prologue_kernel(LP p) {
-  extern __shared__ float cs_all[];  // per wave: cos[K/2], sin[K/2]
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  float* cs = cs_all + wave * p.K;
+// cos/sin of the token's rotary angles into the wave's LDS slice cs[0..K/2) | cs[K/2..K); returns
+// the token index of this wave (clamped) and whether it exists.  All four waves reach the barrier.
+__device__ __forceinline__ int token_angles(const LP& p, float* cs, int wave, int lane, bool* live) {
   const int t_raw = blockIdx.x * TOK_PER_WG + wave;
-  const bool live = t_raw < p.T_tot;
-  const int t = live ? t_raw : p.T_tot - 1;
+  *live = t_raw < p.T_tot;
+  const int t = *live ? t_raw : p.T_tot - 1;
   int pos;
   if (p.cu) {
     int lo = 0, hi = p.N;  // largest n with cu[n] <= t
@@ -99,12 +129,22 @@ __global__ __launch_bounds__(256) void layer_prologue_kernel(LP p) {
     const double ang = (double)((float)pos * p.inv_freq[i]);
     const double turns = rint(ang * 0.15915494309189535);
     const float red = (float)fma(-turns, 6.283185307179586, ang);
-    float s, c;
-    sincosf(red, &s, &c);
+    float sn, c;
+    sincosf(red, &sn, &c);
     cs[i] = c;
-    cs[half + i] = s;
+    cs[half + i] = sn;
   }
   __syncthreads();
+  return t;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void layer_prologue_kernel(LP p) {
+  extern __shared__ float cs_all[];  // per wave: cos[K/2], sin[K/2]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* cs = cs_all + wave * p.K;
+  bool live;
+  const int t = token_angles(p, cs, wave, lane, &live);
   if (!live) return;
   const size_t tq = (size_t)t * p.HQ * p.K, tk = (size_t)t * p.H * p.K;
   rope_rows<T, VEC>((const T*)p.q + tq, (T*)p.q_swa + tq, p.q_gsa ? (T*)p.q_gsa + tq : nullptr, p.HQ, p.K, cs, p.fm, lane);
@@ -141,6 +181,100 @@ __global__ __launch_bounds__(256) void layer_prologue_kernel(LP p) {
   }
 }
 
+// d silu(x) / dx and the derivative of the feature map
+__device__ __forceinline__ float silu_grad_f(float x) {
+  const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-x));
+  return sg * (1.f + x * (1.f - sg));
+}
+__device__ __forceinline__ float feature_grad_f(float x, int fm) {
+  return fm == 1 ? silu_grad_f(x) : (fm == 2 ? (x > 0.f ? 1.f : 0.f) : 1.f);
+}
+
+// gradient of rope_rows: the rotation by the opposite angle of the window cotangent plus the
+// feature map's derivative times the slot cotangent
+template <typename T, int VEC>
+__device__ __forceinline__ void rope_rows_bwd(const T* src, const T* dswa, const T* dgsa, T* dx, int heads, int K,
+                                              const float* cs, int fm, int lane) {
+  const int half = K >> 1, per = half / VEC;
+  for (int u = lane; u < heads * per; u += 64) {
+    const int h = u / per, i = (u - h * per) * VEC;
+    const size_t o1 = (size_t)h * K + i, o2 = o1 + half;
+    float d1[VEC], d2[VEC], r1[VEC], r2[VEC];
+    ldv<T, VEC>(dswa + o1, d1);
+    ldv<T, VEC>(dswa + o2, d2);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float c = cs[i + e], sn = cs[half + i + e];
+      r1[e] = d1[e] * c + d2[e] * sn;
+      r2[e] = d2[e] * c - d1[e] * sn;
+    }
+    if (dgsa) {
+      float x1[VEC], x2[VEC];
+      ldv<T, VEC>(src + o1, x1);
+      ldv<T, VEC>(src + o2, x2);
+      ldv<T, VEC>(dgsa + o1, d1);
+      ldv<T, VEC>(dgsa + o2, d2);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        r1[e] += feature_grad_f(x1[e], fm) * d1[e];
+        r2[e] += feature_grad_f(x2[e], fm) * d2[e];
+      }
+    }
+    stv<T, VEC>(dx + o1, r1);
+    stv<T, VEC>(dx + o2, r2);
+  }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void layer_prologue_bwd_kernel(LP p) {
+  extern __shared__ float cs_all[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* cs = cs_all + wave * p.K;
+  bool live;
+  const int t = token_angles(p, cs, wave, lane, &live);
+  if (!live) return;
+  const size_t tq = (size_t)t * p.HQ * p.K, tk = (size_t)t * p.H * p.K;
+  rope_rows_bwd<T, VEC>((const T*)p.q + tq, (const T*)p.dq_swa + tq, p.dq_gsa ? (const T*)p.dq_gsa + tq : nullptr,
+                        (T*)p.dq + tq, p.HQ, p.K, cs, p.fm, lane);
+  rope_rows_bwd<T, VEC>((const T*)p.k + tk, (const T*)p.dk_swa + tk, p.dk_gsa ? (const T*)p.dk_gsa + tk : nullptr,
+                        (T*)p.dk + tk, p.H, p.K, cs, p.fm, lane);
+  {
+    const int n = p.H * p.V;
+    const T* src = (const T*)p.v + (size_t)t * n;
+    const T* dsrc = (const T*)p.dv_out + (size_t)t * n;
+    T* dst = (T*)p.dv + (size_t)t * n;
+    for (int u = lane * VEC; u < n; u += 64 * VEC) {
+      float x[VEC], d[VEC];
+      ldv<T, VEC>(src + u, x);
+      ldv<T, VEC>(dsrc + u, d);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) d[e] *= silu_grad_f(x[e]);
+      stv<T, VEC>(dst + u, d);
+    }
+  }
+  {
+    // g = logsigmoid(f)/n, s = 1 - exp(g):  df = (dg - ds * exp(g)) / n * sigmoid(-f)
+    const int n = p.H * p.M;
+    const T* src = (const T*)p.f + (size_t)t * n;
+    const T* pdg = (const T*)p.dg + (size_t)t * n;
+    const T* pds = (const T*)p.ds + (size_t)t * n;
+    T* dst = (T*)p.df + (size_t)t * n;
+    for (int u = lane * VEC; u < n; u += 64 * VEC) {
+      float x[VEC], dg[VEC], ds[VEC];
+      ldv<T, VEC>(src + u, x);
+      ldv<T, VEC>(pdg + u, dg);
+      ldv<T, VEC>(pds + u, ds);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float ls = rnd<T>(fminf(x[e], 0.f) - log1pf(expf(-fabsf(x[e]))));
+        const float eg = rnd<T>(expf(rnd<T>(ls * p.inv_norm)));
+        dg[e] = (dg[e] - ds[e] * eg) * p.inv_norm / (1.f + expf(x[e]));
+      }
+      stv<T, VEC>(dst + u, dg);
+    }
+  }
+}
+
 struct EP {
   const void* o;
   void* y;
@@ -168,18 +302,33 @@ __global__ __launch_bounds__(256) void layer_epilogue_kernel(EP p) {
       for (int e = 0; e < VEC; ++e) w[n][e] = 1.f;
       if (p.w && u < p.dim) ldv<float, VEC>(p.w + u, w[n]);
     }
+    // the next row's raw elements are in flight while the current row is reduced and written
+    Raw<T, VEC> nxt[NV];
+    const int r0 = row * ROWS_PER_WAVE;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int u = (n * 64 + lane) * VEC;
+      if (u < p.dim) nxt[n].load((const T*)p.o + (size_t)r0 * p.dim + u);
+    }
     for (int rr = 0; rr < ROWS_PER_WAVE; ++rr) {
-      const int r = row * ROWS_PER_WAVE + rr;
+      const int r = r0 + rr;
       if (r >= p.rows) break;
-      src = (const T*)p.o + (size_t)r * p.dim;
       dst = (T*)p.y + (size_t)r * p.dim;
       float a[NV][VEC];
+#pragma unroll
+      for (int n = 0; n < NV; ++n) nxt[n].unpack(a[n]);
+      if (rr + 1 < ROWS_PER_WAVE && r + 1 < p.rows) {
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+          const int u = (n * 64 + lane) * VEC;
+          if (u < p.dim) nxt[n].load((const T*)p.o + (size_t)(r + 1) * p.dim + u);
+        }
+      }
       ss = 0.f;
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         const int u = (n * 64 + lane) * VEC;
         if (u < p.dim) {
-          ldv<T, VEC>(src + u, a[n]);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             a[n][e] = rnd<T>(silu_f(a[n][e]));
@@ -230,6 +379,109 @@ __global__ __launch_bounds__(256) void layer_epilogue_kernel(EP p) {
   }
 }
 
+struct EPB {
+  const void *o, *dy;
+  void* dout;
+  const float* w;
+  float *dw_part, *db_part;
+  int rows, dim;
+  float eps;
+};
+
+// Backward of y = silu(o) * rstd * w + b for BWD_ROWS rows per workgroup.  Thread `tid` owns the
+// columns (n * 256 + tid) * 8 .. + 8, n < NV, of every row, so its share of the weight and bias
+// gradients accumulates in registers and leaves as one row of the partial-sum arrays
+// dw_part / db_part [gridDim.x, dim] (summed over the first axis by the caller: a fixed order).
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void layer_epilogue_bwd_kernel(EPB p) {
+  __shared__ float red[8];
+  const int tid = threadIdx.x;
+  float w[NV][8], dw[NV][8], db[NV][8];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int u = (n * 256 + tid) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[n][e] = 1.f, dw[n][e] = 0.f, db[n][e] = 0.f;
+    if (p.w && u < p.dim) ldv<float, 8>(p.w + u, w[n]);
+  }
+  const int r0 = blockIdx.x * BWD_ROWS;
+  for (int rr = 0; rr < BWD_ROWS; ++rr) {
+    const int r = r0 + rr;
+    if (r >= p.rows) break;  // uniform over the workgroup
+    const T* src = (const T*)p.o + (size_t)r * p.dim;
+    const T* dsrc = (const T*)p.dy + (size_t)r * p.dim;
+    T* dst = (T*)p.dout + (size_t)r * p.dim;
+    float x[NV][8], a[NV][8], d[NV][8];
+    float ss = 0.f, dot = 0.f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int u = (n * 256 + tid) * 8;
+      if (u < p.dim) {
+        ldv<T, 8>(src + u, x[n]);
+        ldv<T, 8>(dsrc + u, d[n]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          a[n][e] = rnd<T>(silu_f(x[n][e]));
+          ss += a[n][e] * a[n][e];
+          dot += d[n][e] * w[n][e] * a[n][e];
+        }
+      }
+    }
+    // both row sums in one pass over the workgroup
+    ss = wave_sum(ss);
+    dot = wave_sum(dot);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = ss, red[4 + (tid >> 6)] = dot;
+    __syncthreads();
+    ss = (red[0] + red[1]) + (red[2] + red[3]);
+    dot = (red[4] + red[5]) + (red[6] + red[7]);
+    const float rstd = rsqrtf(ss / (float)p.dim + p.eps);
+    const float coef = dot * rstd * rstd * rstd / (float)p.dim;  // rstd * mean(dn * n), n = a * rstd
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int u = (n * 256 + tid) * 8;
+      if (u < p.dim) {
+        float g[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          dw[n][e] += d[n][e] * a[n][e] * rstd;
+          db[n][e] += d[n][e];
+          const float da = rstd * d[n][e] * w[n][e] - coef * a[n][e];
+          g[e] = da * silu_grad_f(x[n][e]);
+        }
+        stv<T, 8>(dst + u, g);
+      }
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int u = (n * 256 + tid) * 8;
+    if (u < p.dim) {
+      if (p.dw_part) stv<float, 8>(p.dw_part + (size_t)blockIdx.x * p.dim + u, dw[n]);
+      if (p.db_part) stv<float, 8>(p.db_part + (size_t)blockIdx.x * p.dim + u, db[n]);
+    }
+  }
+}
+
+template <typename T>
+int launch_epilogue_bwd(const EPB& p, hipStream_t st) {
+  const dim3 grid((p.rows + BWD_ROWS - 1) / BWD_ROWS);
+  if (p.dim <= 2048) hipLaunchKernelGGL((layer_epilogue_bwd_kernel<T, 1>), grid, dim3(256), 0, st, p);
+  else if (p.dim <= 4096) hipLaunchKernelGGL((layer_epilogue_bwd_kernel<T, 2>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((layer_epilogue_bwd_kernel<T, 4>), grid, dim3(256), 0, st, p);
+  return 0;
+}
+
+template <typename T>
+int launch_prologue_bwd(const LP& p, hipStream_t st) {
+  const bool vec = (p.K % 16 == 0) && (p.V % 8 == 0) && (p.M % 8 == 0);
+  const size_t lds = (size_t)TOK_PER_WG * p.K * sizeof(float);
+  const dim3 grid((p.T_tot + TOK_PER_WG - 1) / TOK_PER_WG);
+  if (vec) hipLaunchKernelGGL((layer_prologue_bwd_kernel<T, 8>), grid, dim3(256), lds, st, p);
+  else hipLaunchKernelGGL((layer_prologue_bwd_kernel<T, 1>), grid, dim3(256), lds, st, p);
+  return 0;
+}
+
 template <typename T>
 int launch_prologue(const LP& p, hipStream_t st) {
   const bool vec = (p.K % 16 == 0) && (p.V % 8 == 0) && (p.M % 8 == 0);
@@ -254,7 +506,7 @@ int launch_epilogue(const EP& p, hipStream_t st) {
 }  // namespace
 
 int layer_prologue_impl(const NhaLayerPrologueArgs* a) {
-  LP p;
+  LP p = {};
   p.q = a->q; p.k = a->k; p.v = a->v; p.f = a->f;
   p.q_swa = a->q_swa; p.k_swa = a->k_swa;
   p.q_gsa = a->feature_map ? a->q_gsa : nullptr;
@@ -272,6 +524,52 @@ int layer_prologue_impl(const NhaLayerPrologueArgs* a) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("nha_layer_prologue: launch failed: %s", hipGetErrorString(e));
+    return NHA_ERR_LAUNCH;
+  }
+  return NHA_OK;
+}
+
+int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a) {
+  LP p = {};
+  p.q = a->q; p.k = a->k; p.v = a->v; p.f = a->f;
+  p.dq_swa = a->dq_swa; p.dk_swa = a->dk_swa;
+  p.dq_gsa = a->feature_map ? a->dq_gsa : nullptr;
+  p.dk_gsa = a->feature_map ? a->dk_gsa : nullptr;
+  p.dv_out = a->dv_out; p.ds = a->ds; p.dg = a->dg;
+  p.dq = a->dq; p.dk = a->dk; p.dv = a->dv; p.df = a->df;
+  p.inv_freq = a->inv_freq;
+  p.cu = a->cu_seqlens;
+  p.T_tot = a->T_tot; p.N = a->N; p.T = a->T_tot / a->N;
+  p.HQ = a->HQ; p.H = a->H; p.K = a->K; p.V = a->V; p.M = a->M;
+  p.fm = a->feature_map; p.off = a->seqlen_offset;
+  p.inv_norm = 1.f / a->gate_logit_normalizer;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->dtype == NHA_DTYPE_BF16) launch_prologue_bwd<bf16_t>(p, st);
+  else launch_prologue_bwd<float>(p, st);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("nha_layer_prologue_bwd: launch failed: %s", hipGetErrorString(e));
+    return NHA_ERR_LAUNCH;
+  }
+  return NHA_OK;
+}
+
+int layer_epilogue_bwd_parts(int rows) { return (rows + BWD_ROWS - 1) / BWD_ROWS; }
+
+int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a) {
+  if (a->dim % 8 != 0 || a->dim > 8192) {
+    set_error("nha_layer_epilogue_bwd: dim must be a multiple of 8 and <= 8192, got %d", a->dim);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  EPB p;
+  p.o = a->o; p.dy = a->dy; p.dout = a->dout; p.w = a->weight; p.dw_part = a->dweight_partial; p.db_part = a->dbias_partial;
+  p.rows = a->rows; p.dim = a->dim; p.eps = a->eps;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->dtype == NHA_DTYPE_BF16) launch_epilogue_bwd<bf16_t>(p, st);
+  else launch_epilogue_bwd<float>(p, st);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("nha_layer_epilogue_bwd: launch failed: %s", hipGetErrorString(e));
     return NHA_ERR_LAUNCH;
   }
   return NHA_OK;

@@ -9,8 +9,8 @@ The reference takes RMSNorm, RotaryEmbedding, ShortConvolution, the feature maps
 and the unpad helpers from flash-linear-attention, which is not vendored; they are restated here in
 plain PyTorch from their published behaviour (elementwise / projection glue around the hot path).
 The layer is trainable: chunk_nha carries its own backward, the glue around it is plain autograd.
-With autograd off (inference) the elementwise glue on either side of the op runs as two fused HIP
-launches instead (nha_layer_prologue / nha_layer_epilogue); `fuse_glue = False` keeps the tensor-op chain.
+The elementwise glue on either side of the op runs as two fused HIP launches, each with a fused
+backward (nha_layer_prologue / nha_layer_epilogue); `fuse_glue = False` keeps the tensor-op chain.
 """
 from __future__ import annotations
 
@@ -241,12 +241,12 @@ class NativeHybridAttention(nn.Module):
         self._inv_freq = None
 
     def _fused_glue(self, x: torch.Tensor) -> bool:
-        """The fused prologue/epilogue kernels record no autograd graph and cover the swish, relu and
-        identity feature maps in bf16 / fp32 on the GPU."""
-        return (self.fuse_glue and not torch.is_grad_enabled() and x.is_cuda
-                and x.dtype in (torch.bfloat16, torch.float32)
+        """The fused prologue/epilogue kernels (differentiable) cover the swish, relu and identity
+        feature maps in bf16 / fp32 on the GPU, with a value dimension the epilogue's backward takes."""
+        return (self.fuse_glue and x.is_cuda and x.dtype in (torch.bfloat16, torch.float32)
                 and isinstance(self.feature_map, (SwishFeatureMap, ReLUFeatureMap, type(None)))
-                and self.o_proj.weight.dtype == x.dtype and self.head_k_dim % 2 == 0)
+                and self.o_proj.weight.dtype == x.dtype and self.head_k_dim % 2 == 0
+                and self.value_dim % 8 == 0 and self.value_dim <= 8192)
 
     def forward(
         self,

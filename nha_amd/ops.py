@@ -163,59 +163,157 @@ def nha_prefill_bwd(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, do
 _FMAP = {None: _lib.NHA_FMAP_NONE, "none": _lib.NHA_FMAP_NONE, "swish": _lib.NHA_FMAP_SWISH, "relu": _lib.NHA_FMAP_RELU}
 
 
+def _prologue_dims(q, k, v, f, inv_freq, cu):
+    B, T, HQ, K = q.shape
+    H, V, M = k.shape[2], v.shape[3], f.shape[3]
+    if cu is not None and B != 1:
+        raise ValueError("cu_seqlens needs the packed layout [1, T_tot, ...]")
+    for x in (k, v, f):
+        if x.dtype != q.dtype:
+            raise TypeError("q, k, v, f must share one dtype")
+    if inv_freq.numel() != K // 2:
+        raise ValueError(f"inv_freq must hold K/2 = {K // 2} entries, got {inv_freq.numel()}")
+    return dict(T_tot=B * T, N=(cu.numel() - 1) if cu is not None else B, HQ=HQ, H=H, K=K, V=V, M=M)
+
+
+def _prologue_fwd(q, k, v, f, inv_freq, fm: int, normalizer: float, offset: int, cu):
+    lib = _lib.load()
+    dims = _prologue_dims(q, k, v, f, inv_freq, cu)
+    q_swa, k_swa, v_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    s, g = torch.empty_like(f), torch.empty_like(f)
+    q_gsa = torch.empty_like(q) if fm else None
+    k_gsa = torch.empty_like(k) if fm else None
+    a = _lib.NhaLayerPrologueArgs(
+        q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), q_swa=_ptr(q_swa), k_swa=_ptr(k_swa), q_gsa=_ptr(q_gsa),
+        k_gsa=_ptr(k_gsa), v_out=_ptr(v_out), s=_ptr(s), g=_ptr(g), inv_freq=_ptr(inv_freq), cu_seqlens=_ptr(cu),
+        feature_map=fm, seqlen_offset=int(offset), dtype=_dtype_code(q), gate_logit_normalizer=float(normalizer),
+        stream=_stream(q.device), **dims)
+    _lib.check(lib.nha_layer_prologue(C.byref(a)))
+    return q_swa, k_swa, q_gsa, k_gsa, v_out, s, g
+
+
+def _prologue_bwd(q, k, v, f, inv_freq, fm: int, normalizer: float, offset: int, cu, dq_swa, dk_swa, dq_gsa, dk_gsa,
+                  dv_out, ds, dg):
+    lib = _lib.load()
+    dims = _prologue_dims(q, k, v, f, inv_freq, cu)
+    dq, dk, dv, df = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(f)
+    a = _lib.NhaLayerPrologueBwdArgs(
+        q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), dq_swa=_ptr(dq_swa), dk_swa=_ptr(dk_swa), dq_gsa=_ptr(dq_gsa),
+        dk_gsa=_ptr(dk_gsa), dv_out=_ptr(dv_out), ds=_ptr(ds), dg=_ptr(dg), dq=_ptr(dq), dk=_ptr(dk), dv=_ptr(dv),
+        df=_ptr(df), inv_freq=_ptr(inv_freq), cu_seqlens=_ptr(cu), feature_map=fm, seqlen_offset=int(offset),
+        dtype=_dtype_code(q), gate_logit_normalizer=float(normalizer), stream=_stream(q.device), **dims)
+    _lib.check(lib.nha_layer_prologue_bwd(C.byref(a)))
+    return dq, dk, dv, df
+
+
+class _LayerPrologueFunction(torch.autograd.Function):
+    """Autograd node of the fused prologue: both directions are one HIP launch."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, f, inv_freq, fm, normalizer, offset, cu):
+        outs = _prologue_fwd(q, k, v, f, inv_freq, fm, normalizer, offset, cu)
+        ctx.save_for_backward(q, k, v, f, inv_freq)
+        ctx.cu, ctx.meta = cu, (fm, normalizer, offset)
+        return outs if fm else (outs[0], outs[1], outs[4], outs[5], outs[6])
+
+    @staticmethod
+    def backward(ctx, *grads):
+        q, k, v, f, inv_freq = ctx.saved_tensors
+        fm, normalizer, offset = ctx.meta
+        shapes = (q, k, q, k, v, f, f) if fm else (q, k, v, f, f)
+        grads = [torch.zeros_like(x) if gr is None else gr.contiguous() for gr, x in zip(grads, shapes)]
+        if fm:
+            dq_swa, dk_swa, dq_gsa, dk_gsa, dv_out, ds, dg = grads
+        else:
+            (dq_swa, dk_swa, dv_out, ds, dg), dq_gsa, dk_gsa = grads, None, None
+        dq, dk, dv, df = _prologue_bwd(q, k, v, f, inv_freq, fm, normalizer, offset, ctx.cu, dq_swa, dk_swa, dq_gsa,
+                                       dk_gsa, dv_out, ds, dg)
+        return dq, dk, dv, df, None, None, None, None, None
+
+
 def nha_layer_prologue(q, k, v, f, inv_freq, *, feature_map: Optional[str], gate_logit_normalizer: float,
                        seqlen_offset: int = 0, cu_seqlens: Optional[torch.Tensor] = None):
     """One launch for the elementwise chain of nha_fla/layers/nha.py:214-237 on the raw projections
     q [B,T,HQ,K], k [B,T,H,K], v [B,T,H,V], f [B,T,H,M] (B = 1 with cu_seqlens, an int32 device
     tensor).  Returns (q_swa, k_swa, q_gsa, k_gsa, v, s, g); without a feature map q_gsa / k_gsa
-    are q / k themselves.  Inference only: no autograd graph is recorded."""
-    lib = _lib.load()
+    are q / k themselves.  Differentiable with respect to q, k, v, f (one launch backward too)."""
     _need_cuda(q, k, v, f, inv_freq, cu_seqlens)
     if feature_map not in _FMAP:
         raise NotImplementedError(f"Feature map `{feature_map}` has no fused prologue.")
-    B, T, HQ, K = q.shape
-    H, V, M = k.shape[2], v.shape[3], f.shape[3]
-    if cu_seqlens is not None and B != 1:
-        raise ValueError("cu_seqlens needs the packed layout [1, T_tot, ...]")
-    dt = _dtype_code(q)
+    _dtype_code(q)
     q, k, v, f = (x.contiguous() for x in (q, k, v, f))
-    for x in (k, v, f):
-        if x.dtype != q.dtype:
-            raise TypeError("q, k, v, f must share one dtype")
-    inv_freq = inv_freq.to(torch.float32).contiguous()
-    if inv_freq.numel() != K // 2:
-        raise ValueError(f"inv_freq must hold K/2 = {K // 2} entries, got {inv_freq.numel()}")
+    inv_freq = inv_freq.detach().to(torch.float32).contiguous()
     fm = _FMAP[feature_map]
-    q_swa, k_swa, v_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    s, g = torch.empty_like(f), torch.empty_like(f)
-    q_gsa = torch.empty_like(q) if fm else None
-    k_gsa = torch.empty_like(k) if fm else None
     cu = None if cu_seqlens is None else cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()
-    a = _lib.NhaLayerPrologueArgs(
-        q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), q_swa=_ptr(q_swa), k_swa=_ptr(k_swa), q_gsa=_ptr(q_gsa),
-        k_gsa=_ptr(k_gsa), v_out=_ptr(v_out), s=_ptr(s), g=_ptr(g), inv_freq=_ptr(inv_freq), cu_seqlens=_ptr(cu),
-        T_tot=B * T, N=(cu.numel() - 1) if cu is not None else B, HQ=HQ, H=H, K=K, V=V, M=M, feature_map=fm,
-        seqlen_offset=int(seqlen_offset), dtype=dt, gate_logit_normalizer=float(gate_logit_normalizer),
-        stream=_stream(q.device))
-    _lib.check(lib.nha_layer_prologue(C.byref(a)))
+    args = (q, k, v, f, inv_freq, fm, float(gate_logit_normalizer), int(seqlen_offset), cu)
+    if torch.is_grad_enabled() and any(x.requires_grad for x in (q, k, v, f)):
+        outs = _LayerPrologueFunction.apply(*args)
+        if fm:
+            return outs
+        return outs[0], outs[1], q, k, outs[2], outs[3], outs[4]
+    q_swa, k_swa, q_gsa, k_gsa, v_out, s, g = _prologue_fwd(*args)
     return q_swa, k_swa, (q_gsa if fm else q), (k_gsa if fm else k), v_out, s, g
+
+
+def _epilogue_fwd(o, w, b, eps: float):
+    lib = _lib.load()
+    dim = o.shape[-1]
+    y = torch.empty_like(o)
+    a = _lib.NhaLayerEpilogueArgs(o=_ptr(o), y=_ptr(y), weight=_ptr(w), bias=_ptr(b), rows=o.numel() // dim, dim=dim,
+                                  dtype=_dtype_code(o), eps=float(eps), stream=_stream(o.device))
+    _lib.check(lib.nha_layer_epilogue(C.byref(a)))
+    return y
+
+
+class _LayerEpilogueFunction(torch.autograd.Function):
+    """Autograd node of the fused epilogue; the weight / bias gradients are reduced from the
+    kernel's per-workgroup partial sums in a fixed order."""
+
+    @staticmethod
+    def forward(ctx, o, weight, bias, eps):
+        w = None if weight is None else weight.detach().to(torch.float32).contiguous()
+        b = None if bias is None else bias.detach().to(torch.float32).contiguous()
+        ctx.save_for_backward(o, w)
+        ctx.eps = eps
+        ctx.wb = (None if weight is None else weight.dtype, None if bias is None else bias.dtype)
+        return _epilogue_fwd(o, w, b, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        o, w = ctx.saved_tensors
+        dy = dy.contiguous()
+        dim = o.shape[-1]
+        rows = o.numel() // dim
+        parts = lib.nha_layer_epilogue_bwd_parts(rows)
+        wdt, bdt = ctx.wb
+        need_w = wdt is not None and ctx.needs_input_grad[1]
+        need_b = bdt is not None and ctx.needs_input_grad[2]
+        dwp = torch.empty(parts, dim, dtype=torch.float32, device=o.device) if need_w else None
+        dbp = torch.empty(parts, dim, dtype=torch.float32, device=o.device) if need_b else None
+        do = torch.empty_like(o)
+        a = _lib.NhaLayerEpilogueBwdArgs(o=_ptr(o), dy=_ptr(dy), dout=_ptr(do), weight=_ptr(w), dweight_partial=_ptr(dwp),
+                                         dbias_partial=_ptr(dbp), rows=rows, dim=dim, dtype=_dtype_code(o),
+                                         eps=float(ctx.eps), stream=_stream(o.device))
+        _lib.check(lib.nha_layer_epilogue_bwd(C.byref(a)))
+        return (do, dwp.sum(0).to(wdt) if need_w else None, dbp.sum(0).to(bdt) if need_b else None, None)
 
 
 def nha_layer_epilogue(o, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float):
     """rms_norm(silu(o)) * weight (+ bias) over the last dimension in one launch: the normalisation
-    half of nha_fla/layers/nha.py:278.  Inference only."""
-    lib = _lib.load()
+    half of nha_fla/layers/nha.py:278.  Differentiable with respect to o, weight and bias (last
+    dimension a multiple of 8 and at most 8192 for the backward)."""
     _need_cuda(o, weight, bias)
-    dt = _dtype_code(o)
+    _dtype_code(o)
     o = o.contiguous()
-    dim = o.shape[-1]
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (o, weight, bias)):
+        dim = o.shape[-1]
+        if dim % 8 or dim > 8192:
+            raise NotImplementedError(f"nha_layer_epilogue backward needs a last dimension % 8 == 0 and <= 8192, got {dim}")
+        return _LayerEpilogueFunction.apply(o, weight, bias, float(eps))
     w = None if weight is None else weight.detach().to(torch.float32).contiguous()
     b = None if bias is None else bias.detach().to(torch.float32).contiguous()
-    y = torch.empty_like(o)
-    a = _lib.NhaLayerEpilogueArgs(o=_ptr(o), y=_ptr(y), weight=_ptr(w), bias=_ptr(b), rows=o.numel() // dim, dim=dim,
-                                  dtype=dt, eps=float(eps), stream=_stream(o.device))
-    _lib.check(lib.nha_layer_epilogue(C.byref(a)))
-    return y
+    return _epilogue_fwd(o, w, b, float(eps))
 
 
 class _ChunkNHAFunction(torch.autograd.Function):

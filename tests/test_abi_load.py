@@ -36,9 +36,14 @@ def test_struct_sizes_match_the_header(tmp_path):
     probes += [("NhaLayerPrologueArgs", f) for f in ("q", "q_swa", "g", "inv_freq", "cu_seqlens", "T_tot", "M", "feature_map",
                                                      "seqlen_offset", "dtype", "gate_logit_normalizer", "stream")]
     probes += [("NhaLayerEpilogueArgs", f) for f in ("o", "y", "weight", "bias", "rows", "dim", "dtype", "eps", "stream")]
+    probes += [("NhaLayerPrologueBwdArgs", f) for f in ("q", "dq_swa", "dg", "dq", "df", "inv_freq", "cu_seqlens", "T_tot",
+                                                        "feature_map", "dtype", "gate_logit_normalizer", "stream")]
+    probes += [("NhaLayerEpilogueBwdArgs", f) for f in ("o", "dy", "dout", "weight", "dweight_partial", "dbias_partial",
+                                                        "rows", "dim", "dtype", "eps", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
            'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));',
-           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueArgs), sizeof(NhaLayerEpilogueArgs));']
+           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueArgs), sizeof(NhaLayerEpilogueArgs));',
+           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueBwdArgs), sizeof(NhaLayerEpilogueBwdArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
     src += ['return 0; }']
     cfile = tmp_path / "probe.c"
@@ -49,7 +54,8 @@ def test_struct_sizes_match_the_header(tmp_path):
     assert int(out[0]) == C.sizeof(_lib.NhaPrefillArgs) and int(out[1]) == C.sizeof(_lib.NhaDecodeArgs)
     assert int(out[2]) == C.sizeof(_lib.NhaPrefillBwdArgs)
     assert int(out[3]) == C.sizeof(_lib.NhaLayerPrologueArgs) and int(out[4]) == C.sizeof(_lib.NhaLayerEpilogueArgs)
-    for (t, f), off in zip(probes, out[5:]):
+    assert int(out[5]) == C.sizeof(_lib.NhaLayerPrologueBwdArgs) and int(out[6]) == C.sizeof(_lib.NhaLayerEpilogueBwdArgs)
+    for (t, f), off in zip(probes, out[7:]):
         assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 
@@ -83,6 +89,12 @@ def test_argument_validation_without_gpu():
     assert lib.nha_layer_epilogue(C.byref(le)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
     le.rows, le.dim = 4, 64
     assert lib.nha_layer_epilogue(C.byref(le)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    lpb = _lib.NhaLayerPrologueBwdArgs()
+    assert lib.nha_layer_prologue_bwd(C.byref(lpb)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
+    leb = _lib.NhaLayerEpilogueBwdArgs()
+    leb.rows, leb.dim = 4, 64
+    assert lib.nha_layer_epilogue_bwd(C.byref(leb)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    assert lib.nha_layer_epilogue_bwd_parts(0) == 0 and lib.nha_layer_epilogue_bwd_parts(33) == 2
     with pytest.raises(_lib.NhaError):
         chunk_tables([0, 5, 5])          # zero-length sequence
     with pytest.raises(_lib.NhaError):
