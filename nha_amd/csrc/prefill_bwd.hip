@@ -94,11 +94,21 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
   float* Aj = dov + V;        // [BT] q_gsa . k'_j
   float* Bj = Aj + BT;        // [BT] do . v'_j
   float* gct = Bj + BT;       // [M]
-  const int chunk = blockIdx.x / (BT / 4), r = (blockIdx.x % (BT / 4)) * 4 + wv;
-  const int hq = blockIdx.y, h = hq / NG;
+  // Two launch shapes.  Alone (no flags): grid (NT * 16, HQ), one wave per (token, q-head).  Behind
+  // the matrix-core kernel: grid (NT, H), a workgroup leaves at once unless its (chunk, kv-head) is
+  // flagged and otherwise walks the chunk's 64 * NG (token, q-head) pairs, four at a time.
+  const bool looped = p.big != nullptr;
+  const int chunk = looped ? blockIdx.x : blockIdx.x / (BT / 4);
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
-  if (p.big && !p.big[(int64_t)chunk * H + h]) return;   // the matrix-core kernel has done this chunk
+  if (looped && !p.big[(int64_t)chunk * H + blockIdx.y]) return;   // the matrix-core kernel has done this chunk
+  const int nit = looped ? BT * NG / 4 : 1;
+  for (int itx = 0; itx < nit; ++itx) {
+  if (itx) __syncthreads();   // the previous pair's vectors in LDS are no longer read
+  const int item = 4 * itx + wv;
+  const int r = looped ? item % BT : (blockIdx.x % (BT / 4)) * 4 + wv;
+  const int hq = looped ? blockIdx.y * NG + item / BT : blockIdx.y;
+  const int h = hq / NG;
   const bool valid = bos + it * BT + r < eos;   // waves past the end compute on row 0 and write nothing
   const int rr = valid ? r : 0;
   const int t = bos + it * BT + rr;
@@ -169,6 +179,7 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     }
   }
   if (lane == 0 && valid) p.delta[tq] = delta;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -534,12 +545,31 @@ __global__ __launch_bounds__(256) void bwd_state_scan_kernel(const BP p) {
   const float* dht = isv ? p.dhvt : p.dhkt;
   float E = 0.f;
   if (dht) E = isv ? dht[(((int64_t)n * H + h) * M + m) * X + x] : dht[(((int64_t)n * H + h) * X + x) * M + m];
-  for (int it = nchunks - 1; it >= 0; --it) {
+  // the recurrence is sequential, its operands are not: four chunks' loads are in flight together
+  const int64_t cstride = (int64_t)H * X * M;
+  float* ebn = eb + (((int64_t)p.coff[n] * H + h) * X + x) * M + m;
+  auto gl_of = [&](int it) {
     const int R = (L - it * BT) < BT ? (L - it * BT) : BT;
-    const int64_t idx = (((int64_t)(p.coff[n] + it) * H + h) * X + x) * M + m;
-    const float nc = eb[idx];
-    eb[idx] = E;
-    E = E * expf(p.gc[((int64_t)(bos + it * BT + R - 1) * H + h) * M + m]) + nc;
+    return p.gc[((int64_t)(bos + it * BT + R - 1) * H + h) * M + m];
+  };
+  int it = nchunks - 1;
+  for (; it >= 3; it -= 4) {
+    float nc[4], gl[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      nc[u] = ebn[(it - u) * cstride];
+      gl[u] = gl_of(it - u);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      ebn[(it - u) * cstride] = E;
+      E = E * expf(gl[u]) + nc[u];
+    }
+  }
+  for (; it >= 0; --it) {
+    const float nc = ebn[it * cstride];
+    ebn[it * cstride] = E;
+    E = E * expf(gl_of(it)) + nc;
   }
   float* dh0 = isv ? p.dh0v : p.dh0k;
   if (dh0) {
@@ -655,35 +685,59 @@ __global__ __launch_bounds__(256) void bwd_state_inter_kernel(const BP p) {
 // per chunk the summand, ds and the chunk-local sums (bwd_gate_local_kernel), per sequence the
 // sums of all later chunks plus the end term (bwd_gate_scan_kernel), per chunk the final values
 // (bwd_gate_final_kernel, which also zeroes the gradients of the tokens that never reach the
-// slots: the last `shift` of a sequence).  One thread per slot.
+// slots: the last `shift` of a sequence).
 // ------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void bwd_gate_local_kernel(const BP p) {
+__global__ __launch_bounds__(256) void bwd_gate_local_kernel(const BP p) {
+  // thread = (row group g of 16 rows, slot m): the 16 rows' loads are independent and issued
+  // together; the reverse cumulative sum is a suffix sum in registers plus the sums of the later
+  // groups through LDS
+  __shared__ float gs[4][BT];
   const int M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
   const int chunk = blockIdx.x, h = blockIdx.y;
-  const int m = threadIdx.x;
-  if (m >= M) return;
+  const int m = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   const int nslab = p.nbk + p.nbv;
-  float run = 0.f;
-  for (int r = R - 1; r >= 0; --r) {
-    const int t = c0 + r, sj = t - p.shift;
-    if (sj < bos) break;
-    const int64_t rt = ((int64_t)t * H + h) * M + m;
-    float dstot = p.dsi[rt];
-    for (int b = 0; b < nslab; ++b) dstot += p.dsp[(int64_t)b * p.T_tot * H * M + rt];
-    float x = 0.f;
-    for (int a = 0; a < NG; ++a) x += p.xg[((int64_t)t * HQ + h * NG + a) * M + m];
-    const float sval = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m);
-    run += x - sval * dstot;
-    Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m, dstot);
-    p.dsi[rt] = run;   // chunk-local reverse cumulative sum
+  float z[16], dst[16];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int r = 16 * g + q, t = c0 + r, sj = t - p.shift;
+    z[q] = dst[q] = 0.f;
+    if (m < M && r < R && sj >= bos) {
+      const int64_t rt = ((int64_t)t * H + h) * M + m;
+      float dstot = p.dsi[rt];
+      for (int b = 0; b < nslab; ++b) dstot += p.dsp[(int64_t)b * p.T_tot * H * M + rt];
+      float x = 0.f;
+      for (int a = 0; a < NG; ++a) x += p.xg[((int64_t)t * HQ + h * NG + a) * M + m];
+      const float sval = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m);
+      z[q] = x - sval * dstot;
+      dst[q] = dstot;
+    }
   }
-  p.gtot[((int64_t)chunk * H + h) * M + m] = run;
+  float run = 0.f;
+#pragma unroll
+  for (int q = 15; q >= 0; --q) {
+    run += z[q];
+    z[q] = run;   // suffix sum inside the group
+  }
+  gs[g][m] = run;
+  __syncthreads();
+  float later = 0.f;
+  for (int g2 = 3; g2 > g; --g2) later += gs[g2][m];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int r = 16 * g + q, t = c0 + r, sj = t - p.shift;
+    if (m < M && r < R && sj >= bos) {
+      const int64_t rt = ((int64_t)t * H + h) * M + m;
+      Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m, dst[q]);
+      p.dsi[rt] = z[q] + later;   // chunk-local reverse cumulative sum
+    }
+  }
+  if (g == 0 && m < M) p.gtot[((int64_t)chunk * H + h) * M + m] = run + later;
 }
 
 template <typename T>
@@ -971,7 +1025,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     rc = bwd_slot_products3(a, 0, p.big, p.ap, p.bp, p.ust, p.dpst, p.gc, p.delta, p.dus, p.pp, p.xg, p.ck, p.cv, p.dsi);
     if (rc != NHA_OK) return rc;
   }
-  hipLaunchKernelGGL((bwd_q_kernel<T>), dim3(a->NT * (BT / 4), a->HQ), dim3(256), lds_q, st, p);
+  hipLaunchKernelGGL((bwd_q_kernel<T>), p.big ? dim3(a->NT, a->H) : dim3(a->NT * (BT / 4), a->HQ), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
   if (wmfma) {
     rc = bwd_window_mfma_dq(a, p.delta);
@@ -1010,7 +1064,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     hipLaunchKernelGGL((bwd_state_inter_kernel<T>), dim3(a->NT, a->H * nbmax, 2), dim3(256), lds_s3, st, p);
   }
   NHA_CHECK_LAUNCH("nha_prefill_bwd(state gradients)");
-  hipLaunchKernelGGL((bwd_gate_local_kernel<T>), dim3(a->NT, a->H), dim3(64), 0, st, p);
+  hipLaunchKernelGGL((bwd_gate_local_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_final_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(gate scan)");

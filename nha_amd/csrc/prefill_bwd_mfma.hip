@@ -519,6 +519,19 @@ __device__ __forceinline__ void split_bf16(float x, lbf16* hi, lbf16* lo, int id
   lo[idx] = f32_to_bf16(x - bf16_to_f32(h));
 }
 
+// four consecutive elements at once: two 8-byte LDS writes (idx a multiple of 4)
+__device__ __forceinline__ void split4_bf16(const float4 x, lbf16* hi, lbf16* lo, int idx) {
+  const float v[4] = {x.x, x.y, x.z, x.w};
+  bf16x4 h, l;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    h[e] = (__bf16)v[e];
+    l[e] = (__bf16)(v[e] - (float)h[e]);
+  }
+  *reinterpret_cast<NHA_LDS bf16x4*>(hi + idx) = h;
+  *reinterpret_cast<NHA_LDS bf16x4*>(lo + idx) = l;
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
@@ -556,15 +569,32 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
       rx.store(Xt, tid);
     }
     const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
-    for (int e = tid; e < BT * BT; e += 256) {
-      const int i = e >> 6, c = e & 63;   // coalesced reads over c, transposed writes
-      float w = 0.f, cc = 0.f;
-      if (i < R) {
-        w = wsrc[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
-        if (c <= i) cc = cp[i * BT + c];
+    {
+      // coalesced 16-byte reads over c (all issued before the first use), transposed writes
+      constexpr int NS = BT * BT / 4 / 256;
+      float4 wv[NS], gv[NS], cv[NS];
+#pragma unroll
+      for (int u = 0; u < NS; ++u) {
+        const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+        wv[u] = gv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < R) {
+          wv[u] = *reinterpret_cast<const float4*>(wsrc + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+          gv[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+          if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
+        }
       }
-      split_bf16(w, Wt, Wl, c * TLD + i);
-      split_bf16(cc, Ct, Cl, c * TLD + i);
+#pragma unroll
+      for (int u = 0; u < NS; ++u) {
+        const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+        const float w4[4] = {wv[u].x * __expf(gv[u].x), wv[u].y * __expf(gv[u].y), wv[u].z * __expf(gv[u].z),
+                             wv[u].w * __expf(gv[u].w)};
+        const float c4[4] = {cv[u].x, cv[u].y, cv[u].z, cv[u].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          split_bf16(i < R ? w4[q] : 0.f, Wt, Wl, (c + q) * TLD + i);
+          split_bf16(c + q <= i ? c4[q] : 0.f, Ct, Cl, (c + q) * TLD + i);
+        }
+      }
     }
     lds_barrier();
 #pragma unroll
@@ -628,15 +658,34 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
     rk.store(Kt, tid);
   }
   const float* cp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
-  for (int e = tid; e < BT * BT; e += 256) {
-    const int i = e >> 6, c = e & 63;
-    float w = 0.f, cc = 0.f;
-    if (i < R) {
-      w = p.dus[((int64_t)(c0 + i) * HQ + hq) * BT + c] * __expf(p.gc[((int64_t)(c0 + i) * H + h) * BT + c]);
-      if (c <= i) cc = cp[i * BT + c];
+  {
+    constexpr int NS = BT * BT / 4 / 256;
+    float4 wv[NS], gv[NS], cv[NS];
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+      wv[u] = gv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < R) {
+        wv[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+        gv[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+        if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
+      }
     }
-    split_bf16(w, Wt, Wl, i * TLD + c);
-    split_bf16(cc, Ct, Cl, i * TLD + c);
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+      float4 w, cc;
+      w.x = i < R ? wv[u].x * __expf(gv[u].x) : 0.f;
+      w.y = i < R ? wv[u].y * __expf(gv[u].y) : 0.f;
+      w.z = i < R ? wv[u].z * __expf(gv[u].z) : 0.f;
+      w.w = i < R ? wv[u].w * __expf(gv[u].w) : 0.f;
+      cc.x = c <= i ? cv[u].x : 0.f;
+      cc.y = c + 1 <= i ? cv[u].y : 0.f;
+      cc.z = c + 2 <= i ? cv[u].z : 0.f;
+      cc.w = c + 3 <= i ? cv[u].w : 0.f;
+      split4_bf16(w, Wt, Wl, i * TLD + c);
+      split4_bf16(cc, Ct, Cl, i * TLD + c);
+    }
   }
   lds_barrier();
   const int i = 16 * wave + l16;   // this lane's row of the chunk
@@ -706,15 +755,48 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
     ry.store(Yt, tid);
   }
   const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
-  for (int e = tid; e < D * BT; e += 256) split_bf16(ep[e], Et, El, (e >> 6) * ELD + (e & 63));
   const float* gcb = p.gc + ((int64_t)c0 * H + h) * BT;
-  for (int e = tid; e < BT * BT; e += 256) {
-    const int r = e >> 6, m = e & 63;
-    float v = 0.f;
-    if (r >= vlo && r < R)
-      v = bf16_to_f32(p.s[(((int64_t)c0 + r - p.shift) * H + h) * BT + m]) *
-          __expf(gcb[(int64_t)(R - 1) * H * BT + m] - gcb[(int64_t)r * H * BT + m]);
-    split_bf16(v, St, Sl, r * TLD + m);
+  {
+    // all global loads of a batch are issued before the first conversion waits for one
+    constexpr int NE = D * BT / 4 / 256, EB = NE < 8 ? NE : 8;
+    const float4* ep4 = reinterpret_cast<const float4*>(ep);
+#pragma unroll
+    for (int b0 = 0; b0 < NE; b0 += EB) {
+      float4 buf[EB];
+#pragma unroll
+      for (int u = 0; u < EB; ++u) buf[u] = ep4[tid + 256 * (b0 + u)];
+#pragma unroll
+      for (int u = 0; u < EB; ++u) {
+        const int e = 4 * (tid + 256 * (b0 + u));
+        split4_bf16(buf[u], Et, El, (e >> 6) * ELD + (e & 63));
+      }
+    }
+    constexpr int NS = BT * BT / 4 / 256;
+    float4 gl[NS], gr[NS];
+    uint2 sr[NS];
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), r = e >> 6, m = e & 63;
+      gl[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      sr[u] = make_uint2(0, 0);
+      if (r >= vlo && r < R) {
+        sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + r - p.shift) * H + h) * BT + m);
+        gl[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)(R - 1) * H * BT + m);
+        gr[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)r * H * BT + m);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), r = e >> 6, m = e & 63;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (r >= vlo && r < R) {
+        v.x = __uint_as_float(sr[u].x << 16) * __expf(gl[u].x - gr[u].x);
+        v.y = __uint_as_float(sr[u].x & 0xffff0000u) * __expf(gl[u].y - gr[u].y);
+        v.z = __uint_as_float(sr[u].y << 16) * __expf(gl[u].z - gr[u].z);
+        v.w = __uint_as_float(sr[u].y & 0xffff0000u) * __expf(gl[u].w - gr[u].w);
+      }
+      split4_bf16(v, St, Sl, r * TLD + m);
+    }
   }
   lds_barrier();
   const int col = 16 * wave + l16;
@@ -815,12 +897,32 @@ __device__ __forceinline__ float ref_of(const SP3& p, int c0, int h, int r, int 
 // a telescoping sum), so they are bf16 pairs (split_bf16) and their products hi*hi + hi*lo + lo*hi.
 // rows of Y = s_j[m] e^(ref - gc_j[m]) (zero for rows without a source token)
 __device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int c0, int h, int R, int vlo, int tid) {
-  for (int e = tid; e < BT * BT; e += 256) {
-    const int j = e >> 6, m = e & 63;
-    float v = 0.f;
-    if (j >= vlo && j < R)
-      v = bf16_to_f32(p.s[(((int64_t)c0 + j - p.shift) * p.H + h) * BT + m]) * __expf(ref_of(p, c0, h, j, m) - gc_at(p, c0, h, j, m));
-    split_bf16(v, Yh, Yl, j * TLD + m);
+  // 16-byte reads, all issued before the first conversion waits for one
+  constexpr int NS = BT * BT / 4 / 256;
+  float4 gj[NS], gr[NS];
+  uint2 sr[NS];
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
+    gj[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    sr[u] = make_uint2(0, 0);
+    if (j >= vlo && j < R) {
+      sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + j - p.shift) * p.H + h) * BT + m);
+      gj[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + j) * p.H + h) * BT + m);
+      if (j >= 32) gr[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * p.H + h) * BT + m);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (j >= vlo && j < R) {
+      v.x = __uint_as_float(sr[u].x << 16) * __expf(gr[u].x - gj[u].x);
+      v.y = __uint_as_float(sr[u].x & 0xffff0000u) * __expf(gr[u].y - gj[u].y);
+      v.z = __uint_as_float(sr[u].y << 16) * __expf(gr[u].z - gj[u].z);
+      v.w = __uint_as_float(sr[u].y & 0xffff0000u) * __expf(gr[u].w - gj[u].w);
+    }
+    split4_bf16(v, Yh, Yl, j * TLD + m);
   }
 }
 
@@ -843,11 +945,32 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
   vlo = vlo < 0 ? 0 : vlo;
   const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
   const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
-  for (int e = tid; e < BT * BT; e += 256) {
-    const int i = e >> 6, j = e & 63;
-    const bool in = j <= i && i < R;
-    At[i * TLD + j] = f32_to_bf16(in ? ap[e] : 0.f);
-    Bt[i * TLD + j] = f32_to_bf16(in ? bp[e] : 0.f);
+  {
+    constexpr int NS = BT * BT / 4 / 256;
+    float4 av[NS], bv[NS];
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, j = e & 63;
+      av[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j <= i && i < R) {
+        av[u] = *reinterpret_cast<const float4*>(ap + e);
+        bv[u] = *reinterpret_cast<const float4*>(bp + e);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, j = e & 63;
+      const float a4[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, b4[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
+      bf16x4 pa, pb;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bool in = j + q <= i && i < R;
+        pa[q] = (__bf16)(in ? a4[q] : 0.f);
+        pb[q] = (__bf16)(in ? b4[q] : 0.f);
+      }
+      *reinterpret_cast<NHA_LDS bf16x4*>(At + i * TLD + j) = pa;
+      *reinterpret_cast<NHA_LDS bf16x4*>(Bt + i * TLD + j) = pb;
+    }
   }
   stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
   lds_barrier();
@@ -923,32 +1046,49 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
     if (a > 0) lds_barrier();
     const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
     const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
-    for (int e = tid; e < BT * BT; e += 256) {
-      const int i = e >> 6, c = e & 63;
-      float x0 = 0.f, x1 = 0.f, p0 = 0.f, p1 = 0.f, av = 0.f, bv = 0.f;
-      if (i < R) {
-        const float gi = gc_at(p, c0, h, i, c);
-        const float du = p.dus[((int64_t)(c0 + i) * HQ + hq) * BT + c];
-        const float pv = p.pp[((int64_t)(c0 + i) * HQ + hq) * BT + c];
-        const float e0 = __expf(gi);
-        x0 = du * e0;
-        p0 = pv * e0;
-        if (i >= 32) {
-          const float e1 = __expf(gi - gc_at(p, c0, h, 31, c));
-          x1 = du * e1;
-          p1 = pv * e1;
-        }
-        if (c <= i) {
-          av = ap[e];
-          bv = bp[e];
+#pragma unroll
+    for (int u0 = 0; u0 < BT * BT / 4 / 256; u0 += 2) {
+      // two 4-element groups per thread at a time: their twelve 16-byte reads are in flight together
+      float4 gi[2], g31[2], du[2], pv[2], av[2], bv[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
+        gi[u] = g31[u] = du[u] = pv[u] = av[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < R) {
+          gi[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+          du[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+          pv[u] = *reinterpret_cast<const float4*>(p.pp + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+          if (i >= 32) g31[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
+          if (c <= i) {
+            av[u] = *reinterpret_cast<const float4*>(ap + e);
+            bv[u] = *reinterpret_cast<const float4*>(bp + e);
+          }
         }
       }
-      split_bf16(x0, X0h, X0l, i * TLD + c);
-      split_bf16(x1, X1h, X1l, i * TLD + c);
-      split_bf16(p0, P0h, P0l, i * TLD + c);
-      split_bf16(p1, P1h, P1l, i * TLD + c);
-      AT[c * TLD + i] = f32_to_bf16(av);
-      BT_[c * TLD + i] = f32_to_bf16(bv);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
+        const float g4[4] = {gi[u].x, gi[u].y, gi[u].z, gi[u].w}, r4[4] = {g31[u].x, g31[u].y, g31[u].z, g31[u].w};
+        const float d4[4] = {du[u].x, du[u].y, du[u].z, du[u].w}, q4[4] = {pv[u].x, pv[u].y, pv[u].z, pv[u].w};
+        const float a4[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, b4[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
+        float x0[4], x1[4], p0[4], p1[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float e0 = i < R ? __expf(g4[q]) : 0.f;
+          const float e1 = (i < R && i >= 32) ? __expf(g4[q] - r4[q]) : 0.f;
+          x0[q] = d4[q] * e0;
+          p0[q] = q4[q] * e0;
+          x1[q] = d4[q] * e1;
+          p1[q] = q4[q] * e1;
+          const bool in = i < R && c + q <= i;
+          AT[(c + q) * TLD + i] = f32_to_bf16(in ? a4[q] : 0.f);
+          BT_[(c + q) * TLD + i] = f32_to_bf16(in ? b4[q] : 0.f);
+        }
+        split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
+        split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
+        split4_bf16(make_float4(p0[0], p0[1], p0[2], p0[3]), P0h, P0l, i * TLD + c);
+        split4_bf16(make_float4(p1[0], p1[1], p1[2], p1[3]), P1h, P1l, i * TLD + c);
+      }
     }
     lds_barrier();
     // ck[i][r = col] = sum_m X[i][m] Y[r][m], cv with Xp
