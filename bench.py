@@ -29,8 +29,8 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # device-to-device copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the runs are summarised under
 # profiles/.  Reported as `traffic` only while the workload is the one they were measured on.
 TRAFFIC_BYTES = {
-    "mfma_out_kernel<128,4,8,64>": (281281.8 * 2.0 + 139320.7) * 1024,
-    "decode_mfma_kernel<128,4,2>": (303056.6 * 2.0 + 67517.3) * 1024,
+    "mfma_out_kernel<128,4,8,64>": (289662.6 * 2.0 + 139294.8) * 1024,
+    "decode_mfma_kernel<128,4,2>": (303131.7 * 2.0 + 67519.7) * 1024,
 }
 
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)

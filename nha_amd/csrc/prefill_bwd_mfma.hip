@@ -108,7 +108,9 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const WP p) {
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
   const int hq = blockIdx.x, h = hq / p.NG;
-  const int chunk = blockIdx.y;
+  // last chunk first: the chunks at the start of a sequence see the fewest keys, and short
+  // workgroups at the end of the launch leave the smallest tail
+  const int chunk = gridDim.y - 1 - blockIdx.y;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;

@@ -429,8 +429,10 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   const int H = p.H, HQ = p.HQ, NG = p.NG;
   // grid = (kv-head x head-group, chunk): consecutive workgroup ids are the heads of one chunk, so
   // with 8 (kv-head, group) pairs each XCD (id % 8) streams the chunks of ONE kv-head in order and
-  // the window tiles its resident workgroups share stay in that XCD's L2
-  const int chunk = blockIdx.y;
+  // the window tiles its resident workgroups share stay in that XCD's L2.  Chunks are taken from
+  // the last to the first: the chunks at the start of a sequence have the shortest windows, and
+  // short workgroups at the end of the launch leave the smallest tail.
+  const int chunk = p.NT - 1 - blockIdx.y;
   const int ngrp = NG / G;
   const int h = blockIdx.x / ngrp, grp = blockIdx.x % ngrp;
   const int hq = h * NG + grp * G + wave / WPU;
@@ -942,7 +944,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   }
   PROF_STAGE(5)
 #ifdef NHA_PROF
-  if (blockIdx.y == 200 && blockIdx.x == 3 && lane == 0) {
+  if (chunk == 200 && blockIdx.x == 3 && lane == 0) {
     long long* dbg = (long long*)p.lse_gsa;
     for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
     for (int k = 0; k < 8; ++k) dbg[64 + wave * 8 + k] = ps_[k];
