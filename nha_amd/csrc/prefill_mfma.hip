@@ -605,6 +605,8 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
   // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows
   // j of earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.
+  // All LDS reads of an item are issued before the first exponential waits for one: read one at a
+  // time, the 8 values of an item cost 24 LDS latencies in sequence.
   for (int item = tid; item < (NSEA + NSEB) * 64; item += NTHR) {
     const int f = item >> 6, ln = item & 63;
     const int fl16 = ln & 15, fkb = ln >> 4;
@@ -615,13 +617,19 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       const int pr = rem >> 2, mb = rem & 3;
       const int m = 16 * mb + fl16;
       const float gr = Q > 0 ? gcR[(16 * Q - 1) * GLD + m] : 0.f;
+      float gv[8];
+      bf16_t sv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = 16 * (2 * pr + (e >> 2)) + 4 * fkb + (e & 3);   // j < 64 for every fragment
+        gv[e] = gcR[j * GLD + m];
+        sv[e] = sR[j * SLD + m];
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int jb = 2 * pr + (e >> 2);
-        const int j = 16 * jb + 4 * fkb + (e & 3);
-        float val = 0.f;
-        if (jb <= Q) val = bf16_to_f32(sR[j * SLD + m]) * fexp(fminf(gr - gcR[j * GLD + m], DECAY_CLAMP));
-        out[e] = (__bf16)val;
+        const float val = bf16_to_f32(sv[e]) * fexp(fminf(gr - gv[e], DECAY_CLAMP));
+        out[e] = (__bf16)(jb <= Q ? val : 0.f);
       }
       *reinterpret_cast<NHA_LDS bf16x8*>(SEa + f * 512 + ln * 8) = out;
     } else {
@@ -630,12 +638,19 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       const int rem = g2 - seb_base(Q);
       const int jb = rem >> 1, pr = rem & 1;
       const int j = 16 * jb + fl16;
+      f32x4 gv[2], gr[2];
+      bf16x4 sv[2];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int m = 32 * pr + 16 * (e >> 2) + 4 * fkb + (e & 3);
-        const float gr = Q > 0 ? gcR[(16 * Q - 1) * GLD + m] : 0.f;
-        out[e] = (__bf16)(bf16_to_f32(sR[j * SLD + m]) * fexp(fminf(gr - gcR[j * GLD + m], DECAY_CLAMP)));
+      for (int hh = 0; hh < 2; ++hh) {
+        const int m0 = 32 * pr + 16 * hh + 4 * fkb;   // the lane's 4 consecutive slots of this half
+        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gcR + j * GLD + m0);
+        gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (Q > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gcR + (16 * Q - 1) * GLD + m0);
+        sv[hh] = *reinterpret_cast<const NHA_LDS bf16x4*>(sR + j * SLD + m0);
       }
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        out[e] = (__bf16)((float)sv[e >> 2][e & 3] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
       *reinterpret_cast<NHA_LDS bf16x8*>(SEb + g2 * 512 + ln * 8) = out;
     }
   }
@@ -945,7 +960,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   PROF_STAGE(5)
 #ifdef NHA_PROF
   if (chunk == 200 && blockIdx.x == 3 && lane == 0) {
-    long long* dbg = (long long*)p.lse_gsa;
+    long long* dbg = (long long*)(p.lse_gsa + ((int64_t)p.T_tot - 8) * HQ);   // rows of the chunk that ran first
     for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
     for (int k = 0; k < 8; ++k) dbg[64 + wave * 8 + k] = ps_[k];
   }
