@@ -333,6 +333,9 @@ class NativeHybridAttention(nn.Module):
                 lse_max = torch.maximum(lse_swa, lse_gsa)
                 w_swa, w_gsa = torch.exp(lse_swa - lse_max), torch.exp(lse_gsa - lse_max)
                 self._store_compression_stats(w_swa, w_gsa)
+                if self.gsa_aux_loss_enable:
+                    output, gsa_aux_loss = self._apply_gsa_aux_loss(output, lse_swa, lse_gsa)
+                    self._store_gsa_aux_loss(gsa_aux_loss)
         else:
             raise NotImplementedError(f"Not supported mode `{mode}`.")
         if past_key_values is not None:
@@ -353,6 +356,21 @@ class NativeHybridAttention(nn.Module):
             o = pad_input(o.squeeze(0), indices, batch_size, q_len)
         return o, None, past_key_values
 
+    def _apply_gsa_aux_loss(self, output: torch.Tensor, lse_swa: torch.Tensor, lse_gsa: torch.Tensor):
+        """One-sided auxiliary loss on the slot branch's share of the softmax mass
+        (nha_fla/layers/nha.py:300-317): binary cross-entropy of lse_gsa - stopgrad(lse_swa) against
+        the target ratio; its gradient, scaled by the coefficient, rides on `output`."""
+        delta = lse_gsa.float() - lse_swa.detach().float()
+        target = torch.full_like(delta, self.gsa_aux_loss_target_ratio)
+        loss = F.binary_cross_entropy_with_logits(delta, target, reduction='mean')
+        return _AttachLossGrad.apply(output, loss, self.gsa_aux_loss_coeff), loss
+
+    @torch.no_grad()
+    def _store_gsa_aux_loss(self, gsa_aux_loss: torch.Tensor):
+        if not hasattr(self, '_gsa_aux_losses'):
+            self._gsa_aux_losses = []
+        self._gsa_aux_losses.append(gsa_aux_loss.item())
+
     @torch.no_grad()
     def _store_compression_stats(self, w_swa: torch.Tensor, w_gsa: torch.Tensor):
         """GSA vs SWA share of the softmax mass (nha_fla/layers/nha.py:288-298)."""
@@ -360,3 +378,20 @@ class NativeHybridAttention(nn.Module):
         if not hasattr(self, '_compression_stats'):
             self._compression_stats = []
         self._compression_stats.append({'gsa_ratio': gsa_ratio, 'swa_ratio': 1.0 - gsa_ratio})
+
+
+class _AttachLossGrad(torch.autograd.Function):
+    """Identity on `hidden` whose backward also sends `coeff` into `loss`, so that backpropagating
+    the model's own objective trains the auxiliary loss with weight coeff
+    (nha_fla/layers/nha.py:327-345)."""
+
+    @staticmethod
+    def forward(ctx, hidden, loss, coeff):
+        ctx.coeff, ctx.like = coeff, loss
+        return hidden.view_as(hidden)
+
+    @staticmethod
+    def backward(ctx, dhidden):
+        if not ctx.coeff:
+            return dhidden, None, None
+        return dhidden, torch.full_like(ctx.like, ctx.coeff), None

@@ -52,7 +52,7 @@ def test_layer_forward_matches_oracle_layer():
     assert err <= 3e-2 * max(1.0, ref.abs().max().item()), err
 
 
-def _oracle_layer(w, xc, H, HKV, M, W, D):
+def _oracle_layer(w, xc, H, HKV, M, W, D, aux_target=None):
     """fp64 restatement of nha_fla/layers/nha.py:209-278 (differentiable: built on the oracle's
     per-token recurrence without detaching)."""
     from oracle import nha_ref as R
@@ -70,31 +70,45 @@ def _oracle_layer(w, xc, H, HKV, M, W, D):
     B = xc.shape[0]
     hk = torch.zeros(B, HKV, D, M, dtype=torch.float64)
     hv = torch.zeros(B, HKV, M, D, dtype=torch.float64)
-    out = R._prefill_equal_len(q_swa, k_swa, F.silu(q), F.silu(k), v, s, g, W, 0, 1.0, hk, hv)[0]
+    out, lse_swa, lse_gsa = R._prefill_equal_len(q_swa, k_swa, F.silu(q), F.silu(k), v, s, g, W, 0, 1.0, hk, hv)[:3]
     y = F.silu(out.flatten(-2))
     y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + 1e-5) * w["g_norm.weight"]
-    return y @ w["o_proj.weight"].T
+    y = y @ w["o_proj.weight"].T
+    if aux_target is None:
+        return y
+    # nha_fla/layers/nha.py:300-317: BCE of lse_gsa - stopgrad(lse_swa) against the target ratio
+    delta = lse_gsa - lse_swa.detach()
+    return y, F.binary_cross_entropy_with_logits(delta, torch.full_like(delta, aux_target))
 
 
 @pytest.mark.gpu
-def test_layer_training_step_matches_oracle_layer():
+@pytest.mark.parametrize("aux", [False, True])
+def test_layer_training_step_matches_oracle_layer(aux):
     """One forward + backward through the layer in fp32: the gradient of every parameter and of the
     input against autograd through the fp64 restatement (1e-3 of each gradient's scale: fp32
-    projections and normalisation around the op)."""
+    projections and normalisation around the op).  With the auxiliary loss on, its gradient reaches
+    the parameters through lse_gsa (the op's dlse_gsa cotangent) with weight coeff."""
     from nha_amd.layer import NativeHybridAttention
     torch.manual_seed(1)
     hid, H, HKV, M, W = 128, 4, 2, 32, 16
     D = hid // H
+    coeff, ratio = 3.0, 0.7
     layer = NativeHybridAttention(hidden_size=hid, num_heads=H, num_kv_heads=HKV, num_slots=M, layer_idx=0,
-                                  window_size=W, scale=1.0).cuda().float().train()
+                                  window_size=W, scale=1.0, gsa_aux_loss_enable=aux, gsa_aux_loss_coeff=coeff,
+                                  gsa_aux_loss_target_ratio=ratio).cuda().float().train()
     x = (torch.randn(2, 100, hid) * 0.5).cuda().requires_grad_(True)
     tgt = torch.randn(2, 100, hid)
     o, _, _ = layer(x)
     (o * tgt.cuda()).sum().backward()
     w = {k: v.detach().cpu().double().requires_grad_(True) for k, v in layer.state_dict().items()}
     xc = x.detach().cpu().double().requires_grad_(True)
-    ref = _oracle_layer(w, xc, H, HKV, M, W, D)
-    (ref * tgt.double()).sum().backward()
+    if aux:
+        ref, aux_loss = _oracle_layer(w, xc, H, HKV, M, W, D, aux_target=ratio)
+        ((ref * tgt.double()).sum() + coeff * aux_loss).backward()
+        assert abs(layer._gsa_aux_losses[-1] - aux_loss.item()) <= 1e-4 * abs(aux_loss.item())
+    else:
+        ref = _oracle_layer(w, xc, H, HKV, M, W, D)
+        (ref * tgt.double()).sum().backward()
     assert (o.detach().cpu().double() - ref.detach()).abs().max() <= 1e-3 * max(1.0, ref.abs().max().item())
     named = dict(layer.named_parameters())
     for name, p in list(named.items()) + [("input", x)]:
