@@ -180,3 +180,28 @@ def test_prefill_hands_over_to_ring_decode(W, lens, NG, K):
         oi = ring_decode_step(st, row("q_gsa"), row("q_swa"), row("k_swa"), row("k_gsa"), row("v"), row("g"))
         assert_close(f"decode step {i}", oi, torch.stack([r[0, L + i] for r, L in zip(refs, lens)]), dtype)
     assert st.count.tolist() == [L + steps for L in lens]
+
+
+def test_ring_state_from_fixed_length_prefill():
+    """from_prefill on a [B,T,...] batch (no cu_seqlens): ring slot j % W holds token j of the last W
+    tokens, the state is the prefill's final state, and the next decode step matches the oracle."""
+    import nha_amd
+    from nha_amd import NHARingState, ring_decode_step
+    from tests.util import prefill_inputs
+    dtype, B, T, H, NG, K, M, W = torch.bfloat16, 3, 75, 2, 2, 64, 64, 32
+    HQ, V = H * NG, K
+    names = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+    d = prefill_inputs(7, B, T + 1, HQ, H, K, V, M, dtype=dtype)
+    ref = R.prefill_ref(*[d[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W)[0]
+    c = {k: d[k][:, :T].contiguous().cuda() for k in names}
+    _, _, _, (hk, hv) = nha_amd.chunk_nha(*[c[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W,
+                                          output_final_state=True)
+    st = NHARingState.from_prefill(c["k_swa"], c["k_gsa"], c["v"], c["g"], (hk, hv), W)
+    assert st.count.tolist() == [T] * B
+    for j in range(T - W, T):
+        assert torch.equal(st.ring_k[:, j % W], c["k_swa"][:, j]) and torch.equal(st.ring_g[:, j % W], c["g"][:, j])
+    row = lambda k: d[k][:, T].contiguous().cuda()
+    o = ring_decode_step(st, row("q_gsa"), row("q_swa"), row("k_swa"), row("k_gsa"), row("v"), row("g"))
+    assert_close("first decode step", o, ref[:, T], dtype)
+    with pytest.raises(ValueError):
+        NHARingState.from_prefill(c["k_swa"], c["k_gsa"], c["v"], c["g"], (hk[:1], hv[:1]), W)
