@@ -1,10 +1,11 @@
 """nha_amd: MI355X-native implementation of NHA's fused hybrid-attention hot path.
 
 Public surface mirrors the reference's op API (see nha_amd/ops.py) plus the resident ring-buffer
-decode state (nha_amd/ring.py).  Everything computes through libnha_hip.so (nha_amd/csrc)."""
+decode state (nha_amd/ring.py) and the per-layer cache around it (nha_amd/cache.py).  Everything computes through libnha_hip.so (nha_amd/csrc)."""
 from ._lib import NhaError
 from .ops import chunk_nha, fused_chunk_nha_prefill, fused_recurrent_nha, fused_recurrent_nha_decode
 from .ring import NHARingState, ring_decode_step
+from .cache import NHARingCache
 
 __all__ = ["chunk_nha", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
-           "NHARingState", "ring_decode_step", "NhaError"]
+           "NHARingState", "ring_decode_step", "NHARingCache", "NhaError"]

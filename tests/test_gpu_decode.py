@@ -205,3 +205,41 @@ def test_ring_state_from_fixed_length_prefill():
     assert_close("first decode step", o, ref[:, T], dtype)
     with pytest.raises(ValueError):
         NHARingState.from_prefill(c["k_swa"], c["k_gsa"], c["v"], c["g"], (hk[:1], hv[:1]), W)
+
+
+def test_ring_cache_follows_the_cat_shift_cache():
+    """NHARingCache against a plain restatement of the reference cache's window semantics
+    (nha_fla/models/nha_cache.py:87-131, :143-154): the time-ordered window is the last W tokens, the
+    popped entry is the oldest one once the window is full, and the outputs equal the oracle's."""
+    import nha_amd
+    from nha_amd import NHARingCache
+    from tests.util import prefill_inputs
+    dtype, B, T0, steps, H, NG, K, M, W = torch.bfloat16, 2, 20, 30, 2, 2, 64, 64, 32
+    HQ, V = H * NG, K
+    names = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+    d = prefill_inputs(3, B, T0 + steps, HQ, H, K, V, M, dtype=dtype)
+    ref = R.prefill_ref(*[d[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W)[0]
+    c = {k: d[k][:, :T0].contiguous().cuda() for k in names}
+    _, _, _, fs = nha_amd.chunk_nha(*[c[k] for k in names], window_size_left=W - 1, gsa_kv_shift=W, output_final_state=True)
+    cache = NHARingCache(W)
+    assert cache.get_seq_length(0) == 0 and cache.get_pop_kvf(0) == (None, None, None)
+    cache.prefill(0, c["k_swa"], c["k_gsa"], c["v"], c["g"], fs)
+    for i in range(steps):
+        n = T0 + i                                            # tokens cached before this step
+        assert cache.get_seq_length(0) == n
+        lo = max(0, n - W)
+        wk, wv, wg = cache.window(0)
+        assert torch.equal(wk.cpu(), d["k_swa"][:, lo:n]) and torch.equal(wv.cpu(), d["v"][:, lo:n])
+        pk, pv, pg = cache.get_pop_kvf(0, W)
+        if n < W:
+            assert pk is None
+        else:                                                 # the oldest cached token leaves the window
+            assert torch.equal(pk.cpu(), d["k_gsa"][:, lo:lo + 1].flatten(-2))
+            assert torch.equal(pg.cpu(), d["g"][:, lo:lo + 1].flatten(-2))
+        row = lambda k: d[k][:, n].contiguous().cuda()
+        o = cache.decode(0, row("q_gsa"), row("q_swa"), row("k_swa"), row("k_gsa"), row("v"), row("g"))
+        assert_close(f"cache step {i}", o, ref[:, n], dtype)
+    legacy = cache.to_legacy_cache()
+    assert legacy[0]["attn_state"][0].shape == (B, W, H * K) and legacy[0]["recurrent_state"][0].shape == (B, H, K, M)
+    with pytest.raises(KeyError):
+        cache[1]
