@@ -258,8 +258,12 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
   const int niter = nqt * NG;
   Tile<TQ, D> rq, ro;
   float rl = 0.f, rd = 0.f;
+  // iteration i = (q-head of the group, query tile), tiles innermost: the workgroup of the next
+  // chunk (same XCD, started together) reads the same tile one iteration earlier, so the tile is
+  // still in that XCD's L2; with the heads innermost the reuse distance was four iterations of
+  // every resident workgroup, more than the L2 holds.
   auto issue = [&](int i) {
-    const int qt = i / NG, hq = h * NG + i % NG;
+    const int qt = i % nqt, hq = h * NG + i / nqt;
     const int64_t grow0 = (int64_t)j0 + TQ * qt;
     int vhi = eos - (int)grow0;
     vhi = vhi < 0 ? 0 : (vhi > TQ ? TQ : vhi);
@@ -291,7 +295,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
     const lbf16* Ot = tiles + (2 + cur) * TILE;
     const lfloat* ls = lsb + cur * TQ;
     const lfloat* dl = dlb + cur * TQ;
-    const int ybase = TQ * (i / NG);   // first query of the tile, relative to j0
+    const int ybase = TQ * (i % nqt);   // first query of the tile, relative to j0
     const bool edge = (ybase < 63) || (p.wl >= 0 && ybase + TQ - 1 > p.wl) || (j0 + ybase + TQ > eos);
 #pragma unroll
     for (int hf = 0; hf < NH; ++hf) {
@@ -301,12 +305,25 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
         S[kk] = (f32x4){0.f, 0.f, 0.f, 0.f};
         dP[kk] = (f32x4){0.f, 0.f, 0.f, 0.f};
       }
+      // the fragments of a 16-query block are requested together, then multiplied: one LDS
+      // latency per block instead of one per MFMA
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
+      for (int kk = 0; kk < 2; ++kk) {
+        constexpr int KH = KS > 4 ? 4 : KS;   // fragments in flight per tensor
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          S[kk] = mfma16(lds_frag(Qt, LDT, 32 * hf + 16 * kk + l16, 32 * ks + 8 * kb), kf[ks], S[kk]);
-          if (DO_K) dP[kk] = mfma16(lds_frag(Ot, LDT, 32 * hf + 16 * kk + l16, 32 * ks + 8 * kb), vf[ks], dP[kk]);
+        for (int k0 = 0; k0 < KS; k0 += KH) {
+          bf16x8 qa[KH], oa[DO_K ? KH : 1];
+#pragma unroll
+          for (int u = 0; u < KH; ++u) {
+            qa[u] = lds_frag(Qt, LDT, 32 * hf + 16 * kk + l16, 32 * (k0 + u) + 8 * kb);
+            if (DO_K) oa[u] = lds_frag(Ot, LDT, 32 * hf + 16 * kk + l16, 32 * (k0 + u) + 8 * kb);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < KH; ++u) {
+            S[kk] = mfma16(qa[u], kf[k0 + u], S[kk]);
+            if (DO_K) dP[kk] = mfma16(oa[u], vf[k0 + u], dP[kk]);
+          }
         }
       }
       f32x4 P[2], dS[2];
