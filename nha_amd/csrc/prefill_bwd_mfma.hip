@@ -257,7 +257,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
   const int nqt = (qend - j0 + TQ - 1) / TQ;
   const int niter = nqt * NG;
   Tile<TQ, D> rq, ro;
-  float rl = 0.f, rd = 0.f;
+  float rls = 0.f, rlg = 0.f, rd = 0.f;
   // iteration i = (q-head of the group, query tile), tiles innermost: the workgroup of the next
   // chunk (same XCD, started together) reads the same tile one iteration earlier, so the tile is
   // still in that XCD's L2; with the heads innermost the reuse distance was four iterations of
@@ -269,11 +269,14 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
     vhi = vhi < 0 ? 0 : (vhi > TQ ? TQ : vhi);
     rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, grow0, vhi, tid);
     ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, grow0, vhi, tid);
-    rl = 0.f;
-    rd = 0.f;
+    // only requested here: the merge of the two log-sum-exps waits until the values are staged, a
+    // tile later (used at once, it stalled the first wave for a memory latency in every iteration
+    // and the other waves behind it at the barrier)
+    rls = rlg = rd = 0.f;
     if (tid < TQ && tid < vhi) {
       const int64_t tq = (grow0 + tid) * HQ + hq;
-      rl = logaddexp_f(p.lse_swa[tq], p.lse_gsa[tq]) * LOG2E;
+      rls = p.lse_swa[tq];
+      rlg = p.lse_gsa[tq];
       rd = p.delta[tq];
     }
   };
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
     rq.store(tiles + buf * TILE, tid);
     ro.store(tiles + (2 + buf) * TILE, tid);
     if (tid < TQ) {
-      lsb[buf * TQ + tid] = rl;
+      lsb[buf * TQ + tid] = logaddexp_f(rls, rlg) * LOG2E;
       dlb[buf * TQ + tid] = rd;
     }
   };
