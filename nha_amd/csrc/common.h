@@ -148,7 +148,8 @@ int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, co
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
                        const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs, float* dsp);
 int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap, float* bp, float* ust, float* dpst,
-                      float* delta);
+                      float* delta, const int* big, const float* gc, float* dus, float* pp, float* xg);
+bool bwd_slot_products_fuses_q(const NhaPrefillBwdArgs* a);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);

@@ -955,6 +955,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   float* hkc = (float*)fs;
   fs += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
   float* hvc = (float*)fs;
+  static const bool intra_mfma = getenv("NHA_BWD_INTRA_VALU") == nullptr;
   int rc;
   if (sp.use_mfma) {
     f.impl = NHA_IMPL_MFMA;
@@ -964,8 +965,10 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     // every consumer of the states on this path reads the bf16 copies
     if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (int*)(sc + sp.big));
     // the decay-free products of the slot branch on the matrix cores
+    // (with the decay-coupled terms on the matrix cores too, the per-token stage rides along)
     if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst),
-                                             (float*)(sc + sp.delta));
+                                             (float*)(sc + sp.delta), intra_mfma ? (const int*)(sc + sp.big) : nullptr, gc,
+                                             (float*)(sc + sp.dus), (float*)(sc + sp.pp), (float*)(sc + sp.xg));
   } else {
     f.scratch = sc + sp.fwd;
     f.scratch_bytes = prefill_simple_scratch_bytes(&f);
@@ -985,7 +988,6 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.hkct = (float*)(sc + sp.hkct); p.hvct = (float*)(sc + sp.hvct);
   p.ap = p.bp = p.ust = p.dpst = nullptr;
   p.big = nullptr;
-  static const bool intra_mfma = getenv("NHA_BWD_INTRA_VALU") == nullptr;
   if (sp.use_mfma) {
     if (intra_mfma) p.big = (const int*)(sc + sp.big);
     p.ap = (float*)(sc + sp.ap); p.bp = (float*)(sc + sp.bp);
@@ -1021,7 +1023,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   const bool wmfma = bwd_window_mfma_supported(a);
   if (!sp.use_mfma) hipLaunchKernelGGL(bwd_transpose_states_kernel, dim3(a->NT * a->H), dim3(256), 0, st, p);
-  if (sp.use_mfma && intra_mfma) {
+  if (sp.use_mfma && intra_mfma && !bwd_slot_products_fuses_q(a)) {
     rc = bwd_slot_products3(a, 0, p.big, p.ap, p.bp, p.ust, p.dpst, p.gc, p.delta, p.dus, p.pp, p.xg, p.ck, p.cv, p.dsi);
     if (rc != NHA_OK) return rc;
   }

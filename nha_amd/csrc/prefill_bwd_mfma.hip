@@ -401,96 +401,6 @@ struct SP1 {
   int HQ, H, NG, shift;
 };
 
-template <int D>
-__global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p) {
-  constexpr int KS = D / 32, LDT = D + 16, TILE = BT * LDT;
-  extern __shared__ __align__(16) unsigned char smem[];
-  lbf16* const Qt = (lbf16*)smem;
-  lbf16* const Ot = Qt + TILE;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l16 = lane & 15, kb = lane >> 4;
-  const int H = p.H, HQ = p.HQ;
-  const int hq = blockIdx.x, h = hq / p.NG;
-  const int chunk = blockIdx.y;
-  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
-  const int bos = p.cu[n], eos = p.cu[n + 1];
-  const int c0 = bos + it * BT;
-  const int R = (eos - c0) < BT ? (eos - c0) : BT;
-  {
-    Tile<BT, D> rq, ro;
-    rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
-    ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
-    rq.store(Qt, tid);
-    ro.store(Ot, tid);
-  }
-  // this lane's Y rows: row j = 16 wave + l16 of the chunk (source token c0 + j - shift), slot m = j
-  const int j = 16 * wave + l16;
-  const int tl = it * BT + j - p.shift;
-  const bool has = j < R && tl >= 0;
-  const int64_t sj = ((int64_t)bos + (has ? tl : 0)) * H + h;
-  const int64_t cg = ((int64_t)chunk * H + h) * BT + j;
-  bf16x8 yk[KS], yv[KS], yhk[KS], yhv[KS], yhkl[KS], yhvl[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    uint4 a = make_uint4(0, 0, 0, 0), b = a;
-    if (has) {
-      a = *reinterpret_cast<const uint4*>(p.kg + sj * D + 32 * ks + 8 * kb);
-      b = *reinterpret_cast<const uint4*>(p.v + sj * D + 32 * ks + 8 * kb);
-    }
-    yk[ks] = __builtin_bit_cast(bf16x8, a);
-    yv[ks] = __builtin_bit_cast(bf16x8, b);
-    yhk[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkb + cg * D + 32 * ks + 8 * kb));
-    yhv[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvb + cg * D + 32 * ks + 8 * kb));
-    yhkl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkl + cg * D + 32 * ks + 8 * kb));
-    yhvl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvl + cg * D + 32 * ks + 8 * kb));
-  }
-  lds_barrier();
-  {
-    // delta_i = do_i . o_i: row i = 16 wave + l16, the four lanes sharing l16 split the columns
-    const int i = 16 * wave + l16;
-    float acc = 0.f;
-    if (i < R) {
-      const bf16_t* orow = p.o + ((int64_t)(c0 + i) * HQ + hq) * D;
-      for (int c = 8 * kb; c < D; c += 32) {
-        const bf16x8 ov = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(orow + c));
-        const bf16x8 dv = lds_frag(Ot, LDT, i, c);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
-      }
-    }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
-    if (kb == 0 && i < R) p.delta[(int64_t)(c0 + i) * HQ + hq] = acc;
-  }
-  float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
-  float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
-#pragma unroll
-  for (int blk = 0; blk < 4; ++blk) {
-    f32x4 cA = {0.f, 0.f, 0.f, 0.f}, cB = cA, cU = cA, cP = cA;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 xq = lds_frag(Qt, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
-      const bf16x8 xo = lds_frag(Ot, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
-      cA = mfma16(xq, yk[ks], cA);
-      cU = mfma16(xq, yhk[ks], mfma16(xq, yhkl[ks], cU));
-      cB = mfma16(xo, yv[ks], cB);
-      cP = mfma16(xo, yhv[ks], mfma16(xo, yhvl[ks], cP));
-    }
-    // C[i = 16 blk + 4 kb + r][j = 16 wave + l16]
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int i = 16 * blk + 4 * kb + r;
-      ap[i * BT + j] = cA[r];
-      bp[i * BT + j] = cB[r];
-      if (i < R) {
-        const int64_t tq = ((int64_t)(c0 + i) * HQ + hq) * BT + j;
-        p.ust[tq] = cU[r];
-        p.dpst[tq] = cP[r];
-      }
-    }
-  }
-}
-
 // ------------------------------------------------------------------------------------------
 // Slot branch, products over the rows of a chunk (bf16 operands, fp32 accumulation).
 //
@@ -948,6 +858,50 @@ __device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int 
   }
 }
 
+// u, dp, p and du of the chunk's rows from the tables in LDS (A, B masked to j <= i; Y high and low
+// parts); the lane's values of q.hk0 and do.hv0 come either from the products kernel's accumulators
+// (cU, cP: rows 16 blk + 4 kb + q, slot 16 wave + l16, the same mapping as here) or from scratch.
+template <bool FROM_REGS>
+__device__ __forceinline__ void slot_q_rows(const SP3& p, const lbf16* At, const lbf16* Bt, const lbf16* Yh, const lbf16* Yl,
+                                            int c0, int R, int h, int hq, int wave, int lane, const f32x4* cU,
+                                            const f32x4* cP, const lfloat* dl) {
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int HQ = p.HQ;
+  const int m = 16 * wave + l16;
+  const float g31 = R > 32 ? gc_at(p, c0, h, 31, m) : 0.f;
+#pragma unroll
+  for (int blk = 0; blk < 4; ++blk) {
+    f32x4 cu_[2], cd_[2];   // one accumulator per half of the contraction (= per reference)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const bf16x8 yh = lds_frag_tr(Yh, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);   // Y[j][m]
+      const bf16x8 yl = lds_frag_tr(Yl, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 af = table_frag(At, 16 * blk + l16, hf, kb), bf = table_frag(Bt, 16 * blk + l16, hf, kb);
+      cu_[hf] = mfma16(af, yh, mfma16(af, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
+      cd_[hf] = mfma16(bf, yh, mfma16(bf, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = 16 * blk + 4 * kb + q;
+      if (i >= R) continue;
+      const int64_t tq = (int64_t)(c0 + i) * HQ + hq;
+      const float gi = gc_at(p, c0, h, i, m);
+      const float e0 = __expf(gi);
+      const float e1 = blk >= 2 ? __expf(gi - g31) : 0.f;   // rows before the second half see none of it
+      const float au = p.scale * (e0 * ((FROM_REGS ? cU[blk][q] : p.ust[tq * BT + m]) + cu_[0][q]) + e1 * cu_[1][q]);
+      const float ad = e0 * ((FROM_REGS ? cP[blk][q] : p.dpst[tq * BT + m]) + cd_[0][q]) + e1 * cd_[1][q];
+      const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
+      const float lt = logaddexp_f(ls, lg);
+      const float pm = __expf(au - lt);
+      float du = pm * (ad - (FROM_REGS ? dl[i] : p.delta[tq]));
+      if (p.dlse_gsa) du += p.dlse_gsa[tq] * __expf(au - lg);
+      p.dus[tq * BT + m] = p.scale * du;
+      p.pp[tq * BT + m] = pm;
+      p.xg[tq * BT + m] = du * au + pm * ad;
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
   __shared__ __align__(16) bf16_t sm[4 * BT * TLD];
   lbf16* const At = (lbf16*)sm;          // [64 i][TLD]  A[i][j], zero for j > i
@@ -996,40 +950,126 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
   }
   stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
   lds_barrier();
-  const int m = 16 * wave + l16;
-  const float g31 = R > 32 ? gc_at(p, c0, h, 31, m) : 0.f;
+  slot_q_rows<false>(p, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, nullptr, nullptr, nullptr);
+}
+
+// FUSE: the per-token stage of bwd_slot_q_kernel runs in the same workgroup (same grid, same
+// lane-to-element mapping), so q.hk0 and do.hv0 never leave the registers; chunks flagged for the
+// fp32 fallback, and every chunk without FUSE, get them in scratch instead.
+template <int D, bool FUSE>
+__global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, const SP3 pq) {
+  constexpr int KS = D / 32, LDT = D + 16, TILE = BT * LDT;
+  extern __shared__ __align__(16) unsigned char smem[];
+  lbf16* const Qt = (lbf16*)smem;
+  lbf16* const Ot = Qt + TILE;
+  lbf16* const At = Ot + TILE;           // FUSE only: the four tables of the per-token stage
+  lbf16* const Bt = At + BT * TLD;
+  lbf16* const Yh = Bt + BT * TLD;
+  lbf16* const Yl = Yh + BT * TLD;
+  lfloat* const dlt = (lfloat*)(Yl + BT * TLD);   // [64] delta of the chunk's rows
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ;
+  const int hq = blockIdx.x, h = hq / p.NG;
+  const int chunk = blockIdx.y;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  {
+    Tile<BT, D> rq, ro;
+    rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    rq.store(Qt, tid);
+    ro.store(Ot, tid);
+  }
+  // this lane's Y rows: row j = 16 wave + l16 of the chunk (source token c0 + j - shift), slot m = j
+  const int j = 16 * wave + l16;
+  const int tl = it * BT + j - p.shift;
+  const bool has = j < R && tl >= 0;
+  const int64_t sj = ((int64_t)bos + (has ? tl : 0)) * H + h;
+  const int64_t cg = ((int64_t)chunk * H + h) * BT + j;
+  bf16x8 yk[KS], yv[KS], yhk[KS], yhv[KS], yhkl[KS], yhvl[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    uint4 a = make_uint4(0, 0, 0, 0), b = a;
+    if (has) {
+      a = *reinterpret_cast<const uint4*>(p.kg + sj * D + 32 * ks + 8 * kb);
+      b = *reinterpret_cast<const uint4*>(p.v + sj * D + 32 * ks + 8 * kb);
+    }
+    yk[ks] = __builtin_bit_cast(bf16x8, a);
+    yv[ks] = __builtin_bit_cast(bf16x8, b);
+    yhk[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkb + cg * D + 32 * ks + 8 * kb));
+    yhv[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvb + cg * D + 32 * ks + 8 * kb));
+    yhkl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkl + cg * D + 32 * ks + 8 * kb));
+    yhvl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvl + cg * D + 32 * ks + 8 * kb));
+  }
+  lds_barrier();
+  {
+    // delta_i = do_i . o_i: row i = 16 wave + l16, the four lanes sharing l16 split the columns
+    const int i = 16 * wave + l16;
+    float acc = 0.f;
+    if (i < R) {
+      const bf16_t* orow = p.o + ((int64_t)(c0 + i) * HQ + hq) * D;
+      for (int c = 8 * kb; c < D; c += 32) {
+        const bf16x8 ov = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(orow + c));
+        const bf16x8 dv = lds_frag(Ot, LDT, i, c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
+      }
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (kb == 0 && i < R) p.delta[(int64_t)(c0 + i) * HQ + hq] = acc;
+    if (FUSE && kb == 0) dlt[i] = acc;
+  }
+  float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+  float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+  const bool fused = FUSE && !pq.big[(int64_t)chunk * H + h];
+  f32x4 cUr[FUSE ? 4 : 1], cPr[FUSE ? 4 : 1];
 #pragma unroll
   for (int blk = 0; blk < 4; ++blk) {
-    f32x4 cu_[2], cd_[2];   // one accumulator per half of the contraction (= per reference)
+    f32x4 cA = {0.f, 0.f, 0.f, 0.f}, cB = cA, cU = cA, cP = cA;
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const bf16x8 yh = lds_frag_tr(Yh, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);   // Y[j][m]
-      const bf16x8 yl = lds_frag_tr(Yl, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
-      const bf16x8 af = table_frag(At, 16 * blk + l16, hf, kb), bf = table_frag(Bt, 16 * blk + l16, hf, kb);
-      cu_[hf] = mfma16(af, yh, mfma16(af, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
-      cd_[hf] = mfma16(bf, yh, mfma16(bf, yl, (f32x4){0.f, 0.f, 0.f, 0.f}));
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 xq = lds_frag(Qt, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
+      const bf16x8 xo = lds_frag(Ot, LDT, 16 * blk + l16, 32 * ks + 8 * kb);
+      cA = mfma16(xq, yk[ks], cA);
+      cU = mfma16(xq, yhk[ks], mfma16(xq, yhkl[ks], cU));
+      cB = mfma16(xo, yv[ks], cB);
+      cP = mfma16(xo, yhv[ks], mfma16(xo, yhvl[ks], cP));
     }
+    if (FUSE) {
+      cUr[blk] = cU;
+      cPr[blk] = cP;
+    }
+    // C[i = 16 blk + 4 kb + r][j = 16 wave + l16]
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int i = 16 * blk + 4 * kb + q;
-      if (i >= R) continue;
-      const int64_t tq = (int64_t)(c0 + i) * HQ + hq;
-      const float gi = gc_at(p, c0, h, i, m);
-      const float e0 = __expf(gi);
-      const float e1 = blk >= 2 ? __expf(gi - g31) : 0.f;   // rows before the second half see none of it
-      const float au = p.scale * (e0 * (p.ust[tq * BT + m] + cu_[0][q]) + e1 * cu_[1][q]);
-      const float ad = e0 * (p.dpst[tq * BT + m] + cd_[0][q]) + e1 * cd_[1][q];
-      const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
-      const float lt = logaddexp_f(ls, lg);
-      const float pm = __expf(au - lt);
-      float du = pm * (ad - p.delta[tq]);
-      if (p.dlse_gsa) du += p.dlse_gsa[tq] * __expf(au - lg);
-      p.dus[tq * BT + m] = p.scale * du;
-      p.pp[tq * BT + m] = pm;
-      p.xg[tq * BT + m] = du * au + pm * ad;
+    for (int r = 0; r < 4; ++r) {
+      const int i = 16 * blk + 4 * kb + r;
+      ap[i * BT + j] = cA[r];
+      bp[i * BT + j] = cB[r];
+      if (fused) {
+        const bool in = j <= i && i < R;
+        At[i * TLD + j] = f32_to_bf16(in ? cA[r] : 0.f);
+        Bt[i * TLD + j] = f32_to_bf16(in ? cB[r] : 0.f);
+      } else if (i < R) {
+        const int64_t tq = ((int64_t)(c0 + i) * HQ + hq) * BT + j;
+        p.ust[tq] = cU[r];
+        p.dpst[tq] = cP[r];
+      }
     }
   }
+  if constexpr (FUSE) {
+    if (!fused) return;   // uniform over the workgroup
+    int vlo = p.shift - it * BT;
+    vlo = vlo < 0 ? 0 : vlo;
+    stage_y(Yh, Yl, pq, c0, h, R, vlo, tid);
+    lds_barrier();
+    slot_q_rows<true>(pq, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, cUr, cPr, dlt);
+  }
 }
+
 
 __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -1244,26 +1284,43 @@ int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const fl
   return launch_dkv<256, 32, 2>(p, a->NT, st);
 }
 
-template <int D>
-static int launch_slot_products(const SP1& p, int NT, hipStream_t st) {
-  const size_t lds = (size_t)2 * BT * (D + 16) * 2;
+template <int D, bool FUSE>
+static int launch_slot_products(const SP1& p, const SP3& pq, int NT, hipStream_t st) {
+  const size_t lds = (size_t)2 * BT * (D + 16) * 2 + (FUSE ? (size_t)4 * BT * TLD * 2 + BT * 4 : 0);
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_products_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_products_kernel<D, FUSE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
       set_error("nha_prefill_bwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
       return NHA_ERR_LAUNCH;
     }
     configured = true;
   }
-  hipLaunchKernelGGL((bwd_slot_products_kernel<D>), dim3(p.HQ, NT), dim3(256), lds, st, p);
+  hipLaunchKernelGGL((bwd_slot_products_kernel<D, FUSE>), dim3(p.HQ, NT), dim3(256), lds, st, p, pq);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products)");
   return NHA_OK;
 }
 
-// bf16, K == V in {64,128,256}, M == 64 (the shapes of the matrix-core state pass)
+static SP3 make_sp3(const NhaPrefillBwdArgs* a, const int* big, const float* ap, const float* bp, const float* ust,
+                    const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
+                    float* cv, float* dsi) {
+  SP3 p;
+  p.s = (const bf16_t*)a->s;
+  p.ap = ap; p.bp = bp; p.ust = ust; p.dpst = dpst; p.gc = gc; p.delta = delta;
+  p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa; p.dlse_gsa = a->dlse_gsa;
+  p.dus = dus; p.pp = pp; p.xg = xg; p.ck = ck; p.cv = cv; p.dsi = dsi; p.big = big;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
+  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift; p.scale = a->scale;
+  return p;
+}
+
+// With `big` (the decay flags) and head dims up to 128 the per-token stage is fused in and
+// bwd_slot_products_fuses_q() tells the caller to skip bwd_slot_products3(which = 0).
+bool bwd_slot_products_fuses_q(const NhaPrefillBwdArgs* a) { return a->K <= 128; }
+
 int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap,
-                      float* bp, float* ust, float* dpst, float* delta) {
+                      float* bp, float* ust, float* dpst, float* delta, const int* big, const float* gc, float* dus, float* pp,
+                      float* xg) {
   SP1 p;
   p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.v = (const bf16_t*)a->v;
   p.hkb = (const bf16_t*)hkb; p.hvb = (const bf16_t*)hvb;
@@ -1272,10 +1329,12 @@ int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* h
   p.o = (const bf16_t*)a->o; p.delta = delta;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
   p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift;
+  const SP3 pq = make_sp3(a, big, ap, bp, ust, dpst, gc, delta, dus, pp, xg, nullptr, nullptr, nullptr);
   hipStream_t st = (hipStream_t)a->stream;
-  if (a->K == 64) return launch_slot_products<64>(p, a->NT, st);
-  if (a->K == 128) return launch_slot_products<128>(p, a->NT, st);
-  return launch_slot_products<256>(p, a->NT, st);
+  const bool fuse = big != nullptr && bwd_slot_products_fuses_q(a);
+  if (a->K == 64) return fuse ? launch_slot_products<64, true>(p, pq, a->NT, st) : launch_slot_products<64, false>(p, pq, a->NT, st);
+  if (a->K == 128) return fuse ? launch_slot_products<128, true>(p, pq, a->NT, st) : launch_slot_products<128, false>(p, pq, a->NT, st);
+  return launch_slot_products<256, false>(p, pq, a->NT, st);
 }
 
 template <int D>
@@ -1328,13 +1387,7 @@ int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, c
 int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const float* ap, const float* bp, const float* ust,
                        const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
                        float* cv, float* dsi) {
-  SP3 p;
-  p.s = (const bf16_t*)a->s;
-  p.ap = ap; p.bp = bp; p.ust = ust; p.dpst = dpst; p.gc = gc; p.delta = delta;
-  p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa; p.dlse_gsa = a->dlse_gsa;
-  p.dus = dus; p.pp = pp; p.xg = xg; p.ck = ck; p.cv = cv; p.dsi = dsi; p.big = big;
-  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
-  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.shift = a->shift; p.scale = a->scale;
+  const SP3 p = make_sp3(a, big, ap, bp, ust, dpst, gc, delta, dus, pp, xg, ck, cv, dsi);
   hipStream_t st = (hipStream_t)a->stream;
   if (which == 0) hipLaunchKernelGGL(bwd_slot_q_kernel, dim3(a->HQ, a->NT), dim3(256), 0, st, p);
   else {
