@@ -31,6 +31,8 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 TRAFFIC_BYTES = {
     "mfma_out_kernel<128,4,8,64>": (289662.6 * 2.0 + 139294.8) * 1024,
     "decode_mfma_kernel<128,4,2>": (303131.7 * 2.0 + 67519.7) * 1024,
+    "layer_prologue_kernel": (106610.8 * 2.0 + 393216.0) * 1024,
+    "layer_epilogue_kernel": (65759.4 * 2.0 + 131072.0) * 1024,
 }
 
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
@@ -399,9 +401,11 @@ def main():
                        "prologue_us": gl["prologue_us"], "epilogue_us": gl["epilogue_us"],
                        "roofline": {"bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                     "prologue": {"achieved": gl["prologue_gbs"], "frac": gl["prologue_gbs"] / PEAK_HBM_GBS,
-                                                 "algorithmic_bytes": gl["prologue_bytes"]},
+                                                 "algorithmic_bytes": gl["prologue_bytes"],
+                                                 "traffic": TRAFFIC_BYTES["layer_prologue_kernel"]},
                                     "epilogue": {"achieved": gl["epilogue_gbs"], "frac": gl["epilogue_gbs"] / PEAK_HBM_GBS,
-                                                 "algorithmic_bytes": gl["epilogue_bytes"]}}},
+                                                 "algorithmic_bytes": gl["epilogue_bytes"],
+                                                 "traffic": TRAFFIC_BYTES["layer_epilogue_kernel"]}}},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
