@@ -296,9 +296,12 @@ def cpu_baseline(torch):
     # cost per token grows with the window fill; aim at ~15 s of CPU work, at most the full T
     T = 256
     est = t_probe
-    while T < cfg["T"] and est * 4.5 < 15.0:
+    while T < cfg["T"]:
+        grow = 4.5 if 2 * T <= W else 2.2
+        if est * grow > 20.0:
+            break
         T *= 2
-        est *= 4.5 if T <= W else 2.2
+        est *= grow
     t = timed(T)
     pre = dict(value=T / t, unit="tokens/s", cores=cores, kind="port",
                sample=f"B=1 slice, first {T} tokens of the T={cfg['T']} workload, fp32, {t:.1f} s")
