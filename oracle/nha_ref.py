@@ -16,6 +16,9 @@ It restates, as plain PyTorch on CPU, the semantics of the reference op
   nha_fla/ops/nha/fused_recurrent.py:309-329)
 * caller-supplied-window-logit step (scripts/verify_opt_parity.py:128-144)
 
+A second, independent restatement of the prefill in plain C lives in nha_ref_c.c
+(front: nha_ref_c.py); it is pinned against this module.
+
 Pinning (see tests/test_oracle_pins.py): every function below is checked against
 something that is *not* a retyping of its own formula -- torch's
 scaled_dot_product_attention (slots degenerate to zero sinks), the explicit

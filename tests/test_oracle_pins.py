@@ -357,3 +357,40 @@ def test_layer_glue_against_library_routines_and_invariants():
     assert torch.allclose(R.layer_epilogue_ref(o, w, b, 1e-5), ref, atol=1e-12)
     y = R.layer_epilogue_ref(o, None, None, 0.0)
     assert torch.allclose(y.pow(2).mean(-1), torch.ones(B, T, dtype=DT), atol=1e-12)
+
+
+@pytest.mark.parametrize("wl,shift,varlen,NG", [(15, 16, False, 2), (16, 0, True, 1), (-1, 3, True, 4), (0, 1, False, 1)])
+def test_c_restatement_matches_torch_oracle(wl, shift, varlen, NG):
+    """oracle/nha_ref_c.c (plain C, written independently of the torch code: explicit loops, one task
+    per q-head carrying its kv-head's recurrence) against prefill_ref on random cases: both
+    conventions, GQA, packed sequences shorter and longer than window and shift, initial states.
+    float32 in and out, so agreement to float32 rounding."""
+    from oracle.nha_ref_c import prefill_ref_c
+    torch.manual_seed(7)
+    H, K, V, M = 2, 12, 10, 7
+    HQ = H * NG
+    B, T = (1, 90) if varlen else (2, 45)
+    cu = [0, 3, 40, 41, 90] if varlen else None
+    N = 4 if varlen else B
+    r = lambda *s: torch.randn(*s, dtype=torch.float32)
+    g = F.logsigmoid(r(B, T, H, M))
+    x = [r(B, T, HQ, K), r(B, T, H, K), r(B, T, HQ, K), r(B, T, H, K), r(B, T, H, V), 1 - g.exp(), g]
+    h0 = (r(N, H, K, M), r(N, H, M, V))
+    kw = dict(window_size_left=wl, gsa_kv_shift=shift, cu_seqlens=cu, initial_state=h0, scale=0.3)
+    ref = R.prefill_ref(*x, **kw)
+    got = prefill_ref_c(*x, **kw)
+    for name, a, b in zip(("o", "lse_swa", "lse_gsa", "hkt", "hvt"), got, ref):
+        assert a.dtype == torch.float32 and a.shape == b.shape, name
+        assert (a.double() - b).abs().max() <= 2e-6 * max(1.0, b.abs().max().item()), name
+    # zero slots and zero initial state: plain banded softmax attention from the library routine
+    if wl >= 0 and not varlen:
+        z = [x[0], x[1], x[2], x[3], x[4], torch.zeros_like(x[5]), x[6]]
+        o = prefill_ref_c(*z, window_size_left=wl, gsa_kv_shift=shift, scale=0.3)[0]
+        i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+        band = (j <= i) & (j >= i - wl)
+        kx = torch.cat([torch.zeros(B, M, H, K), x[1]], 1).repeat_interleave(NG, 2)     # M zero-logit, zero-value sinks
+        vx = torch.cat([torch.zeros(B, M, H, V), x[4]], 1).repeat_interleave(NG, 2)
+        mask = torch.cat([torch.ones(T, M, dtype=torch.bool), band], 1)
+        sd = F.scaled_dot_product_attention(x[0].transpose(1, 2).double(), kx.transpose(1, 2).double(),
+                                            vx.transpose(1, 2).double(), attn_mask=mask, scale=0.3).transpose(1, 2)
+        assert (o.double() - sd).abs().max() <= 2e-6
