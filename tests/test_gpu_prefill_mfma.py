@@ -110,3 +110,27 @@ def test_mfma_matches_simple_kernels_at_size():
     assert_close("lse_gsa", a[2], b[2].double(), BF)
     assert_close("hk", a[3][0], b[3][0].double(), BF)
     assert_close("hv", a[3][1], b[3][1].double(), BF)
+
+
+def test_mfma_headline_shape_matches_c_oracle():
+    """The benchmark's own shape (T=8192, 32/8 heads, D=128, M=64, W=2048; one of its two sequences)
+    element by element against the plain-C restatement of the oracle, which gets through it in
+    seconds on the host cores."""
+    import bench
+    from nha_amd import chunk_nha
+    from oracle.nha_ref_c import prefill_ref_c
+    cfg = bench.PREFILL
+    xs = bench.make_prefill_inputs(torch, cfg, "cpu", seed=5, B=1)
+    W = cfg["W"]
+    ref = prefill_ref_c(*xs, window_size_left=W - 1, gsa_kv_shift=W)
+    got = chunk_nha(*[x.cuda() for x in xs], window_size_left=W - 1, gsa_kv_shift=W, output_final_state=True, impl="mfma")
+    assert_close("o", got[0], ref[0].double(), BF)
+    assert_close("lse_swa", got[1], ref[1].double(), BF)
+    assert_close("lse_gsa", got[2], ref[2].double(), BF)
+    assert_close("hk", got[3][0], ref[3].double(), BF)
+    assert_close("hv", got[3][1], ref[4].double(), BF)
+    # the workload's values are small next to the absolute bar above: relative L2 error as well
+    # (bf16 output rounding alone is 2^-9)
+    for name, a, b in (("o", got[0], ref[0]), ("hk", got[3][0], ref[3]), ("hv", got[3][1], ref[4])):
+        rel = ((a.double().cpu() - b.double()).norm() / b.double().norm()).item()
+        assert rel <= 5e-3, f"{name}: relative L2 error {rel:.3e}"
