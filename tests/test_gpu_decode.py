@@ -243,3 +243,39 @@ def test_ring_cache_follows_the_cat_shift_cache():
     assert legacy[0]["attn_state"][0].shape == (B, W, H * K) and legacy[0]["recurrent_state"][0].shape == (B, H, K, M)
     with pytest.raises(KeyError):
         cache[1]
+
+
+def test_ring_decode_at_benchmark_shape():
+    """Two steps of the benchmark's decode workload (B=128, 32/8 heads, D=128, M=64, W=1024: full
+    windows at random ring positions) against the oracle's ring recurrence."""
+    import bench
+    from nha_amd import NHARingState, ring_decode_step
+    cfg = bench.DECODE
+    B, HQ, H, D, M, W = (cfg[k] for k in ("B", "HQ", "H", "D", "M", "W"))
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(21)
+    r = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    st = NHARingState.empty(B, H, D, D, M, W, dtype=dtype)
+    st.hk.copy_(r(B, H, D, M) * 0.1)
+    st.hv.copy_(r(B, H, M, D) * 0.1)
+    st.ring_k.copy_(r(B, W, H, D))
+    st.ring_kg.copy_(r(B, W, H, D))
+    st.ring_v.copy_(r(B, W, H, D))
+    st.ring_g.copy_(F.logsigmoid(r(B, W, H, M)))
+    counts = torch.randint(W, 3 * W, (B,), generator=gen, dtype=torch.int32)
+    st.count.copy_(counts)
+    ref = dict(hk=st.hk.cpu().double(), hv=st.hv.cpu().double(),
+               rings=tuple(x.cpu().double() for x in (st.ring_k, st.ring_kg, st.ring_v, st.ring_g)), count=counts.clone())
+    for step in range(2):
+        q, sq = (r(B, HQ, D) * D ** -0.5).to(dtype), (r(B, HQ, D) * D ** -0.5).to(dtype)
+        kn, kgn, vn = r(B, H, D).to(dtype), r(B, H, D).to(dtype), r(B, H, D).to(dtype)
+        gn = F.logsigmoid(r(B, H, M)).to(dtype)
+        o = ring_decode_step(st, q.cuda(), sq.cuda(), kn.cuda(), kgn.cuda(), vn.cuda(), gn.cuda())
+        ro, ref["hk"], ref["hv"], ref["rings"] = R.decode_ring_ref(q, sq, kn, kgn, vn, gn, *ref["rings"], ref["count"],
+                                                                   ref["hk"], ref["hv"])
+        ref["count"] += 1
+        assert_close(f"step {step} o", o, ro, dtype)
+        rel = ((o.double().cpu() - ro).norm() / ro.norm()).item()
+        assert rel <= 5e-3, f"step {step}: relative L2 error {rel:.3e}"
+    assert_close("hk", st.hk, ref["hk"], dtype)
+    assert_close("hv", st.hv, ref["hv"], dtype)
