@@ -7,6 +7,8 @@
  *   nha_fla/ops/nha/chunk_fused.py:291-303      fused_chunk_nha_prefill
  *   nha_fla/ops/nha/fused_recurrent.py:431-445  fused_recurrent_nha_decode
  *   nha_fla/ops/nha/fused_recurrent.py:588-598  fused_recurrent_nha
+ * and, one level up, the layer nha_fla/layers/nha.py:147-282, whose elementwise glue around the
+ * op (lines 214-237 and 278) has entry points here too.
  * Each entry point below states which of those it sits behind.  The host-side mirror of that
  * Python API (same names, argument meaning and error behaviour) is nha_amd/ops.py, which binds
  * this library with ctypes; no torch type crosses this boundary.
