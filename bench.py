@@ -229,6 +229,50 @@ def bench_glue(torch, steps, warmup, cfg=PREFILL):
                 epilogue_us=us_e, epilogue_bytes=by_e, epilogue_gbs=by_e / us_e / 1e3)
 
 
+def bench_layer(torch, steps, warmup):
+    """NativeHybridAttention (hidden 1024, 4 heads of 256, 64 slots, window 512: the 340M layer) on
+    B=8 T=2048 bf16: milliseconds per forward (autograd off) and per forward + backward, with the
+    fused glue launches and with the tensor-op chain."""
+    from nha_amd.layer import NativeHybridAttention
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    layer = NativeHybridAttention(hidden_size=1024, num_heads=4, num_kv_heads=4, num_slots=64, layer_idx=0,
+                                  window_size=512).to(dev).to(torch.bfloat16)
+    x = (torch.randn(8, 2048, 1024) * 0.5).to(torch.bfloat16).to(dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record(stream)
+        for _ in range(steps):
+            fn()
+        ev[1].record(stream)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / steps
+
+    def fwd():
+        with torch.no_grad():
+            layer(x)
+
+    def fwd_bwd():
+        xg = x.detach().requires_grad_(True)
+        y = layer(xg)[0]
+        y.backward(torch.ones_like(y))
+
+    out = {}
+    for fuse in (True, False):
+        layer.fuse_glue = fuse
+        layer.eval()
+        out[("fused" if fuse else "chain") + "_fwd_ms"] = timed(fwd)
+        layer.train()
+        layer._compression_stats = []
+        out[("fused" if fuse else "chain") + "_fwd_bwd_ms"] = timed(fwd_bwd)
+    return out
+
+
 def bench_decode(torch, warmup):
     from nha_amd import NHARingState, ring_decode_step
     cfg = DECODE
@@ -336,7 +380,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--only", choices=["prefill", "decode", "glue"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "glue", "layer"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
     ap.add_argument("--backward", action="store_true",
                     help="with --workload: also time the backward of the prefill op")
@@ -368,7 +412,8 @@ def main():
         return
     if args.only:
         res = (bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else
-               bench_glue(torch, args.steps, args.warmup) if args.only == "glue" else bench_decode(torch, args.warmup))
+               bench_glue(torch, args.steps, args.warmup) if args.only == "glue" else
+               bench_layer(torch, args.steps, args.warmup) if args.only == "layer" else bench_decode(torch, args.warmup))
         print(json.dumps(res))
         return
     pf = bench_prefill(torch, args.steps, args.warmup)
