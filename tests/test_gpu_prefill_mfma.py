@@ -136,16 +136,18 @@ def test_mfma_headline_shape_matches_c_oracle():
         assert rel <= 5e-3, f"{name}: relative L2 error {rel:.3e}"
 
 
-@pytest.mark.parametrize("name", ["cfg2", "cfg3"])
+@pytest.mark.parametrize("name", ["cfg2", "cfg3", "cfg5"])
 def test_mfma_layer_workloads_match_c_oracle(name):
-    """The D=256 workloads of the benchmark (layer convention wl = W, shift = 0; cfg3 is the packed
-    varlen draw of 64..4096-token sequences) against the C restatement, with initial states."""
+    """The other workloads of the benchmark against the C restatement, with initial states: the D=256
+    ones (layer convention wl = W, shift = 0; cfg3 is the packed varlen draw of 64..4096-token
+    sequences) and one T=16384 sequence of the long-context hybrid shape (32/8 heads, D=128,
+    W=2048, shifted convention)."""
     import bench
     from nha_amd import chunk_nha
     from oracle.nha_ref_c import prefill_ref_c
     cfg = dict(bench.WORKLOADS[name])
     if not cfg.get("varlen"):
-        cfg["B"] = 2                                          # two of its eight sequences
+        cfg["B"] = 1 if name == "cfg5" else 2                 # a part of its batch
     lens = bench.workload_lengths(torch, cfg)
     B, T, H, D, M = cfg["B"], cfg["T"], cfg["H"], cfg["D"], cfg["M"]
     xs = bench.make_prefill_inputs(torch, cfg, "cpu", seed=9)
@@ -155,7 +157,7 @@ def test_mfma_layer_workloads_match_c_oracle(name):
     N = len(lens)
     gen = torch.Generator().manual_seed(4)
     h0 = (torch.randn(N, H, D, M, generator=gen) * 0.05, torch.randn(N, H, M, D, generator=gen) * 0.05)
-    kw = dict(window_size_left=cfg["wl"], gsa_kv_shift=cfg["shift"])
+    kw = dict(window_size_left=cfg.get("wl", cfg["W"] - 1), gsa_kv_shift=cfg.get("shift", cfg["W"]))
     ref = prefill_ref_c(*xs, cu_seqlens=None if cu is None else cu.tolist(), initial_state=h0, **kw)
     got = chunk_nha(*[x.cuda() for x in xs], cu_seqlens=None if cu is None else cu.cuda(),
                     initial_state=(h0[0].cuda(), h0[1].cuda()), output_final_state=True, impl="mfma", **kw)
