@@ -961,9 +961,9 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     f.impl = NHA_IMPL_MFMA;
     f.scratch = sc + sp.mfma;
     f.scratch_bytes = prefill_mfma_scratch_bytes(&f);
-    rc = prefill_mfma_impl(&f);
-    // every consumer of the states on this path reads the bf16 copies
-    if (rc == NHA_OK) rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (int*)(sc + sp.big));
+    // state pass (segment form) and its export; every consumer of the states on this path reads
+    // the bf16 copies
+    rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (int*)(sc + sp.big));
     // the decay-free products of the slot branch on the matrix cores
     // (with the decay-coupled terms on the matrix cores too, the per-token stage rides along)
     if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst),

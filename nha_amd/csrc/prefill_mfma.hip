@@ -15,99 +15,14 @@
 //   state pass  (mfma_state_kernel): per (sequence, kv-head, 16-slot block) sweep over 64-row chunks
 //               with the fp32 state held in MFMA accumulators (chunk_fused.py:30-113).
 //   output pass (mfma_out_kernel)  : per (chunk, kv-head, group of <=4 q-heads).
-#include "common.h"
+#include "mfma_common.h"
+
+#include <mutex>
 
 namespace nha {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-// explicit LDS address space: keeps every tile access a ds_* instruction (never a flat access)
-#define NHA_LDS __attribute__((address_space(3)))
-typedef NHA_LDS bf16_t lbf16;
-typedef NHA_LDS float lfloat;
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ void lds_st16(lbf16* p, uint4 v) { *reinterpret_cast<NHA_LDS u32x4*>(p) = (u32x4){v.x, v.y, v.z, v.w}; }
-__device__ __forceinline__ float4 lds_ld_f4(const lfloat* p) {
-  const f32x4 v = *reinterpret_cast<const NHA_LDS f32x4*>(p);
-  return make_float4(v[0], v[1], v[2], v[3]);
-}
-
-constexpr int BT = 64;        // chunk rows == window tile keys
-constexpr int MS = 64;        // slots
-constexpr int GLD = 68;       // LDS row stride (floats) of the gate-cumsum tables
-constexpr int SLD = 72;       // LDS row stride (bf16) of the s tables
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
-constexpr float DECAY_CLAMP = 80.f;   // largest positive decay exponent formed on the MFMA path
-
-struct MP {
-  const bf16_t *q_swa, *k_swa, *q_gsa, *k_gsa, *v, *s, *g;
-  bf16_t* o;
-  float *lse_swa, *lse_gsa;
-  const float *h0k, *h0v;
-  float *hkt, *hvt;
-  const int32_t *cu, *cidx, *coff;
-  bf16_t* hkT;   // [NT][H][MS][D]   segment-local chunk-start k-state, transposed ([m][d])
-  bf16_t* hvc;   // [NT][H][MS][D]   segment-local chunk-start v-state ([m][d])
-  float* gc;     // [NT][H][BT][MS]  chunk-local inclusive gate cumsum
-  float* dcum;   // [NT][H][MS]      decay from the segment start to the chunk start
-  float *hend_k, *hend_v;   // [NSLOT][H][MS][D]  segment-local end states
-  float *hseg_k, *hseg_v;   // [NSLOT][H][MS][D]  true segment-start states
-  float* dtot;   // [NSLOT][H][MS]   total decay of a segment
-  int* flags;    // [NT][H][4]       per 16-slot block: bit q = sub-block q decays past DECAY_CLAMP
-  int T_tot, N, NT, HQ, H, NG, wl, shift;
-  float scale;
-};
-
-__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-__device__ __forceinline__ bf16x8 as_bf16x8(uint4 u) { return __builtin_bit_cast(bf16x8, u); }
-__device__ __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float fexp(float x) { return __builtin_amdgcn_exp2f(x * LOG2E); }
-
-__device__ __forceinline__ bf16x8 pack8(f32x4 a, f32x4 b) {
-  bf16x8 r;
-  r[0] = (__bf16)a[0]; r[1] = (__bf16)a[1]; r[2] = (__bf16)a[2]; r[3] = (__bf16)a[3];
-  r[4] = (__bf16)b[0]; r[5] = (__bf16)b[1]; r[6] = (__bf16)b[2]; r[7] = (__bf16)b[3];
-  return r;
-}
-
-// workgroup barrier that orders LDS traffic only: outstanding global loads (tile prefetches) stay
-// in flight across it
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-// max over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), VALU only
-__device__ __forceinline__ float max_over_rows(float x) {
-  const unsigned u = __float_as_uint(x);
-  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  const unsigned v = __float_as_uint(x);
-  const auto b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-
-// A/B fragment of a row-major LDS tile: 8 consecutive elements of row `row` starting at `col`.
-__device__ __forceinline__ bf16x8 lds_frag(const lbf16* tile, int ld, int row, int col) {
-  return *reinterpret_cast<const NHA_LDS bf16x8*>(tile + row * ld + col);
-}
-
-// Transposed fragment of a row-major [rows][ld] bf16 LDS tile: the lane (c = l%16, kb = l/16)
-// receives X[r0a + 4*kb + e][col0 + c] for e = 0..3 and X[r0b + 4*kb + e][col0 + c] for e = 4..7.
-__device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a, int r0b, int col0, int lane) {
-  const int l16 = lane & 15, kb = lane >> 4;
-  const lbf16* pa = tile + (r0a + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
-  const lbf16* pb = tile + (r0b + 4 * kb + (l16 >> 2)) * ld + col0 + 4 * (l16 & 3);
-  struct { s16x4 a, b; } t;
-  t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
-  t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pb);
-  return __builtin_bit_cast(bf16x8, t);
-}
+using namespace mf;
 
 // ------------------------------------------------------------------------------------------
 // cooperative 64-row tile copy, global -> registers -> LDS (16-byte pieces, zero fill)
@@ -148,13 +63,12 @@ __device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<ROWS, D, NTH
 // per 16-slot block) runs the recurrence of chunk_fused.py:30-113 from a ZERO state over its
 // segment and stores, per chunk, the local chunk-start states, the gate cumsum table and the
 // decay accumulated since the segment start; per segment, the local end state and total decay.
-// Level 2 (state_scan_kernel) carries the true state across segments element-wise:
-//   h_seg[s+1] = h_seg[s] * dtot[s] + hend[s].
-// The true chunk-start state, h_loc + h_seg * dcum, is formed by the output pass while it stages
-// the state tiles into LDS.  Both states are kept as C[d][m] accumulators (slot m = lane % 16).
-constexpr int SEG = 4;
-
-__device__ __forceinline__ int seg_slot(const int32_t* coff, int n, int it) { return coff[n] / SEG + it / SEG + n; }
+// Level 2 carries the true state across segments element-wise, h_seg[s+1] = h_seg[s] * dtot[s] + hend[s],
+// in one of two forms.  The forward (state_final_kernel) turns every chunk-start state of the
+// segment into the true one on the way, h_loc + h_seg * dcum, rounded to bf16 in place, so that the
+// output pass reads plain operand tiles.  The backward (state_scan_kernel) keeps the segment-local
+// states and writes the segment-start states h_seg beside them: it needs the sum in fp32.
+// Both states are kept as C[d][m] accumulators (slot m = lane % 16).
 
 template <int D>
 __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
@@ -363,6 +277,89 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
   }
 }
 
+// Level 2, forward form: four consecutive d of one slot per thread, sequential over the segments
+// of its sequence; the loads of the next segment are requested before the current one is combined.
+// grid (N*H, 2*MS*D/1024): the first MS*D/4 groups are the k-state ([m][d]), the rest the v-state.
+template <int D>
+__global__ __launch_bounds__(256) void state_final_kernel(const MP p) {
+  const int H = p.H;
+  const int n = blockIdx.x / H, h = blockIdx.x % H;
+  const int e4 = blockIdx.y * 256 + threadIdx.x;
+  const bool isv = e4 >= MS * D / 4;
+  const int em = (isv ? e4 - MS * D / 4 : e4) * 4;
+  const int m = em / D, d = em % D;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int nchunks = (eos - bos + BT - 1) / BT;
+  const int nseg = (nchunks + SEG - 1) / SEG;
+  float hcur[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.h0k) {
+    if (isv) {
+      const float4 x = *reinterpret_cast<const float4*>(p.h0v + (((int64_t)n * H + h) * MS + m) * D + d);
+      hcur[0] = x.x; hcur[1] = x.y; hcur[2] = x.z; hcur[3] = x.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) hcur[i] = p.h0k[(((int64_t)n * H + h) * D + d + i) * MS + m];
+    }
+  }
+  const float* hend = isv ? p.hend_v : p.hend_k;
+  bf16_t* hloc = isv ? p.hvc : p.hkT;
+  const int chunk0 = p.coff[n];
+  const int slot0 = chunk0 / SEG + n;
+  struct SegRegs {
+    uint2 loc[SEG];
+    float dc[SEG];
+    float dt;
+    float4 he;
+  };
+  auto request = [&](SegRegs& r, int sg) {
+    const int64_t sl = (int64_t)(slot0 + sg) * H + h;
+#pragma unroll
+    for (int jc = 0; jc < SEG; ++jc) {
+      r.loc[jc] = make_uint2(0, 0);
+      r.dc[jc] = 0.f;
+      if (sg * SEG + jc < nchunks) {
+        const int64_t cg = (int64_t)(chunk0 + sg * SEG + jc) * H + h;
+        r.loc[jc] = *reinterpret_cast<const uint2*>(hloc + (cg * MS + m) * D + d);
+        r.dc[jc] = p.dcum[cg * MS + m];
+      }
+    }
+    r.dt = p.dtot[sl * MS + m];
+    r.he = *reinterpret_cast<const float4*>(hend + (sl * MS + m) * D + d);
+  };
+  SegRegs cur, nxt;
+  request(cur, 0);
+  for (int sg = 0; sg < nseg; ++sg) {
+    if (sg + 1 < nseg) request(nxt, sg + 1);
+#pragma unroll
+    for (int jc = 0; jc < SEG; ++jc) {
+      if (sg * SEG + jc < nchunks) {
+        const int64_t cg = (int64_t)(chunk0 + sg * SEG + jc) * H + h;
+        const uint32_t w[2] = {cur.loc[jc].x, cur.loc[jc].y};
+        bf16x4 o4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float a0 = __uint_as_float((i & 1) ? (w[i >> 1] & 0xffff0000u) : (w[i >> 1] << 16));
+          o4[i] = (__bf16)(a0 + hcur[i] * cur.dc[jc]);
+        }
+        *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + d) = o4;
+      }
+    }
+    hcur[0] = hcur[0] * cur.dt + cur.he.x;
+    hcur[1] = hcur[1] * cur.dt + cur.he.y;
+    hcur[2] = hcur[2] * cur.dt + cur.he.z;
+    hcur[3] = hcur[3] * cur.dt + cur.he.w;
+    cur = nxt;
+  }
+  if (p.hkt) {
+    if (isv) {
+      *reinterpret_cast<float4*>(p.hvt + (((int64_t)n * H + h) * MS + m) * D + d) = make_float4(hcur[0], hcur[1], hcur[2], hcur[3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p.hkt[(((int64_t)n * H + h) * D + d + i) * MS + m] = hcur[i];
+    }
+  }
+}
+
 // ==========================================================================================
 // output pass
 #ifdef NHA_PROF
@@ -382,8 +379,6 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
 // chunk-start k-state, k_gsa rows, chunk-start v-state, v rows) fit at once when TK = 64 and
 // in two stages when TK = 32.  The decay factors s_j[m] exp(gr[m] - gc_j[m]) that every wave
 // needs are computed once per workgroup into LDS, already in MFMA fragment order.
-constexpr int NSEA = 24;   // fragments s*decay with rows = slots  (A operand of the logit update)
-constexpr int NSEB = 20;   // fragments s*decay with rows = tokens (A operand of the slot-read weights)
 
 template <int D, int TK>
 struct OutSmem {
@@ -393,8 +388,6 @@ struct OutSmem {
       4 * tile_bytes + (size_t)BT * GLD * 4 + (size_t)BT * SLD * 2 + (size_t)(NSEA + NSEB) * 512 * 2;
 };
 
-__device__ __forceinline__ int sea_base(int Q) { return Q == 0 ? 0 : Q == 1 ? 4 : Q == 2 ? 8 : 16; }
-__device__ __forceinline__ int seb_base(int Q) { return Q == 0 ? 0 : Q == 1 ? 2 : Q == 2 ? 6 : 12; }
 
 template <int D, int G, int NW, int TK>
 __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
@@ -503,46 +496,14 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   const int64_t grow_s = (int64_t)c0 - p.shift;
   // Every global load of this phase is issued before the first result is used, so the phase costs
   // one memory latency, not one per tile.
-  constexpr int NPS = BT * D / 8 / NTHR;   // 16-byte pieces per thread of a 64-row tile
-  struct StateRegs {
-    uint4 lk[NPS];        // segment-local state, bf16
-    float4 k0[NPS], k1[NPS];   // segment-start state, fp32
-    float dc[NPS];        // decay from the segment start to the chunk start
+  // chunk-start states are plain [m][d] bf16 tiles (the state pass leaves the true states)
+  auto issue_state = [&](TileRegs<BT, D, NTHR>& r, const bf16_t* hst) {
+    tile_g2r<BT, D, NTHR>(r, hst + cg * MS * D, (int64_t)D, 0, 0, BT, tid);
   };
-  // true chunk-start state = segment-local state + decayed segment-start state
-  auto issue_state = [&](StateRegs& r, const bf16_t* hloc, const float* hseg) {
-    const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
-#pragma unroll
-    for (int u = 0; u < NPS; ++u) {
-      const int c = tid + NTHR * u;
-      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
-      r.dc[u] = p.dcum[cg * MS + row];
-      r.lk[u] = *reinterpret_cast<const uint4*>(hloc + (cg * MS + row) * D + col);
-      const float* sk = hseg + (sl * MS + row) * D + col;
-      r.k0[u] = *reinterpret_cast<const float4*>(sk);
-      r.k1[u] = *reinterpret_cast<const float4*>(sk + 4);
-    }
-  };
-  auto commit_state = [&](lbf16* dst, const StateRegs& r) {
-#pragma unroll
-    for (int u = 0; u < NPS; ++u) {
-      const int c = tid + NTHR * u;
-      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
-      const float kf[8] = {r.k0[u].x, r.k0[u].y, r.k0[u].z, r.k0[u].w, r.k1[u].x, r.k1[u].y, r.k1[u].z, r.k1[u].w};
-      const uint32_t lkw[4] = {r.lk[u].x, r.lk[u].y, r.lk[u].z, r.lk[u].w};
-      bf16x8 o8;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float a0 = __uint_as_float((e & 1) ? (lkw[e >> 1] & 0xffff0000u) : (lkw[e >> 1] << 16));
-        o8[e] = (__bf16)(a0 + kf[e] * r.dc[u]);
-      }
-      *reinterpret_cast<NHA_LDS bf16x8*>(dst + row * LDT + col) = o8;
-    }
-  };
-  auto load_state_tile = [&](lbf16* dst, const bf16_t* hloc, const float* hseg) {
-    StateRegs r;
-    issue_state(r, hloc, hseg);
-    commit_state(dst, r);
+  auto load_state_tile = [&](lbf16* dst, const bf16_t* hst) {
+    TileRegs<BT, D, NTHR> r;
+    issue_state(r, hst);
+    tile_r2l<BT, D, NTHR>(dst, r, tid);
   };
   auto load_rows_tile = [&](lbf16* dst, const bf16_t* src) {
     TileRegs<BT, D, NTHR> t;
@@ -550,15 +511,14 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     tile_r2l<BT, D, NTHR>(dst, t, tid);
   };
   {
-    StateRegs ra, rc;
-    TileRegs<BT, D, NTHR> tb, td;
+    TileRegs<BT, D, NTHR> ra, rc, tb, td;
     constexpr int NG4 = 1024 / NTHR, NS8 = (512 + NTHR - 1) / NTHR;
     float4 gx[NG4];
     uint4 sx[NS8];
-    issue_state(ra, p.hkT, p.hseg_k);
+    issue_state(ra, p.hkT);
     tile_g2r<BT, D, NTHR>(tb, p.k_gsa + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
     if (TK == 64) {
-      issue_state(rc, p.hvc, p.hseg_v);
+      issue_state(rc, p.hvc);
       tile_g2r<BT, D, NTHR>(td, p.v + (int64_t)h * D, (int64_t)H * D, grow_s, vlo, rows, tid);
     }
     // gate cumsum table (fp32 [64][64]); rows past the sequence end are zero
@@ -581,10 +541,10 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     issue_window(0);
     PROF_STAGE(6)
     __builtin_amdgcn_sched_barrier(0);
-    commit_state(tA, ra);
+    tile_r2l<BT, D, NTHR>(tA, ra, tid);
     tile_r2l<BT, D, NTHR>(tB, tb, tid);
     if (TK == 64) {
-      commit_state(tC, rc);
+      tile_r2l<BT, D, NTHR>(tC, rc, tid);
       tile_r2l<BT, D, NTHR>(tD, td, tid);
     }
 #pragma unroll
@@ -788,7 +748,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   if (TK == 32) {
     // second stage of the slot-branch tiles: the state / row tiles of the value side
     __syncthreads();
-    load_state_tile(tC, p.hvc, p.hseg_v);
+    load_state_tile(tC, p.hvc);
     load_rows_tile(tD, p.v);
     __syncthreads();
   }
@@ -1033,12 +993,10 @@ __global__ __launch_bounds__(256) void mfma_repair_kernel(const MP p) {
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int rows = (eos - c0) < BT ? (eos - c0) : BT;
-  const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
   for (int e = tid; e < MS * D; e += 256) {
     const int m = e / D, d = e % D;
-    const float dc = p.dcum[cg * MS + m];
-    hk[m * LDH + d] = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
-    hv[m * D + d] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
+    hk[m * LDH + d] = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]);
+    hv[m * D + d] = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]);
   }
   for (int e = tid; e < BT * MS; e += 256) gcl[e] = p.gc[cg * BT * MS + e];
 
@@ -1134,15 +1092,13 @@ __global__ __launch_bounds__(256) void mfma_repair_kernel(const MP p) {
 
 template <int D>
 int launch_repair(const MP& p, hipStream_t st) {
-  static bool configured = false;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
   const size_t lds = RepairSmem<D>::floats * 4;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)mfma_repair_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) {
-      set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-      return NHA_ERR_LAUNCH;
-    }
-    configured = true;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)mfma_repair_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
   }
   hipLaunchKernelGGL((mfma_repair_kernel<D>), dim3(p.NT, p.H), dim3(256), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma repair pass)");
@@ -1199,18 +1155,36 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
 
 template <int D, int G, int NW, int TK>
 int launch_out(const MP& p, hipStream_t st) {
-  static bool configured = false;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
   const size_t lds = OutSmem<D, TK>::bytes;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G, NW, TK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) {
-      set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-      return NHA_ERR_LAUNCH;
-    }
-    configured = true;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)mfma_out_kernel<D, G, NW, TK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
   }
   hipLaunchKernelGGL((mfma_out_kernel<D, G, NW, TK>), dim3(p.H * (p.NG / G), p.NT), dim3(64 * NW), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass)");
+  return NHA_OK;
+}
+
+// state pass: level 1, then level 2 in the forward form (true chunk-start states in place) or, for
+// the backward's state export, in the segment form (segment-start states beside the local ones)
+template <int D>
+int run_state_pass(const MP& p, bool segment_form, hipStream_t st) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  const size_t lds = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H, 2), dim3(256), lds, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
+  if (segment_form) hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((state_final_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
   return NHA_OK;
 }
 
@@ -1221,20 +1195,8 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     return NHA_ERR_UNSUPPORTED;
   }
   if (phases != 2) {
-    static bool configured = false;
-    const size_t lds = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) {
-        set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        return NHA_ERR_LAUNCH;
-      }
-      configured = true;
-    }
-    hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H, 2), dim3(256), lds, st, p);
-    NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
-    hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
-    NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
+    const int rc = run_state_pass<D>(p, false, st);
+    if (rc != NHA_OK) return rc;
   }
   if (phases != 1) {
     // G query heads of one kv-head share a workgroup.  D <= 128: 64-key tiles, 8 waves of 32 (G = 4)
@@ -1326,7 +1288,7 @@ int prefill_mfma_impl(const NhaPrefillArgs* a) {
   return run_mfma<256>(p, a->phases, st);
 }
 
-// `a` describes a finished state pass (phases = 1) with its scratch; gc [T_tot][H][M], hkc
+// Runs the state pass of `a` in the segment form and exports it; gc [T_tot][H][M], hkc
 // [NT][H][K][M], hkct [NT][H][M][K], hvct [NT][H][V][M] receive fp32 copies, hkb [NT][H][M][K] and
 // hvb [NT][H][M][V] bf16 copies with their low parts hkl, hvl (hkc, hkct, hvct may be NULL together), big [NT][H] the flag of
 // chunks with a decay beyond e^-80
@@ -1334,6 +1296,12 @@ int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, f
                                void* hkl, void* hvl, int* big) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
+  if (p.NT > 65535) {
+    set_error("nha_prefill_bwd(mfma): more than 65535 chunks (%d) in one call", p.NT);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  const int rcs = a->K == 64 ? run_state_pass<64>(p, true, st) : a->K == 128 ? run_state_pass<128>(p, true, st) : run_state_pass<256>(p, true, st);
+  if (rcs != NHA_OK) return rcs;
   const dim3 grid(a->NT, a->H);
   if (a->K == 64) hipLaunchKernelGGL((export_states_kernel<64>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb, (bf16_t*)hkl, (bf16_t*)hvl, big);
   else if (a->K == 128) hipLaunchKernelGGL((export_states_kernel<128>), grid, dim3(256), 0, st, p, gc, hkc, hkct, hvct, (bf16_t*)hkb, (bf16_t*)hvb, (bf16_t*)hkl, (bf16_t*)hvl, big);
