@@ -21,7 +21,7 @@ FLAGS = [
 
 # the MFMA kernels never produce NaN on purpose; without this flag every fmaxf operand is
 # canonicalised by an extra VALU instruction in the softmax inner loop
-EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "decode_mfma.hip": ["-fno-honor-nans"],
+EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "prefill_ring.hip": ["-fno-honor-nans"], "decode_mfma.hip": ["-fno-honor-nans"],
          "prefill_bwd_mfma.hip": ["-fno-honor-nans"]}
 
 

@@ -18,6 +18,7 @@
 #include "mfma_common.h"
 
 #include <mutex>
+#include <stdlib.h>
 
 namespace nha {
 namespace {
@@ -1203,7 +1204,10 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     // or 16 (G = 2) query rows, two per SIMD; D = 256: 32-key tiles and 16-row waves to fit the
     // register file and LDS
     int rc;
-    if constexpr (D <= 128) {
+    static const bool ring_off = getenv("NHA_PREFILL_NO_RING") != nullptr;   // A/B switch for measurements
+    if (!ring_off && prefill_ring_supported(p, D)) {
+      rc = prefill_ring_launch(p, D, st);
+    } else if constexpr (D <= 128) {
       if (p.NG % 4 == 0) rc = launch_out<D, 4, 8, 64>(p, st);
       else if (p.NG % 2 == 0) rc = launch_out<D, 2, 8, 64>(p, st);
       else rc = launch_out<D, 1, 4, 64>(p, st);

@@ -1,6 +1,742 @@
-// placeholder translation unit, filled in below
+// Output pass of the bf16 matrix-core prefill for groups of four query heads per kv-head (K == V == D
+// in {64, 128}, M == 64): same mathematics as mfma_out_kernel (prefill_mfma.hip; chunk algebra of
+// nha_fla/ops/nha/chunk_fused.py:186-283, one softmax over [slots | window] as in
+// nha_fla/ops/nha/chunk.py:459-470), different data movement and order.
+//
+//  * Every operand tile goes from global memory straight into LDS (global_load_lds_dwordx4, 1 KB
+//    per wave instruction): no staging registers, no LDS stores, and the loads of the slot branch
+//    are requested at the start and land while the window loop runs.
+//  * The sliding window is walked first, in units of 32 keys through a ring of NR unit buffers; the
+//    slot branch (which only needs the chunk-start states and the chunk's own rows) is folded into
+//    the running softmax afterwards.
+//  * The window loop is software-pipelined inside each wave: while the matrix core forms the scores
+//    of unit u+1, the VALU exponentiates unit u; while it accumulates P.V of unit u, the VALU takes
+//    the row maxima of unit u+1.  The scale and the running maximum are folded into the score
+//    product itself (pre-scaled queries, accumulator started at -max), so a score needs one
+//    v_exp_f32 and half a v_cvt_pk_bf16_f32 and nothing else on the common path.
+//
+// LDS layouts (bank-conflict free for the two fragment reads without padding, which a 1 KB wave
+// load cannot produce): a 32-row unit is cut into 16-row x 32-column blocks of 1 KB, a row of a block
+// is 64 contiguous bytes.  "K layout" (row fragments, ds_read_b128) XORs the 16-byte piece index
+// inside a row with (row / 4) % 4; "V layout" (transposing ds_read_b64_tr_b16) stores pieces in order.
 #include "mfma_common.h"
+
+#include <mutex>
+
 namespace nha {
-bool prefill_ring_supported(const mf::MP&, int) { return false; }
-int prefill_ring_launch(const mf::MP&, int, hipStream_t) { return NHA_ERR_UNSUPPORTED; }
+namespace {
+using namespace mf;
+
+typedef NHA_LDS unsigned char lbyte;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// nothing crosses: the instruction order of the loop is the source order
+#define NHA_FENCE() __builtin_amdgcn_sched_barrier(0)
+// keeps a value, and the arithmetic that made it, where the source has it
+#define NHA_PIN(x) asm volatile("" : "+v"(x))
+
+__device__ __forceinline__ unsigned cvt2(float a, float b) {
+  bf16x2 t;
+  t[0] = (__bf16)a;
+  t[1] = (__bf16)b;
+  return __builtin_bit_cast(unsigned, t);
+}
+
+// 16 bytes per lane from global memory into LDS at lds_base + 16 * lane (lds_base wave-uniform).
+// Issued outside the compiler's memory model: every wait on these loads is written by hand.
+__device__ __forceinline__ void g2l16(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int D>
+struct RingCfg {
+  static constexpr int KS = D / 32;            // 32-column blocks per row == contraction steps of q.k
+  static constexpr int DB = D / 16;            // 16-row blocks of O^T
+  static constexpr int UB = 32 * D * 2;        // bytes of a 32-row unit
+  static constexpr int HB = UB / 2;            // bytes of its 16-row half
+  static constexpr int NR = 512 / D;           // ring slots (64 KB of K and V units together)
+  static constexpr int LPW = KS / 2;           // LDS-direct loads per wave for a unit (K and V) or a 64-row tile
+  static constexpr int RING_K = 0, RING_V = NR * UB;
+  static constexpr int TA = 2 * NR * UB;       // chunk-start k-state [m][d], K layout
+  static constexpr int TB = TA + 2 * UB;       // k_gsa rows, K layout
+  static constexpr int TC = TB + 2 * UB;       // chunk-start v-state [m][d], V layout
+  static constexpr int TD = TC + 2 * UB;       // v rows, V layout
+  static constexpr int GC = TD + 2 * UB;       // gate cumsum fp32 [64][64], pieces XORed with row % 16
+  static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
+  static constexpr int BYTES = SS + 8192;
+  static constexpr int SEA = 0;                // decay-factor fragments, over the ring once the window is done
+  static constexpr int SEB = NSEA * 1024;
+  static constexpr int NSLOT_LOADS = 4 * LPW + 3;   // per wave: four tiles, two gate blocks, one s block
+  static_assert((NSEA + NSEB) * 1024 <= 2 * NR * UB, "decay fragments must fit the ring");
+};
+
+template <int D>
+__global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
+  using C = RingCfg<D>;
+  constexpr int KS = C::KS, DB = C::DB, UB = C::UB, HB = C::HB, NR = C::NR, LPW = C::LPW;
+  constexpr int RQB = 2;                        // 16-row query blocks per wave
+  constexpr int NPRE = NR - 1;                  // units requested before the loop
+  extern __shared__ __align__(1024) unsigned char smem_[];
+#ifdef NHA_RING_STAMPS
+  long long st_[8];
+  st_[0] = __builtin_amdgcn_s_memtime();
+#define NHA_STAMP(k) st_[k] = __builtin_amdgcn_s_memtime()
+#else
+#define NHA_STAMP(k)
+#endif
+  lbyte* const lds = (lbyte*)smem_;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ, NG = p.NG;
+  // grid = (kv-head x group of four q-heads, chunk), chunks from the last to the first (prefill_mfma.hip)
+  const int chunk = p.NT - 1 - blockIdx.y;
+  const int ngrp = NG / 4;
+  const int h = blockIdx.x / ngrp, grp = blockIdx.x % ngrp;
+  const int hq = h * NG + grp * 4 + wave / 2;
+  const int qb0 = (wave % 2) * RQB;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int rows = (eos - c0) < BT ? (eos - c0) : BT;
+  const float cs = p.scale * LOG2E;
+  const int64_t cg = (int64_t)chunk * H + h;
+
+  // window units: unit u covers keys [c0 + 32 - 32 u, c0 + 64 - 32 u); c0 - bos is a multiple of 64, so no
+  // unit starts before its sequence; units 0 and 1 are the chunk's own rows and may run past eos
+  int lowest = bos;
+  if (p.wl >= 0 && c0 - p.wl > bos) lowest = c0 - p.wl;
+  const int nunits = (c0 + 64 - lowest + 31) / 32;   // >= 2
+
+  // ---- load descriptors of this wave: LDS-direct load i of a unit / a 64-row tile ------------------
+  // block index b = wave + 8 i; per lane: row lane / 4 of the block, piece lane % 4 of its 64-byte row
+  const int lrow16 = lane >> 2, lsl = lane & 3, lswz = lsl ^ ((lane >> 4) & 3);
+  uint32_t u_off[LPW];          // byte offset from the unit's first row (token rows, stride H*D)
+  uint32_t u_lds[LPW];          // LDS address of the block inside ring slot 0
+  bool u_isv[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int b = wave + 8 * i;
+    const bool isv = b >= 2 * KS;
+    const int bb = isv ? b - 2 * KS : b;
+    const int rh = bb / KS, cq = bb % KS;
+    u_isv[i] = isv;
+    u_off[i] = ((uint32_t)(16 * rh + lrow16) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lsl : lswz)) * 8) * 2;
+    u_lds[i] = lds0 + (isv ? C::RING_V : C::RING_K) + rh * HB + cq * 1024;
+  }
+  // request unit u; rows past eos (units 0 and 1 only) are read from row eos - 1: always masked, always finite
+  auto issue_unit_checked = [&](int u) {
+    const int key0 = c0 + 32 - 32 * u;
+    const int slot = u & (NR - 1);
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int b = wave + 8 * i;
+      const bool isv = b >= 2 * KS;
+      const int bb = isv ? b - 2 * KS : b;
+      const int rh = bb / KS, cq = bb % KS;
+      int row = key0 + 16 * rh + lrow16;
+      row = row < eos ? row : eos - 1;
+      const uint32_t off = ((uint32_t)(row - bos) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lsl : lswz)) * 8) * 2;
+      const bf16_t* base = (isv ? p.v : p.k_swa) + ((int64_t)bos * H + h) * D;
+      g2l16(base, off, u_lds[i] + slot * UB);
+    }
+  };
+  // 64-row tile of the slot branch: kind 0 = K layout, 1 = V layout; rows of `src` with `stride` elements,
+  // row r of the tile is global row rowmap(r)
+  auto issue_tile = [&](int lds_tile, bool vlay, const bf16_t* src, uint32_t stride, auto rowmap) {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int b = wave + 8 * i;            // < 4 KS
+      const int unit = b / (2 * KS), bb = b % (2 * KS);
+      const int rh = bb / KS, cq = bb % KS;
+      const int r = 32 * unit + 16 * rh + lrow16;
+      const uint32_t off = ((uint32_t)rowmap(r) * stride + (uint32_t)(4 * cq + (vlay ? lsl : lswz)) * 8) * 2;
+      g2l16(src, off, lds0 + lds_tile + unit * UB + rh * HB + cq * 1024);
+    }
+  };
+
+  // ---- requests: the first window units, then the query fragments ---------------------------------
+#pragma unroll
+  for (int u = 0; u < NPRE; ++u)
+    if (u < nunits) issue_unit_checked(u);
+
+  // window-query fragments, pre-scaled by scale * log2(e): scores come out of the matrix core in the
+  // units the exponential wants
+  bf16x8 qs[RQB][KS];
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const int irow = 16 * (qb0 + qb) + l16;
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+      bf16x8 r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+        r[e] = (__bf16)(f * cs);
+      }
+      qs[qb][ks] = r;
+    }
+  }
+  // (the compiler has waited for the query loads, and with them for the unit loads before them)
+
+  // ---- requests of the slot branch: made in the first loop iteration, they land while the window loop runs
+  const int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);   // first row of the chunk whose source token exists
+  auto issue_slot_operands = [&]() {
+    const int grow_s = c0 - p.shift;   // source token of row 0
+    auto tok = [&](int r) {            // source token of row r, kept inside the sequence (rows outside [vlo, rows) carry no weight)
+      int t = grow_s + r;
+      t = t < bos ? bos : t;
+      t = t < eos ? t : eos - 1;
+      return t - bos;
+    };
+    auto ident = [&](int r) { return r; };
+    issue_tile(C::TA, false, p.hkT + cg * MS * D, (uint32_t)D, ident);
+    issue_tile(C::TB, false, p.k_gsa + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
+    issue_tile(C::TC, true, p.hvc + cg * MS * D, (uint32_t)D, ident);
+    issue_tile(C::TD, true, p.v + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
+    // gate cumsums: 16 blocks of 4 rows; rows >= `rows` were never written by the state pass and stay unused
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int b = wave + 8 * i;
+      const int r = 4 * b + (lane >> 4);
+      const int c = (lane & 15) ^ (r & 15);
+      g2l16(p.gc + cg * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + C::GC + b * 1024);
+    }
+    {
+      const int r = 8 * wave + (lane >> 3);
+      const int c = (lane & 7) ^ (r & 7);
+      g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok(r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + wave * 1024);
+    }
+  };
+
+  // ---- window loop state ------------------------------------------------------------------------
+  f32x4 O[DB][RQB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) O[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  f32x4 Lw[RQB];
+  float nm[RQB];     // minus the running reference maximum, log2 units
+  f32x4 nmv[RQB];    // nm broadcast: the accumulator the score products start from
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    Lw[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    nm[qb] = 0.f;
+    nmv[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
+  // lazy rescaling: the reference only moves when a score exceeds it by more than 2^THR
+  constexpr float THR = 8.f;
+
+  const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
+  const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 64 + 8 * (l16 & 3));
+  // row fragment (rows 16 kk + l16 of a unit, columns 32 ks + 8 kb ..) of a K-layout unit at byte address a
+  auto kfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {
+    return *reinterpret_cast<const NHA_LDS bf16x8*>(lds + a + kk * HB + ks * 1024);
+  };
+  // transposed fragment of a V-layout unit: X[4 kb + e][16 db + l16] (e < 4) and X[16 + 4 kb + e - 4][..]
+  auto vfrag = [&](uint32_t a, int db) -> bf16x8 {
+    const lbyte* pa = lds + a + (db >> 1) * 1024 + (db & 1) * 32;
+    struct { s16x4 a, b; } t;
+    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + HB));
+    return __builtin_bit_cast(bf16x8, t);
+  };
+  auto mask_unit = [&](f32x4 (&S)[2][RQB], int u) {
+    const int xbase = 32 - 32 * u;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) {
+        const int y = 16 * (qb0 + qb) + l16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int x = xbase + 16 * kk + 4 * kb + r;
+          const bool ok = (x <= y) && (p.wl < 0 || x >= y - p.wl);
+          if (!ok) S[kk][qb][r] = -INFINITY;
+        }
+      }
+  };
+  auto is_edge = [&](int u) -> bool { return (63 - 32 * u > 0) || (p.wl >= 0 && 32 - 32 * u < 63 - p.wl); };
+  // the reference of column qb moves up by delta: everything accumulated so far shrinks by 2^-delta
+  auto rescale_acc = [&](int qb, float delta) {
+    const float alpha = fexp2(-delta);
+    nm[qb] -= delta;
+    nmv[qb] = (f32x4){nm[qb], nm[qb], nm[qb], nm[qb]};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Lw[qb][r] *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[db][qb][r] *= alpha;
+  };
+  auto rescale = [&](f32x4 (&S)[2][RQB], const float (&rmax)[RQB]) {
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      const float delta = fmaxf(max_over_rows(rmax[qb]), 0.f);
+      rescale_acc(qb, delta);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[kk][qb][r] -= delta;
+    }
+  };
+
+  f32x4 Sc[2][RQB], Sn[2][RQB];
+  bf16x8 kf[KS][2];
+  bf16x8 vf[DB];
+  // ---- prologue: scores of unit 0, K fragments of unit 1 -----------------------------------------------
+  // units 0 .. NPRE-1 have landed for this wave
+  NHA_STAMP(1);
+  wait_vm<0>();
+  lds_barrier();
+  {
+    const uint32_t k0 = C::RING_K + kaddr;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) Sc[kk][qb] = nmv[qb];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 a0 = kfrag(k0, 0, ks), a1 = kfrag(k0, 1, ks);
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) {
+        Sc[0][qb] = mfma16(a0, qs[qb][ks], Sc[0][qb]);
+        Sc[1][qb] = mfma16(a1, qs[qb][ks], Sc[1][qb]);
+      }
+    }
+    mask_unit(Sc, 0);   // unit 0 is always an edge unit
+    float rmax[RQB];
+    bool need = false;
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      float x = fmaxf(fmaxf(Sc[0][qb][0], Sc[0][qb][1]), fmaxf(Sc[0][qb][2], Sc[0][qb][3]));
+      x = fmaxf(x, fmaxf(fmaxf(Sc[1][qb][0], Sc[1][qb][1]), fmaxf(Sc[1][qb][2], Sc[1][qb][3])));
+      rmax[qb] = x;
+      need |= x > THR;
+    }
+    if (__any(need)) rescale(Sc, rmax);
+    const uint32_t k1 = C::RING_K + (1 & (NR - 1)) * UB + kaddr;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks][0] = kfrag(k1, 0, ks);
+      kf[ks][1] = kfrag(k1, 1, ks);
+    }
+  }
+  // global position of the next unit to request (unit NPRE at u = 0), 32 rows back per iteration
+  const bf16_t* kreq = p.k_swa + (((int64_t)c0 + 32 - 32 * NPRE) * H + h) * D;
+  const bf16_t* vreq = p.v + (((int64_t)c0 + 32 - 32 * NPRE) * H + h) * D;
+  const int64_t ustep = (int64_t)32 * H * D;
+
+  NHA_STAMP(2);
+  for (int u = 0; u < nunits; ++u) {
+    const uint32_t k_nn = C::RING_K + ((u + 2) & (NR - 1)) * UB + kaddr;   // K of unit u+2 (after the barrier)
+    const uint32_t v_c = C::RING_V + (u & (NR - 1)) * UB + vaddr;           // V of unit u
+    const bool has_next = u + 1 < nunits;
+    // ---- phase A: scores of unit u+1 on the matrix core, exponentials of unit u on the VALU,
+    //      V fragments of unit u requested from LDS ----
+    unsigned pw[RQB][4];
+    NHA_FENCE();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kk = j & 1, qb = j >> 1;
+        // DB / (4 KS) = 1/2 V fragment per score product
+        if ((j & 1) == 0) vf[2 * ks + (j >> 1)] = vfrag(v_c, 2 * ks + (j >> 1));
+        Sn[kk][qb] = mfma16(kf[ks][kk], qs[qb][ks], ks == 0 ? nmv[qb] : Sn[kk][qb]);
+        // a score block of the current unit per contraction step: with KS = 4 block (ks & 1, ks >> 1),
+        // with KS = 2 blocks (0, ks) and (1, ks)
+        if (KS == 4) {
+          Sc[ks & 1][ks >> 1][j] = fexp2(Sc[ks & 1][ks >> 1][j]);
+          NHA_PIN(Sc[ks & 1][ks >> 1][j]);
+        } else {
+          Sc[0][ks][j] = fexp2(Sc[0][ks][j]);
+          NHA_PIN(Sc[0][ks][j]);
+          Sc[1][ks][j] = fexp2(Sc[1][ks][j]);
+          NHA_PIN(Sc[1][ks][j]);
+        }
+        NHA_FENCE();
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      pw[qb][0] = cvt2(Sc[0][qb][0], Sc[0][qb][1]);
+      pw[qb][1] = cvt2(Sc[0][qb][2], Sc[0][qb][3]);
+      pw[qb][2] = cvt2(Sc[1][qb][0], Sc[1][qb][1]);
+      pw[qb][3] = cvt2(Sc[1][qb][2], Sc[1][qb][3]);
+    }
+    bf16x8 Pq[RQB];
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      const u32x4 t = {pw[qb][0], pw[qb][1], pw[qb][2], pw[qb][3]};
+      Pq[qb] = __builtin_bit_cast(bf16x8, t);
+      NHA_PIN(Pq[qb]);
+    }
+    NHA_FENCE();
+    // unit u+2 has landed (this wave's part; at most the requests of unit u+3 stay in flight), then
+    // everybody's; after the barrier the slot of unit u-1 is free and takes unit u+NPRE
+    // (the requests younger than unit u+2: units u+3 .. u+NR-2, and the slot-branch operands while
+    // u <= NR-3, which were queued behind unit NR-1 in iteration 0)
+    if (u + 2 < nunits) {
+      if (u + NR - 2 < nunits) {
+        if (u >= 1 && u <= NR - 3) wait_vm<LPW * (NR - 4) + C::NSLOT_LOADS>();
+        else wait_vm<LPW * (NR - 4)>();
+      } else {
+        wait_vm<0>();
+      }
+    }
+    lds_barrier();
+    if (u + NPRE < nunits) {
+      const int slot = (u + NPRE) & (NR - 1);
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) g2l16(u_isv[i] ? vreq : kreq, u_off[i], u_lds[i] + slot * UB);
+    }
+    if (u == 0) issue_slot_operands();
+    kreq -= ustep;
+    vreq -= ustep;
+    NHA_FENCE();
+    // ---- phase B: value products of unit u on the matrix core, row maxima of unit u+1 on the VALU,
+    //      K fragments of unit u+2 requested from LDS ----
+    float m0[RQB], m1[RQB];
+    auto max_step = [&](int step) {
+      const int q2 = step >> 3, s2 = step & 7;
+      if (s2 == 0) m0[q2] = fmaxf(Sn[0][q2][0], Sn[0][q2][1]);
+      if (s2 == 1) m1[q2] = fmaxf(Sn[0][q2][2], Sn[0][q2][3]);
+      if (s2 == 2) m0[q2] = fmaxf(fmaxf(m0[q2], Sn[1][q2][0]), Sn[1][q2][1]);
+      if (s2 == 3) m1[q2] = fmaxf(fmaxf(m1[q2], Sn[1][q2][2]), Sn[1][q2][3]);
+      if (s2 == 4) m0[q2] = fmaxf(m0[q2], m1[q2]);
+      if (s2 == 0 || s2 == 2 || s2 == 4) NHA_PIN(m0[q2]);
+      if (s2 == 1 || s2 == 3) NHA_PIN(m1[q2]);
+    };
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      Lw[qb] = mfma16(ones, Pq[qb], Lw[qb]);
+      NHA_FENCE();
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      if (db < 2 * KS) kf[db >> 1][db & 1] = kfrag(k_nn, db & 1, db >> 1);
+      NHA_FENCE();
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) {
+        O[db][qb] = mfma16(vf[db], Pq[qb], O[db][qb]);
+        // the row maxima of the next unit take 10 steps (5 per query block) spread over the 2 DB products
+        if (DB >= 8) {
+          max_step(2 * db + qb);
+        } else {
+          max_step(2 * (2 * db + qb));
+          max_step(2 * (2 * db + qb) + 1);
+        }
+        NHA_FENCE();
+      }
+    }
+    if (has_next) {
+      if (is_edge(u + 1)) {
+        mask_unit(Sn, u + 1);
+#pragma unroll
+        for (int qb = 0; qb < RQB; ++qb) {
+          float x = fmaxf(fmaxf(Sn[0][qb][0], Sn[0][qb][1]), fmaxf(Sn[0][qb][2], Sn[0][qb][3]));
+          m0[qb] = fmaxf(x, fmaxf(fmaxf(Sn[1][qb][0], Sn[1][qb][1]), fmaxf(Sn[1][qb][2], Sn[1][qb][3])));
+        }
+      }
+      bool need = false;
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) need |= m0[qb] > THR;
+      if (__any(need)) rescale(Sn, m0);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) Sc[kk][qb] = Sn[kk][qb];
+  }
+
+  NHA_STAMP(3);
+  // ================= slot branch, folded into the running softmax =================================
+  // slot-branch query fragments of the first query block: requested now, used after the decay fragments
+  // are built; those of the second block are requested while the first is worked on
+  auto load_qg = [&](bf16x8 (&q)[KS], int qb) {
+    const int irow = 16 * (qb0 + qb) + l16;
+    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      q[ks] = as_bf16x8(x);
+    }
+  };
+  bf16x8 qg[KS];
+  load_qg(qg, 0);
+  // every LDS-direct request of this wave has landed, every wave is done with the ring
+  wait_vm<0>();
+  lds_barrier();
+  NHA_STAMP(4);
+  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
+  auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
+  // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
+  // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows j of
+  // earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.  Rows whose
+  // source token does not exist (before the sequence, past its end) carry no weight.
+  for (int item = tid; item < (NSEA + NSEB) * 64; item += 512) {
+    const int f = item >> 6, ln = item & 63;
+    const int fl16 = ln & 15, fkb = ln >> 4;
+    bf16x8 out;
+    if (f < NSEA) {
+      const int Q = f < 4 ? 0 : f < 8 ? 1 : f < 16 ? 2 : 3;
+      const int rem = f - sea_base(Q);
+      const int pr = rem >> 2, mb = rem & 3;
+      const int m = 16 * mb + fl16;
+      const float gr = Q > 0 ? *gc_at(16 * Q - 1, m) : 0.f;
+      float gv[8];
+      bf16_t sv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = 16 * (2 * pr + (e >> 2)) + 4 * fkb + (e & 3);   // j < 64 for every fragment
+        gv[e] = *gc_at(j, m);
+        sv[e] = *s_at(j, m);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int jb = 2 * pr + (e >> 2);
+        const int j = 16 * jb + 4 * fkb + (e & 3);
+        const float val = bf16_to_f32(sv[e]) * fexp(fminf(gr - gv[e], DECAY_CLAMP));
+        out[e] = (__bf16)((jb <= Q && j >= vlo && j < rows) ? val : 0.f);
+      }
+      *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::SEA + f * 1024 + ln * 16) = out;
+    } else {
+      const int g2 = f - NSEA;
+      const int Q = g2 < 2 ? 0 : g2 < 6 ? 1 : g2 < 12 ? 2 : 3;
+      const int rem = g2 - seb_base(Q);
+      const int jb = rem >> 1, pr = rem & 1;
+      const int j = 16 * jb + fl16;
+      const bool jok = j >= vlo && j < rows;
+      f32x4 gv[2], gr[2];
+      bf16x4 sv[2];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int m0s = 32 * pr + 16 * hh + 4 * fkb;   // the lane's 4 consecutive slots of this half
+        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m0s));
+        gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (Q > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Q - 1, m0s));
+        sv[hh] = *reinterpret_cast<const NHA_LDS bf16x4*>(s_at(j, m0s));
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float val = (float)sv[e >> 2][e & 3] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP));
+        out[e] = (__bf16)(jok ? val : 0.f);
+      }
+      *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::SEB + g2 * 1024 + ln * 16) = out;
+    }
+  }
+  __syncthreads();
+  NHA_STAMP(5);
+
+  float lg[RQB];
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const int Q = qb0 + qb;                // sub-block index inside the chunk
+    const int irow = 16 * Q + l16;         // this lane's query row inside the chunk
+    // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
+    f32x4 ok[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(C::TA + (mb >> 1) * UB + kaddr, mb & 1, ks), qg[ks], ok[mb]);
+    // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
+    bf16x8 bA[2];
+    {
+      f32x4 at[4];
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb)
+          if (jb <= Q) at[jb] = mfma16(kfrag(C::TB + (jb >> 1) * UB + kaddr, jb & 1, ks), qg[ks], at[jb]);
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+        if (jb == Q) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (4 * kb + r > l16) at[jb][r] = 0.f;
+        }
+      bA[0] = pack8(at[0], at[1]);
+      bA[1] = pack8(at[2], at[3]);
+    }
+    if (qb + 1 < RQB) load_qg(qg, qb + 1);
+    // okT_intra[m][i] = sum_j s_j[m] exp(gr[m] - gc_j[m]) AT[j][i]
+    f32x4 oki[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      oki[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr)
+        if (2 * pr <= Q) {
+          const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(lds + C::SEA + (sea_base(Q) + 4 * pr + mb) * 1024 + lane * 16);
+          oki[mb] = mfma16(se, bA[pr], oki[mb]);
+        }
+    }
+    // combine; the slot logits join the running softmax as one more set of keys
+    const int rref = 16 * Q - 1;
+    f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
+    float xmax = -INFINITY;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(irow, 16 * mb + 4 * kb));
+      f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (Q > 0) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(rref, 16 * mb + 4 * kb));
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        egi[mb][r] = fexp(gi[r]);
+        egr[mb][r] = fexp(gi[r] - gr4[r]);
+        ok[mb][r] = (ok[mb][r] * egi[mb][r] + oki[mb][r] * egr[mb][r]) * cs;   // slot logit, log2 units
+        xmax = fmaxf(xmax, ok[mb][r]);
+      }
+    }
+    // relative to the reference of the window pass; the reference moves if a slot logit tops it by 2^THR
+    if (__any(xmax + nm[qb] > THR)) {
+      const float delta = fmaxf(max_over_rows(xmax) + nm[qb], 0.f);
+      rescale_acc(qb, delta);
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        ok[mb][r] = fexp2(ok[mb][r] + nm[qb]);   // unnormalised slot probabilities
+        psum += ok[mb][r];
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    lg[qb] = psum;
+    if (p.lse_gsa && kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(psum) - nm[qb]) * LN2;
+    bf16x8 bp[2], bpr[2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      f32x4 x0, x1, y0, y1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        x0[r] = ok[2 * pr][r] * egi[2 * pr][r];
+        x1[r] = ok[2 * pr + 1][r] * egi[2 * pr + 1][r];
+        y0[r] = ok[2 * pr][r] * egr[2 * pr][r];
+        y1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
+      }
+      bp[pr] = pack8(x0, x1);
+      bpr[pr] = pack8(y0, y1);
+    }
+    // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) O[db][qb] = mfma16(vfrag(C::TC + pr * UB + vaddr, db), bp[pr], O[db][qb]);
+    // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
+    bf16x8 bAv[2];
+    {
+      f32x4 av[4];
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        av[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (jb <= Q) {
+#pragma unroll
+          for (int pr = 0; pr < 2; ++pr) {
+            const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(lds + C::SEB + (seb_base(Q) + 2 * jb + pr) * 1024 + lane * 16);
+            av[jb] = mfma16(se, bpr[pr], av[jb]);
+          }
+          if (jb == Q) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (4 * kb + r > l16) av[jb][r] = 0.f;
+          }
+        }
+      }
+      bAv[0] = pack8(av[0], av[1]);
+      bAv[1] = pack8(av[2], av[3]);
+    }
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+      if (2 * pr <= Q) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) O[db][qb] = mfma16(vfrag(C::TD + pr * UB + vaddr, db), bAv[pr], O[db][qb]);
+      }
+  }
+
+  NHA_STAMP(6);
+  // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
+  //      row block db + 1, and the two trade their halves) -------------------------------------------
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const int irow = 16 * (qb0 + qb) + l16;
+    const float lwt = Lw[qb][0];
+    const float inv = 1.f / (lwt + lg[qb]);
+    bf16_t* op = p.o + ((int64_t)(c0 + irow) * HQ + hq) * D;
+#pragma unroll
+    for (int db = 0; db < DB; db += 2) {
+      unsigned a[2], b[2];
+      a[0] = cvt2(O[db][qb][0] * inv, O[db][qb][1] * inv);
+      a[1] = cvt2(O[db][qb][2] * inv, O[db][qb][3] * inv);
+      b[0] = cvt2(O[db + 1][qb][0] * inv, O[db + 1][qb][1] * inv);
+      b[1] = cvt2(O[db + 1][qb][2] * inv, O[db + 1][qb][3] * inv);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(a[e], b[e], false, false);
+        a[e] = sw[0];
+        b[e] = sw[1];
+      }
+      const int dcol = 16 * (db + (kb & 1)) + 8 * (kb >> 1);
+      if (irow < rows) *reinterpret_cast<uint4*>(op + dcol) = make_uint4(a[0], a[1], b[0], b[1]);
+    }
+    if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(lwt) - nm[qb]) * LN2;
+  }
+#ifdef NHA_RING_STAMPS
+  if (lane == 0 && (wave == 0 || wave == 4)) {
+    st_[7] = __builtin_amdgcn_s_memtime();
+    long long* d = (long long*)p.hseg_k + (((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 10;
+    for (int k = 0; k < 8; ++k) d[k] = st_[k];
+    d[8] = nunits;
+    d[9] = __builtin_amdgcn_s_memrealtime();
+  }
+#endif
+}
+
+template <int D>
+int launch_ring(const MP& p, hipStream_t st) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  const size_t lds = RingCfg<D>::BYTES;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring_out_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((ring_out_kernel<D>), dim3(p.H * (p.NG / 4), p.NT), dim3(512), lds, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass, ring)");
+  return NHA_OK;
+}
+
+}  // namespace
+
+// Served: four (or a multiple of four) query heads per kv-head at D = 64 or 128.  The per-lane byte
+// offsets of the LDS-direct loads are 32 bits: the tensors of one sequence must stay below 4 GiB, which
+// the caller's 32-bit token count times the row size decides.
+bool prefill_ring_supported(const mf::MP& p, int D) {
+  if (!(D == 64 || D == 128) || p.NG % 4 != 0) return false;
+  return (int64_t)p.T_tot * p.H * D * 2 < ((int64_t)1 << 32) && (int64_t)p.T_tot * p.H * MS * 2 < ((int64_t)1 << 32);
+}
+
+int prefill_ring_launch(const mf::MP& p, int D, hipStream_t st) {
+  return D == 64 ? launch_ring<64>(p, st) : launch_ring<128>(p, st);
+}
+
 }  // namespace nha
