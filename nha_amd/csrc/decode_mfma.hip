@@ -88,14 +88,8 @@ static size_t lds_bytes_for(int D, int G, int NW) {
 // once (4 workgroups per CU), so nothing waits for a second round.  The slot branch issues every
 // load it needs up front (popped entry first, then all state rows): its dependent chain is
 // count -> popped row, and no workgroup's state rows queue behind another's window stream.
-// With -DNHA_PROF the kernel records per-wave time stamps (100 MHz) into the buffer whose address
-// is given by the environment variable NHA_PROF_PTR (hex): entry, end of slot branch, end of window
-// branch, exit, then one stamp per window block.
 template <int D, int G, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecodeArgs a, long long* prof) {
-#ifdef NHA_PROF
-  const long long pt0 = __builtin_amdgcn_s_memrealtime();
-#endif
+__global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecodeArgs a) {
   constexpr int NT = 64 * NW;
   constexpr int LDT = D + 16;   // bf16 row stride of a V tile
   constexpr int KS = D / 32;    // MFMA k-steps over the head dim
@@ -436,9 +430,6 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
         O[vt] = mfma16(lds_frag_tr(X, LDT, 16 * vt, lane), P, O[vt]);
       }
       __builtin_amdgcn_sched_barrier(0);
-#ifdef NHA_PROF
-      if (prof && lane == 0 && blk / NW < 28) prof[((int64_t)blockIdx.x * NW + wave) * 32 + 4 + blk / NW] = __builtin_amdgcn_s_memrealtime();
-#endif
     };
     for (int blk = wave; blk < nblk; blk += 2 * NW) {
       process(kr0, vr0, blk);
@@ -457,18 +448,8 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
     }
   };
 
-#ifdef NHA_PROF
-  long long pt1;
-#define PROF_MID { __builtin_amdgcn_sched_barrier(0); pt1 = __builtin_amdgcn_s_memrealtime(); __builtin_amdgcn_sched_barrier(0); }
-#else
-#define PROF_MID
-#endif
   slot_branch();
-  PROF_MID
   window_branch();
-#ifdef NHA_PROF
-  const long long pt2 = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // ---- merge: slots + window partials under one softmax ----------------------------------------
   lds_barrier();
@@ -496,12 +477,6 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
       ((bf16_t*)a.o)[((int64_t)b * HQ + h * NG + g) * D + v] = f32_to_bf16(num / den);
     }
   }
-#ifdef NHA_PROF
-  if (prof && lane == 0) {
-    long long* pr = prof + ((int64_t)blockIdx.x * NW + wave) * 32;
-    pr[0] = pt0; pr[1] = pt1; pr[2] = pt2; pr[3] = __builtin_amdgcn_s_memrealtime();
-  }
-#endif
 }
 
 #ifndef NHA_DEC_NW
@@ -512,7 +487,7 @@ template <int D, int G>
 int launch(const NhaDecodeArgs* a) {
   constexpr int NW = NHA_DEC_NW;
   const size_t lds = lds_bytes_for(D, G, NW);
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured && lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)decode_mfma_kernel<D, G, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
@@ -521,11 +496,7 @@ int launch(const NhaDecodeArgs* a) {
     }
     configured = true;
   }
-  long long* prof = nullptr;
-#ifdef NHA_PROF
-  if (const char* e = getenv("NHA_PROF_PTR")) prof = (long long*)strtoull(e, nullptr, 16);
-#endif
-  hipLaunchKernelGGL((decode_mfma_kernel<D, G, NW>), dim3(a->B * a->H), dim3(64 * NW), lds, (hipStream_t)a->stream, *a, prof);
+  hipLaunchKernelGGL((decode_mfma_kernel<D, G, NW>), dim3(a->B * a->H), dim3(64 * NW), lds, (hipStream_t)a->stream, *a);
   NHA_CHECK_LAUNCH("nha_decode_step");
   return NHA_OK;
 }

@@ -1011,7 +1011,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   const size_t lds_s1 = ((size_t)2 * BT * LM + BT * (BT + 1) + BT * (CB + 1)) * 4 + BT * 4;
   const size_t lds_s3 = ((size_t)CB * LM + 3 * BT * LM + BT * (CB + 1)) * 4 + BT * 4;
   const size_t lds_w = ((size_t)K + V + 512) * 4;
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
     hipError_t e1 = hipFuncSetAttribute((const void*)bwd_intra_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     hipError_t e2 = hipFuncSetAttribute((const void*)bwd_state_inter_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

@@ -1217,7 +1217,7 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
 template <int D, int TK>
 int launch_dq(const WP& p, int NT, hipStream_t st) {
   const size_t lds = (size_t)4 * TK * (D + 16) * 2;
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)bwd_dq_kernel<D, TK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
@@ -1234,7 +1234,7 @@ int launch_dq(const WP& p, int NT, hipStream_t st) {
 template <int D, int TQ, int MODE>
 int launch_dkv(const WP& p, int NT, hipStream_t st) {
   const size_t lds = (size_t)4 * TQ * (D + 16) * 2 + 4 * TQ * 4;
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)bwd_dkv_kernel<D, TQ, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
@@ -1287,7 +1287,7 @@ int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const fl
 template <int D, bool FUSE>
 static int launch_slot_products(const SP1& p, const SP3& pq, int NT, hipStream_t st) {
   const size_t lds = (size_t)2 * BT * (D + 16) * 2 + (FUSE ? (size_t)4 * BT * TLD * 2 + BT * 4 : 0);
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_products_kernel<D, FUSE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
@@ -1342,7 +1342,7 @@ static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
   const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
   const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
   const size_t lds_i = (size_t)BT * (D + 16) * 2 + (size_t)2 * D * (BT + 8) * 2 + (size_t)2 * BT * TLD * 2;
-  static bool configured = false;
+  static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
     hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
     hipError_t e2 = hipFuncSetAttribute((const void*)bwd_slot_dq_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
@@ -1392,7 +1392,7 @@ int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, co
   if (which == 0) hipLaunchKernelGGL(bwd_slot_q_kernel, dim3(a->HQ, a->NT), dim3(256), 0, st, p);
   else {
     const size_t lds = (size_t)12 * BT * TLD * 2;
-    static bool configured = false;
+    static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
     if (!configured) {
       hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_intra_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) {

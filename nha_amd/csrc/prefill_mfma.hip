@@ -363,15 +363,6 @@ __global__ __launch_bounds__(256) void state_final_kernel(const MP p) {
 
 // ==========================================================================================
 // output pass
-#ifdef NHA_PROF
-#define PROF_DECL long long pt_[8] = {0,0,0,0,0,0,0,0}; long long pl_ = __builtin_amdgcn_s_memtime();
-#define PROF_STAGE(k) { __builtin_amdgcn_sched_barrier(0); ps_[k] = __builtin_amdgcn_s_memtime(); __builtin_amdgcn_sched_barrier(0); }
-#define PROF_MARK(k) { __builtin_amdgcn_sched_barrier(0); long long n_ = __builtin_amdgcn_s_memtime(); pt_[k] += n_ - pl_; pl_ = n_; }
-#else
-#define PROF_DECL
-#define PROF_STAGE(k)
-#define PROF_MARK(k)
-#endif
 // ==========================================================================================
 // One workgroup = one 64-row chunk x G query heads of one kv-head; its NW waves split the
 // 64 x G query rows into RQB blocks of 16 rows per wave.  Window K/V stream through four LDS
@@ -486,11 +477,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       lds_st16(vdst + loff[u], rv.r[u]);
     }
   };
-
-#ifdef NHA_PROF
-  long long ps_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
-  PROF_STAGE(0)
   // ---- phase 0: slot-branch operands -> LDS --------------------------------------------------
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
@@ -540,7 +526,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       if (c8 < 512 && j >= vlo && j < rows) sx[u] = *reinterpret_cast<const uint4*>(p.s + ((grow_s + j) * H + h) * MS + m8);
     }
     issue_window(0);
-    PROF_STAGE(6)
     __builtin_amdgcn_sched_barrier(0);
     tile_r2l<BT, D, NTHR>(tA, ra, tid);
     tile_r2l<BT, D, NTHR>(tB, tb, tid);
@@ -562,7 +547,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     }
   }
   __syncthreads();
-  PROF_STAGE(7)
   // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
   // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows
   // j of earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.
@@ -639,7 +623,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
       qs[qb][ks] = as_bf16x8(x);
     }
   }
-  PROF_STAGE(1)
   // ---- phase 1a: slot logits and the slot "tile" of the softmax, one 16-row block at a time ----
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -753,7 +736,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
     load_rows_tile(tD, p.v);
     __syncthreads();
   }
-  PROF_STAGE(2)
   // ---- phase 1b: slot read ----------------------------------------------------------------------
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -795,8 +777,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
           O[db][qb] = mfma16(lds_frag_tr(tD, LDT, 32 * pr, 32 * pr + 16, 16 * db, lane), bAv[pr], O[db][qb]);
       }
   }
-
-  PROF_STAGE(3)
   // ---- phase 2: sliding window, streamed in TK-key tiles --------------------------------------
   lds_barrier();   // every wave is done with the slot-branch tiles
   stage_window(Kb0, Vb0);
@@ -816,10 +796,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   // every load issued before the prefetch of tile 1 (queries, tile 0) has landed here, so inside
   // the loop only the tile prefetch of the previous iteration is ever outstanding
   __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NPC));   // vmcnt(2 * NPC), other counters untouched
-  PROF_STAGE(4)
-  PROF_DECL
   for (int i = 0; i < ntiles; ++i) {
-    PROF_MARK(7)
     const int cur = i & 1;
     const lbf16* Kt = cur ? Kb1 : Kb0;
     const lbf16* Vt = cur ? Vb1 : Vb0;
@@ -844,7 +821,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
           S[1][qb] = mfma16(a1, qs[qb][ks], S[1][qb]);
         }
       }
-      PROF_MARK(0)
       if (edge) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
@@ -872,7 +848,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
         rmax[qb] = x;
         need |= x > mrun[qb] + thr;
       }
-      PROF_MARK(1)
       if (__any(need)) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) {
@@ -899,7 +874,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
         // window row sums on the matrix core: every row of ones^T P is the sum over the 32 keys
         Lw[qb] = mfma16(ones, P[qb], Lw[qb]);
       }
-      PROF_MARK(2)
       // O^T[d][q] += V^T P^T over the 32 keys of this half
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
@@ -907,25 +881,13 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
 #pragma unroll
         for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(a, P[qb], O[db][qb]);
       }
-      PROF_MARK(3)
     }
     if (i + 1 < ntiles) {
       stage_window(cur ? Kb0 : Kb1, cur ? Vb0 : Vb1);
-      PROF_MARK(6)
       if (i + 2 < ntiles) issue_window_fast(i + 2);   // tiles >= 2 lie wholly before the chunk
     }
-    PROF_MARK(4)
     lds_barrier();
-    PROF_MARK(5)
   }
-  PROF_STAGE(5)
-#ifdef NHA_PROF
-  if (chunk == 200 && blockIdx.x == 3 && lane == 0) {
-    long long* dbg = (long long*)(p.lse_gsa + ((int64_t)p.T_tot - 8) * HQ);   // rows of the chunk that ran first
-    for (int k = 0; k < 8; ++k) dbg[wave * 8 + k] = pt_[k];
-    for (int k = 0; k < 8; ++k) dbg[64 + wave * 8 + k] = ps_[k];
-  }
-#endif
 
   // ---- epilogue -------------------------------------------------------------------------------
 #pragma unroll

@@ -68,10 +68,9 @@ struct RingCfg {
   static constexpr int GC = TD + 2 * UB;       // gate cumsum fp32 [64][64], pieces XORed with row % 16
   static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
   static constexpr int BYTES = SS + 8192;
-  static constexpr int SEA = 0;                // decay-factor fragments, over the ring once the window is done
-  static constexpr int SEB = NSEA * 1024;
+  static constexpr int ETAB = 0;               // decay tables (6 units of 4 KB), over the ring once the window is done
   static constexpr int NSLOT_LOADS = 4 * LPW + 3;   // per wave: four tiles, two gate blocks, one s block
-  static_assert((NSEA + NSEB) * 1024 <= 2 * NR * UB, "decay fragments must fit the ring");
+  static_assert(6 * 4096 <= 2 * NR * UB, "decay tables must fit the ring");
 };
 
 template <int D>
@@ -81,13 +80,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   constexpr int RQB = 2;                        // 16-row query blocks per wave
   constexpr int NPRE = NR - 1;                  // units requested before the loop
   extern __shared__ __align__(1024) unsigned char smem_[];
-#ifdef NHA_RING_STAMPS
-  long long st_[8];
-  st_[0] = __builtin_amdgcn_s_memtime();
-#define NHA_STAMP(k) st_[k] = __builtin_amdgcn_s_memtime()
-#else
-#define NHA_STAMP(k)
-#endif
   lbyte* const lds = (lbyte*)smem_;
   const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -297,7 +289,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   bf16x8 vf[DB];
   // ---- prologue: scores of unit 0, K fragments of unit 1 -----------------------------------------------
   // units 0 .. NPRE-1 have landed for this wave
-  NHA_STAMP(1);
   wait_vm<0>();
   lds_barrier();
   {
@@ -338,14 +329,44 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   const bf16_t* vreq = p.v + (((int64_t)c0 + 32 - 32 * NPRE) * H + h) * D;
   const int64_t ustep = (int64_t)32 * H * D;
 
-  NHA_STAMP(2);
-  for (int u = 0; u < nunits; ++u) {
+  // slot-branch query fragments of one query block (requested while the last unit is worked on)
+  auto load_qg = [&](bf16x8 (&q)[KS], int qb) {
+    const int irow = 16 * (qb0 + qb) + l16;
+    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      q[ks] = as_bf16x8(x);
+    }
+  };
+  // exponentials of the current unit's block for contraction step ks, element j (see phase A)
+  auto exp_step = [&](int ks, int j) {
+    if (KS == 4) {
+      Sc[ks & 1][ks >> 1][j] = fexp2(Sc[ks & 1][ks >> 1][j]);
+      NHA_PIN(Sc[ks & 1][ks >> 1][j]);
+    } else {
+      Sc[0][ks][j] = fexp2(Sc[0][ks][j]);
+      NHA_PIN(Sc[0][ks][j]);
+      Sc[1][ks][j] = fexp2(Sc[1][ks][j]);
+      NHA_PIN(Sc[1][ks][j]);
+    }
+  };
+  auto pack_p = [&](bf16x8 (&Pq)[RQB]) {
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      const u32x4 t = {cvt2(Sc[0][qb][0], Sc[0][qb][1]), cvt2(Sc[0][qb][2], Sc[0][qb][3]), cvt2(Sc[1][qb][0], Sc[1][qb][1]),
+                       cvt2(Sc[1][qb][2], Sc[1][qb][3])};
+      Pq[qb] = __builtin_bit_cast(bf16x8, t);
+      NHA_PIN(Pq[qb]);
+    }
+  };
+
+  for (int u = 0; u + 1 < nunits; ++u) {
     const uint32_t k_nn = C::RING_K + ((u + 2) & (NR - 1)) * UB + kaddr;   // K of unit u+2 (after the barrier)
     const uint32_t v_c = C::RING_V + (u & (NR - 1)) * UB + vaddr;           // V of unit u
-    const bool has_next = u + 1 < nunits;
     // ---- phase A: scores of unit u+1 on the matrix core, exponentials of unit u on the VALU,
     //      V fragments of unit u requested from LDS ----
-    unsigned pw[RQB][4];
     NHA_FENCE();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -357,37 +378,16 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
         Sn[kk][qb] = mfma16(kf[ks][kk], qs[qb][ks], ks == 0 ? nmv[qb] : Sn[kk][qb]);
         // a score block of the current unit per contraction step: with KS = 4 block (ks & 1, ks >> 1),
         // with KS = 2 blocks (0, ks) and (1, ks)
-        if (KS == 4) {
-          Sc[ks & 1][ks >> 1][j] = fexp2(Sc[ks & 1][ks >> 1][j]);
-          NHA_PIN(Sc[ks & 1][ks >> 1][j]);
-        } else {
-          Sc[0][ks][j] = fexp2(Sc[0][ks][j]);
-          NHA_PIN(Sc[0][ks][j]);
-          Sc[1][ks][j] = fexp2(Sc[1][ks][j]);
-          NHA_PIN(Sc[1][ks][j]);
-        }
+        exp_step(ks, j);
         NHA_FENCE();
       }
     }
-#pragma unroll
-    for (int qb = 0; qb < RQB; ++qb) {
-      pw[qb][0] = cvt2(Sc[0][qb][0], Sc[0][qb][1]);
-      pw[qb][1] = cvt2(Sc[0][qb][2], Sc[0][qb][3]);
-      pw[qb][2] = cvt2(Sc[1][qb][0], Sc[1][qb][1]);
-      pw[qb][3] = cvt2(Sc[1][qb][2], Sc[1][qb][3]);
-    }
     bf16x8 Pq[RQB];
-#pragma unroll
-    for (int qb = 0; qb < RQB; ++qb) {
-      const u32x4 t = {pw[qb][0], pw[qb][1], pw[qb][2], pw[qb][3]};
-      Pq[qb] = __builtin_bit_cast(bf16x8, t);
-      NHA_PIN(Pq[qb]);
-    }
+    pack_p(Pq);
     NHA_FENCE();
-    // unit u+2 has landed (this wave's part; at most the requests of unit u+3 stay in flight), then
-    // everybody's; after the barrier the slot of unit u-1 is free and takes unit u+NPRE
-    // (the requests younger than unit u+2: units u+3 .. u+NR-2, and the slot-branch operands while
-    // u <= NR-3, which were queued behind unit NR-1 in iteration 0)
+    // unit u+2 has landed (this wave's part), then everybody's; after the barrier the slot of unit u-1
+    // is free and takes unit u+NPRE.  Requests younger than unit u+2 may stay in flight: units
+    // u+3 .. u+NR-2, and the slot-branch operands while u <= NR-3 (queued behind unit NR-1 in iteration 0)
     if (u + 2 < nunits) {
       if (u + NR - 2 < nunits) {
         if (u >= 1 && u <= NR - 3) wait_vm<LPW * (NR - 4) + C::NSLOT_LOADS>();
@@ -426,7 +426,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     }
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      if (db < 2 * KS) kf[db >> 1][db & 1] = kfrag(k_nn, db & 1, db >> 1);
+      kf[db >> 1][db & 1] = kfrag(k_nn, db & 1, db >> 1);
       NHA_FENCE();
 #pragma unroll
       for (int qb = 0; qb < RQB; ++qb) {
@@ -441,106 +441,100 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
         NHA_FENCE();
       }
     }
-    if (has_next) {
-      if (is_edge(u + 1)) {
-        mask_unit(Sn, u + 1);
+    if (is_edge(u + 1)) {
+      mask_unit(Sn, u + 1);
 #pragma unroll
-        for (int qb = 0; qb < RQB; ++qb) {
-          float x = fmaxf(fmaxf(Sn[0][qb][0], Sn[0][qb][1]), fmaxf(Sn[0][qb][2], Sn[0][qb][3]));
-          m0[qb] = fmaxf(x, fmaxf(fmaxf(Sn[1][qb][0], Sn[1][qb][1]), fmaxf(Sn[1][qb][2], Sn[1][qb][3])));
-        }
+      for (int qb = 0; qb < RQB; ++qb) {
+        float x = fmaxf(fmaxf(Sn[0][qb][0], Sn[0][qb][1]), fmaxf(Sn[0][qb][2], Sn[0][qb][3]));
+        m0[qb] = fmaxf(x, fmaxf(fmaxf(Sn[1][qb][0], Sn[1][qb][1]), fmaxf(Sn[1][qb][2], Sn[1][qb][3])));
       }
-      bool need = false;
-#pragma unroll
-      for (int qb = 0; qb < RQB; ++qb) need |= m0[qb] > THR;
-      if (__any(need)) rescale(Sn, m0);
     }
+    bool need = false;
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) need |= m0[qb] > THR;
+    if (__any(need)) rescale(Sn, m0);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int qb = 0; qb < RQB; ++qb) Sc[kk][qb] = Sn[kk][qb];
   }
-
-  NHA_STAMP(3);
-  // ================= slot branch, folded into the running softmax =================================
-  // slot-branch query fragments of the first query block: requested now, used after the decay fragments
-  // are built; those of the second block are requested while the first is worked on
-  auto load_qg = [&](bf16x8 (&q)[KS], int qb) {
-    const int irow = 16 * (qb0 + qb) + l16;
-    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
-      q[ks] = as_bf16x8(x);
-    }
-  };
+  // ---- the last unit: no further scores; the slot-branch queries of the first query block are
+  //      requested into the registers the window queries leave ----
   bf16x8 qg[KS];
-  load_qg(qg, 0);
+  {
+    const int u = nunits - 1;
+    const uint32_t v_c = C::RING_V + (u & (NR - 1)) * UB + vaddr;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) vf[db] = vfrag(v_c, db);
+    load_qg(qg, 0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) exp_step(ks, j);
+    bf16x8 Pq[RQB];
+    pack_p(Pq);
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) Lw[qb] = mfma16(ones, Pq[qb], Lw[qb]);
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(vf[db], Pq[qb], O[db][qb]);
+  }
+
+  // ================= slot branch, folded into the running softmax =================================
   // every LDS-direct request of this wave has landed, every wave is done with the ring
   wait_vm<0>();
   lds_barrier();
-  NHA_STAMP(4);
   auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
   auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
-  // decay-factor fragments, one (fragment, lane) item = 8 values.  Sub-block Q (16 query rows)
-  // references the gate cumsum gr of the row before it: exponent gr[m] - gc_j[m] <= 0 for rows j of
-  // earlier sub-blocks, and bounded by the sub-block's own decay for its diagonal rows.  Rows whose
-  // source token does not exist (before the sequence, past its end) carry no weight.
-  for (int item = tid; item < (NSEA + NSEB) * 64; item += 512) {
-    const int f = item >> 6, ln = item & 63;
-    const int fl16 = ln & 15, fkb = ln >> 4;
+  // decay tables E_Q[j][m] = s_j[m] exp(min(gr_Q[m] - gc_j[m], DECAY_CLAMP)) for the rows j of the 16-row
+  // blocks jb <= Q, zero elsewhere: query sub-block Q (16 rows) references the gate cumsum gr_Q of the
+  // row before it (0 for Q = 0), so the exponent is <= 0 for rows of earlier blocks and bounded by the
+  // block's own decay on the diagonal.  Rows whose source token does not exist (before the sequence,
+  // past its end) carry no weight.  Stored as 32-row units in the V layout (64 columns): the logit
+  // update reads them transposed (rows = slots), the slot-read weights row by row (rows = tokens).
+  // Units: E_0 -> 0, E_1 -> 1, E_2 -> 2,3, E_3 -> 4,5; a thread makes 8 consecutive slots of a row.
+  for (int item = tid; item < 6 * 256; item += 512) {
+    const int U = item >> 8, r32 = (item >> 3) & 31, m = (item & 7) * 8;
+    const int Q = U == 0 ? 0 : U == 1 ? 1 : U < 4 ? 2 : 3;
+    const int pr = (U == 3 || U == 5) ? 1 : 0;
+    const int j = 32 * pr + r32;
+    const bool ok = (j >> 4) <= Q && j >= vlo && j < rows;
     bf16x8 out;
-    if (f < NSEA) {
-      const int Q = f < 4 ? 0 : f < 8 ? 1 : f < 16 ? 2 : 3;
-      const int rem = f - sea_base(Q);
-      const int pr = rem >> 2, mb = rem & 3;
-      const int m = 16 * mb + fl16;
-      const float gr = Q > 0 ? *gc_at(16 * Q - 1, m) : 0.f;
-      float gv[8];
-      bf16_t sv[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int j = 16 * (2 * pr + (e >> 2)) + 4 * fkb + (e & 3);   // j < 64 for every fragment
-        gv[e] = *gc_at(j, m);
-        sv[e] = *s_at(j, m);
-      }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int jb = 2 * pr + (e >> 2);
-        const int j = 16 * jb + 4 * fkb + (e & 3);
-        const float val = bf16_to_f32(sv[e]) * fexp(fminf(gr - gv[e], DECAY_CLAMP));
-        out[e] = (__bf16)((jb <= Q && j >= vlo && j < rows) ? val : 0.f);
-      }
-      *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::SEA + f * 1024 + ln * 16) = out;
-    } else {
-      const int g2 = f - NSEA;
-      const int Q = g2 < 2 ? 0 : g2 < 6 ? 1 : g2 < 12 ? 2 : 3;
-      const int rem = g2 - seb_base(Q);
-      const int jb = rem >> 1, pr = rem & 1;
-      const int j = 16 * jb + fl16;
-      const bool jok = j >= vlo && j < rows;
+    for (int e = 0; e < 8; ++e) out[e] = (__bf16)0.f;
+    if (ok) {
       f32x4 gv[2], gr[2];
-      bf16x4 sv[2];
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
-        const int m0s = 32 * pr + 16 * hh + 4 * fkb;   // the lane's 4 consecutive slots of this half
-        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m0s));
+        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m + 4 * hh));
         gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        if (Q > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Q - 1, m0s));
-        sv[hh] = *reinterpret_cast<const NHA_LDS bf16x4*>(s_at(j, m0s));
+        if (Q > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Q - 1, m + 4 * hh));
       }
+      const bf16x8 sv = *reinterpret_cast<const NHA_LDS bf16x8*>(s_at(j, m));
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float val = (float)sv[e >> 2][e & 3] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP));
-        out[e] = (__bf16)(jok ? val : 0.f);
-      }
-      *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::SEB + g2 * 1024 + ln * 16) = out;
+      for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)sv[e] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
     }
+    *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + (r32 & 15) * 64 + (m & 31) * 2) = out;
   }
   __syncthreads();
-  NHA_STAMP(5);
 
+  // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+  auto etab_tr = [&](int Q, int pr, int mb) -> bf16x8 {
+    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 32 + vaddr;
+    struct { s16x4 a, b; } t;
+    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + 2048));
+    return __builtin_bit_cast(bf16x8, t);
+  };
+  // E_Q by rows: row = token 16 jb + l16, contraction over the slots 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+  auto etab_row = [&](int Q, int jb, int pr) -> bf16x8 {
+    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 64 + 8 * kb;
+    struct { bf16x4 a, b; } t;
+    t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(pa);
+    t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 32);
+    return __builtin_bit_cast(bf16x8, t);
+  };
   float lg[RQB];
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -584,8 +578,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
       for (int pr = 0; pr < 2; ++pr)
         if (2 * pr <= Q) {
-          const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(lds + C::SEA + (sea_base(Q) + 4 * pr + mb) * 1024 + lane * 16);
-          oki[mb] = mfma16(se, bA[pr], oki[mb]);
+          oki[mb] = mfma16(etab_tr(Q, pr, mb), bA[pr], oki[mb]);
         }
     }
     // combine; the slot logits join the running softmax as one more set of keys
@@ -651,8 +644,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
         if (jb <= Q) {
 #pragma unroll
           for (int pr = 0; pr < 2; ++pr) {
-            const bf16x8 se = *reinterpret_cast<const NHA_LDS bf16x8*>(lds + C::SEB + (seb_base(Q) + 2 * jb + pr) * 1024 + lane * 16);
-            av[jb] = mfma16(se, bpr[pr], av[jb]);
+            av[jb] = mfma16(etab_row(Q, jb, pr), bpr[pr], av[jb]);
           }
           if (jb == Q) {
 #pragma unroll
@@ -672,7 +664,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       }
   }
 
-  NHA_STAMP(6);
   // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
   //      row block db + 1, and the two trade their halves) -------------------------------------------
 #pragma unroll
@@ -699,15 +690,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     }
     if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(lwt) - nm[qb]) * LN2;
   }
-#ifdef NHA_RING_STAMPS
-  if (lane == 0 && (wave == 0 || wave == 4)) {
-    st_[7] = __builtin_amdgcn_s_memtime();
-    long long* d = (long long*)p.hseg_k + (((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 10;
-    for (int k = 0; k < 8; ++k) d[k] = st_[k];
-    d[8] = nunits;
-    d[9] = __builtin_amdgcn_s_memrealtime();
-  }
-#endif
 }
 
 template <int D>
