@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 5
+#define NHA_ABI_VERSION 6
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -93,6 +93,19 @@ typedef struct NhaPrefillArgs {
  * cumsums, staging).  Only the integer/dtype/impl fields of `a` are read. */
 size_t nha_prefill_scratch_bytes(const NhaPrefillArgs* a);
 int nha_prefill_fwd(const NhaPrefillArgs* a);
+
+/* nha_prefill_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments, kernels and results, but
+ * `scratch` / `scratch_bytes` are ignored and the workspace is an array of
+ * NHA_NOALLOC_SCRATCH_BYTES that is part of the loaded library (one per GPU, held until the process
+ * ends).  The call allocates and frees nothing.  It returns NHA_ERR_SCRATCH when
+ * nha_prefill_scratch_bytes(a) exceeds NHA_NOALLOC_SCRATCH_BYTES (bf16, D = 128: about 400 chunks x
+ * kv-heads, e.g. 3200 tokens at 8 kv-heads).  Every call on a GPU shares that GPU's array: calls
+ * that overlap on one GPU (different streams or threads) race and must be serialised by the
+ * caller; successive calls on one stream are ordered by the stream.  No counterpart in the
+ * reference, whose ops allocate their intermediates through torch. */
+#define NHA_NOALLOC_SCRATCH_BYTES (32u << 20)
+int nha_prefill_fwd_noalloc(const NhaPrefillArgs* a);
 
 /* ------------------------------------------------------------------------------------------
  * Chunked prefill backward.  Replaces ChunkNativeHybridAttentionFunction.backward

@@ -14,11 +14,12 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 5
+ABI_VERSION = 6
+NHA_NOALLOC_SCRATCH_BYTES = 32 << 20   # workspace of nha_prefill_fwd_noalloc (include/nha_hip.h)
 NHA_FMAP_NONE, NHA_FMAP_SWISH, NHA_FMAP_RELU = 0, 1, 2
 
 EXPORTS = (
-    "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
+    "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_fwd_noalloc", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
     "nha_decode_step", "nha_decode_advance", "nha_layer_prologue", "nha_layer_epilogue",
     "nha_layer_prologue_bwd", "nha_layer_epilogue_bwd", "nha_layer_epilogue_bwd_parts",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
@@ -142,6 +143,8 @@ def load() -> C.CDLL:
     lib.nha_prefill_scratch_bytes.argtypes = [C.POINTER(NhaPrefillArgs)]
     lib.nha_prefill_fwd.restype = C.c_int
     lib.nha_prefill_fwd.argtypes = [C.POINTER(NhaPrefillArgs)]
+    lib.nha_prefill_fwd_noalloc.restype = C.c_int
+    lib.nha_prefill_fwd_noalloc.argtypes = [C.POINTER(NhaPrefillArgs)]
     lib.nha_prefill_bwd_scratch_bytes.restype = C.c_size_t
     lib.nha_prefill_bwd_scratch_bytes.argtypes = [C.POINTER(NhaPrefillBwdArgs)]
     lib.nha_prefill_bwd.restype = C.c_int

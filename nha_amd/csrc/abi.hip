@@ -4,6 +4,8 @@
 
 #include <string.h>
 
+#include <mutex>
+
 namespace nha {
 
 static thread_local char g_err[512] = "";
@@ -15,7 +17,7 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-static int check_prefill(const NhaPrefillArgs* a, bool pointers) {
+static int check_prefill(const NhaPrefillArgs* a, bool pointers, bool own_scratch = false) {
   NHA_CHECK_ARG(a != nullptr, "nha_prefill: null args");
   NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->NT > 0 && a->HQ > 0 && a->H > 0 && a->K > 0 && a->V > 0 && a->M > 0,
                 "nha_prefill: non-positive dimension");
@@ -31,8 +33,39 @@ static int check_prefill(const NhaPrefillArgs* a, bool pointers) {
                   "nha_prefill_fwd: cu_seqlens, chunk_indices and chunk_offsets are required");
     NHA_CHECK_ARG((a->h0k == nullptr) == (a->h0v == nullptr), "nha_prefill_fwd: pass both initial states or neither");
     NHA_CHECK_ARG((a->hkt == nullptr) == (a->hvt == nullptr), "nha_prefill_fwd: pass both final states or neither");
-    NHA_CHECK_ARG(a->scratch != nullptr, "nha_prefill_fwd: scratch is required");
+    NHA_CHECK_ARG(own_scratch || a->scratch != nullptr, "nha_prefill_fwd: scratch is required");
   }
+  return NHA_OK;
+}
+
+// Scratch of nha_prefill_fwd_noalloc: device memory that is part of the loaded library, one copy per
+// GPU at its own address, held until the process ends.  The name is a host-side handle only; host code
+// uses the address hipGetSymbolAddress reports for the current device.
+static __device__ __align__(256) unsigned char scratch[NHA_NOALLOC_SCRATCH_BYTES];
+
+static int noalloc_scratch(void** out) {
+  constexpr int MAX_DEV = 64;
+  static std::mutex mu;
+  static void* addr[MAX_DEV];
+  static bool known[MAX_DEV];
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+    set_error("nha_prefill_fwd_noalloc: no usable current device (%s, ordinal %d)", hipGetErrorString(e), dev);
+    return NHA_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!known[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("nha_prefill_fwd_noalloc: cannot locate the library's scratch array on device %d: %s", dev, hipGetErrorString(e));
+      return NHA_ERR_LAUNCH;
+    }
+    addr[dev] = ptr;
+    known[dev] = true;
+  }
+  *out = addr[dev];
   return NHA_OK;
 }
 
@@ -90,6 +123,32 @@ int nha_prefill_fwd(const NhaPrefillArgs* a) {
     return NHA_ERR_SCRATCH;
   }
   return mfma ? prefill_mfma_impl(a) : prefill_simple_impl(a);
+}
+
+int nha_prefill_fwd_noalloc(const NhaPrefillArgs* a) {
+  int rc = check_prefill(a, true, true);
+  if (rc != NHA_OK) return rc;
+  const bool mfma = use_mfma(a);
+  if (a->impl == NHA_IMPL_MFMA && !mfma) {
+    set_error("nha_prefill_fwd_noalloc: the MFMA kernels are not built for dtype=%d K=%d V=%d M=%d HQ/H=%d", a->dtype, a->K,
+              a->V, a->M, a->HQ / a->H);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  const size_t need = mfma ? prefill_mfma_scratch_bytes(a) : prefill_simple_scratch_bytes(a);
+  if (need > (size_t)NHA_NOALLOC_SCRATCH_BYTES) {
+    set_error("nha_prefill_fwd_noalloc: this call needs %zu bytes of scratch, the library's array holds %zu "
+              "(use nha_prefill_fwd with a workspace of nha_prefill_scratch_bytes() bytes)", need, (size_t)NHA_NOALLOC_SCRATCH_BYTES);
+    return NHA_ERR_SCRATCH;
+  }
+  void* ptr = nullptr;
+  rc = noalloc_scratch(&ptr);
+  if (rc != NHA_OK) return rc;
+  // nothing in the scratch has to start at zero: the state pass writes every table the output pass
+  // reads (rows past a sequence's end are never read), so the previous call's contents are harmless
+  NhaPrefillArgs b = *a;
+  b.scratch = ptr;
+  b.scratch_bytes = (size_t)NHA_NOALLOC_SCRATCH_BYTES;
+  return mfma ? prefill_mfma_impl(&b) : prefill_simple_impl(&b);
 }
 
 size_t nha_prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a) {
