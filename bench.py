@@ -35,16 +35,25 @@ TRAFFIC_BYTES = {
     "layer_epilogue_kernel": (65759.4 * 2.0 + 131072.0) * 1024,
 }
 
+# where each figure above comes from: the counters are read in separate rocprofv3 runs, not in this one
+TRAFFIC_SOURCE = {
+    "mfma_out_kernel<128,4,8,64>": "profiles/mfma_out_kernel_prefill_T8192.md (rocprofv3 --pmc, not measured in this run)",
+    "decode_mfma_kernel<128,4,2>": "profiles/decode_mfma_kernel_B128_W1024.md (rocprofv3 --pmc, not measured in this run)",
+}
+OUT_KERNEL = "mfma_out_kernel<128,4,8,64>"
+
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
 DECODE = dict(B=128, HQ=32, H=8, D=128, M=64, W=1024, steps=256)
 # the other prefill shapes of the reference's configurations (parity-test cases; `--workload NAME`
 # times one of them with the same method as the headline).  wl/shift default to the shifted
 # convention (W-1, W); "layer" = (W, 0).  cfg3 packs sequences of 64..4096 tokens into 32768.
+# gate_mean: mean of the gate logits before logsigmoid (N(-1,1) for the long-context shapes, N(0,1)
+# for the 340M-layer shapes); h0_std: standard deviation of the per-sequence initial slot states.
 WORKLOADS = dict(
     headline=PREFILL,
-    cfg2=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0),
-    cfg2_shifted=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512),
-    cfg3=dict(B=1, T=32768, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0, varlen=True),
+    cfg2=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0, gate_mean=0.0),
+    cfg2_shifted=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512, gate_mean=0.0),
+    cfg3=dict(B=1, T=32768, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0, varlen=True, gate_mean=0.0, h0_std=0.1),
     cfg5=dict(B=2, T=16384, HQ=32, H=8, D=128, M=64, W=2048),
 )
 
@@ -72,6 +81,16 @@ def workload_lengths(torch, cfg):
     return lens
 
 
+def min_prefill_bytes(cfg, N):
+    """Minimal HBM bytes of a prefill call: every operand read once, the output written once (bf16),
+    initial states read when the workload has them."""
+    B, T, HQ, H, D, M = (cfg[k] for k in ("B", "T", "HQ", "H", "D", "M"))
+    b = 2 * B * T * (HQ * 3 * D + H * (3 * D + 2 * M))
+    if cfg.get("h0_std"):
+        b += 4 * N * H * 2 * D * M
+    return b
+
+
 def decode_bytes(B, HQ, H, D, M, W):
     """Algorithmic HBM bytes of one decode step: fp32 state read+write, bf16 K/V window read,
     q/o/new-token/popped-entry traffic."""
@@ -90,13 +109,23 @@ def make_prefill_inputs(torch, cfg, device, seed=0, B=None, T=None):
     q = (r(B, T, HQ, D) * D ** -0.5).to(torch.bfloat16)
     k = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
     v = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
-    g = torch.nn.functional.logsigmoid(r(B, T, H, M) - 1.0).to(torch.bfloat16)   # slow-forgetting gates
+    g = torch.nn.functional.logsigmoid(r(B, T, H, M) + cfg.get("gate_mean", -1.0)).to(torch.bfloat16)
     s = (1 - g.float().exp()).to(torch.bfloat16)
     # the window branch and the slot branch see different (rotated / raw) q and k in the hybrid
     # models; a second draw keeps the two operand streams distinct as they are in production
     q2 = (r(B, T, HQ, D) * D ** -0.5).to(torch.bfloat16)
     k2 = (r(B, T, H, D) * D ** -0.5).to(torch.bfloat16)
     return [x.to(device) for x in (q2, k2, q, k, v, s, g)]
+
+
+def make_initial_state(torch, cfg, N, device, seed=4):
+    """Per-sequence initial slot states ~ N(0, h0_std) of a workload that has them, else None."""
+    if not cfg.get("h0_std"):
+        return None
+    gen = torch.Generator().manual_seed(seed)
+    H, D, M = cfg["H"], cfg["D"], cfg["M"]
+    return ((torch.randn(N, H, D, M, generator=gen) * cfg["h0_std"]).to(device),
+            (torch.randn(N, H, M, D, generator=gen) * cfg["h0_std"]).to(device))
 
 
 def bench_prefill(torch, steps, warmup, cfg=PREFILL):
@@ -120,6 +149,9 @@ def bench_prefill(torch, steps, warmup, cfg=PREFILL):
     a = _lib.NhaPrefillArgs()
     a.q_swa, a.k_swa, a.q_gsa, a.k_gsa, a.v, a.s, a.g = (_ptr(x) for x in xs)
     a.o, a.lse_swa, a.lse_gsa, a.hkt, a.hvt = _ptr(o), _ptr(lse_s), _ptr(lse_g), _ptr(hkt), _ptr(hvt)
+    h0 = make_initial_state(torch, cfg, N, dev)
+    if h0 is not None:
+        a.h0k, a.h0v = _ptr(h0[0]), _ptr(h0[1])
     a.cu_seqlens, a.chunk_indices, a.chunk_offsets = _ptr(cu_d), _ptr(idx_d), _ptr(off_d)
     a.T_tot, a.N, a.NT, a.HQ, a.H, a.K, a.V, a.M = B * T, N, NT, HQ, H, D, D, M
     a.wl, a.shift, a.dtype, a.impl, a.scale = wl, shift, _lib.NHA_DTYPE_BF16, _lib.NHA_IMPL_MFMA, D ** -0.5
@@ -322,6 +354,68 @@ def bench_decode(torch, warmup):
     return dict(us_per_step=us_step, us_kernel=us_kernel, bytes=nbytes, achieved_gbs=nbytes / (us_kernel * 1e-6) / 1e9)
 
 
+def bench_api(torch, steps, warmup):
+    """The drop-in Python ops, called the way the reference's callers call them (outputs allocated per
+    call, tables and workspace found in the ops' caches): milliseconds / microseconds per call with HIP
+    events on the launch stream.  chunk_nha at the headline shape and on the packed varlen
+    configuration (cu_seqlens tensor on the GPU, initial and final states); fused_recurrent_nha_decode
+    in its window form (time-ordered [B,W,H,D] window tensors, explicit popped entry) at the decode
+    configuration, once with a pre-rotated query and once with in-kernel rotary (cos / sin)."""
+    import itertools
+    from nha_amd import chunk_nha, fused_recurrent_nha_decode
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+
+    def timed(fn, n):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record(stream)
+        for _ in range(n):
+            fn()
+        ev[1].record(stream)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / n
+
+    out = {}
+    with torch.no_grad():
+        cfg = PREFILL
+        xs = make_prefill_inputs(torch, cfg, dev)
+        W = cfg["W"]
+        out["chunk_nha_ms"] = timed(lambda: chunk_nha(*xs, window_size_left=W - 1, gsa_kv_shift=W), steps)
+        del xs
+        cfg = WORKLOADS["cfg3"]
+        lens = workload_lengths(torch, cfg)
+        xs = make_prefill_inputs(torch, cfg, dev)
+        cu = torch.tensor([0] + list(itertools.accumulate(lens)), dtype=torch.int32, device=dev)
+        h0 = make_initial_state(torch, cfg, len(lens), dev)
+        out["chunk_nha_varlen_cfg3_ms"] = timed(lambda: chunk_nha(*xs, cu_seqlens=cu, window_size_left=cfg["wl"],
+                                                                  gsa_kv_shift=cfg["shift"], initial_state=h0,
+                                                                  output_final_state=True), steps)
+        del xs
+        d = DECODE
+        B, HQ, H, D, M, Wd = (d[k] for k in ("B", "HQ", "H", "D", "M", "W"))
+        gen = torch.Generator().manual_seed(3)
+        r = lambda *sh: torch.randn(*sh, generator=gen, dtype=torch.float32)
+        bf = lambda x: x.to(torch.bfloat16).to(dev)
+        q, sq = bf(r(B, 1, HQ, D) * D ** -0.5), bf(r(B, 1, HQ, D) * D ** -0.5)
+        k, v = bf(r(B, 1, H, D)), bf(r(B, 1, H, D))
+        g = bf(torch.nn.functional.logsigmoid(r(B, 1, H, M)))
+        swk, swv = bf(r(B, Wd, H, D)), bf(r(B, Wd, H, D))
+        hk, hv = (r(B, H, D, M) * 0.1).to(dev), (r(B, H, M, D) * 0.1).to(dev)
+        pos = torch.arange(Wd, dtype=torch.float32)
+        inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+        ang = torch.cat([pos[:, None] * inv[None], pos[:, None] * inv[None]], -1)[None]
+        cos, sin = bf(ang.cos()), bf(ang.sin())
+        n = d["steps"]
+        out["decode_window_eager_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
+            q, k, v, g, swk, swv, sq=sq, initial_state=(hk, hv), output_final_state=True), n)
+        out["decode_window_rotary_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
+            q, k, v, g, swk, swv, cos=cos, sin=sin, initial_state=(hk, hv), output_final_state=True), n)
+    return out
+
+
 def cpu_baseline(torch):
     """The oracle on the host cores, bounded sample: the plain-C restatement (oracle/nha_ref_c.c,
     OpenMP over sequences x q-heads, double arithmetic) for the prefill, the torch restatement for a
@@ -368,7 +462,44 @@ def cpu_baseline(torch):
         R.decode_ref(**args, sq=args["q"], initial_state=h0, dtype=torch.float32)
     pre["decode_us_per_step"] = (time.perf_counter() - t0) / nrep * 1e6
     pre["decode_sample"] = f"{nrep} steps of the B={B} decode workload, fp32"
+    pre["torch_naive"] = cpu_baseline_torch_naive(torch, cores, (args, h0))
     return pre
+
+
+def cpu_baseline_torch_naive(torch, cores, decode_inputs):
+    """The naive PyTorch per-token path (oracle.prefill_ref / oracle.decode_ref: the shape of computation of
+    the reference's scripts/verify_opt_parity.py:88-191), fp32, all host cores: one warm-up, then the
+    median of three runs, on a B=1 slice of the prefill workload sized to a few seconds per run."""
+    import statistics
+    from oracle import nha_ref as R
+    cfg = PREFILL
+    W = cfg["W"]
+    keys = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+
+    def run(T):
+        xs = make_prefill_inputs(torch, cfg, "cpu", B=1, T=T)
+        t0 = time.perf_counter()
+        R.prefill_ref(*xs, window_size_left=W - 1, gsa_kv_shift=W, dtype=torch.float32)
+        return time.perf_counter() - t0
+
+    T = 256
+    t = run(T)                                       # warm-up and probe
+    while T < cfg["T"] and t * 2.5 <= 8.0:           # per-token cost grows until the window is full
+        T *= 2
+        t *= 2.5
+    ts = sorted(run(T) for _ in range(3))
+    a, h0 = decode_inputs
+    R.decode_ref(**a, sq=a["q"], initial_state=h0, dtype=torch.float32)
+    td = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        R.decode_ref(**a, sq=a["q"], initial_state=h0, dtype=torch.float32)
+        td.append(time.perf_counter() - t0)
+    return dict(value=T / ts[1], unit="tokens/s", cores=cores, kind="port",
+                sample=f"B=1 slice, first {T} tokens of the T={cfg['T']} workload, fp32 torch per-token loop, "
+                       f"1 warm-up + median of 3 ({ts[1]:.1f} s)",
+                decode_us_per_step=statistics.median(td) * 1e6,
+                decode_sample=f"median of 3 steps after a warm-up, B={DECODE['B']} decode workload, fp32 torch")
 
 
 def main():
@@ -404,7 +535,7 @@ def main():
         cfg = WORKLOADS[args.workload]
         res = bench_prefill(torch, args.steps, args.warmup, cfg)
         res["workload"] = {k: v for k, v in cfg.items()}
-        res["min_bytes"] = 2 * cfg["B"] * cfg["T"] * (cfg["HQ"] * 3 * cfg["D"] + cfg["H"] * (3 * cfg["D"] + 2 * cfg["M"]))
+        res["min_bytes"] = min_prefill_bytes(cfg, len(workload_lengths(torch, cfg)))
         res["min_bytes_gbs"] = res["min_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9
         if args.backward:
             res.update(bench_backward(torch, args.steps, args.warmup, cfg))
@@ -420,6 +551,17 @@ def main():
     bw = bench_backward(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     dc = bench_decode(torch, args.warmup)
     gl = bench_glue(torch, args.steps, args.warmup)
+    api = bench_api(torch, max(args.steps // 2, 1), min(args.warmup, 2))
+    others = {}
+    for name in ("cfg2", "cfg3", "cfg5"):
+        cfg = WORKLOADS[name]
+        r = bench_prefill(torch, max(args.steps // 2, 1), min(args.warmup, 2), cfg)
+        mb = min_prefill_bytes(cfg, len(workload_lengths(torch, cfg)))
+        others[name] = {"ms": r["ms_per_step"], "state_pass_ms": r["t_state_ms"], "output_pass_ms": r["t_out_ms"],
+                        "tokens_per_s": r["tokens_per_s"], "tflops": r["whole_op_tflops"],
+                        "mfma_frac": r["whole_op_tflops"] / PEAK_MFMA_BF16_TFLOPS, "min_bytes": mb,
+                        "min_bytes_gbs": mb / (r["ms_per_step"] * 1e-3) / 1e9,
+                        "shape": {k: v for k, v in cfg.items()}}
     cpu = None if args.no_cpu_baseline else cpu_baseline(torch)
     out = {
         "metric": "NHA prefill tokens/s @T=8K bf16",
@@ -438,15 +580,18 @@ def main():
                                "(window W keys, slots hold tokens <= t-W), gate logits N(-1,1)->logsigmoid",
                    "decode_workload": "B=128 HQ=32 H=8 D=128 M=64 W=1024 ring buffer, full windows at random "
                                       "ring positions, 256 consecutive steps"},
-        "roofline": {"bound": "mfma", "kernel": "mfma_out_kernel<128,4,8,64>", "achieved": pf["achieved_tflops"],
+        "roofline": {"bound": "mfma", "kernel": OUT_KERNEL, "achieved": pf["achieved_tflops"],
                      "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": pf["achieved_tflops"] / PEAK_MFMA_BF16_TFLOPS,
-                     "traffic": TRAFFIC_BYTES["mfma_out_kernel<128,4,8,64>"], "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
+                     "traffic": TRAFFIC_BYTES[OUT_KERNEL], "traffic_source": TRAFFIC_SOURCE[OUT_KERNEL],
+                     "kernel_ms": pf["t_out_ms"], "state_pass_ms": pf["t_state_ms"],
                      "whole_op_tflops": pf["whole_op_tflops"], "algorithmic_flop": pf["flops"]},
         "decode": {"metric": "decode step us @B=128", "value": dc["us_per_step"], "unit": "us/step",
                    "higher_is_better": False,
                    "roofline": {"bound": "hbm", "kernel": "decode_mfma_kernel<128,4,2>", "achieved": dc["achieved_gbs"],
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
-                                "traffic": TRAFFIC_BYTES["decode_mfma_kernel<128,4,2>"], "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
+                                "traffic": TRAFFIC_BYTES["decode_mfma_kernel<128,4,2>"],
+                                "traffic_source": TRAFFIC_SOURCE["decode_mfma_kernel<128,4,2>"],
+                                "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
         "backward": {"metric": "backward of the same prefill call", "ms_per_call": bw["bwd_ms"], "unit": "ms",
                      "tokens_per_s": bw["bwd_tokens_per_s"], "tflops": bw["bwd_tflops"],
                      "flop": bw["bwd_flops"], "note": "2.5 x the forward's algorithmic flop"},
@@ -459,6 +604,13 @@ def main():
                                     "epilogue": {"achieved": gl["epilogue_gbs"], "frac": gl["epilogue_gbs"] / PEAK_HBM_GBS,
                                                  "algorithmic_bytes": gl["epilogue_bytes"],
                                                  "traffic": TRAFFIC_BYTES["layer_epilogue_kernel"]}}},
+        "api": {"note": "the drop-in Python ops as their callers use them (outputs allocated per call); the headline "
+                        "value above times the C-ABI call with pre-allocated outputs",
+                "chunk_nha_ms": api["chunk_nha_ms"], "chunk_nha_vs_abi": api["chunk_nha_ms"] / pf["ms_per_step"],
+                "chunk_nha_varlen_cfg3_ms": api["chunk_nha_varlen_cfg3_ms"],
+                "fused_recurrent_nha_decode_window_eager_us": api["decode_window_eager_us"],
+                "fused_recurrent_nha_decode_window_rotary_us": api["decode_window_rotary_us"]},
+        "workloads": others,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

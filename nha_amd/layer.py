@@ -132,7 +132,19 @@ class ShortConvolution(nn.Module):
                 y = y + self.bias[None, :, None]
         else:
             y = F.conv1d(xs, self.weight, self.bias, groups=Dm)
-        final = xs[..., -(self.kernel_size - 1):].contiguous() if output_final_state else None
+        final = None
+        if output_final_state:
+            if cu_seqlens is not None and cache is None:
+                # one state per packed sequence: its last kernel_size - 1 inputs, zeros where it is shorter
+                cu = cu_seqlens.to(x.device).long()
+                ends = cu[1:]
+                back = torch.arange(self.kernel_size - 1, 0, -1, device=x.device)              # W-1 .. 1
+                idx = ends[:, None] - back[None, :]                                            # [N, W-1]
+                ok = idx >= cu[:-1, None]
+                gathered = x[0][idx.clamp(min=0)]                                              # [N, W-1, Dm]
+                final = (gathered * ok[..., None].to(x.dtype)).transpose(1, 2).contiguous()     # [N, Dm, W-1]
+            else:
+                final = xs[..., -(self.kernel_size - 1):].contiguous()
         if self.activation in ("silu", "swish"):
             y = F.silu(y)
         return y.transpose(1, 2), final

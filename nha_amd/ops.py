@@ -15,6 +15,7 @@ is a HIP kernel behind the C ABI.  There is no CPU / eager fallback.
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Optional, Tuple
 
 import numpy as np
@@ -67,9 +68,42 @@ def prefill_tables(cu_host: np.ndarray, device) -> Tuple[torch.Tensor, torch.Ten
     out = (torch.from_numpy(cu_host.astype(np.int32)).to(device), torch.from_numpy(idx).to(device),
            torch.from_numpy(off).to(device), int(idx.shape[0]))
     if len(_TABLE_CACHE) > 64:
-        _TABLE_CACHE.clear()
+        _TABLE_CACHE.pop(next(iter(_TABLE_CACHE)))      # oldest entry
     _TABLE_CACHE[key] = out
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# forward workspace: one buffer per (device, stream), grown when a call needs more.  Calls on one
+# stream are ordered by the stream, so they can share it; another stream gets its own.
+# ---------------------------------------------------------------------------------------------
+_WORKSPACE: dict = {}
+
+
+def _workspace(nbytes: int, dev, stream: int) -> torch.Tensor:
+    key = (str(dev), stream)
+    ws = _WORKSPACE.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _WORKSPACE[key] = ws
+    return ws
+
+
+# host copies of cu_seqlens tensors, keyed by the tensor OBJECT (weakly) and its version counter, so that
+# the layers of a model, which all receive the same tensor, wait for one device-to-host copy, not one each
+_CU_HOST: dict = {}      # id(tensor) -> (weak reference, version, host copy)
+
+
+def _cu_to_host(cu: torch.Tensor) -> np.ndarray:
+    if not cu.is_cuda:
+        return cu.detach().to(torch.int32).numpy()
+    key = id(cu)
+    hit = _CU_HOST.get(key)
+    if hit is not None and hit[0]() is cu and hit[1] == cu._version:
+        return hit[2]
+    host = cu.detach().to("cpu", torch.int32).numpy()
+    _CU_HOST[key] = (weakref.ref(cu, lambda _, k=key: _CU_HOST.pop(k, None)), cu._version, host)
+    return host
 
 
 def nha_prefill(q_swa, k_swa, q_gsa, k_gsa, v, s, g, cu_host: np.ndarray, *, wl: int, shift: int, scale: float,
@@ -109,8 +143,8 @@ def nha_prefill(q_swa, k_swa, q_gsa, k_gsa, v, s, g, cu_host: np.ndarray, *, wl:
     nbytes = lib.nha_prefill_scratch_bytes(C.byref(a))
     if nbytes == 0:
         _lib.check(_lib.NHA_ERR_INVALID)
-    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
+    scratch = _workspace(nbytes, dev, a.stream or 0)
+    a.scratch, a.scratch_bytes = _ptr(scratch), scratch.numel()
     _lib.check(lib.nha_prefill_fwd(C.byref(a)))
     return o, lse_swa, lse_gsa, hkt, hvt
 
@@ -401,7 +435,7 @@ def chunk_nha(
     if cu_seqlens is not None:
         if B != 1:
             raise ValueError("varlen (cu_seqlens) inputs must be packed with batch size 1")
-        cu_host = cu_seqlens.detach().to("cpu", torch.int32).numpy()
+        cu_host = _cu_to_host(cu_seqlens)
         if int(cu_host[-1]) != T:
             raise ValueError(f"cu_seqlens[-1] = {int(cu_host[-1])} does not match the packed length {T}")
     else:
@@ -409,13 +443,32 @@ def chunk_nha(
     dt = q_swa.dtype
     args = [_flat(x.to(dt)) for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)]
     h0 = (None, None) if initial_state is None or initial_state[0] is None else tuple(initial_state)
+    # empty sequences (a fully padded batch row after unpadding yields a repeated cu_seqlens entry): the
+    # kernels see the packing without them; their final state is their initial state
+    lens = np.diff(cu_host)
+    if (lens < 0).any():
+        raise ValueError("cu_seqlens must be non-decreasing")
+    keep = None
+    if (lens == 0).any():
+        keep = torch.from_numpy(np.nonzero(lens > 0)[0]).to(q_swa.device)
+        n_all = lens.size
+        cu_host = np.concatenate([[0], np.cumsum(lens[lens > 0])]).astype(np.int32)
+        h0_all = h0
+        if h0[0] is not None:
+            h0 = (h0[0][keep], h0[1][keep])
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (*args, *h0)):
         o, lse_swa, lse_gsa, hkt, hvt = _ChunkNHAFunction.apply(
             *args, h0[0], h0[1], cu_host, window_size_left, gsa_kv_shift, scale, output_final_state, impl)
     else:
         o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(
             *args, cu_host, wl=window_size_left, shift=gsa_kv_shift, scale=scale,
-            h0=initial_state, want_state=output_final_state, impl=impl)
+            h0=None if h0[0] is None else h0, want_state=output_final_state, impl=impl)
+    if keep is not None and output_final_state:
+        def spread(part, init):
+            full = torch.zeros(n_all, *part.shape[1:], dtype=part.dtype, device=part.device) if init is None \
+                else init.to(part.dtype).clone()
+            return full.index_copy(0, keep, part)
+        hkt, hvt = spread(hkt, h0_all[0]), spread(hvt, h0_all[1])
     o = o.view(B, T, HQ, -1)
     lse_swa = lse_swa.view(B, T, HQ)
     lse_gsa = lse_gsa.view(B, T, HQ)

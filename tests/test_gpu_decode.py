@@ -279,3 +279,43 @@ def test_ring_decode_at_benchmark_shape():
         assert rel <= 5e-3, f"step {step}: relative L2 error {rel:.3e}"
     assert_close("hk", st.hk, ref["hk"], dtype)
     assert_close("hv", st.hv, ref["hv"], dtype)
+
+
+def test_ring_decode_benchmark_shape_partial_windows_16_steps():
+    """The decode configuration as written: B=128 sequences, 32/8 heads, D=128, M=64, a W=1024 ring
+    whose fill is drawn per sequence from [1, W] (some rings fill up and start popping within the
+    run), state ~ N(0, 0.1), 16 consecutive steps, every step against the oracle's ring recurrence."""
+    import bench
+    from nha_amd import NHARingState, ring_decode_step
+    cfg = bench.DECODE
+    B, HQ, H, D, M, W = (cfg[k] for k in ("B", "HQ", "H", "D", "M", "W"))
+    dtype, steps = torch.bfloat16, 16
+    gen = torch.Generator().manual_seed(22)
+    r = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    st = NHARingState.empty(B, H, D, D, M, W, dtype=dtype)
+    st.hk.copy_(r(B, H, D, M) * 0.1)
+    st.hv.copy_(r(B, H, M, D) * 0.1)
+    st.ring_k.copy_(r(B, W, H, D))
+    st.ring_kg.copy_(r(B, W, H, D))
+    st.ring_v.copy_(r(B, W, H, D))
+    st.ring_g.copy_(F.logsigmoid(r(B, W, H, M)))
+    counts = torch.randint(0, W, (B,), generator=gen, dtype=torch.int32)    # fill after the first step in [1, W]
+    counts[:8] = torch.tensor([0, 1, W - 1, W - 2, W - steps, W - 5, 63, 64], dtype=torch.int32)
+    st.count.copy_(counts)
+    ref = dict(hk=st.hk.cpu().double(), hv=st.hv.cpu().double(),
+               rings=tuple(x.cpu().double() for x in (st.ring_k, st.ring_kg, st.ring_v, st.ring_g)), count=counts.clone())
+    for step in range(steps):
+        q, sq = (r(B, HQ, D) * D ** -0.5).to(dtype), (r(B, HQ, D) * D ** -0.5).to(dtype)
+        kn, kgn, vn = r(B, H, D).to(dtype), r(B, H, D).to(dtype), r(B, H, D).to(dtype)
+        gn = F.logsigmoid(r(B, H, M)).to(dtype)
+        o = ring_decode_step(st, q.cuda(), sq.cuda(), kn.cuda(), kgn.cuda(), vn.cuda(), gn.cuda())
+        ro, ref["hk"], ref["hv"], ref["rings"] = R.decode_ring_ref(q, sq, kn, kgn, vn, gn, *ref["rings"], ref["count"],
+                                                                   ref["hk"], ref["hv"], dtype=torch.float32)
+        ref["count"] += 1
+        assert_close(f"step {step} o", o, ro, dtype)
+        rel = ((o.double().cpu() - ro.double()).norm() / ro.double().norm()).item()
+        assert rel <= 5e-3, f"step {step}: relative L2 error {rel:.3e}"
+    assert torch.equal(st.count.cpu(), ref["count"])
+    assert (ref["count"] > W).any() and (ref["count"] < W).any()
+    assert_close("hk", st.hk, ref["hk"], dtype)
+    assert_close("hv", st.hv, ref["hv"], dtype)

@@ -109,3 +109,27 @@ def test_api_errors():
         chunk_nha(*[d[k] for k in KEYS])                     # CPU tensors: no fallback
     with pytest.raises(ValueError):
         chunk_nha(*[x.expand(2, -1, -1, -1) for x in c], cu_seqlens=torch.tensor([0, 32], dtype=torch.int32).cuda())
+
+
+@pytest.mark.gpu
+def test_varlen_tables_on_the_device_bit_exact_vs_oracle():
+    """The chunk tables the kernels consume (built by the host-side C entry points, copied to the GPU by
+    prefill_tables) equal the integer oracle bit for bit: the reference test's length lists
+    (tests/test_varlen.py:60-73 of the reference) and the benchmark's 32768-token varlen draw."""
+    import random
+    import numpy as np
+    import bench
+    from nha_amd.ops import prefill_tables
+    from oracle import varlen_index as VI
+    random.seed(0)
+    cases = [[128] * 4, [128, 64, 200, 10], [4096, 2048, 1, 1024, 2], [random.randint(1, 100) for _ in range(256)],
+             [1, 2000, 3, 50, 4, 3000, 2, 7], bench.workload_lengths(torch, bench.WORKLOADS["cfg3"])]
+    for lens in cases:
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        cu_d, idx_d, off_d, NT = prefill_tables(cu, torch.device("cuda:0"))
+        ridx, roff = VI.chunk_tables_brute(cu.tolist(), 64)
+        assert cu_d.dtype == idx_d.dtype == off_d.dtype == torch.int32
+        assert torch.equal(cu_d.cpu(), torch.from_numpy(cu))
+        assert torch.equal(idx_d.cpu(), torch.from_numpy(ridx))
+        assert torch.equal(off_d.cpu(), torch.from_numpy(roff))
+        assert NT == ridx.shape[0]

@@ -138,10 +138,11 @@ def test_mfma_headline_shape_matches_c_oracle():
 
 @pytest.mark.parametrize("name", ["cfg2", "cfg3", "cfg5"])
 def test_mfma_layer_workloads_match_c_oracle(name):
-    """The other workloads of the benchmark against the C restatement, with initial states: the D=256
-    ones (layer convention wl = W, shift = 0; cfg3 is the packed varlen draw of 64..4096-token
-    sequences) and one T=16384 sequence of the long-context hybrid shape (32/8 heads, D=128,
-    W=2048, shifted convention)."""
+    """The other configurations, with their own input distributions, against the C restatement:
+    cfg2 (340M-layer shape, D=256, layer convention wl = W, shift = 0, gate logits N(0,1), no
+    initial state; 2 of its 8 independent sequences), cfg3 (the packed varlen draw of 64..4096-token
+    sequences, 32768 tokens, initial states ~ N(0, 0.1)) and cfg5 (32/8 heads, D=128, W=2048,
+    gate logits N(-1,1), shifted convention; 1 of its 2 independent T=16384 sequences)."""
     import bench
     from nha_amd import chunk_nha
     from oracle.nha_ref_c import prefill_ref_c
@@ -149,19 +150,19 @@ def test_mfma_layer_workloads_match_c_oracle(name):
     if not cfg.get("varlen"):
         cfg["B"] = 1 if name == "cfg5" else 2                 # a part of its batch
     lens = bench.workload_lengths(torch, cfg)
-    B, T, H, D, M = cfg["B"], cfg["T"], cfg["H"], cfg["D"], cfg["M"]
     xs = bench.make_prefill_inputs(torch, cfg, "cpu", seed=9)
     cu = None
     if cfg.get("varlen"):
         cu = torch.tensor([0] + list(itertools.accumulate(lens)), dtype=torch.int32)
-    N = len(lens)
-    gen = torch.Generator().manual_seed(4)
-    h0 = (torch.randn(N, H, D, M, generator=gen) * 0.05, torch.randn(N, H, M, D, generator=gen) * 0.05)
+    h0 = bench.make_initial_state(torch, cfg, len(lens), "cpu")
+    assert (h0 is not None) == (name == "cfg3")
     kw = dict(window_size_left=cfg.get("wl", cfg["W"] - 1), gsa_kv_shift=cfg.get("shift", cfg["W"]))
     ref = prefill_ref_c(*xs, cu_seqlens=None if cu is None else cu.tolist(), initial_state=h0, **kw)
     got = chunk_nha(*[x.cuda() for x in xs], cu_seqlens=None if cu is None else cu.cuda(),
-                    initial_state=(h0[0].cuda(), h0[1].cuda()), output_final_state=True, impl="mfma", **kw)
+                    initial_state=None if h0 is None else (h0[0].cuda(), h0[1].cuda()), output_final_state=True,
+                    impl="mfma", **kw)
     assert_close("o", got[0], ref[0].double(), BF)
+    assert_close("lse_swa", got[1], ref[1].double(), BF)
     assert_close("lse_gsa", got[2], ref[2].double(), BF)
     assert_close("hk", got[3][0], ref[3].double(), BF)
     assert_close("hv", got[3][1], ref[4].double(), BF)

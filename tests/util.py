@@ -29,7 +29,9 @@ def prefill_inputs(seed, B, T, HQ, H, K, V, M, dtype=torch.bfloat16, gate_div=8.
 
 
 def assert_close(name, got, ref, dtype):
-    """bf16: 2e-2 abs / 1e-2 rel elementwise; fp32: 1e-4 relative to the tensor's scale."""
+    """bf16: 2e-2 abs / 1e-2 rel element by element.  fp32: 1e-4 relative element by element, with an
+    absolute floor of 2e-6 of the tensor's largest magnitude (the rounding noise of fp32 sums of that
+    size; elements that cancel to nearly zero have no meaningful relative error)."""
     got = got.detach().double().cpu()
     ref = ref.detach().double().cpu()
     assert got.shape == ref.shape, (name, got.shape, ref.shape)
@@ -40,5 +42,7 @@ def assert_close(name, got, ref, dtype):
         assert not bad.any(), f"{name}: {int(bad.sum())} elements out of tolerance, max abs err {diff.max():.3e}"
     else:
         scale = max(ref.abs().max().item(), 1e-30)
-        assert diff.max().item() <= 1e-4 * scale, f"{name}: max err {diff.max():.3e} vs scale {scale:.3e}"
+        bad = diff > (1e-4 * ref.abs() + 2e-6 * scale)
+        assert not bad.any(), (f"{name}: {int(bad.sum())} elements out of tolerance, worst excess "
+                               f"{(diff - 1e-4 * ref.abs()).max().item() / scale:.3e} of the scale {scale:.3e}")
     return diff.max().item()
