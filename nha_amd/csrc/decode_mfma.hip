@@ -1,5 +1,7 @@
-// Matrix-core decode step for gfx950: bf16, K == V == D in {64,128}, M == 64 slots, window or ring
-// mode with a pre-rotated window query, up to 8 query heads per kv-head.
+// Matrix-core decode step for gfx950: bf16, K == V == D in {64,128}, M == 64 slots, up to 8 query
+// heads per kv-head; window or ring mode with a pre-rotated window query, or window mode with
+// in-kernel rotate-half RoPE of the raw query and window keys (cos / sin tables,
+// nha_fla/ops/nha/fused_recurrent.py:309-329).
 //
 // Same work split as decode.hip (one workgroup per (sequence, kv-head), state and window read
 // once), but the window is streamed ONCE, in 32-key blocks dealt round-robin to the waves:
@@ -78,9 +80,45 @@ __device__ __forceinline__ uint4 ld16_stream(const bf16_t* p) {
 
 constexpr int MS = 64;   // slots
 
-static size_t lds_bytes_for(int D, int G, int NW) {
+static size_t lds_bytes_for(int D, int G, int NW, bool rot) {
   const size_t fl = (size_t)2 * MS + 2 * D + (size_t)G * D + (size_t)G * MS + (size_t)NW * G * (D > MS ? D : MS) + 16 * NW * 2 + 32;
-  return fl * 4 + (size_t)NW * 32 * (D + 16) * 2;
+  // rotary: per wave the cos and sin pieces of one 32-key block, 16 bytes per lane and piece
+  return fl * 4 + (size_t)NW * 32 * (D + 16) * 2 + (rot ? (size_t)NW * 4 * (D / 32) * 1024 : 0);
+}
+
+// 16 bytes per lane from global memory into LDS at lds_base + 16 * lane (lds_base wave-uniform): the
+// cos / sin pieces of the next block wait there instead of in registers.  Outside the compiler's
+// memory model; it is issued before the register loads that the next wait counts, so that wait
+// covers it.
+__device__ __forceinline__ void g2l16(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
+}
+
+// rotate-half of the column pair (c, c + D/2), 8 columns at a time: xa holds columns c.., xb columns
+// c + D/2..; out_a = xa cos_a - xb sin_a, out_b = xb cos_b + xa sin_b (fp32, rounded to bf16 once)
+__device__ __forceinline__ void rope8(uint4& xa, uint4& xb, uint4 ca, uint4 sa, uint4 cb, uint4 sb) {
+  const uint32_t a[4] = {xa.x, xa.y, xa.z, xa.w}, b[4] = {xb.x, xb.y, xb.z, xb.w};
+  const uint32_t c0[4] = {ca.x, ca.y, ca.z, ca.w}, s0[4] = {sa.x, sa.y, sa.z, sa.w};
+  const uint32_t c1[4] = {cb.x, cb.y, cb.z, cb.w}, s1[4] = {sb.x, sb.y, sb.z, sb.w};
+  uint32_t oa[4], ob[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float ra[2], rb[2];
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      auto f = [&](uint32_t w) { return __uint_as_float(hlf ? (w & 0xffff0000u) : (w << 16)); };
+      ra[hlf] = f(a[i]) * f(c0[i]) - f(b[i]) * f(s0[i]);
+      rb[hlf] = f(b[i]) * f(c1[i]) + f(a[i]) * f(s1[i]);
+    }
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 pa, pb;
+    pa[0] = (__bf16)ra[0]; pa[1] = (__bf16)ra[1];
+    pb[0] = (__bf16)rb[0]; pb[1] = (__bf16)rb[1];
+    oa[i] = __builtin_bit_cast(uint32_t, pa);
+    ob[i] = __builtin_bit_cast(uint32_t, pb);
+  }
+  xa = make_uint4(oa[0], oa[1], oa[2], oa[3]);
+  xb = make_uint4(ob[0], ob[1], ob[2], ob[3]);
 }
 
 // One workgroup of NW waves per (sequence, kv-head): slot branch, then window branch, then the
@@ -88,7 +126,12 @@ static size_t lds_bytes_for(int D, int G, int NW) {
 // once (4 workgroups per CU), so nothing waits for a second round.  The slot branch issues every
 // load it needs up front (popped entry first, then all state rows): its dependent chain is
 // count -> popped row, and no workgroup's state rows queue behind another's window stream.
-template <int D, int G, int NW>
+// ROT: window mode with cos / sin tables.  Row w of the window is rotated by row w of the tables (the
+// tables' last W rows, ascending in time like the window), the query by row W-1.  A column and its
+// partner at +-D/2 sit in the same lane (k-steps j and j +- KS/2), so the rotation moves nothing
+// between lanes; the cos / sin pieces of a block are as many bytes again as twice its keys, so they
+// wait in a per-wave LDS area (requested one block ahead) instead of doubling the register buffers.
+template <int D, int G, int NW, bool ROT>
 __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecodeArgs a) {
   constexpr int NT = 64 * NW;
   constexpr int LDT = D + 16;   // bf16 row stride of a V tile
@@ -117,6 +160,9 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, qd = lane >> 4;
   lbf16* X = (lbf16*)(NHA_LDS void*)(ms + 32) + wave * 32 * LDT;   // wave-private V tile [32][LDT]
+  // rotary: [table cos|sin][row half t][k-step j] x 1 KB (16 bytes per lane), per wave
+  NHA_LDS unsigned char* const CS = (NHA_LDS unsigned char*)((lbf16*)(NHA_LDS void*)(ms + 32) + NW * 32 * LDT) + wave * (4 * KS * 1024);
+  const uint32_t cs_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)CS);   // wave-uniform: it goes to m0
   const int b = blockIdx.x / H, h = blockIdx.x % H;
   const int64_t bh = (int64_t)b * H + h;
   const float qscale = a.scale * LOG2E;
@@ -365,16 +411,53 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
 
   // ================= window branch: one pass, 32 keys per block, blocks wave, wave+NW, ... =======
   auto window_branch = [&]() {
+    // cos / sin pieces of block `blk` for this lane's two rows -> the wave's LDS area
+    const bf16_t* ctab = ROT ? (const bf16_t*)a.cos + (int64_t)b * a.cos_sb : nullptr;
+    const bf16_t* stab = ROT ? (const bf16_t*)a.sin + (int64_t)b * a.cos_sb : nullptr;
+    auto request_cs = [&](int blk) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        int w = 32 * blk + 16 * t + l16;
+        w = w < nvalid ? w : nvalid - 1;
+        const uint32_t off = ((uint32_t)w * (uint32_t)a.cos_sw + 8 * qd) * 2;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+          g2l16(ctab, off + 64 * j, cs_lds + ((0 * 2 + t) * KS + j) * 1024);
+          g2l16(stab, off + 64 * j, cs_lds + ((1 * 2 + t) * KS + j) * 1024);
+        }
+      }
+    };
+    auto cs_piece = [&](int tab, int t, int j) -> uint4 {
+      const u32x4 x = *reinterpret_cast<const NHA_LDS u32x4*>(CS + ((tab * 2 + t) * KS + j) * 1024 + lane * 16);
+      return make_uint4(x[0], x[1], x[2], x[3]);
+    };
     // window-query B fragments: lane (head l%16, piece l/16) of each 32-wide k-step
     bf16x8 qf[KS];
+    {
+      uint4 qx[KS];
+      const bf16_t* qsrc = ROT ? (const bf16_t*)a.q : (const bf16_t*)a.sq;
 #pragma unroll
-    for (int j = 0; j < KS; ++j) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (l16 < NG) x = *reinterpret_cast<const uint4*>((const bf16_t*)a.sq + ((int64_t)b * HQ + h * NG + l16) * D + 32 * j + 8 * qd);
-      qf[j] = as_bf16x8(x);
+      for (int j = 0; j < KS; ++j) {
+        qx[j] = make_uint4(0, 0, 0, 0);
+        if (l16 < NG) qx[j] = *reinterpret_cast<const uint4*>(qsrc + ((int64_t)b * HQ + h * NG + l16) * D + 32 * j + 8 * qd);
+      }
+      if (ROT) {   // the query's own position is the last row of the tables
+        const bf16_t* cq = ctab + (int64_t)(W - 1) * a.cos_sw + 8 * qd;
+        const bf16_t* sq_ = stab + (int64_t)(W - 1) * a.cos_sw + 8 * qd;
+#pragma unroll
+        for (int j = 0; j < KS / 2; ++j) {
+          const uint4 ca = *reinterpret_cast<const uint4*>(cq + 32 * j), sa = *reinterpret_cast<const uint4*>(sq_ + 32 * j);
+          const uint4 cb = *reinterpret_cast<const uint4*>(cq + 32 * (j + KS / 2)), sb = *reinterpret_cast<const uint4*>(sq_ + 32 * (j + KS / 2));
+          rope8(qx[j], qx[j + KS / 2], ca, sa, cb, sb);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < KS; ++j) qf[j] = as_bf16x8(qx[j]);
     }
     uint4 kr0[2 * KS], vr0[NVT], kr1[2 * KS], vr1[NVT];
     // issue order is the consumption order (the waits count loads still in flight)
+    __builtin_amdgcn_sched_barrier(0);
+    if (ROT) request_cs(wave);
     __builtin_amdgcn_sched_barrier(0);
     load_block(kr0, vr0, wave);
     __builtin_amdgcn_sched_barrier(0);
@@ -387,6 +470,20 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
 
     // consumes the block held in (kr, vr) and refills the registers as soon as they are free
     auto process = [&](uint4(&kr)[2 * KS], uint4(&vr)[NVT], int blk) {
+      if (ROT) {
+        // the block's keys are here (the compiler waits on kr), and with them the cos / sin pieces
+        // requested before them; rotate in place, then ask for the next block's pieces
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < KS / 2; ++j)
+            rope8(kr[t * KS + j], kr[t * KS + j + KS / 2], cs_piece(0, t, j), cs_piece(1, t, j), cs_piece(0, t, j + KS / 2),
+                  cs_piece(1, t, j + KS / 2));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the pieces have left LDS before new ones may land
+        __builtin_amdgcn_sched_barrier(0);
+        request_cs(blk + NW);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < KS; ++j) S0 = mfma16(as_bf16x8(kr[j]), qf[j], S0);
@@ -483,31 +580,31 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
 #define NHA_DEC_NW 2
 #endif
 
-template <int D, int G>
+template <int D, int G, bool ROT>
 int launch(const NhaDecodeArgs* a) {
   constexpr int NW = NHA_DEC_NW;
-  const size_t lds = lds_bytes_for(D, G, NW);
+  const size_t lds = lds_bytes_for(D, G, NW, ROT);
   static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)decode_mfma_kernel<D, G, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)decode_mfma_kernel<D, G, NW, ROT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) {
       set_error("decode: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
       return NHA_ERR_LAUNCH;
     }
     configured = true;
   }
-  hipLaunchKernelGGL((decode_mfma_kernel<D, G, NW>), dim3(a->B * a->H), dim3(64 * NW), lds, (hipStream_t)a->stream, *a);
+  hipLaunchKernelGGL((decode_mfma_kernel<D, G, NW, ROT>), dim3(a->B * a->H), dim3(64 * NW), lds, (hipStream_t)a->stream, *a);
   NHA_CHECK_LAUNCH("nha_decode_step");
   return NHA_OK;
 }
 
-template <int D>
+template <int D, bool ROT>
 int dispatch(const NhaDecodeArgs* a, int G) {
   switch (G) {
-    case 1: return launch<D, 1>(a);
-    case 2: return launch<D, 2>(a);
-    case 4: return launch<D, 4>(a);
-    default: return launch<D, 8>(a);
+    case 1: return launch<D, 1, ROT>(a);
+    case 2: return launch<D, 2, ROT>(a);
+    case 4: return launch<D, 4, ROT>(a);
+    default: return launch<D, 8, ROT>(a);
   }
 }
 
@@ -516,7 +613,15 @@ int dispatch(const NhaDecodeArgs* a, int G) {
 bool decode_mfma_supported(const NhaDecodeArgs* a) {
   if (a->dtype != NHA_DTYPE_BF16 || a->K != a->V || (a->K != 64 && a->K != 128)) return false;
   if (a->mode != NHA_DECODE_WINDOW && a->mode != NHA_DECODE_RING) return false;
-  if (!a->sq || a->cos) return false;
+  // either a pre-rotated query, or (window mode) cos / sin tables whose rows are 16-byte aligned pieces
+  const bool rot = a->cos != nullptr;
+  if (rot) {
+    if (a->mode != NHA_DECODE_WINDOW || !a->sin || a->sq) return false;
+    if (a->cos_sw % 8 != 0 || a->cos_sb % 8 != 0 || ((uintptr_t)a->cos & 15) || ((uintptr_t)a->sin & 15)) return false;
+    if (a->cos_sw * (int64_t)a->W >= ((int64_t)1 << 30)) return false;
+  } else if (!a->sq) {
+    return false;
+  }
   const int NG = a->HQ / a->H;
   // window rows are addressed with 32-bit element offsets
   return NG <= 8 && a->M == MS && (int64_t)a->W * a->H * a->K < ((int64_t)1 << 31);
@@ -526,7 +631,8 @@ int decode_mfma_impl(const NhaDecodeArgs* a) {
   const int NG = a->HQ / a->H;
   int G = 1;
   while (G < NG) G <<= 1;
-  return a->K == 64 ? dispatch<64>(a, G) : dispatch<128>(a, G);
+  if (a->cos) return a->K == 64 ? dispatch<64, true>(a, G) : dispatch<128, true>(a, G);
+  return a->K == 64 ? dispatch<64, false>(a, G) : dispatch<128, false>(a, G);
 }
 
 }  // namespace nha
