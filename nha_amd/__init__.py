@@ -6,6 +6,9 @@ from ._lib import NhaError
 from .ops import chunk_nha, fused_chunk_nha_prefill, fused_recurrent_nha, fused_recurrent_nha_decode
 from .ring import NHARingState, ring_decode_step
 from .cache import NHARingCache
+from .hybrid import (HybridNHAConfig, LlamaNativeHybridAttention, Qwen3MoeNativeHybridAttention, init_gates_from_keys,
+                     pool_k_to_g)
 
 __all__ = ["chunk_nha", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
-           "NHARingState", "ring_decode_step", "NHARingCache", "NhaError"]
+           "NHARingState", "ring_decode_step", "NHARingCache", "NhaError", "HybridNHAConfig",
+           "LlamaNativeHybridAttention", "Qwen3MoeNativeHybridAttention", "init_gates_from_keys", "pool_k_to_g"]

@@ -32,6 +32,7 @@ class NHARingCache:
         self.extra: List[Dict[str, object]] = []           # what `update` was given: recurrent / conv / ffn / attn state
         self.former_tokens = seen_tokens
         self._seen_tokens = seen_tokens
+        self._layer_tokens: Dict[int, int] = {}            # tokens a layer's ring has taken so far (longest sequence)
 
     def __len__(self) -> int:
         return max(len(self.states), len(self.extra))
@@ -133,20 +134,35 @@ class NHARingCache:
             raise ValueError("time-ordered views need sequences of equal length; use the ring buffers directly")
         return c[0]
 
-    def prefill(self, layer_idx: int, k_swa, k_gsa, v, g, final_state, cu_seqlens=None) -> NHARingState:
+    def prefill(self, layer_idx: int, k_swa, k_gsa, v, g, final_state, cu_seqlens=None,
+                window_size: Optional[int] = None) -> NHARingState:
         """Hand a prompt's prefill (operands and final state of chunk_nha / fused_chunk_nha_prefill
-        with (window_size_left, gsa_kv_shift) = (W-1, W)) over to the ring buffers of `layer_idx`."""
-        st = NHARingState.from_prefill(k_swa, k_gsa, v, g, final_state, self.window_size, cu_seqlens=cu_seqlens)
+        with (window_size_left, gsa_kv_shift) = (W-1, W)) over to the ring buffers of `layer_idx`.
+        `window_size` overrides the cache's window for this layer (models mix short-window layers with
+        2048-token ones)."""
+        W = self.window_size if window_size is None else int(window_size)
+        st = NHARingState.from_prefill(k_swa, k_gsa, v, g, final_state, W, cu_seqlens=cu_seqlens)
         self._grow(layer_idx)
         self.states[layer_idx] = st
-        self._count_tokens(layer_idx, int(st.count.max().item()), whole_step=True)
+        longest = k_swa.shape[1] if cu_seqlens is None else int(st.count.max().item())
+        self._layer_tokens[layer_idx] = longest
+        self._count_tokens(layer_idx, longest, whole_step=True)
         return st
+
+    def has_ring(self, layer_idx: int) -> bool:
+        """Whether `layer_idx` holds ring buffers (a prompt was handed over with `prefill`)."""
+        return self._ring(layer_idx) is not None
+
+    def layer_tokens(self, layer_idx: int) -> int:
+        """Tokens the ring of `layer_idx` has taken (its longest sequence): the next token's position."""
+        return self._layer_tokens.get(layer_idx, 0)
 
     def decode(self, layer_idx: int, q_gsa, q_swa, k_swa, k_gsa, v, g, scale: Optional[float] = None) -> torch.Tensor:
         """One token per sequence through layer `layer_idx`: pops the entry leaving the window into the
         slots, stores the new token, attends (one launch).  Tensors `[B, heads, dim]`; returns o."""
         st = self.states[layer_idx]
         o = ring_decode_step(st, q_gsa, q_swa, k_swa, k_gsa, v, g, scale=scale)
+        self._layer_tokens[layer_idx] = self._layer_tokens.get(layer_idx, 0) + 1
         self._count_tokens(layer_idx, 1, whole_step=True)
         return o
 

@@ -1,0 +1,269 @@
+"""Attention modules of the hybrid decoder models, on the GQA-native prefill and the ring-buffer decode.
+
+The reference's converted decoder models (nha_fla/models/qwen3_moe_nha/qwennha.py:43-413, the MoE
+flavour with per-head q/k RMSNorm; nha_fla/models/llama3_nha/llamanha.py:30-270, the dense flavour)
+replace every softmax-attention block by one of two kinds of layer, chosen per layer index
+(qwennha.py:64-68, llamanha.py:58-62):
+
+* an NHA layer (window <= 64): M gated slots + a short sliding window under one softmax.  Prefill is
+  one `fused_chunk_nha_prefill` call on the kv-head layout (qwennha.py:308-321; the dense flavour's
+  repeat-to-query-heads chain, llamanha.py:186-203, computes the same numbers).  Decode is one
+  `ring_decode_step` launch on the layer's resident ring buffers instead of the reference's
+  pop / cat-shift / re-rotate / decode-op sequence (qwennha.py:151-176, :200-226, :351-365): keys are
+  rotated once, at their own position, when they enter the ring.
+* a "full attention" layer (window 2048): plain sliding-window softmax attention preceded by
+  `num_slots` all-zero key/value rows (qwennha.py:323-336, llamanha.py:204-216).  Query t therefore
+  sees `clamp(W-1-t, 0, M)` zero-logit sinks next to its window.  Here that is the same NHA kernel with
+  slot states that stay zero (s = 0, g = 0: M zero logits with zero values at every t), rescaled per
+  query by (e^lse_swa + M) / (e^lse_swa + sinks(t)) from the window log-sum-exp the kernel returns.
+  Decode keeps all M sinks at every step, as the reference's torch path does (llamanha.py:238-246,
+  qwennha.py:377-389; its optional flash-attn call, qwennha.py:371-375, has none, and that package is
+  no part of this build).
+
+The cache is `NHARingCache`; a layer hands its prompt over with `cache.prefill` and steps with
+`cache.decode`.  Everything heavy runs in libnha_hip.so; the projections are torch GEMMs.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .cache import NHARingCache
+from .ops import chunk_nha, fused_chunk_nha_prefill
+
+GATE_LOGIT_NORMALIZER = 8          # qwennha.py:62, llamanha.py:96
+FULL_ATTENTION_WINDOW = 2048       # qwennha.py:66, llamanha.py:60
+NHA_MAX_WINDOW = 64                # layers with a longer window are the zero-sink kind (qwennha.py:307, llamanha.py:187)
+
+
+@dataclass
+class HybridNHAConfig:
+    """The fields of the reference's model configurations that the attention modules read
+    (configuration_qwen3_moe_nha.py:36-109, configuration_llama3_nha.py:13-73); any object with
+    these attributes (a transformers config among them) works in its place."""
+    hidden_size: int = 2048
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 4
+    head_dim: Optional[int] = None
+    num_slots: int = 64
+    window_size: int = 32
+    block_size: Optional[int] = None
+    transformer_idx: Optional[int] = None
+    attention_bias: bool = False
+    attention_dropout: float = 0.0
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 10000.0
+    max_position_embeddings: int = 32768
+
+
+class HeadRMSNorm(nn.Module):
+    """RMSNorm over the last (head) dimension, statistics in fp32, as the q/k norms of the MoE flavour
+    (qwennha.py:83-84)."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.variance_epsilon = eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        dt = x.dtype
+        x = x.to(torch.float32)
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * x.to(dt)
+
+
+class RotaryTables(nn.Module):
+    """cos / sin of the default rotary embedding, `[B, T, head_dim]` for integer positions `[B, T]`
+    (two copies of the head_dim/2 angles side by side: the rotate-half convention)."""
+
+    def __init__(self, head_dim: int, base: float = 10000.0):
+        super().__init__()
+        inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, position_ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        ang = position_ids.to(self.inv_freq.device, torch.float32)[..., None] * self.inv_freq
+        emb = torch.cat([ang, ang], -1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
+def rotate_half_apply(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x `[B, T, heads, D]`, cos / sin `[B, T, D]`: x cos + rotate_half(x) sin, evaluated in fp32 and
+    rounded to x's dtype once (as the decode kernel's in-kernel rotary does)."""
+    half = x.shape[-1] // 2
+    xf = x.to(torch.float32)
+    rot = torch.cat([-xf[..., half:], xf[..., :half]], -1)
+    return (xf * cos[:, :, None, :].to(torch.float32) + rot * sin[:, :, None, :].to(torch.float32)).to(x.dtype)
+
+
+def zero_sink_count(T: int, window: int, num_sinks: int, device) -> torch.Tensor:
+    """How many of the `num_sinks` zero rows in front of the sequence the W-wide window of query t still
+    covers: positions are shifted by num_sinks, the window spans [t + num_sinks - W + 1, t + num_sinks]."""
+    t = torch.arange(T, device=device)
+    return (window - 1 - t).clamp(0, num_sinks)
+
+
+def pool_k_to_g(k_weight: torch.Tensor, target_rows: int) -> torch.Tensor:
+    """Gate-projection initialisation from a key projection (training/convert_weight.py:7-22): the
+    `[rows, hidden]` key weight is averaged over groups of rows/target_rows consecutive rows."""
+    rows, hidden = k_weight.shape
+    if rows % target_rows != 0:
+        raise ValueError(f"The source dimension {rows} must be divisible by the target dimension {target_rows}.")
+    return k_weight.reshape(target_rows, rows // target_rows, hidden).mean(1)
+
+
+@torch.no_grad()
+def init_gates_from_keys(model: nn.Module) -> int:
+    """For every `...g_proj.weight` of `model` with a sibling `...k_proj.weight`, copy the pooled key
+    weight into it (training/convert_weight.py:36-48).  Returns the number of gate projections set."""
+    params = dict(model.named_parameters())
+    done = 0
+    for name, p in params.items():
+        if "g_proj" in name and "weight" in name:
+            kp = params.get(name.replace("g_proj", "k_proj"))
+            if kp is None:
+                continue
+            p.copy_(pool_k_to_g(kp.detach().to(torch.float32), p.shape[0]).to(p.dtype))
+            done += 1
+    return done
+
+
+class HybridNHAAttention(nn.Module):
+    """One attention block of a hybrid decoder: projections, gates, rotary, the NHA kernels, o_proj.
+    `forward` has the reference modules' signature and returns `(output, None)`."""
+
+    qk_norm = False
+
+    def __init__(self, config, layer_idx: int = 0):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_key_value_heads = config.num_key_value_heads or config.num_attention_heads
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.head_dim = getattr(config, "head_dim", None) or self.hidden_size // self.num_heads
+        self.scaling = self.head_dim ** -0.5
+        self.num_slots = config.num_slots
+        self.gate_logit_normalizer = GATE_LOGIT_NORMALIZER
+        self.window_size = config.window_size
+        block, which = getattr(config, "block_size", None), getattr(config, "transformer_idx", None)
+        if block is not None and which is not None and layer_idx % block == which:
+            self.window_size = FULL_ATTENTION_WINDOW
+        bias = bool(getattr(config, "attention_bias", False)) and self.qk_norm
+        HQ, H, D = self.num_heads, self.num_key_value_heads, self.head_dim
+        self.q_proj = nn.Linear(self.hidden_size, HQ * D, bias=bias)
+        self.k_proj = nn.Linear(self.hidden_size, H * D, bias=bias)
+        self.v_proj = nn.Linear(self.hidden_size, H * D, bias=bias)
+        self.o_proj = nn.Linear(HQ * D, self.hidden_size, bias=bias)
+        self.g_proj = nn.Linear(self.hidden_size, H * self.num_slots, bias=False)
+        if self.qk_norm:
+            eps = getattr(config, "rms_norm_eps", 1e-6)
+            self.q_norm = HeadRMSNorm(D, eps)
+            self.k_norm = HeadRMSNorm(D, eps)
+        self.rotary_emb = RotaryTables(D, getattr(config, "rope_theta", 10000.0))
+
+    @property
+    def is_nha_layer(self) -> bool:
+        return self.window_size <= NHA_MAX_WINDOW
+
+    def _tables(self, x, position_ids, position_embeddings, past, T):
+        if position_embeddings is not None:
+            cos, sin = position_embeddings
+            return cos[:, -T:], sin[:, -T:]
+        if position_ids is None:
+            start = past.layer_tokens(self.layer_idx) if past is not None else 0
+            position_ids = torch.arange(start, start + T, device=x.device)[None].expand(x.shape[0], T)
+        return self.rotary_emb(x, position_ids)
+
+    def forward(
+        self,
+        hidden_states: torch.Tensor,
+        attention_mask: Optional[torch.Tensor] = None,
+        position_ids: Optional[torch.LongTensor] = None,
+        past_key_value: Optional[NHARingCache] = None,
+        use_cache: bool = False,
+        cache_position: Optional[torch.LongTensor] = None,
+        position_embeddings: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+        **kwargs,
+    ) -> Tuple[torch.Tensor, None]:
+        if past_key_value is None:
+            past_key_value = kwargs.get("past_key_values")
+        if past_key_value is not None and not isinstance(past_key_value, NHARingCache):
+            raise TypeError("the hybrid attention modules keep their decode state in an nha_amd.NHARingCache "
+                            f"(NHARingCache.from_legacy_cache converts), got {type(past_key_value).__name__}")
+        B, T, _ = hidden_states.shape
+        HQ, H, D, M, W = self.num_heads, self.num_key_value_heads, self.head_dim, self.num_slots, self.window_size
+        q = self.q_proj(hidden_states).view(B, T, HQ, D)
+        k = self.k_proj(hidden_states).view(B, T, H, D)
+        v = self.v_proj(hidden_states).view(B, T, H, D)
+        if self.qk_norm:
+            q, k = self.q_norm(q), self.k_norm(k)
+        nha = self.is_nha_layer
+        if nha:
+            g = F.logsigmoid(self.g_proj(hidden_states).view(B, T, H, M)) / self.gate_logit_normalizer
+        else:                                  # the slots of a full-attention layer never absorb anything
+            g = torch.zeros(B, T, H, M, dtype=v.dtype, device=v.device)
+        has_state = past_key_value is not None and past_key_value.has_ring(self.layer_idx)
+        decode_step = (not self.training) and T == 1 and has_state
+        mask_t = None
+        if attention_mask is not None:         # left padding: a padded token writes nothing into the slots
+            if attention_mask.dim() != 2:
+                raise ValueError(f"attention_mask must be the [batch, tokens] padding mask, got {tuple(attention_mask.shape)}")
+            mask_t = attention_mask[:, -T:].to(v.dtype)[:, :, None, None]
+            v = v * mask_t
+        cos, sin = self._tables(v, position_ids, position_embeddings, past_key_value, T)
+        sq, sk = rotate_half_apply(q, cos, sin), rotate_half_apply(k, cos, sin)
+        dt = q.dtype
+        if dt == torch.float32 and torch.is_autocast_enabled():
+            dt = torch.get_autocast_gpu_dtype()
+        q, k, v, g, sq, sk = (x.to(dt).contiguous() for x in (q, k, v, g, sq, sk))
+
+        if decode_step:
+            o = past_key_value.decode(self.layer_idx, q[:, 0], sq[:, 0], sk[:, 0], k[:, 0], v[:, 0], g[:, 0],
+                                      scale=self.scaling)[:, None]
+        else:
+            if has_state:
+                raise NotImplementedError("a multi-token step on top of a cached prompt is not supported "
+                                          "(the reference's modules do not support it either)")
+            if nha:
+                s = 1 - torch.exp(g).to(g.dtype)
+                if mask_t is not None:
+                    s = s * mask_t
+            else:
+                s = torch.zeros_like(g)
+            want_state = use_cache or past_key_value is not None
+            if nha and not torch.is_grad_enabled():
+                o, state = fused_chunk_nha_prefill(q=q, k=k, v=v, rotary_q=sq, rotary_k=sk, s=s, g=g, window_size=W,
+                                                   output_final_state=want_state, scale=self.scaling)
+            else:
+                out = chunk_nha(sq, sk, q, k, v, s, g, window_size_left=W - 1, window_size_right=0, gsa_kv_shift=W,
+                                output_final_state=want_state, scale=self.scaling)
+                o, lse_swa = out[0], out[1]
+                state = out[3] if want_state else (None, None)
+                if not nha:
+                    # M zero-logit sinks were in the softmax at every t; the reference's window covers
+                    # zero_sink_count(t) of them
+                    e = torch.exp(-lse_swa)                                         # [B,T,HQ] fp32
+                    n0 = zero_sink_count(T, W, M, e.device).to(e.dtype)[None, :, None]
+                    o = (o.to(torch.float32) * ((1 + M * e) / (1 + n0 * e))[..., None]).to(o.dtype)
+            if past_key_value is not None:
+                past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W)
+        o = self.o_proj(o.reshape(B, T, HQ * D))
+        return o, None
+
+
+class Qwen3MoeNativeHybridAttention(HybridNHAAttention):
+    """The MoE flavour's block: RMSNorm on every q and k head before rotary, optional projection biases
+    (nha_fla/models/qwen3_moe_nha/qwennha.py:43-86)."""
+    qk_norm = True
+
+
+class LlamaNativeHybridAttention(HybridNHAAttention):
+    """The dense flavour's block: bias-free projections, no q/k norm (nha_fla/models/llama3_nha/llamanha.py:30-62)."""
+    qk_norm = False
