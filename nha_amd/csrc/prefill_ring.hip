@@ -17,8 +17,12 @@
 //
 // LDS layouts (bank-conflict free for the two fragment reads without padding, which a 1 KB wave
 // load cannot produce): a 32-row unit is cut into 16-row x 32-column blocks of 1 KB, a row of a block
-// is 64 contiguous bytes.  "K layout" (row fragments, ds_read_b128) XORs the 16-byte piece index
-// inside a row with (row / 4) % 4; "V layout" (transposing ds_read_b64_tr_b16) stores pieces in order.
+// is 64 bytes.  "K layout" (row fragments, ds_read_b128): the row's 64 bytes are contiguous and the
+// 16-byte piece index inside it is XORed with (row / 4) % 4.  "V layout" (transposing
+// ds_read_b64_tr_b16, which takes 16 columns = 32 bytes of each of 16 rows per wave instruction): the
+// block is two planes of 16 rows x 32 bytes, columns 0..15 then columns 16..31, so that the 512 bytes
+// of one instruction are contiguous and use every bank twice (with 64-byte rows they used half the
+// banks four times: SQ_LDS_BANK_CONFLICT 9.8e7 -> 3.9e7 cycles per launch at the T = 8192 shape).
 #include "mfma_common.h"
 
 #include <mutex>
@@ -107,6 +111,8 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   // ---- load descriptors of this wave: LDS-direct load i of a unit / a 64-row tile ------------------
   // block index b = wave + 8 i; per lane: row lane / 4 of the block, piece lane % 4 of its 64-byte row
   const int lrow16 = lane >> 2, lsl = lane & 3, lswz = lsl ^ ((lane >> 4) & 3);
+  // V layout: the lane's 16 bytes are piece lane % 2 of plane lane / 32, row (lane % 32) / 2
+  const int lrowv = (lane & 31) >> 1, lpv = 2 * (lane >> 5) + (lane & 1);
   uint32_t u_off[LPW];          // byte offset from the unit's first row (token rows, stride H*D)
   uint32_t u_lds[LPW];          // LDS address of the block inside ring slot 0
   bool u_isv[LPW];
@@ -117,7 +123,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     const int bb = isv ? b - 2 * KS : b;
     const int rh = bb / KS, cq = bb % KS;
     u_isv[i] = isv;
-    u_off[i] = ((uint32_t)(16 * rh + lrow16) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lsl : lswz)) * 8) * 2;
+    u_off[i] = ((uint32_t)(16 * rh + (isv ? lrowv : lrow16)) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lpv : lswz)) * 8) * 2;
     u_lds[i] = lds0 + (isv ? C::RING_V : C::RING_K) + rh * HB + cq * 1024;
   }
   // request unit u; rows past eos (units 0 and 1 only) are read from row eos - 1: always masked, always finite
@@ -130,9 +136,9 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       const bool isv = b >= 2 * KS;
       const int bb = isv ? b - 2 * KS : b;
       const int rh = bb / KS, cq = bb % KS;
-      int row = key0 + 16 * rh + lrow16;
+      int row = key0 + 16 * rh + (isv ? lrowv : lrow16);
       row = row < eos ? row : eos - 1;
-      const uint32_t off = ((uint32_t)(row - bos) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lsl : lswz)) * 8) * 2;
+      const uint32_t off = ((uint32_t)(row - bos) * (uint32_t)(H * D) + (uint32_t)(4 * cq + (isv ? lpv : lswz)) * 8) * 2;
       const bf16_t* base = (isv ? p.v : p.k_swa) + ((int64_t)bos * H + h) * D;
       g2l16(base, off, u_lds[i] + slot * UB);
     }
@@ -145,8 +151,8 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       const int b = wave + 8 * i;            // < 4 KS
       const int unit = b / (2 * KS), bb = b % (2 * KS);
       const int rh = bb / KS, cq = bb % KS;
-      const int r = 32 * unit + 16 * rh + lrow16;
-      const uint32_t off = ((uint32_t)rowmap(r) * stride + (uint32_t)(4 * cq + (vlay ? lsl : lswz)) * 8) * 2;
+      const int r = 32 * unit + 16 * rh + (vlay ? lrowv : lrow16);
+      const uint32_t off = ((uint32_t)rowmap(r) * stride + (uint32_t)(4 * cq + (vlay ? lpv : lswz)) * 8) * 2;
       g2l16(src, off, lds0 + lds_tile + unit * UB + rh * HB + cq * 1024);
     }
   };
@@ -231,14 +237,14 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   constexpr float THR = 8.f;
 
   const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
-  const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 64 + 8 * (l16 & 3));
+  const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
   // row fragment (rows 16 kk + l16 of a unit, columns 32 ks + 8 kb ..) of a K-layout unit at byte address a
   auto kfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {
     return *reinterpret_cast<const NHA_LDS bf16x8*>(lds + a + kk * HB + ks * 1024);
   };
   // transposed fragment of a V-layout unit: X[4 kb + e][16 db + l16] (e < 4) and X[16 + 4 kb + e - 4][..]
   auto vfrag = [&](uint32_t a, int db) -> bf16x8 {
-    const lbyte* pa = lds + a + (db >> 1) * 1024 + (db & 1) * 32;
+    const lbyte* pa = lds + a + (db >> 1) * 1024 + (db & 1) * 512;
     struct { s16x4 a, b; } t;
     t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
     t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + HB));
@@ -515,13 +521,13 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)sv[e] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
     }
-    *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + (r32 & 15) * 64 + (m & 31) * 2) = out;
+    *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
   }
   __syncthreads();
 
   // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
   auto etab_tr = [&](int Q, int pr, int mb) -> bf16x8 {
-    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 32 + vaddr;
+    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 512 + vaddr;
     struct { s16x4 a, b; } t;
     t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
     t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + 2048));
@@ -529,10 +535,10 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   };
   // E_Q by rows: row = token 16 jb + l16, contraction over the slots 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
   auto etab_row = [&](int Q, int jb, int pr) -> bf16x8 {
-    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 64 + 8 * kb;
+    const lbyte* pa = lds + C::ETAB + ((Q < 2 ? Q : 2 * Q - 2) + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 32 + 8 * kb;
     struct { bf16x4 a, b; } t;
     t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(pa);
-    t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 32);
+    t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 512);
     return __builtin_bit_cast(bf16x8, t);
   };
   float lg[RQB];
