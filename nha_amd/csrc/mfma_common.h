@@ -29,7 +29,10 @@ constexpr int GLD = 68;       // LDS row stride (floats) of the gate-cumsum tabl
 constexpr int SLD = 72;       // LDS row stride (bf16) of the s tables
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
-constexpr float DECAY_CLAMP = 80.f;   // largest positive decay exponent formed on the MFMA path
+// Largest positive decay exponent formed on the MFMA path.  A factor s exp(60) = 1.1e26 still multiplies
+// unscaled intra-chunk scores (the layer's default scale is 1) summed over 16 rows with e^28 of fp32
+// range to spare; sub-blocks that decay faster are flagged and recomputed exactly.
+constexpr float DECAY_CLAMP = 60.f;
 
 struct MP {
   const bf16_t *q_swa, *k_swa, *q_gsa, *k_gsa, *v, *s, *g;

@@ -546,6 +546,9 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   for (int qb = 0; qb < RQB; ++qb) {
     const int Q = qb0 + qb;                // sub-block index inside the chunk
     const int irow = 16 * Q + l16;         // this lane's query row inside the chunk
+    // the window's own log-sum-exp, taken before the slots join: afterwards the window sum is only known
+    // relative to the joint maximum and underflows when the slot logits top the window's by 2^126
+    if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[qb][0]) - nm[qb]) * LN2;
     // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
     f32x4 ok[4];
 #pragma unroll
@@ -610,6 +613,9 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       rescale_acc(qb, delta);
     }
     float psum = 0.f;
+    f32x4 sl[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) sl[mb] = ok[mb];
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -620,7 +626,18 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     psum += __shfl_xor(psum, 16, 64);
     psum += __shfl_xor(psum, 32, 64);
     lg[qb] = psum;
-    if (p.lse_gsa && kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(psum) - nm[qb]) * LN2;
+    if (p.lse_gsa) {
+      // the slots' own log-sum-exp, relative to their own maximum (log2 units; logits were saved in `sl`)
+      const float ms = max_over_rows(xmax);
+      float pown = 0.f;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pown += fexp2(sl[mb][r] - ms);
+      pown += __shfl_xor(pown, 16, 64);
+      pown += __shfl_xor(pown, 32, 64);
+      if (kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(pown) + ms) * LN2;
+    }
     bf16x8 bp[2], bpr[2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr) {
@@ -694,7 +711,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       const int dcol = 16 * (db + (kb & 1)) + 8 * (kb >> 1);
       if (irow < rows) *reinterpret_cast<uint4*>(op + dcol) = make_uint4(a[0], a[1], b[0], b[1]);
     }
-    if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(lwt) - nm[qb]) * LN2;
   }
 }
 

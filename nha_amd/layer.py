@@ -151,16 +151,20 @@ class ShortConvolution(nn.Module):
 
 
 def get_unpad_data(attention_mask: torch.Tensor):
-    seqlens = attention_mask.sum(-1, dtype=torch.int32)
-    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
-    cu = F.pad(torch.cumsum(seqlens, 0, dtype=torch.int32), (1, 0))
-    return indices, cu, int(seqlens.max())
+    """Positions of the kept tokens in the flattened `[batch * seqlen]` order, the packed sequences'
+    boundaries (int32, leading zero) and the longest sequence, from a `[batch, seqlen]` 0/1 mask."""
+    kept = attention_mask.reshape(-1).nonzero().squeeze(-1)
+    lengths = attention_mask.to(torch.int32).sum(dim=-1)
+    bounds = torch.zeros(lengths.numel() + 1, dtype=torch.int32, device=attention_mask.device)
+    bounds[1:] = lengths.cumsum(0)
+    return kept, bounds, int(lengths.max())
 
 
 def pad_input(x: torch.Tensor, indices: torch.Tensor, batch: int, seqlen: int):
-    out = x.new_zeros(batch * seqlen, *x.shape[1:])
-    out[indices] = x
-    return out.view(batch, seqlen, *x.shape[1:])
+    """Inverse of the unpadding: rows of the packed `x` go back to their `[batch, seqlen]` places, zeros elsewhere."""
+    full = torch.zeros(batch * seqlen, *x.shape[1:], dtype=x.dtype, device=x.device)
+    full.index_copy_(0, indices, x)
+    return full.view(batch, seqlen, *x.shape[1:])
 
 
 class NativeHybridAttention(nn.Module):
@@ -197,58 +201,42 @@ class NativeHybridAttention(nn.Module):
         **kwargs,
     ):
         super().__init__()
-        self.mode = mode
-        self.hidden_size = hidden_size
-        self.expand_k, self.expand_v = expand_k, expand_v
-        self.num_heads = num_heads
-        self.num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
-        self.num_kv_groups = self.num_heads // self.num_kv_heads
-        self.key_dim = int(hidden_size * expand_k)
-        self.value_dim = int(hidden_size * expand_v)
-        self.key_dim_per_group = self.key_dim // self.num_kv_groups
-        self.value_dim_per_group = self.value_dim // self.num_kv_groups
-        self.head_k_dim = self.key_dim // self.num_heads
-        self.head_v_dim = self.value_dim // self.num_heads
-        self.use_short_conv, self.conv_size, self.conv_bias = use_short_conv, conv_size, conv_bias
-        self.gate_logit_normalizer = gate_logit_normalizer
-        self.use_output_gate, self.use_norm, self.fuse_norm = use_output_gate, use_norm, fuse_norm
-        self.scale = scale
-        self.window_size = window_size
-        self.rope_theta = rope_theta
-        self.max_position_embeddings = max_position_embeddings
-        self.gsa_aux_loss_enable = gsa_aux_loss_enable
-        self.gsa_aux_loss_coeff = gsa_aux_loss_coeff
-        self.gsa_aux_loss_target_ratio = gsa_aux_loss_target_ratio
-        self.gsa_kv_shift = gsa_kv_shift
-        self.num_slots = self.head_k_dim if num_slots is None else num_slots
-        self.layer_idx = layer_idx
-        self.norm_eps = norm_eps
-        if layer_idx is None:
-            warnings.warn(
-                f"Instantiating {self.__class__.__name__} without passing `layer_idx` is not recommended and will "
-                "to errors during the forward call, if caching is used. Please make sure to provide a `layer_idx` "
-                "when creating this class.",
-            )
-        self.register_module('feature_map', None)
-        if feature_map == 'swish':
-            self.feature_map = SwishFeatureMap()
-        elif feature_map == 'relu':
-            self.feature_map = ReLUFeatureMap()
-        elif feature_map == 't2r':
-            self.feature_map = T2RFeatureMap(self.head_k_dim, self.head_k_dim)
-        else:
+        if feature_map not in ('swish', 'relu', 't2r'):
             raise NotImplementedError(f"Feature map `{feature_map}` is not supported now.")
-        self.q_proj = nn.Linear(self.hidden_size, self.key_dim, bias=False)
-        self.k_proj = nn.Linear(self.hidden_size, self.key_dim_per_group, bias=False)
-        self.v_proj = nn.Linear(self.hidden_size, self.value_dim_per_group, bias=False)
-        self.f_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.num_slots, bias=False)
+        if layer_idx is None:
+            warnings.warn(f"{type(self).__name__} was built without `layer_idx`: a forward call that uses a cache "
+                          "needs it to find this layer's states and will fail.")
+        kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        groups = num_heads // kv_heads
+        key_dim, value_dim = int(hidden_size * expand_k), int(hidden_size * expand_v)
+        # the attributes the reference layer exposes (nha_fla/layers/nha.py:59-98), under the same names
+        for name, value in dict(
+                mode=mode, hidden_size=hidden_size, expand_k=expand_k, expand_v=expand_v, num_heads=num_heads,
+                num_kv_heads=kv_heads, num_kv_groups=groups, key_dim=key_dim, value_dim=value_dim,
+                key_dim_per_group=key_dim // groups, value_dim_per_group=value_dim // groups,
+                head_k_dim=key_dim // num_heads, head_v_dim=value_dim // num_heads,
+                use_short_conv=use_short_conv, conv_size=conv_size, conv_bias=conv_bias,
+                gate_logit_normalizer=gate_logit_normalizer, use_output_gate=use_output_gate, use_norm=use_norm,
+                fuse_norm=fuse_norm, scale=scale, window_size=window_size, rope_theta=rope_theta,
+                max_position_embeddings=max_position_embeddings, gsa_aux_loss_enable=gsa_aux_loss_enable,
+                gsa_aux_loss_coeff=gsa_aux_loss_coeff, gsa_aux_loss_target_ratio=gsa_aux_loss_target_ratio,
+                gsa_kv_shift=gsa_kv_shift, layer_idx=layer_idx, norm_eps=norm_eps).items():
+            setattr(self, name, value)
+        self.num_slots = self.head_k_dim if num_slots is None else num_slots
+        maps = {'swish': SwishFeatureMap, 'relu': ReLUFeatureMap, 't2r': lambda: T2RFeatureMap(self.head_k_dim, self.head_k_dim)}
+        self.feature_map = maps[feature_map]()
+        # projections: queries at the q-head count, keys / values / gate logits at the kv-head count
+        widths = dict(q_proj=key_dim, k_proj=self.key_dim_per_group, v_proj=self.value_dim_per_group,
+                      f_proj=kv_heads * self.num_slots)
+        for name, width in widths.items():
+            setattr(self, name, nn.Linear(hidden_size, width, bias=False))
         if use_short_conv:
-            self.q_conv1d = ShortConvolution(self.key_dim, conv_size, bias=conv_bias, activation='silu')
-            self.k_conv1d = ShortConvolution(self.key_dim_per_group, conv_size, bias=conv_bias, activation='silu')
-            self.v_conv1d = ShortConvolution(self.value_dim_per_group, conv_size, bias=conv_bias, activation='silu')
-        self.g_norm = RMSNorm(self.hidden_size, elementwise_affine, eps=norm_eps, dtype=torch.float32)
-        self.o_proj = nn.Linear(self.value_dim, self.hidden_size, bias=False)
-        self.rotary = RotaryEmbedding(dim=self.head_k_dim, base=self.rope_theta)
+            for name in ('q', 'k', 'v'):
+                setattr(self, name + '_conv1d',
+                        ShortConvolution(widths[name + '_proj'], conv_size, bias=conv_bias, activation='silu'))
+        self.g_norm = RMSNorm(hidden_size, elementwise_affine, eps=norm_eps, dtype=torch.float32)
+        self.o_proj = nn.Linear(value_dim, hidden_size, bias=False)
+        self.rotary = RotaryEmbedding(dim=self.head_k_dim, base=rope_theta)
         self.fuse_glue = True
         self._inv_freq = None
 
@@ -270,11 +258,9 @@ class NativeHybridAttention(nn.Module):
         **kwargs,
     ) -> Tuple[torch.Tensor, None, object]:
         if attention_mask is not None:
-            assert len(attention_mask.shape) == 2, (
-                "Expected attention_mask as a 0-1 matrix with shape [batch_size, seq_len] "
-                "for padding purposes (0 indicating padding). "
-                "Arbitrary attention masks of shape [batch_size, seq_len, seq_len] are not allowed."
-            )
+            assert attention_mask.dim() == 2, (
+                f"attention_mask must be the [batch, tokens] padding mask (1 = token, 0 = padding); got shape "
+                f"{tuple(attention_mask.shape)}.  Per-query masks [batch, tokens, tokens] are not supported.")
         batch_size, q_len, _ = hidden_states.shape
         last_state = None
         if past_key_values is not None and len(past_key_values) > self.layer_idx:
@@ -282,10 +268,8 @@ class NativeHybridAttention(nn.Module):
         recurrent_state = last_state['recurrent_state'] if last_state is not None else None
         if q_len == 1 and last_state is not None:
             raise NotImplementedError(
-                "Single-token decode for the NHA layer was removed: its only "
-                "implementation called the never-released fused_recurrent_nha_step. "
-                "Run the chunk path (prefill-style) instead."
-            )
+                "this layer has no single-token step on top of a cached state (the reference layer raises here "
+                "too); call it on the whole chunk, or decode with nha_amd.NHARingCache / the hybrid attention blocks")
         mode = self.mode
         cu_seqlens = kwargs.get('cu_seqlens')
         max_seqlen = kwargs.get('max_seqlen')

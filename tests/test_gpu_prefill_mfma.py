@@ -97,6 +97,33 @@ def test_mfma_isolated_strong_decay(D, HQ, H):
     run_case("isolated decay shifted", d, wl=31, shift=32, dtype=BF, impl="mfma", cu=cu)
 
 
+@pytest.mark.parametrize("HQ,H", [(8, 2), (2, 2)])
+@pytest.mark.parametrize("per_row", [-3.55, -4.6])
+def test_mfma_decay_near_the_clamp_at_scale_one(HQ, H, per_row):
+    """scale = 1 (the layer's default) with q / k of magnitude 2, and slots whose gates decay a 16-row
+    sub-block by e^-57 (just inside what the matrix cores factor: s exp(57) times unscaled scores summed
+    over 16 rows must stay inside fp32) or by e^-74 (flagged, recomputed exactly).  Logits of this size
+    make the softmax sharp, so bf16 rounding of the states moves single outputs by more than the
+    element-wise bar: finite everywhere, relative L2 within 3e-2."""
+    from nha_amd import chunk_nha
+    d = prefill_inputs(870, 2, 192, HQ, H, 64, 64, 64, dtype=BF, gate_div=8.0, qk_scale=2.0)
+    g = d["g"].float()
+    g[:, 16:32, :, 3] = per_row
+    g[:, 80:96, 0, 40:44] = per_row
+    g[:, 160:176, H - 1, 63] = per_row
+    d["g"] = g.to(BF)
+    d["s"] = (1 - d["g"].float().exp()).to(BF)
+    for wl, shift in ((31, 32), (64, 0)):
+        c = [d[k].cuda() for k in KEYS]
+        o, ls, lg = chunk_nha(*c, window_size_left=wl, gsa_kv_shift=shift, scale=1.0, impl="mfma")
+        ro, rls, rlg, _, _ = R.prefill_ref(*[d[k] for k in KEYS], window_size_left=wl, gsa_kv_shift=shift, scale=1.0)
+        for name, got, ref in (("o", o, ro), ("lse_swa", ls, rls), ("lse_gsa", lg, rlg)):
+            got = got.double().cpu()
+            assert torch.isfinite(got).all(), name
+            rel = ((got - ref).norm() / ref.norm()).item()
+            assert rel <= 3e-2, (name, wl, shift, rel)
+
+
 def test_mfma_matches_simple_kernels_at_size():
     """A shape the CPU recurrence cannot reach in seconds: MFMA kernels vs the fp32-math kernels."""
     from nha_amd import chunk_nha
