@@ -114,5 +114,8 @@ __device__ __forceinline__ int seb_base(int Q) { return Q == 0 ? 0 : Q == 1 ? 2 
 // output pass with LDS-direct window loads (prefill_ring.hip); false when the shape is not served
 bool prefill_ring_supported(const mf::MP& p, int D);
 int prefill_ring_launch(const mf::MP& p, int D, hipStream_t st);
+// the same for head size 256, one query head per workgroup (prefill_ring256.hip)
+bool prefill_ring256_supported(const mf::MP& p, int D);
+int prefill_ring256_launch(const mf::MP& p, hipStream_t st);
 
 }  // namespace nha

@@ -1169,6 +1169,8 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     static const bool ring_off = getenv("NHA_PREFILL_NO_RING") != nullptr;   // A/B switch for measurements
     if (!ring_off && prefill_ring_supported(p, D)) {
       rc = prefill_ring_launch(p, D, st);
+    } else if (!ring_off && prefill_ring256_supported(p, D)) {
+      rc = prefill_ring256_launch(p, st);
     } else if constexpr (D <= 128) {
       if (p.NG % 4 == 0) rc = launch_out<D, 4, 8, 64>(p, st);
       else if (p.NG % 2 == 0) rc = launch_out<D, 2, 8, 64>(p, st);

@@ -1,0 +1,660 @@
+// Output pass of the bf16 matrix-core prefill at head size 256 (K == V == 256, M == 64), one query head
+// per workgroup: the data movement and loop of prefill_ring.hip (operands straight from global memory
+// into LDS, the window walked first in 32-key units, the slot branch folded into the running softmax
+// afterwards; chunk algebra of nha_fla/ops/nha/chunk_fused.py:186-283, one softmax over
+// [slots | window] as in nha_fla/ops/nha/chunk.py:459-470) re-proportioned for rows of 512 bytes:
+//
+//  * One workgroup = one 64-row chunk of one query head, 4 waves of 16 query rows: the accumulators of
+//    16 rows x 256 columns are 64 registers, those of 32 rows would not leave room for the fragments.
+//  * A unit of 32 keys is 16 KB of K and 16 KB of V.  K and V units live in two rings of three buffers
+//    with their own schedules: iteration u forms the scores of unit u + 1 and the products of unit u, so
+//    after its barrier the K buffer of unit u + 1 and the V buffer of unit u - 1 are free and take K of
+//    unit u + 4 and V of unit u + 2; both have two iterations to land.
+//  * Fragments are read from LDS a few matrix instructions before their use and not earlier: sixteen K
+//    and sixteen V fragments held at once (128 registers) would push the accumulators out of the
+//    register file.
+//  * The slot-branch operands (four 64 x 256 tiles, 128 KB) do not fit beside the rings: they pass
+//    through the ring buffers after the window loop, three tiles at once (their latency is covered by
+//    building the decay tables) and the fourth while the first three are worked on.
+#include "mfma_common.h"
+
+#include <mutex>
+
+namespace nha {
+namespace {
+using namespace mf;
+
+typedef NHA_LDS unsigned char lbyte;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+#define NHA_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define NHA_PIN(x) asm volatile("" : "+v"(x))
+
+__device__ __forceinline__ unsigned cvt2(float a, float b) {
+  bf16x2 t;
+  t[0] = (__bf16)a;
+  t[1] = (__bf16)b;
+  return __builtin_bit_cast(unsigned, t);
+}
+
+// 16 bytes per lane from global memory into LDS at lds_base + 16 * lane (lds_base wave-uniform).
+// Issued outside the compiler's memory model: every wait on these loads is written by hand.
+__device__ __forceinline__ void g2l16(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+struct Cfg {
+  static constexpr int D = 256;
+  static constexpr int KS = D / 32;            // 32-column blocks per row == contraction steps of q.k
+  static constexpr int DB = D / 16;            // 16-row blocks of O^T
+  static constexpr int UB = 32 * D * 2;        // bytes of a 32-row unit buffer (16 KB)
+  static constexpr int HB = UB / 2;            // bytes of its 16-row half
+  static constexpr int NR = 3;                 // buffers per ring
+  static constexpr int NW = 4;                 // waves
+  static constexpr int BPU = 2 * KS;           // 1 KB blocks of a unit buffer (16)
+  static constexpr int LPB = BPU / NW;         // LDS-direct loads per wave for one buffer (4)
+  static constexpr int RING_K = 0, RING_V = NR * UB;
+  static constexpr int GC = 2 * NR * UB;       // gate cumsum fp32 [64][64], pieces XORed with row % 16
+  static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
+  static constexpr int ETAB = SS + 8192;       // decay tables, 6 units of 4 KB
+  static constexpr int BYTES = ETAB + 6 * 4096;
+  static constexpr int NGS = 16 / NW + 8 / NW; // loads per wave for the gate and s blocks (6)
+};
+
+// LDS layouts as in prefill_ring.hip: a 32-row buffer is cut into 16-row x 32-column blocks of 1 KB
+// (half h, column block c at h * HB + c * 1024).  K layout: 64-byte rows, 16-byte piece index XORed
+// with (row / 4) % 4.  V layout: two planes of 16 rows x 32 bytes (columns 0..15, then 16..31).
+__global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
+  using C = Cfg;
+  constexpr int D = C::D, KS = C::KS, DB = C::DB, UB = C::UB, HB = C::HB, NR = C::NR, NW = C::NW, LPB = C::LPB;
+  extern __shared__ __align__(1024) unsigned char smem_[];
+  lbyte* const lds = (lbyte*)smem_;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ, NG = p.NG;
+  // grid = (query head, chunk), chunks from the last to the first
+  const int chunk = p.NT - 1 - blockIdx.y;
+  const int hq = blockIdx.x, h = hq / NG;
+  const int Q = wave;                          // this wave's 16-row sub-block of the chunk
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int rows = (eos - c0) < BT ? (eos - c0) : BT;
+  const float cs = p.scale * LOG2E;
+  const int64_t cg = (int64_t)chunk * H + h;
+  const int irow = 16 * Q + l16;               // this lane's query row inside the chunk
+
+  // window units: unit u covers keys [c0 + 32 - 32 u, c0 + 64 - 32 u); c0 - bos is a multiple of 64, so no
+  // unit starts before its sequence; units 0 and 1 are the chunk's own rows and may run past eos
+  int lowest = bos;
+  if (p.wl >= 0 && c0 - p.wl > bos) lowest = c0 - p.wl;
+  const int nunits = (c0 + 64 - lowest + 31) / 32;   // >= 2
+
+  // ---- LDS-direct loads: block b = wave + 4 i of a buffer; per lane a row of the block and a 16-byte piece
+  const int lrow16 = lane >> 2, lswz = (lane & 3) ^ ((lane >> 4) & 3);          // K layout
+  const int lrowv = (lane & 31) >> 1, lpv = 2 * (lane >> 5) + (lane & 1);         // V layout
+  // one 32-row buffer from rows of `src` (row stride in elements): row r of the buffer is global row rowmap(r)
+  auto issue_buffer = [&](uint32_t lds_buf, bool vlay, const bf16_t* src, uint32_t stride, auto rowmap) {
+#pragma unroll
+    for (int i = 0; i < LPB; ++i) {
+      const int b = wave + NW * i;           // < 16
+      const int rh = b / KS, cq = b % KS;
+      const int r = 16 * rh + (vlay ? lrowv : lrow16);
+      const uint32_t off = ((uint32_t)rowmap(r) * stride + (uint32_t)(4 * cq + (vlay ? lpv : lswz)) * 8) * 2;
+      g2l16(src, off, lds0 + lds_buf + rh * HB + cq * 1024);
+    }
+  };
+  const bf16_t* const kbase = p.k_swa + ((int64_t)bos * H + h) * D;
+  const bf16_t* const vbase = p.v + ((int64_t)bos * H + h) * D;
+  // rows past eos (units 0 and 1 only) are read from row eos - 1: always masked, always finite
+  auto unit_row = [&](int u) {
+    const int key0 = c0 + 32 - 32 * u - bos;
+    const int last = eos - 1 - bos;
+    return [=](int r) { return key0 + r < last ? key0 + r : last; };
+  };
+  auto issue_k = [&](int u) { issue_buffer(C::RING_K + (u % NR) * UB, false, kbase, (uint32_t)(H * D), unit_row(u)); };
+  auto issue_v = [&](int u) { issue_buffer(C::RING_V + (u % NR) * UB, true, vbase, (uint32_t)(H * D), unit_row(u)); };
+  // units >= 2 lie wholly before the chunk (never past eos): fixed per-lane offsets from a wave-uniform row pointer
+  uint32_t koff[LPB], voff[LPB], boff[LPB];
+#pragma unroll
+  for (int i = 0; i < LPB; ++i) {
+    const int b = wave + NW * i;
+    const int rh = b / KS, cq = b % KS;
+    koff[i] = ((uint32_t)(16 * rh + lrow16) * (uint32_t)(H * D) + (uint32_t)(4 * cq + lswz) * 8) * 2;
+    voff[i] = ((uint32_t)(16 * rh + lrowv) * (uint32_t)(H * D) + (uint32_t)(4 * cq + lpv) * 8) * 2;
+    boff[i] = lds0 + rh * HB + cq * 1024;
+  }
+  auto issue_k_fast = [&](int u, uint32_t slot_off) {
+    const bf16_t* src = p.k_swa + (((int64_t)c0 + 32 - 32 * u) * H + h) * D;
+#pragma unroll
+    for (int i = 0; i < LPB; ++i) g2l16(src, koff[i], boff[i] + C::RING_K + slot_off);
+  };
+  auto issue_v_fast = [&](int u, uint32_t slot_off) {
+    const bf16_t* src = p.v + (((int64_t)c0 + 32 - 32 * u) * H + h) * D;
+#pragma unroll
+    for (int i = 0; i < LPB; ++i) g2l16(src, voff[i], boff[i] + C::RING_V + slot_off);
+  };
+
+  // ---- requests: K and V of the first units, then the query fragments ---------------------------------
+  issue_k(0);
+  issue_v(0);
+  issue_k(1);
+  issue_v(1);
+  if (2 < nunits) issue_k_fast(2, 2 * UB);
+  // window-query fragments, pre-scaled by scale * log2(e)
+  bf16x8 qs[KS];
+  {
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+      bf16x8 r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+        r[e] = (__bf16)(f * cs);
+      }
+      qs[ks] = r;
+    }
+  }
+
+  const int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);   // first row of the chunk whose source token exists
+  const int grow_s = c0 - p.shift;                                       // source token of row 0
+  auto tok = [&](int r) {   // source token of row r, kept inside the sequence (rows outside [vlo, rows) carry no weight)
+    int t = grow_s + r;
+    t = t < bos ? bos : t;
+    t = t < eos ? t : eos - 1;
+    return t - bos;
+  };
+  // gate cumsums (16 blocks of 4 rows; rows >= `rows` were never written by the state pass and stay unused) and s
+  auto issue_gates = [&]() {
+#pragma unroll
+    for (int i = 0; i < 16 / NW; ++i) {
+      const int b = wave + NW * i;
+      const int r = 4 * b + (lane >> 4);
+      const int c = (lane & 15) ^ (r & 15);
+      g2l16(p.gc + cg * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + C::GC + b * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < 8 / NW; ++i) {
+      const int b = wave + NW * i;
+      const int r = 8 * b + (lane >> 3);
+      const int c = (lane & 7) ^ (r & 7);
+      g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok(r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + b * 1024);
+    }
+  };
+
+  // ---- window loop state ------------------------------------------------------------------------
+  f32x4 O[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) O[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  f32x4 Lw = {0.f, 0.f, 0.f, 0.f};
+  float nm = 0.f;                      // minus the running reference maximum, log2 units
+  f32x4 nmv = {0.f, 0.f, 0.f, 0.f};    // nm broadcast: the accumulator the score products start from
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
+  constexpr float THR = 8.f;           // the reference moves (prologue, slot branch) when a score tops it by more than 2^THR
+  constexpr float BIG = 96.f;          // scores this far above the reference leave the matrix-core path
+
+  const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
+  const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
+  // row fragment (rows 16 kk + l16 of a buffer, columns 32 ks + 8 kb ..) of a K-layout buffer at byte address a
+  auto kfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {
+    const lbyte* base = lds + (a + kaddr);     // one address per buffer; the fragment is a constant offset from it
+    return *reinterpret_cast<const NHA_LDS bf16x8*>(base + (kk * HB + ks * 1024));
+  };
+  // transposed fragment of a V-layout buffer: X[4 kb + e][16 db + l16] (e < 4) and X[16 + 4 kb + e - 4][..]
+  auto vfrag = [&](uint32_t a, int db) -> bf16x8 {
+    const lbyte* base = lds + (a + vaddr);
+    const lbyte* pa = base + ((db >> 1) * 1024 + (db & 1) * 512);
+    struct { s16x4 a, b; } t;
+    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + HB));
+    return __builtin_bit_cast(bf16x8, t);
+  };
+  auto mask_unit = [&](f32x4 (&S)[2], int u) {
+    const int xbase = 32 - 32 * u;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int x = xbase + 16 * kk + 4 * kb + r;
+        const bool ok = (x <= irow) && (p.wl < 0 || x >= irow - p.wl);
+        if (!ok) S[kk][r] = -INFINITY;
+      }
+  };
+  auto is_edge = [&](int u) -> bool { return (63 - 32 * u > 0) || (p.wl >= 0 && 32 - 32 * u < 63 - p.wl); };
+  // the reference moves up by delta: everything accumulated so far shrinks by 2^-delta
+  auto rescale_acc = [&](float delta) {
+    const float alpha = fexp2(-delta);
+    nm -= delta;
+    nmv = (f32x4){nm, nm, nm, nm};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Lw[r] *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[db][r] *= alpha;
+  };
+  auto rescale = [&](f32x4 (&S)[2], float rmax) {
+    const float delta = fmaxf(max_over_rows(rmax), 0.f);
+    rescale_acc(delta);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) S[kk][r] -= delta;
+  };
+  auto max8 = [&](const f32x4 (&S)[2]) -> float {
+    const float a = fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3]));
+    return fmaxf(a, fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
+  };
+
+  f32x4 Sc[2], Sn[2];
+  constexpr int PD = 6;   // fragments requested from LDS ahead of the matrix instruction that takes them
+  // ---- prologue: scores of unit 0, K fragments of unit 1 -----------------------------------------------
+  wait_vm<0>();
+  lds_barrier();
+  {
+    Sc[0] = nmv;
+    Sc[1] = nmv;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Sc[0] = mfma16(kfrag(C::RING_K, 0, ks), qs[ks], Sc[0]);
+      Sc[1] = mfma16(kfrag(C::RING_K, 1, ks), qs[ks], Sc[1]);
+    }
+    mask_unit(Sc, 0);   // unit 0 is always an edge unit
+    const float x = max8(Sc);
+    if (__any(x > THR)) rescale(Sc, x);
+  }
+  // every wave has read the K buffer of unit 0: unit 3 takes it
+  lds_barrier();
+  if (3 < nunits) issue_k_fast(3, 0);
+
+  // slot-branch query fragments (requested while the last unit is worked on)
+  bf16x8 qg[KS];
+  auto load_qg = [&]() {
+    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 x = make_uint4(0, 0, 0, 0);
+      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+      qg[ks] = as_bf16x8(x);
+    }
+  };
+  auto pack_p = [&]() -> bf16x8 {
+    const u32x4 t = {cvt2(Sc[0][0], Sc[0][1]), cvt2(Sc[0][2], Sc[0][3]), cvt2(Sc[1][0], Sc[1][1]), cvt2(Sc[1][2], Sc[1][3])};
+    bf16x8 P = __builtin_bit_cast(bf16x8, t);
+    NHA_PIN(P);
+    return P;
+  };
+
+  // ring positions as rotating buffer offsets: s0 = buffer of unit u, s1 of unit u+1, s2 of unit u+2
+  uint32_t s0 = 0, s1 = UB, s2 = 2 * UB;
+  for (int u = 0; u + 1 < nunits; ++u) {
+    const uint32_t k_n = C::RING_K + s1;    // K of unit u+1
+    const uint32_t v_c = C::RING_V + s0;    // V of unit u
+    // ---- phase A: scores of unit u+1 on the matrix core (two accumulators in turn), exponentials of
+    //      unit u on the VALU (one per two products); K fragment i = 2 ks + kk is read PD products ahead ----
+    bf16x8 kfr[2 * KS];
+    NHA_FENCE();
+#pragma unroll
+    for (int i = 0; i < PD; ++i) kfr[i] = kfrag(k_n, i & 1, i >> 1);
+    NHA_FENCE();
+#pragma unroll
+    for (int i = 0; i < 2 * KS; ++i) {
+      const int ks = i >> 1, kk = i & 1;
+      if (i + PD < 2 * KS) kfr[i + PD] = kfrag(k_n, (i + PD) & 1, (i + PD) >> 1);
+      Sn[kk] = mfma16(kfr[i], qs[ks], ks == 0 ? nmv : Sn[kk]);
+      if (kk == 1) {
+        Sc[ks >> 2][ks & 3] = fexp2(Sc[ks >> 2][ks & 3]);
+        NHA_PIN(Sc[ks >> 2][ks & 3]);
+      }
+      NHA_FENCE();
+    }
+    const bf16x8 Pq = pack_p();
+    NHA_FENCE();
+    // K of unit u+2 and V of unit u (requested two iterations ago) have landed for this wave, then for
+    // everybody.  What may stay in flight: the requests of the previous iteration (and, right after the
+    // start, K of unit 3 and the gate blocks).
+    if (u >= 1) {
+      if (u + 3 < nunits) {          // the previous iteration made a full request (K of u+3, V of u+1)
+        if (u <= 2) wait_vm<2 * LPB + C::NGS>();
+        else wait_vm<2 * LPB>();
+      } else {
+        wait_vm<0>();
+      }
+    }
+    lds_barrier();
+    if (u + 4 < nunits) issue_k_fast(u + 4, s1);   // unit u+4 takes the buffer of unit u+1
+    if (u + 2 < nunits) issue_v_fast(u + 2, s2);
+    if (u == 0) issue_gates();
+    NHA_FENCE();
+    // ---- phase B: value products of unit u on the matrix core, row maximum of unit u+1 on the VALU;
+    //      V fragment db is read PD products ahead ----
+    float m0 = 0.f, m1 = 0.f;
+    auto max_step = [&](int s2) {
+      if (s2 == 0) m0 = fmaxf(Sn[0][0], Sn[0][1]);
+      if (s2 == 1) m1 = fmaxf(Sn[0][2], Sn[0][3]);
+      if (s2 == 2) m0 = fmaxf(fmaxf(m0, Sn[1][0]), Sn[1][1]);
+      if (s2 == 3) m1 = fmaxf(fmaxf(m1, Sn[1][2]), Sn[1][3]);
+      if (s2 == 4) m0 = fmaxf(m0, m1);
+      if (s2 == 0 || s2 == 2 || s2 == 4) NHA_PIN(m0);
+      if (s2 == 1 || s2 == 3) NHA_PIN(m1);
+    };
+    bf16x8 vfr[DB];
+#pragma unroll
+    for (int i = 0; i < PD; ++i) vfr[i] = vfrag(v_c, i);
+    Lw = mfma16(ones, Pq, Lw);
+    NHA_FENCE();
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      if (db + PD < DB) vfr[db + PD] = vfrag(v_c, db + PD);
+      O[db] = mfma16(vfr[db], Pq, O[db]);
+      if (db % 3 == 0 && db / 3 < 5) max_step(db / 3);
+      NHA_FENCE();
+    }
+    if (is_edge(u + 1)) {
+      mask_unit(Sn, u + 1);
+      m0 = max8(Sn);
+    }
+    // The reference of the window stays where the prologue put it: moving it would mean rescaling 64
+    // accumulator registers inside this loop, which costs the loop its registers whether or not the branch
+    // is ever taken.  fp32 sums and bf16 probabilities hold 2^BIG above it; a score beyond that sends the
+    // wave's 16 rows to the exact pass (mfma_repair_kernel recomputes flagged sub-blocks) and is clamped.
+    if (__any(m0 > BIG)) {
+      if (lane == 0) atomicOr(p.flags + cg * 4, 1 << Q);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Sn[kk][r] = fminf(Sn[kk][r], BIG);
+    }
+    Sc[0] = Sn[0];
+    Sc[1] = Sn[1];
+    const uint32_t t0 = s0;
+    s0 = s1;
+    s1 = s2;
+    s2 = t0;
+  }
+  // ---- the last unit: no further scores; the slot-branch queries are requested meanwhile ----
+  {
+    const int u = nunits - 1;
+    const uint32_t v_c = C::RING_V + (u % NR) * UB;
+    bf16x8 vf[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) vf[db] = vfrag(v_c, db);
+    load_qg();
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Sc[kk][r] = fexp2(Sc[kk][r]);
+    const bf16x8 Pq = pack_p();
+    Lw = mfma16(ones, Pq, Lw);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) O[db] = mfma16(vf[db], Pq, O[db]);
+  }
+
+  // ================= slot branch, folded into the running softmax =================================
+  // every request of this wave has landed, every wave is done with the rings
+  wait_vm<0>();
+  lds_barrier();
+  // the tiles take ring buffers: chunk-start k-state [m][d] (K layout), the chunk's k_gsa rows (K layout),
+  // chunk-start v-state [m][d] (V layout); the v rows (V layout) follow into the first two once they are free
+  struct Tiles {
+    static constexpr uint32_t a(int i) { return C::RING_K + i * UB; }                      // k-state: K buffers 0, 1
+    static constexpr uint32_t b(int i) { return i == 0 ? C::RING_K + 2 * UB : C::RING_V; } // k_gsa rows: K buffer 2, V buffer 0
+    static constexpr uint32_t c(int i) { return C::RING_V + (1 + i) * UB; }                // v-state: V buffers 1, 2
+    static constexpr uint32_t d(int i) { return C::RING_K + i * UB; }                      // v rows: K buffers 0, 1 again
+  };
+  {
+    const bf16_t* hk = p.hkT + cg * MS * D;
+    const bf16_t* hv = p.hvc + cg * MS * D;
+    const bf16_t* kg = p.k_gsa + ((int64_t)bos * H + h) * D;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      issue_buffer(Tiles::a(half), false, hk, (uint32_t)D, [=](int r) { return 32 * half + r; });
+      issue_buffer(Tiles::b(half), false, kg, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
+      issue_buffer(Tiles::c(half), true, hv, (uint32_t)D, [=](int r) { return 32 * half + r; });
+    }
+  }
+  // the window's own log-sum-exp, before the slots join the running softmax
+  if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[0]) - nm) * LN2;
+
+  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
+  auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
+  // decay tables E_Q[j][m] = s_j[m] exp(min(gr_Q[m] - gc_j[m], DECAY_CLAMP)) for the rows j of the 16-row
+  // blocks jb <= Q, zero elsewhere (gr_Q: gate cumsum of the row before sub-block Q, 0 for Q = 0); rows
+  // whose source token does not exist carry no weight.  32-row units in the V layout (64 columns):
+  // E_0 -> unit 0, E_1 -> 1, E_2 -> 2,3, E_3 -> 4,5; a thread makes 8 consecutive slots of a row.
+  for (int item = tid; item < 6 * 256; item += 64 * NW) {
+    const int U = item >> 8, r32 = (item >> 3) & 31, m = (item & 7) * 8;
+    const int Qt = U == 0 ? 0 : U == 1 ? 1 : U < 4 ? 2 : 3;
+    const int pr = (U == 3 || U == 5) ? 1 : 0;
+    const int j = 32 * pr + r32;
+    const bool ok = (j >> 4) <= Qt && j >= vlo && j < rows;
+    bf16x8 out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = (__bf16)0.f;
+    if (ok) {
+      f32x4 gv[2], gr[2];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m + 4 * hh));
+        gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (Qt > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Qt - 1, m + 4 * hh));
+      }
+      const bf16x8 sv = *reinterpret_cast<const NHA_LDS bf16x8*>(s_at(j, m));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)sv[e] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
+    }
+    *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
+  }
+  // the three tiles have landed, the tables are written
+  wait_vm<0>();
+  __syncthreads();
+
+  const int etu = Q < 2 ? Q : 2 * Q - 2;   // first table unit of this wave's sub-block
+  // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+  auto etab_tr = [&](int pr, int mb) -> bf16x8 {
+    const lbyte* pa = lds + C::ETAB + (etu + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 512 + vaddr;
+    struct { s16x4 a, b; } t;
+    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + 2048));
+    return __builtin_bit_cast(bf16x8, t);
+  };
+  // E_Q by rows: row = token 16 jb + l16, contraction over the slots 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+  auto etab_row = [&](int jb, int pr) -> bf16x8 {
+    const lbyte* pa = lds + C::ETAB + (etu + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 32 + 8 * kb;
+    struct { bf16x4 a, b; } t;
+    t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(pa);
+    t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 512);
+    return __builtin_bit_cast(bf16x8, t);
+  };
+
+  // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
+  f32x4 ok[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(Tiles::a(mb >> 1), mb & 1, ks), qg[ks], ok[mb]);
+  // every wave is done with the k-state tile: the v rows take its buffers and land during what follows
+  lds_barrier();
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+    issue_buffer(Tiles::d(half), true, vbase, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
+  // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
+  bf16x8 bA[2];
+  {
+    f32x4 at[4];
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+        if (jb <= Q) at[jb] = mfma16(kfrag(Tiles::b(jb >> 1), jb & 1, ks), qg[ks], at[jb]);
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb)
+      if (jb == Q) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (4 * kb + r > l16) at[jb][r] = 0.f;
+      }
+    bA[0] = pack8(at[0], at[1]);
+    bA[1] = pack8(at[2], at[3]);
+  }
+  // okT_intra[m][i] = sum_j s_j[m] exp(gr[m] - gc_j[m]) AT[j][i]
+  f32x4 oki[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    oki[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+      if (2 * pr <= Q) oki[mb] = mfma16(etab_tr(pr, mb), bA[pr], oki[mb]);
+  }
+  // combine; the slot logits join the running softmax as one more set of keys
+  const int rref = 16 * Q - 1;
+  f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
+  float xmax = -INFINITY;
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(irow, 16 * mb + 4 * kb));
+    f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (Q > 0) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(rref, 16 * mb + 4 * kb));
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      egi[mb][r] = fexp(gi[r]);
+      egr[mb][r] = fexp(gi[r] - gr4[r]);
+      ok[mb][r] = (ok[mb][r] * egi[mb][r] + oki[mb][r] * egr[mb][r]) * cs;   // slot logit, log2 units
+      xmax = fmaxf(xmax, ok[mb][r]);
+    }
+  }
+  const float ms = max_over_rows(xmax);   // the slots' own maximum
+  if (__any(ms + nm > THR)) rescale_acc(fmaxf(ms + nm, 0.f));
+  if (p.lse_gsa) {
+    float pown = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pown += fexp2(ok[mb][r] - ms);
+    pown += __shfl_xor(pown, 16, 64);
+    pown += __shfl_xor(pown, 32, 64);
+    if (kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(pown) + ms) * LN2;
+  }
+  float psum = 0.f;
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      ok[mb][r] = fexp2(ok[mb][r] + nm);   // unnormalised slot probabilities
+      psum += ok[mb][r];
+    }
+  psum += __shfl_xor(psum, 16, 64);
+  psum += __shfl_xor(psum, 32, 64);
+  bf16x8 bp[2], bpr[2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr) {
+    f32x4 x0, x1, y0, y1;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      x0[r] = ok[2 * pr][r] * egi[2 * pr][r];
+      x1[r] = ok[2 * pr + 1][r] * egi[2 * pr + 1][r];
+      y0[r] = ok[2 * pr][r] * egr[2 * pr][r];
+      y1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
+    }
+    bp[pr] = pack8(x0, x1);
+    bpr[pr] = pack8(y0, y1);
+  }
+  // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+    for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag(Tiles::c(pr), db), bp[pr], O[db]);
+  // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
+  bf16x8 bAv[2];
+  {
+    f32x4 av[4];
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      av[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (jb <= Q) {
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) av[jb] = mfma16(etab_row(jb, pr), bpr[pr], av[jb]);
+        if (jb == Q) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (4 * kb + r > l16) av[jb][r] = 0.f;
+        }
+      }
+    }
+    bAv[0] = pack8(av[0], av[1]);
+    bAv[1] = pack8(av[2], av[3]);
+  }
+  // the v rows have landed (this wave's part, then everybody's)
+  wait_vm<0>();
+  lds_barrier();
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr)
+    if (2 * pr <= Q) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag(Tiles::d(pr), db), bAv[pr], O[db]);
+    }
+
+  // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
+  //      row block db + 1, and the two trade their halves) -------------------------------------------
+  {
+    const float inv = 1.f / (Lw[0] + psum);
+    bf16_t* op = p.o + ((int64_t)(c0 + irow) * HQ + hq) * D;
+#pragma unroll
+    for (int db = 0; db < DB; db += 2) {
+      unsigned a[2], b[2];
+      a[0] = cvt2(O[db][0] * inv, O[db][1] * inv);
+      a[1] = cvt2(O[db][2] * inv, O[db][3] * inv);
+      b[0] = cvt2(O[db + 1][0] * inv, O[db + 1][1] * inv);
+      b[1] = cvt2(O[db + 1][2] * inv, O[db + 1][3] * inv);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(a[e], b[e], false, false);
+        a[e] = sw[0];
+        b[e] = sw[1];
+      }
+      const int dcol = 16 * (db + (kb & 1)) + 8 * (kb >> 1);
+      if (irow < rows) *reinterpret_cast<uint4*>(op + dcol) = make_uint4(a[0], a[1], b[0], b[1]);
+    }
+  }
+}
+
+}  // namespace
+
+// Served: K == V == 256 with any grouping of query heads (each head walks its kv-head's window on its
+// own).  The per-lane byte offsets of the LDS-direct loads are 32 bits: the tensors of one call must
+// stay below 4 GiB.
+bool prefill_ring256_supported(const mf::MP& p, int D) {
+  if (D != 256) return false;
+  return (int64_t)p.T_tot * p.H * D * 2 < ((int64_t)1 << 32) && (int64_t)p.T_tot * p.H * MS * 2 < ((int64_t)1 << 32);
+}
+
+int prefill_ring256_launch(const mf::MP& p, hipStream_t st) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  const size_t lds = Cfg::BYTES;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(ring256_out_kernel, dim3(p.HQ, p.NT), dim3(256), lds, st, p);
+  NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass, ring, head size 256)");
+  return NHA_OK;
+}
+
+}  // namespace nha

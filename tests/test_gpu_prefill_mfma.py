@@ -124,6 +124,25 @@ def test_mfma_decay_near_the_clamp_at_scale_one(HQ, H, per_row):
             assert rel <= 3e-2, (name, wl, shift, rel)
 
 
+@pytest.mark.parametrize("qk_scale", [1.0, 3.0])
+def test_mfma_head_size_256_scores_far_above_the_first_units(qk_scale):
+    """Head size 256 at scale 1 with unnormalised q / k: window scores of a few hundred.  The output pass
+    for this head size keeps the softmax reference of the chunk's own keys; rows in which a later key tops
+    it by more than 2^96 are handed to the exact pass.  Finite everywhere, relative L2 within 3e-2 (logits of
+    this size make single outputs move by more than the element-wise bar under bf16 rounding of the states)."""
+    from nha_amd import chunk_nha
+    d = prefill_inputs(880, 2, 200, 4, 2, 256, 256, 64, dtype=BF, gate_div=8.0, qk_scale=qk_scale)
+    for wl, shift in ((99, 100), (64, 0)):
+        c = [d[k].cuda() for k in KEYS]
+        o, ls, lg = chunk_nha(*c, window_size_left=wl, gsa_kv_shift=shift, scale=1.0, impl="mfma")
+        ro, rls, rlg, _, _ = R.prefill_ref(*[d[k] for k in KEYS], window_size_left=wl, gsa_kv_shift=shift, scale=1.0)
+        for name, got, ref in (("o", o, ro), ("lse_swa", ls, rls), ("lse_gsa", lg, rlg)):
+            got = got.double().cpu()
+            assert torch.isfinite(got).all(), (name, wl, shift)
+            rel = ((got - ref).norm() / ref.norm()).item()
+            assert rel <= 3e-2, (name, wl, shift, rel)
+
+
 def test_mfma_matches_simple_kernels_at_size():
     """A shape the CPU recurrence cannot reach in seconds: MFMA kernels vs the fp32-math kernels."""
     from nha_amd import chunk_nha
