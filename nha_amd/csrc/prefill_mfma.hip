@@ -71,10 +71,12 @@ __device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<ROWS, D, NTH
 // states and writes the segment-start states h_seg beside them: it needs the sum in fp32.
 // Both states are kept as C[d][m] accumulators (slot m = lane % 16).
 
-template <int D>
+// DW: columns of the state one workgroup carries (D, or D/2: twice the workgroups with half the
+// tile, which this latency-bound kernel turns into bandwidth; the gates are then read once more).
+template <int D, int DW>
 __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
-  constexpr int LDT = D + 16;
-  constexpr int NB = D / 16;
+  constexpr int LDT = DW + 16;
+  constexpr int NB = DW / 16;
   extern __shared__ __align__(16) unsigned char smem[];
   lbf16* Xt = (lbf16*)smem;
   lbf16* St = Xt + BT * LDT;
@@ -85,8 +87,10 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   // blockIdx.z picks the state: 0 = k-state (rows of k_gsa; it also writes the gate tables),
   // 1 = v-state (rows of v).  The two recurrences share nothing but the gates, and twice the
   // workgroups of half the size fill the chip better.
-  const bool isv = blockIdx.z != 0;
-  const bf16_t* xsrc = isv ? p.v : p.k_gsa;
+  const bool isv = (blockIdx.z & 1) != 0;
+  const int dcol0 = (blockIdx.z >> 1) * DW;   // first state column of this workgroup
+  const bool lead = dcol0 == 0;                // writes what does not depend on the column range
+  const bf16_t* xsrc = (isv ? p.v : p.k_gsa) + dcol0;
   bf16_t* hloc = isv ? p.hvc : p.hkT;
   float* hend = isv ? p.hend_v : p.hend_k;
   // blockIdx.x is a segment slot (seg_slot); slots are dense up to a few gaps per sequence, so
@@ -116,14 +120,14 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   for (int b = 0; b < NB; ++b) hx[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float gsum = 0.f;   // sum of the chunk-end gate cumsums since the segment start, this lane's slot
 
-  TileRegs<BT, D, 256> rx;
+  TileRegs<BT, DW, 256> rx;
   uint4 rs[2], rg[2];
   auto issue = [&](int it) {
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     const int64_t grow0 = (int64_t)bos + it * BT - p.shift;
     int vlo = p.shift - it * BT;
     vlo = vlo < 0 ? 0 : vlo;
-    tile_g2r<BT, D, 256>(rx, xsrc + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
+    tile_g2r<BT, DW, 256>(rx, xsrc + (int64_t)h * D, (int64_t)H * D, grow0, vlo, rows, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     const int chunk = chunk0 + jc;
     const int rows = (L - it * BT) < BT ? (L - it * BT) : BT;
     if (jc > 0) __syncthreads();   // everyone is done reading the previous chunk's tiles
-    tile_r2l<BT, D, 256>(Xt, rx, tid);
+    tile_r2l<BT, DW, 256>(Xt, rx, tid);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c8 = tid + 256 * u;
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
       glast = __shfl(cand, l16 + 16 * src_kb, 64);
     }
     const int64_t cg = (int64_t)chunk * H + h;
-    if (!isv) {
+    if (!isv && lead) {
       float* gout = p.gc + cg * BT * MS + m;
 #pragma unroll
       for (int e = 0; e < 16; ++e) gout[(16 * (e >> 2) + 4 * kb + (e & 3)) * MS] = gcv[e];
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
       bf16x4 pk;
 #pragma unroll
       for (int r = 0; r < 4; ++r) pk[r] = (__bf16)hx[b][r];
-      *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + 16 * b + 4 * kb) = pk;
+      *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + dcol0 + 16 * b + 4 * kb) = pk;
     }
     const float dk = fexp(glast);
     gsum += glast;
@@ -245,8 +249,8 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   const int64_t sl = (int64_t)seg_slot(p.coff, n, it0) * H + h;
 #pragma unroll
   for (int b = 0; b < NB; ++b)
-    *reinterpret_cast<float4*>(hend + (sl * MS + m) * D + 16 * b + 4 * kb) = make_float4(hx[b][0], hx[b][1], hx[b][2], hx[b][3]);
-  if (kb == 0 && !isv) p.dtot[sl * MS + m] = fexp(gsum);
+    *reinterpret_cast<float4*>(hend + (sl * MS + m) * D + dcol0 + 16 * b + 4 * kb) = make_float4(hx[b][0], hx[b][1], hx[b][2], hx[b][3]);
+  if (kb == 0 && !isv && lead) p.dtot[sl * MS + m] = fexp(gsum);
 }
 
 // Level 2: one thread per state element, sequential over the segments of its sequence.
@@ -1137,13 +1141,14 @@ template <int D>
 int run_state_pass(const MP& p, bool segment_form, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  const size_t lds = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * SLD * 2;
-  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  constexpr int DW = D >= 256 ? D / 2 : D;   // measured: 96 -> 88 us at B=8 T=2048 H=4 D=256; no gain at D = 128
+  const size_t lds = (size_t)BT * (DW + 16) * 2 + (size_t)2 * BT * SLD * 2;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)mfma_state_local_kernel<D, DW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
   if (attr_err != hipSuccess) {
     set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((mfma_state_local_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H, 2), dim3(256), lds, st, p);
+  hipLaunchKernelGGL((mfma_state_local_kernel<D, DW>), dim3(p.NT / SEG + p.N + 1, p.H, 2 * (D / DW)), dim3(256), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
   if (segment_form) hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
   else hipLaunchKernelGGL((state_final_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);

@@ -296,6 +296,20 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     return P;
   };
 
+  // The slot-branch tiles (k-state, k_gsa rows, v-state as two 32-row halves each) take ring buffers as the
+  // window loop retires them: with at least five units the last three K buffers and the last V buffer to
+  // come free receive four of the six halves while the loop still runs (a half is as many loads as a
+  // unit buffer, so the in-flight counts of the loop stay what they are); the two v-state halves follow
+  // after the loop, and shorter windows request everything then.
+  const bf16_t* const t_hk = p.hkT + cg * MS * D;
+  const bf16_t* const t_hv = p.hvc + cg * MS * D;
+  const bf16_t* const t_kg = p.k_gsa + ((int64_t)bos * H + h) * D;
+  auto issue_ta = [&](uint32_t off, int half) { issue_buffer(off, false, t_hk, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
+  auto issue_tb = [&](uint32_t off, int half) { issue_buffer(off, false, t_kg, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); }); };
+  auto issue_tc = [&](uint32_t off, int half) { issue_buffer(off, true, t_hv, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
+  const bool early = nunits >= 5;
+  uint32_t oA0 = C::RING_K, oA1 = C::RING_K + UB, oB0 = C::RING_K + 2 * UB, oB1 = C::RING_V;   // where the halves lie
+  uint32_t oC0 = C::RING_V + UB, oC1 = C::RING_V + 2 * UB;
   // ring positions as rotating buffer offsets: s0 = buffer of unit u, s1 of unit u+1, s2 of unit u+2
   uint32_t s0 = 0, s1 = UB, s2 = 2 * UB;
   for (int u = 0; u + 1 < nunits; ++u) {
@@ -325,16 +339,36 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     // everybody.  What may stay in flight: the requests of the previous iteration (and, right after the
     // start, K of unit 3 and the gate blocks).
     if (u >= 1) {
-      if (u + 3 < nunits) {          // the previous iteration made a full request (K of u+3, V of u+1)
-        if (u <= 2) wait_vm<2 * LPB + C::NGS>();
+      if (early) {                    // every iteration requests two buffers' worth, V side first
+        if (u + 2 == nunits) wait_vm<LPB>();   // last iteration: also V of the last unit; the tile half behind it may fly
+        else if (u <= 2) wait_vm<2 * LPB + C::NGS>();
         else wait_vm<2 * LPB>();
       } else {
         wait_vm<0>();
       }
     }
     lds_barrier();
-    if (u + 4 < nunits) issue_k_fast(u + 4, s1);   // unit u+4 takes the buffer of unit u+1
-    if (u + 2 < nunits) issue_v_fast(u + 2, s2);
+    if (u + 2 < nunits) {
+      issue_v_fast(u + 2, s2);
+    } else if (early) {
+      oB1 = C::RING_V + s2;
+      issue_tb(oB1, 1);
+    }
+    if (u + 4 < nunits) {
+      issue_k_fast(u + 4, s1);   // unit u+4 takes the buffer of unit u+1
+    } else if (early) {
+      const uint32_t off = C::RING_K + s1;
+      if (u + 4 == nunits) {
+        oA0 = off;
+        issue_ta(off, 0);
+      } else if (u + 3 == nunits) {
+        oA1 = off;
+        issue_ta(off, 1);
+      } else {
+        oB0 = off;
+        issue_tb(off, 0);
+      }
+    }
     if (u == 0) issue_gates();
     NHA_FENCE();
     // ---- phase B: value products of unit u on the matrix core, row maximum of unit u+1 on the VALU;
@@ -405,25 +439,17 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   // every request of this wave has landed, every wave is done with the rings
   wait_vm<0>();
   lds_barrier();
-  // the tiles take ring buffers: chunk-start k-state [m][d] (K layout), the chunk's k_gsa rows (K layout),
-  // chunk-start v-state [m][d] (V layout); the v rows (V layout) follow into the first two once they are free
-  struct Tiles {
-    static constexpr uint32_t a(int i) { return C::RING_K + i * UB; }                      // k-state: K buffers 0, 1
-    static constexpr uint32_t b(int i) { return i == 0 ? C::RING_K + 2 * UB : C::RING_V; } // k_gsa rows: K buffer 2, V buffer 0
-    static constexpr uint32_t c(int i) { return C::RING_V + (1 + i) * UB; }                // v-state: V buffers 1, 2
-    static constexpr uint32_t d(int i) { return C::RING_K + i * UB; }                      // v rows: K buffers 0, 1 again
-  };
-  {
-    const bf16_t* hk = p.hkT + cg * MS * D;
-    const bf16_t* hv = p.hvc + cg * MS * D;
-    const bf16_t* kg = p.k_gsa + ((int64_t)bos * H + h) * D;
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      issue_buffer(Tiles::a(half), false, hk, (uint32_t)D, [=](int r) { return 32 * half + r; });
-      issue_buffer(Tiles::b(half), false, kg, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
-      issue_buffer(Tiles::c(half), true, hv, (uint32_t)D, [=](int r) { return 32 * half + r; });
-    }
+  if (!early) {
+    issue_ta(oA0, 0);
+    issue_ta(oA1, 1);
+    issue_tb(oB0, 0);
+    issue_tb(oB1, 1);
+  } else {   // the V buffers of the last two units (s0, s2 after the loop's last rotation) are the free ones
+    oC0 = C::RING_V + s2;
+    oC1 = C::RING_V + s0;
   }
+  issue_tc(oC0, 0);
+  issue_tc(oC1, 1);
   // the window's own log-sum-exp, before the slots join the running softmax
   if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[0]) - nm) * LN2;
 
@@ -456,8 +482,8 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     }
     *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
   }
-  // the three tiles have landed, the tables are written
-  wait_vm<0>();
+  // k-state and k_gsa rows have landed (the two v-state halves may still fly), the tables are written
+  wait_vm<2 * LPB>();
   __syncthreads();
 
   const int etu = Q < 2 ? Q : 2 * Q - 2;   // first table unit of this wave's sub-block
@@ -485,12 +511,12 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(Tiles::a(mb >> 1), mb & 1, ks), qg[ks], ok[mb]);
+    for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(((mb >> 1) ? oA1 : oA0), mb & 1, ks), qg[ks], ok[mb]);
   // every wave is done with the k-state tile: the v rows take its buffers and land during what follows
   lds_barrier();
 #pragma unroll
   for (int half = 0; half < 2; ++half)
-    issue_buffer(Tiles::d(half), true, vbase, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
+    issue_buffer(half ? oA1 : oA0, true, vbase, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
   // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
   bf16x8 bA[2];
   {
@@ -501,7 +527,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb)
-        if (jb <= Q) at[jb] = mfma16(kfrag(Tiles::b(jb >> 1), jb & 1, ks), qg[ks], at[jb]);
+        if (jb <= Q) at[jb] = mfma16(kfrag(((jb >> 1) ? oB1 : oB0), jb & 1, ks), qg[ks], at[jb]);
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb)
       if (jb == Q) {
@@ -574,11 +600,14 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     bp[pr] = pack8(x0, x1);
     bpr[pr] = pack8(y0, y1);
   }
+  // the v-state halves have landed (this wave's part, then everybody's); the v rows behind them may fly
+  wait_vm<2 * LPB>();
+  lds_barrier();
   // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
 #pragma unroll
   for (int pr = 0; pr < 2; ++pr)
 #pragma unroll
-    for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag(Tiles::c(pr), db), bp[pr], O[db]);
+    for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oC1 : oC0), db), bp[pr], O[db]);
   // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
   bf16x8 bAv[2];
   {
@@ -606,7 +635,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   for (int pr = 0; pr < 2; ++pr)
     if (2 * pr <= Q) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag(Tiles::d(pr), db), bAv[pr], O[db]);
+      for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oA1 : oA0), db), bAv[pr], O[db]);
     }
 
   // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
