@@ -10,10 +10,14 @@
 //    slot branch (which only needs the chunk-start states and the chunk's own rows) is folded into
 //    the running softmax afterwards.
 //  * The window loop is software-pipelined inside each wave: while the matrix core forms the scores
-//    of unit u+1, the VALU exponentiates unit u; while it accumulates P.V of unit u, the VALU takes
-//    the row maxima of unit u+1.  The scale and the running maximum are folded into the score
-//    product itself (pre-scaled queries, accumulator started at -max), so a score needs one
-//    v_exp_f32 and half a v_cvt_pk_bf16_f32 and nothing else on the common path.
+//    of unit u+1, the VALU exponentiates unit u.  The scale and the softmax reference are folded into
+//    the score product itself (pre-scaled queries, accumulator started at -reference), so a score
+//    needs one v_exp_f32 and half a v_cvt_pk_bf16_f32 and nothing else.
+//  * The softmax reference of a query row is fixed once, from the first unit (the row's own and
+//    nearest keys; 0 for rows that unit does not reach): fp32 sums relative to a fixed reference are
+//    exact while every score stays within 2^+-100 of it, and the loop carries no maxima, no
+//    comparisons and no rescaling of the accumulators.  A row whose window sum leaves that range
+//    (overflowed, or below 2^-100) is flagged for mfma_repair_kernel, which recomputes it exactly.
 //
 // LDS layouts (bank-conflict free for the two fragment reads without padding, which a 1 KB wave
 // load cannot produce): a 32-row unit is cut into 16-row x 32-column blocks of 1 KB, a row of a block
@@ -222,7 +226,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
     for (int qb = 0; qb < RQB; ++qb) O[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
   f32x4 Lw[RQB];
-  float nm[RQB];     // minus the running reference maximum, log2 units
+  float nm[RQB];     // minus the softmax reference of the row, log2 units
   f32x4 nmv[RQB];    // nm broadcast: the accumulator the score products start from
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   bf16x8 ones;
 #pragma unroll
   for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
-  // lazy rescaling: the reference only moves when a score exceeds it by more than 2^THR
+  // the reference is taken from unit 0 when a score there exceeds 2^THR, and kept from then on
   constexpr float THR = 8.f;
 
   const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
@@ -412,19 +416,8 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     kreq -= ustep;
     vreq -= ustep;
     NHA_FENCE();
-    // ---- phase B: value products of unit u on the matrix core, row maxima of unit u+1 on the VALU,
+    // ---- phase B: value products of unit u on the matrix core,
     //      K fragments of unit u+2 requested from LDS ----
-    float m0[RQB], m1[RQB];
-    auto max_step = [&](int step) {
-      const int q2 = step >> 3, s2 = step & 7;
-      if (s2 == 0) m0[q2] = fmaxf(Sn[0][q2][0], Sn[0][q2][1]);
-      if (s2 == 1) m1[q2] = fmaxf(Sn[0][q2][2], Sn[0][q2][3]);
-      if (s2 == 2) m0[q2] = fmaxf(fmaxf(m0[q2], Sn[1][q2][0]), Sn[1][q2][1]);
-      if (s2 == 3) m1[q2] = fmaxf(fmaxf(m1[q2], Sn[1][q2][2]), Sn[1][q2][3]);
-      if (s2 == 4) m0[q2] = fmaxf(m0[q2], m1[q2]);
-      if (s2 == 0 || s2 == 2 || s2 == 4) NHA_PIN(m0[q2]);
-      if (s2 == 1 || s2 == 3) NHA_PIN(m1[q2]);
-    };
 #pragma unroll
     for (int qb = 0; qb < RQB; ++qb) {
       Lw[qb] = mfma16(ones, Pq[qb], Lw[qb]);
@@ -437,28 +430,10 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
       for (int qb = 0; qb < RQB; ++qb) {
         O[db][qb] = mfma16(vf[db], Pq[qb], O[db][qb]);
-        // the row maxima of the next unit take 10 steps (5 per query block) spread over the 2 DB products
-        if (DB >= 8) {
-          max_step(2 * db + qb);
-        } else {
-          max_step(2 * (2 * db + qb));
-          max_step(2 * (2 * db + qb) + 1);
-        }
         NHA_FENCE();
       }
     }
-    if (is_edge(u + 1)) {
-      mask_unit(Sn, u + 1);
-#pragma unroll
-      for (int qb = 0; qb < RQB; ++qb) {
-        float x = fmaxf(fmaxf(Sn[0][qb][0], Sn[0][qb][1]), fmaxf(Sn[0][qb][2], Sn[0][qb][3]));
-        m0[qb] = fmaxf(x, fmaxf(fmaxf(Sn[1][qb][0], Sn[1][qb][1]), fmaxf(Sn[1][qb][2], Sn[1][qb][3])));
-      }
-    }
-    bool need = false;
-#pragma unroll
-    for (int qb = 0; qb < RQB; ++qb) need |= m0[qb] > THR;
-    if (__any(need)) rescale(Sn, m0);
+    if (is_edge(u + 1)) mask_unit(Sn, u + 1);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
@@ -487,6 +462,14 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       for (int qb = 0; qb < RQB; ++qb) O[db][qb] = mfma16(vf[db], Pq[qb], O[db][qb]);
   }
 
+  // a window sum outside 2^+-100 of the fixed reference (overflowed sums are +inf: beyond the upper bound):
+  // products with the values may have left fp32, or bf16 probabilities may have been flushed to zero
+  // that matter against the sum; the exact pass redoes the rows of the sub-block
+#pragma unroll
+  for (int qb = 0; qb < RQB; ++qb) {
+    const bool bad = (16 * (qb0 + qb) + l16 < rows) && (Lw[qb][0] >= 0x1p100f || Lw[qb][0] < 0x1p-100f);
+    if (__any(bad) && lane == 0) atomicOr(p.flags + cg * 4, 1 << (qb0 + qb));
+  }
   // ================= slot branch, folded into the running softmax =================================
   // every LDS-direct request of this wave has landed, every wave is done with the ring
   wait_vm<0>();

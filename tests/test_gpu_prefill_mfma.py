@@ -124,14 +124,17 @@ def test_mfma_decay_near_the_clamp_at_scale_one(HQ, H, per_row):
             assert rel <= 3e-2, (name, wl, shift, rel)
 
 
+@pytest.mark.parametrize("HQ,H,D", [(4, 2, 256), (8, 2, 128), (8, 2, 64)])
 @pytest.mark.parametrize("qk_scale", [1.0, 3.0])
-def test_mfma_head_size_256_scores_far_above_the_first_units(qk_scale):
-    """Head size 256 at scale 1 with unnormalised q / k: window scores of a few hundred.  The output pass
-    for this head size keeps the softmax reference of the chunk's own keys; rows in which a later key tops
-    it by more than 2^96 are handed to the exact pass.  Finite everywhere, relative L2 within 3e-2 (logits of
-    this size make single outputs move by more than the element-wise bar under bf16 rounding of the states)."""
+def test_mfma_scores_far_from_the_fixed_softmax_reference(qk_scale, HQ, H, D):
+    """Scale 1 with unnormalised q / k: window scores of a few hundred, far above and far below those of the
+    chunk's own keys.  The LDS-direct output passes (four query heads per kv-head at D <= 128, any grouping
+    at D = 256) fix the softmax reference of a row from its first keys and hand rows whose sums leave the
+    fp32 range they allow (2^+-100 around the reference at D <= 128, 2^96 above it at D = 256) to the exact
+    pass.  Finite everywhere, relative L2 within 3e-2 (logits of this size make single outputs move by more
+    than the element-wise bar under bf16 rounding of the states)."""
     from nha_amd import chunk_nha
-    d = prefill_inputs(880, 2, 200, 4, 2, 256, 256, 64, dtype=BF, gate_div=8.0, qk_scale=qk_scale)
+    d = prefill_inputs(880, 2, 200, HQ, H, D, D, 64, dtype=BF, gate_div=8.0, qk_scale=qk_scale)
     for wl, shift in ((99, 100), (64, 0)):
         c = [d[k].cuda() for k in KEYS]
         o, ls, lg = chunk_nha(*c, window_size_left=wl, gsa_kv_shift=shift, scale=1.0, impl="mfma")
