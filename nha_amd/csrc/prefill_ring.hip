@@ -19,14 +19,16 @@
 //    comparisons and no rescaling of the accumulators.  A row whose window sum leaves that range
 //    (overflowed, or below 2^-100) is flagged for mfma_repair_kernel, which recomputes it exactly.
 //
-// LDS layouts (bank-conflict free for the two fragment reads without padding, which a 1 KB wave
-// load cannot produce): a 32-row unit is cut into 16-row x 32-column blocks of 1 KB, a row of a block
-// is 64 bytes.  "K layout" (row fragments, ds_read_b128): the row's 64 bytes are contiguous and the
-// 16-byte piece index inside it is XORed with (row / 4) % 4.  "V layout" (transposing
+// LDS layouts (no padding, which a 1 KB wave load cannot produce; the 16-byte pieces of a wave load may
+// come from anywhere, so any order of pieces inside a 1 KB block is free): a 32-row unit is cut into
+// 16-row x 32-column blocks of 1 KB.  "K layout" (row fragments, ds_read_b128): the 16-byte piece c of
+// row r sits at 256 c + 16 r, which is exactly 16 x the number of the lane that reads it as its MFMA
+// operand, so a wave reads a block as 1 KB of consecutive bytes (with 64-byte rows and the piece index
+// XORed with (row / 4) % 4 a read took 12 LDS cycles instead of 4: SQ_LDS_BANK_CONFLICT 3.9e7 -> 5.1e6,
+// SQ_LDS_IDX_ACTIVE 1.12e8 -> 7.8e7 cycles per launch at the T = 8192 shape).  "V layout" (transposing
 // ds_read_b64_tr_b16, which takes 16 columns = 32 bytes of each of 16 rows per wave instruction): the
 // block is two planes of 16 rows x 32 bytes, columns 0..15 then columns 16..31, so that the 512 bytes
-// of one instruction are contiguous and use every bank twice (with 64-byte rows they used half the
-// banks four times: SQ_LDS_BANK_CONFLICT 9.8e7 -> 3.9e7 cycles per launch at the T = 8192 shape).
+// of one instruction are contiguous (with 64-byte rows: SQ_LDS_BANK_CONFLICT 9.8e7 -> 3.9e7).
 #include "mfma_common.h"
 
 #include <mutex>
@@ -113,8 +115,8 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   const int nunits = (c0 + 64 - lowest + 31) / 32;   // >= 2
 
   // ---- load descriptors of this wave: LDS-direct load i of a unit / a 64-row tile ------------------
-  // block index b = wave + 8 i; per lane: row lane / 4 of the block, piece lane % 4 of its 64-byte row
-  const int lrow16 = lane >> 2, lsl = lane & 3, lswz = lsl ^ ((lane >> 4) & 3);
+  // block index b = wave + 8 i; K layout: the lane's 16 bytes are piece lane / 16 of row lane % 16 of the block
+  const int lrow16 = lane & 15, lswz = lane >> 4;
   // V layout: the lane's 16 bytes are piece lane % 2 of plane lane / 32, row (lane % 32) / 2
   const int lrowv = (lane & 31) >> 1, lpv = 2 * (lane >> 5) + (lane & 1);
   uint32_t u_off[LPW];          // byte offset from the unit's first row (token rows, stride H*D)
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   // the reference is taken from unit 0 when a score there exceeds 2^THR, and kept from then on
   constexpr float THR = 8.f;
 
-  const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
+  const uint32_t kaddr = (uint32_t)(lane * 16);
   const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
   // row fragment (rows 16 kk + l16 of a unit, columns 32 ks + 8 kb ..) of a K-layout unit at byte address a
   auto kfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {

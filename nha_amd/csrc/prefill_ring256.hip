@@ -66,8 +66,8 @@ struct Cfg {
 };
 
 // LDS layouts as in prefill_ring.hip: a 32-row buffer is cut into 16-row x 32-column blocks of 1 KB
-// (half h, column block c at h * HB + c * 1024).  K layout: 64-byte rows, 16-byte piece index XORed
-// with (row / 4) % 4.  V layout: two planes of 16 rows x 32 bytes (columns 0..15, then 16..31).
+// (half h, column block c at h * HB + c * 1024).  K layout: 16-byte piece c of row r at 256 c + 16 r (a wave's
+// row fragments are 1 KB of consecutive bytes).  V layout: two planes of 16 rows x 32 bytes (columns 0..15, then 16..31).
 __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   using C = Cfg;
   constexpr int D = C::D, KS = C::KS, DB = C::DB, UB = C::UB, HB = C::HB, NR = C::NR, NW = C::NW, LPB = C::LPB;
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   const int nunits = (c0 + 64 - lowest + 31) / 32;   // >= 2
 
   // ---- LDS-direct loads: block b = wave + 4 i of a buffer; per lane a row of the block and a 16-byte piece
-  const int lrow16 = lane >> 2, lswz = (lane & 3) ^ ((lane >> 4) & 3);          // K layout
+  const int lrow16 = lane & 15, lswz = lane >> 4;          // K layout
   const int lrowv = (lane & 31) >> 1, lpv = 2 * (lane >> 5) + (lane & 1);         // V layout
   // one 32-row buffer from rows of `src` (row stride in elements): row r of the buffer is global row rowmap(r)
   auto issue_buffer = [&](uint32_t lds_buf, bool vlay, const bf16_t* src, uint32_t stride, auto rowmap) {
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   constexpr float THR = 8.f;           // the reference moves (prologue, slot branch) when a score tops it by more than 2^THR
   constexpr float BIG = 96.f;          // scores this far above the reference leave the matrix-core path
 
-  const uint32_t kaddr = (uint32_t)(l16 * 64 + ((kb ^ (l16 >> 2)) & 3) * 16);
+  const uint32_t kaddr = (uint32_t)(lane * 16);
   const uint32_t vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
   // row fragment (rows 16 kk + l16 of a buffer, columns 32 ks + 8 kb ..) of a K-layout buffer at byte address a
   auto kfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {
