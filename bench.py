@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # device-to-device copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the runs are summarised under
 # profiles/.  Reported as `traffic` only while the workload is the one they were measured on.
 TRAFFIC_BYTES = {
-    "ring_out_kernel<128>": (257433.0 * 2.0 + 139281.0) * 1024,
+    "ring_out_kernel<128>": (256759.0 * 2.0 + 139275.0) * 1024,
     "decode_mfma_kernel<128,4,2>": (302939.0 * 2.0 + 67216.0) * 1024,
     "layer_prologue_kernel": (106610.8 * 2.0 + 393216.0) * 1024,
     "layer_epilogue_kernel": (65759.4 * 2.0 + 131072.0) * 1024,
