@@ -33,6 +33,11 @@ constexpr float LN2 = 0.6931471805599453f;
 // unscaled intra-chunk scores (the layer's default scale is 1) summed over 16 rows with e^28 of fp32
 // range to spare; sub-blocks that decay faster are flagged and recomputed exactly.
 constexpr float DECAY_CLAMP = 60.f;
+// The backward's factored products use one reference per 32-row half of a chunk; the large factor
+// s exp(ref - gc_j) <= e^70 = 2.5e30 meets gradient-sized weights there (p (dp - delta), not raw scores), so
+// e^18 of fp32 range is enough, and gates drawn as logsigmoid(N(-1, 1)) (32 rows decay by e^-42 +- e^-4.5)
+// stay on the matrix-core path; chunks beyond it take the fp32 kernels.
+constexpr float BWD_DECAY_CLAMP = 70.f;
 
 struct MP {
   const bf16_t *q_swa, *k_swa, *q_gsa, *k_gsa, *v, *s, *g;

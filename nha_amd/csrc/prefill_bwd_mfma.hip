@@ -794,7 +794,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
 // into e^(gc_i - ref) <= 1 for the later row and e^(ref - gc_j) >= 1 for the earlier one, ref taken
 // at the start of j's half, and the terms become plain products of 64 x 64 tables
 //   X^(b) = scale du o e^(gc - ref_b), Xp^(b) = p o e^(gc - ref_b) (rows i), Y = s o e^(ref - gc) (rows j)
-// as long as no slot decays by more than e^-80 within a half (bf16 and fp32 share the exponent
+// as long as no slot decays by more than e^-70 within a half (bf16 and fp32 share the exponent
 // range); chunks beyond that are flagged by the state export and take the fp32 VALU kernels.
 //
 // bwd_slot_q_kernel, grid (HQ, NT): u = scale (E o q.hk0 + sum_b e^(gc - ref_b) o (A_masked Y)_b),

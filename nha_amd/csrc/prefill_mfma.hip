@@ -1106,7 +1106,7 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
     hvl[(cg * MS + m) * D + d] = f32_to_bf16(hv - bf16_to_f32(hvh));
   }
   for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
-  // chunks in which some slot decays by more than e^-DECAY_CLAMP over one of the two 32-row halves: the
+  // chunks in which some slot decays by more than e^-BWD_DECAY_CLAMP over one of the two 32-row halves: the
   // backward's factored products (e^(gc_i - ref) e^(ref - gc_j) as two operands, ref = the start of
   // j's half) leave the bf16 / fp32 range there
   if (tid == 0) {
@@ -1114,7 +1114,7 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
     const float* g = p.gc + cg * BT * MS;
     for (int m = 0; m < MS; ++m) {
       const float g31 = g[(R > 32 ? 31 : R - 1) * MS + m];
-      b |= (g31 < -DECAY_CLAMP) | (g[(R - 1) * MS + m] - g31 < -DECAY_CLAMP);
+      b |= (g31 < -BWD_DECAY_CLAMP) | (g[(R - 1) * MS + m] - g31 < -BWD_DECAY_CLAMP);
     }
     big[cg] = b;
   }
