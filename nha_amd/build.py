@@ -8,7 +8,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnha_hip.so")
-SOURCES = ["abi.hip", "decode.hip", "decode_mfma.hip", "prefill_simple.hip", "prefill_mfma.hip", "prefill_ring.hip", "prefill_ring256.hip", "prefill_bwd.hip", "prefill_bwd_mfma.hip",
+SOURCES = ["abi.hip", "decode.hip", "decode_mfma.hip", "prefill_simple.hip", "prefill_mfma.hip", "prefill_ring.hip", "prefill_ring256.hip", "prefill_bwd.hip", "prefill_bwd_mfma.hip", "prefill_bwd_ring.hip",
            "layer_fuse.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -22,7 +22,7 @@ FLAGS = [
 # the MFMA kernels never produce NaN on purpose; without this flag every fmaxf operand is
 # canonicalised by an extra VALU instruction in the softmax inner loop
 EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "prefill_ring.hip": ["-fno-honor-nans"], "prefill_ring256.hip": ["-fno-honor-nans"], "decode_mfma.hip": ["-fno-honor-nans"],
-         "prefill_bwd_mfma.hip": ["-fno-honor-nans"]}
+         "prefill_bwd_mfma.hip": ["-fno-honor-nans"], "prefill_bwd_ring.hip": ["-fno-honor-nans"]}
 
 
 def build_library(verbose: bool = False, jobs: int = 4) -> str:

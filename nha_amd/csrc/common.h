@@ -156,6 +156,9 @@ size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);
 bool bwd_window_mfma_supported(const NhaPrefillBwdArgs* a);
 int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta);
+// prefill_bwd_ring.hip: dq_swa with LDS-direct units for four query heads per kv-head at K = V = 128
+bool bwd_ring_dq_supported(const NhaPrefillBwdArgs* a);
+int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta);
 int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs);
 
 }  // namespace nha

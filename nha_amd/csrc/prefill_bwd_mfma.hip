@@ -1267,6 +1267,7 @@ bool bwd_window_mfma_supported(const NhaPrefillBwdArgs* a) {
 }
 
 int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta) {
+  if (bwd_ring_dq_supported(a)) return bwd_ring_dq(a, delta);
   const WP p = make_wp(a, delta, nullptr);
   hipStream_t st = (hipStream_t)a->stream;
   if (a->K == 64) return launch_dq<64, 64>(p, a->NT, st);

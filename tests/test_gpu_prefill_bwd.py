@@ -99,20 +99,22 @@ def test_bwd_head_dims_of_the_models():
     run_bwd_case("D256", d, wl=64, shift=0, dtype=BF, impl="mfma")
 
 
+@pytest.mark.parametrize("HQ,D,M", [(4, 64, 16), (8, 128, 64)])
 @pytest.mark.parametrize("wl,shift", [(-1, 0), (5, 6), (31, 32), (45, 0), (63, 64), (64, 0), (200, 201), (1000, 0)])
-def test_bwd_window_edges_on_the_matrix_cores(wl, shift):
-    """bf16, K == V == 64: the window gradients come from the matrix-core kernels.  Packed ragged
-    sequences (1 token, mid-chunk ends, longer than several key tiles), windows shorter than a
-    32-key half tile, not a multiple of it, longer than every sequence, and unbounded."""
+def test_bwd_window_edges_on_the_matrix_cores(wl, shift, HQ, D, M):
+    """bf16, K == V: the window gradients come from the matrix-core kernels (at D = 128 with four query
+    heads per kv-head dq_swa comes from the kernel that streams the window through LDS-direct units).
+    Packed ragged sequences (1 token, mid-chunk ends, longer than several key tiles), windows shorter
+    than a 32-key half tile, not a multiple of it, longer than every sequence, and unbounded."""
     cu = [0, 1, 66, 130, 450, 519]
-    d = prefill_inputs(7400 + wl, 1, cu[-1], 4, 2, 64, 64, 16, dtype=BF, qk_scale=1.0, with_state=True, N=5)
-    run_bwd_case(f"window wl={wl}", d, wl=wl, shift=shift, dtype=BF, cu=cu, scale=0.125, with_dht=True)
+    d = prefill_inputs(7400 + wl + D, 1, cu[-1], HQ, 2, D, D, M, dtype=BF, qk_scale=1.0, with_state=True, N=5)
+    run_bwd_case(f"window wl={wl} D={D}", d, wl=wl, shift=shift, dtype=BF, cu=cu, scale=D ** -0.5, with_dht=True)
 
 
 @pytest.mark.parametrize("gate_mean", [-1.0, -2.0, -4.0])
 def test_bwd_strong_gates(gate_mean):
     """Gate logits N(gate_mean, 1) -> logsigmoid without the /8: a 32-row half of a chunk decays by
-    about e^-45 / e^-70 / e^-130.  Up to e^-80 the matrix-core slot kernels factor the decay
+    about e^-45 / e^-70 / e^-130.  Up to e^-70 the matrix-core slot kernels factor the decay
     around the half's start; beyond, the state export flags the chunk and the fp32 VALU kernels
     take it.  Mixed within one call for gate_mean = -2 (some slots cross the bound, most do not).
     dg is a telescoping sum (large per-row terms that cancel against the final-state term); with a
