@@ -42,6 +42,23 @@ TRAFFIC_SOURCE = {
 }
 OUT_KERNEL = "ring_out_kernel<128>"
 
+# Seconds of back-to-back launches before every timed region, on top of the --warmup steps.  An idle
+# MI355X parks its shader clock near 100 MHz and needs about a second of load to reach the level it then
+# holds (2.3 GHz under the prefill here); the default 20 timed steps of 0.7 ms would otherwise be measured
+# on the ramp (about 2.0 GHz on these boxes).  `--clock-warmup 0` switches it off.
+CLOCK_WARM_S = 1.5
+
+
+def keep_busy(torch, fn, seconds=None, batch=20):
+    """Launch `fn` back to back for `seconds` of wall time (untimed)."""
+    seconds = CLOCK_WARM_S if seconds is None else seconds
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(batch):
+            fn()
+        torch.cuda.synchronize()
+
+
 PREFILL = dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=2048)
 DECODE = dict(B=128, HQ=32, H=8, D=128, M=64, W=1024, steps=256)
 # the other prefill shapes of the reference's configurations (parity-test cases; `--workload NAME`
@@ -165,6 +182,7 @@ def bench_prefill(torch, steps, warmup, cfg=PREFILL):
         a.phases = phases
         _lib.check(lib.nha_prefill_fwd(C.byref(a)))
 
+    keep_busy(torch, lambda: run(0))
     for _ in range(warmup):
         run(0)
     torch.cuda.synchronize()
@@ -211,6 +229,7 @@ def bench_backward(torch, steps, warmup, cfg=PREFILL):
     do = torch.randn(o.shape, generator=gen, device=dev, dtype=torch.float32).to(o.dtype)
     stream = torch.cuda.current_stream(dev)
     run = lambda: nha_prefill_bwd(*xs, o, ls, lg, do, cu_host, wl=wl, shift=shift, scale=D ** -0.5)
+    keep_busy(torch, run, batch=5)
     for _ in range(warmup):
         run()
     torch.cuda.synchronize()
@@ -242,6 +261,7 @@ def bench_glue(torch, steps, warmup, cfg=PREFILL):
     stream = torch.cuda.current_stream(dev)
 
     def timed(fn):
+        keep_busy(torch, fn)
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -274,6 +294,7 @@ def bench_layer(torch, steps, warmup):
     stream = torch.cuda.current_stream(dev)
 
     def timed(fn):
+        keep_busy(torch, fn)
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -336,6 +357,7 @@ def bench_decode(torch, warmup):
             j = i % pool
             ring_decode_step(st, q[j], sq[j], kn[j], kgn[j], vn[j], gn[j], out=o, advance=advance)
 
+    keep_busy(torch, lambda: loop(pool, False), batch=4)
     loop(warmup, True)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -367,6 +389,7 @@ def bench_api(torch, steps, warmup):
     stream = torch.cuda.current_stream(dev)
 
     def timed(fn, n):
+        keep_busy(torch, fn)
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -506,11 +529,15 @@ def cpu_baseline_torch_naive(torch, cores, decode_inputs):
 
 
 def main():
+    global CLOCK_WARM_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARM_S,
+                    help="seconds of untimed back-to-back launches before each timed region (the shader clock of an "
+                         "idle GPU needs about a second of load to reach its sustained level); 0 = off")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -521,6 +548,7 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
                     help="time the prefill of another of the reference's configurations and print its raw numbers")
     args = ap.parse_args()
+    CLOCK_WARM_S = max(args.clock_warmup, 0.0)
     if args.gpus != 1:
         print("bench.py measures one GPU: this path shards by sequence / kv-head with no communication and "
               "no multi-GPU figure is produced (run with --gpus 1)", file=sys.stderr)
@@ -573,6 +601,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "clock_warmup_s": CLOCK_WARM_S,
         "ms_per_step": pf["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
