@@ -155,11 +155,13 @@ bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);
 size_t prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a);
 int prefill_bwd_impl(const NhaPrefillBwdArgs* a);
 bool bwd_window_mfma_supported(const NhaPrefillBwdArgs* a);
-int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta);
-// prefill_bwd_ring.hip: dq_swa with LDS-direct units for four query heads per kv-head at K = V = 128
-bool bwd_ring_dq_supported(const NhaPrefillBwdArgs* a);
-int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta);
-int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs);
+int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta, void* ld);
+// prefill_bwd_ring.hip: the window gradients with LDS-direct operands for four query heads per kv-head at
+// K = V = 128; `ld` [T_tot, HQ] pairs of floats is written by the dq call and read by the dk / dv call
+bool bwd_ring_supported(const NhaPrefillBwdArgs* a);
+int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta, float2* ld);
+int bwd_ring_dkv(const NhaPrefillBwdArgs* a, const float2* ld, const float* dvs);
+int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs, const void* ld);
 
 }  // namespace nha
 

@@ -879,7 +879,7 @@ __global__ __launch_bounds__(256) void bwd_kv_window_kernel(const BP p) {
 size_t aligned(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct BwdPlan {
-  size_t fwd, mfma, hkct, hvct, hkb, hvb, hkl, hvl, ap, bp, ust, dpst, big, hkT, hvT, dus, pp, xg, delta, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
+  size_t fwd, mfma, hkct, hvct, hkb, hvb, hkl, hvl, ap, bp, ust, dpst, big, hkT, hvT, dus, pp, xg, delta, ld, ck, cv, dsi, dsp, dvs, gtot, dks, ek, ev, total;
   bool use_mfma;
   int nbk, nbv;
 };
@@ -914,6 +914,7 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
   s.pp = off; off += tqm;
   s.xg = off; off += tqm;
   s.delta = off; off += aligned((size_t)a->T_tot * a->HQ * 4);
+  s.ld = off; off += aligned((size_t)a->T_tot * a->HQ * 8);   // (-lse / scale, -delta) pairs of the LDS-direct window kernels
   const size_t cc = aligned((size_t)a->NT * a->HQ * BT * BT * 4);
   s.ck = off; off += cc;
   s.cv = off; off += cc;
@@ -1030,7 +1031,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipLaunchKernelGGL((bwd_q_kernel<T>), p.big ? dim3(a->NT, a->H) : dim3(a->NT * (BT / 4), a->HQ), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(query pass)");
   if (wmfma) {
-    rc = bwd_window_mfma_dq(a, p.delta);
+    rc = bwd_window_mfma_dq(a, p.delta, sc + sp.ld);
     if (rc != NHA_OK) return rc;
   } else {
     hipLaunchKernelGGL((bwd_q_window_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds_qw, st, p);
@@ -1070,7 +1071,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   hipLaunchKernelGGL((bwd_gate_scan_kernel<T>), dim3(a->N * a->H), dim3(64), 0, st, p);
   hipLaunchKernelGGL((bwd_gate_final_kernel<T>), dim3(a->NT, a->H), dim3(256), 0, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(gate scan)");
-  if (wmfma) return bwd_window_mfma_dkv(a, p.delta, p.dvs);
+  if (wmfma) return bwd_window_mfma_dkv(a, p.delta, p.dvs, sc + sp.ld);
   hipLaunchKernelGGL((bwd_kv_window_kernel<T>), dim3(a->T_tot, a->H), dim3(256), lds_w, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(key pass)");
   return NHA_OK;

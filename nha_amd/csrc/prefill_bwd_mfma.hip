@@ -1266,8 +1266,8 @@ bool bwd_window_mfma_supported(const NhaPrefillBwdArgs* a) {
          a->dlse_swa == nullptr && a->NT <= 65535;
 }
 
-int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta) {
-  if (bwd_ring_dq_supported(a)) return bwd_ring_dq(a, delta);
+int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta, void* ld) {
+  if (bwd_ring_supported(a)) return bwd_ring_dq(a, delta, (float2*)ld);
   const WP p = make_wp(a, delta, nullptr);
   hipStream_t st = (hipStream_t)a->stream;
   if (a->K == 64) return launch_dq<64, 64>(p, a->NT, st);
@@ -1275,7 +1275,8 @@ int bwd_window_mfma_dq(const NhaPrefillBwdArgs* a, const float* delta) {
   return launch_dq<256, 32>(p, a->NT, st);
 }
 
-int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs) {
+int bwd_window_mfma_dkv(const NhaPrefillBwdArgs* a, const float* delta, const float* dvs, const void* ld) {
+  if (bwd_ring_supported(a)) return bwd_ring_dkv(a, (const float2*)ld, dvs);
   const WP p = make_wp(a, delta, dvs);
   hipStream_t st = (hipStream_t)a->stream;
   if (a->K == 64) return launch_dkv<64, 64, 0>(p, a->NT, st);

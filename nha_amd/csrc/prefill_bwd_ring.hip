@@ -1,15 +1,24 @@
-// Window branch of the NHA prefill backward, dq_swa, for groups of four query heads per kv-head at
-// K == V == D == 128 (bf16): the data movement of ring_out_kernel (prefill_ring.hip) applied to the
-// products of bwd_dq_kernel (prefill_bwd_mfma.hip; the part nha_fla/ops/nha/chunk.py:499-511 hands to
-// flash-attn's backward).  With the merged log-sum-exp and delta = do . o of the whole op per (token,
-// q-head):
-//   S^T = K Q^T (log2 units, started at -lse),  dP^T = V dO^T,  dS^T = 2^S (dP^T - delta),
-//   dQ^T += K^T dS^T,   dq_swa = scale dQ.
-// One workgroup of 8 waves = one 64-token chunk x 4 query heads of one kv-head (32 queries per wave), so
-// the K / V rows of the window are fetched once for the four heads; they go from global memory straight
-// into LDS (global_load_lds_dwordx4) in units of 32 keys through a ring of four unit buffers.  A unit is
-// three tiles: K and V as row fragments (A operands of the two score products) and K once more in the
-// layout of the transposing read (A operand of K^T dS^T).  LDS layouts as in prefill_ring.hip.
+// Window branch of the NHA prefill backward for K == V == D == 128 (bf16) with four (or a multiple of
+// four) query heads per kv-head: the data movement of ring_out_kernel (prefill_ring.hip) applied to the
+// products of bwd_dq_kernel / bwd_dkv_kernel (prefill_bwd_mfma.hip; the part
+// nha_fla/ops/nha/chunk.py:499-511 hands to flash-attn's backward).  With the merged log-sum-exp and
+// delta = do . o of the whole op per (token, q-head), window logits w = scale q.k:
+//   pi = e^(w - lse),  dw = pi (do.v - delta),
+//   dq_swa_q = scale sum_j dw k_j,   dk_swa_j = scale sum_q dw q_q,   dv_j += sum_q pi do_q.
+// Every streamed operand goes from global memory straight into LDS (global_load_lds_dwordx4) through a
+// ring of four buffers; LDS layouts as in prefill_ring.hip (row-fragment tiles read as consecutive
+// bytes, tiles for the transposing read in two planes of 32-byte rows).
+//
+// ring_dq_kernel: one workgroup of 8 waves = one 64-token chunk x 4 query heads of one kv-head (a query
+//   per lane, 32 queries per wave), so the K / V rows of the window are fetched once for the four heads,
+//   in units of 32 keys.  A unit is three tiles: K and V as row fragments (A operands of S^T = K Q^T and
+//   dP^T = V dO^T) and K once more for the transposing read (A operand of dQ^T += K^T dS^T).  It also
+//   leaves (-lse / scale, -delta) per (token, q-head) as pairs for the kernel below, whose score and
+//   dP accumulators start from them.
+// ring_dkv_kernel: one workgroup of 8 waves = 256 keys of one kv-head (a key per lane and 16-key block, 32 keys per wave,
+//   K and V rows in registers); the q / do rows of every query head of the group stream through the ring
+//   in items of 32 queries: four tiles (q and do as row fragments for S = Q K^T and dP = dO V^T, and once
+//   more for the transposing read: dV^T += dO^T P, dK^T += Q^T dS) plus the 32 (lse, delta) pairs.
 #include "common.h"
 #include "mfma_common.h"
 
@@ -32,6 +41,7 @@ __device__ __forceinline__ void wait_vm() {
 struct DqP {
   const bf16_t *q, *k, *v, *dout;          // q_swa [T,HQ,D]; k_swa, v [T,H,D]; dout [T,HQ,D]
   const float *lse_swa, *lse_gsa, *delta;  // [T,HQ]
+  float2* ld;                              // [T,HQ] out: (-lse / scale, -delta) of the merged softmax
   bf16_t* dq;
   const int32_t *cu, *cidx;
   int HQ, H, NG, NT, wl;
@@ -132,6 +142,7 @@ __global__ __launch_bounds__(512, 1) void ring_dq_kernel(const DqP p) {
     const float mx = fmaxf(ls, lg);
     nlse[qb] = valid ? -(mx + __logf(__expf(ls - mx) + __expf(lg - mx))) * LOG2E : 0.f;
     dl[qb] = valid ? p.delta[tq] : 0.f;
+    if (valid && kb == 0) p.ld[tq] = make_float2(nlse[qb] / cs, -dl[qb]);
   }
   f32x4 dQ[DB][RQB];
 #pragma unroll
@@ -232,21 +243,306 @@ __global__ __launch_bounds__(512, 1) void ring_dq_kernel(const DqP p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------------
+struct DkvP {
+  const bf16_t *q, *k, *v, *dout;          // q_swa [T,HQ,D]; k_swa, v [T,H,D]; dout [T,HQ,D]
+  const float2* ld;                        // [T,HQ] (-lse / scale, -delta): what the two score accumulators start from
+  const float* dvs;                        // [T,H,D] slot-branch part of dv
+  bf16_t *dk, *dv;
+  const int32_t *cu, *cidx;
+  int HQ, H, NG, NT, wl;
+  float scale;
+};
+
+constexpr int KV_ITEM = 4 * UB + 1024;   // q rows | do rows | q transposing | do transposing | 32 (lse, delta) pairs
+constexpr int KV_QR = 0, KV_OR = UB, KV_QT = 2 * UB, KV_OT = 3 * UB, KV_LD = 4 * UB;
+constexpr int KV_BYTES = NR * KV_ITEM;
+constexpr int KEYS = 256;                // keys per workgroup
+constexpr int NKB = 2;                   // 16-key blocks per wave
+
+__device__ __forceinline__ void g2l4(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
+}
+
+__global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
+  constexpr int KV_LPW = 4;   // tile loads per wave and item (32 blocks of 1 KB, 8 waves)
+  extern __shared__ __align__(1024) unsigned char smem_[];
+  lbyte* const lds = (lbyte*)smem_;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int H = p.H, HQ = p.HQ, NG = p.NG;
+  // grid = (kv-head, chunk): the workgroup of every fourth chunk of a sequence takes that chunk and the next
+  // three; the others leave at once.  Workgroups are handed to the shader engines in turn, in launch order: were the working ones every
+  // fourth of that order they would all land on the same engine.  The launch order therefore walks the
+  // chunks with stride 4 (chunks 0, 4, 8, ... first, then 1, 5, 9, ...), so that the chunks of a sequence that
+  // start a group of four are neighbours in it; chunks from the last to the first.
+  const int nq = (p.NT + 3) >> 2;
+  const int cperm = 4 * (blockIdx.y % nq) + blockIdx.y / nq;
+  if (cperm >= p.NT) return;
+  const int chunk = p.NT - 1 - cperm;
+  const int h = blockIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  if (it & 3) return;
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int kspan = (eos - c0) < KEYS ? (eos - c0) : KEYS;
+  const float cs = p.scale * LOG2E;
+  // queries that see a key of the workgroup: [c0, qend), in items of 32 per query head
+  int qend = eos;
+  if (p.wl >= 0 && c0 + kspan + p.wl < eos) qend = c0 + kspan + p.wl;
+  const int nun = (qend - c0 + 31) / 32;   // >= 1
+  const int total = NG * nun;
+
+  // block (16-row half wave / 4, 32-column block wave % 4) of each of the four tiles of an item
+  const int rh = wave >> 2, cq = wave & 3;
+  // item (g, u): rows [c0 + 32 u, c0 + 32 u + 32) of query head h NG + g; rows past eos are read from row
+  // eos - 1 (always masked, always finite)
+  auto issue_item = [&](int g, int u, int slot) {
+    // what follows from the lane number is derived again at every request: kept across the loop it would
+    // cost registers the accumulators need
+    int ln = threadIdx.x & 63;
+    asm volatile("" : "+v"(ln));
+    const int lrow16 = ln & 15, lpk = ln >> 4;
+    const int lrowv = (ln & 31) >> 1, lpv = 2 * (ln >> 5) + (ln & 1);
+    const int hq = h * NG + g;
+    const int q0 = c0 + 32 * u;
+    const bf16_t* const qbase = p.q + ((int64_t)bos * HQ + hq) * D;
+    const bf16_t* const obase = p.dout + ((int64_t)bos * HQ + hq) * D;
+    int rr = q0 + 16 * rh + lrow16;
+    rr = rr < eos ? rr : eos - 1;
+    int rt = q0 + 16 * rh + lrowv;
+    rt = rt < eos ? rt : eos - 1;
+    const uint32_t offr = ((uint32_t)(rr - bos) * (uint32_t)(HQ * D) + (uint32_t)(4 * cq + lpk) * 8) * 2;
+    const uint32_t offt = ((uint32_t)(rt - bos) * (uint32_t)(HQ * D) + (uint32_t)(4 * cq + lpv) * 8) * 2;
+    const uint32_t dst = lds0 + slot * KV_ITEM + rh * HB + cq * 1024;
+    g2l16(qbase, offr, dst + KV_QR);
+    g2l16(obase, offr, dst + KV_OR);
+    g2l16(qbase, offt, dst + KV_QT);
+    g2l16(obase, offt, dst + KV_OT);
+    if (wave == 0) {
+      int r = q0 + (ln >> 1);
+      r = r < eos ? r : eos - 1;
+      g2l4(p.ld, (uint32_t)(((int64_t)r * HQ + hq) * 2 + (ln & 1)) * 4u, lds0 + slot * KV_ITEM + KV_LD);
+    }
+  };
+  int ig = 0, iu = 0;   // next item to request
+  auto issue_next = [&](int slot) {
+    issue_item(ig, iu, slot);
+    if (++iu == nun) {
+      iu = 0;
+      ++ig;
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < NR - 1; ++i)
+    if (i < total) issue_next(i);
+
+  // this lane's keys (one per 16-key block of the wave) and their K / V rows (B operands: K[key][32 ks + 8 kb ..])
+  const int kbase = 16 * NKB * wave;               // first key of the wave, relative to c0
+  bf16x8 kfr[NKB][KS], vfr[NKB][KS];
+#pragma unroll
+  for (int kk = 0; kk < NKB; ++kk) {
+    const int tk = c0 + kbase + 16 * kk + l16;
+    const int64_t jk = (int64_t)(tk < eos ? tk : eos - 1) * H + h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kfr[kk][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(p.k + jk * D + 32 * ks + 8 * kb));
+      vfr[kk][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(p.v + jk * D + 32 * ks + 8 * kb));
+    }
+  }
+  // the K / V rows are in their registers before the loop starts: left to the compiler, the wait for them sits
+  // at their first use inside the loop, as a wait for every load in flight, the LDS-direct ones included
+#pragma unroll
+  for (int kk = 0; kk < NKB; ++kk)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+v"(kfr[kk][ks]));
+      asm volatile("" : "+v"(vfr[kk][ks]));
+    }
+  f32x4 dK[DB][NKB], dV[DB][NKB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int kk = 0; kk < NKB; ++kk) {
+      dK[db][kk] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      dV[db][kk] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+  uint32_t kaddr, vaddr;   // set per item (see issue_item)
+  auto rfrag = [&](uint32_t a, int kk, int ks) -> bf16x8 {
+    return *reinterpret_cast<const NHA_LDS bf16x8*>(lds + (a + kaddr) + kk * HB + ks * 1024);
+  };
+  auto tfrag = [&](uint32_t a, int db) -> bf16x8 {
+    const lbyte* pa = lds + (a + vaddr) + (db >> 1) * 1024 + (db & 1) * 512;
+    struct { s16x4 a, b; } t;
+    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + HB));
+    return __builtin_bit_cast(bf16x8, t);
+  };
+
+  int u = 0;   // unit of the item being worked on
+  for (int i = 0; i < total; ++i) {
+    // item i has landed (this wave's part; wave 0 carries one more load per item), then everybody's
+    if (i + 2 < total) {
+      if (wave == 0) wait_vm<2 * (KV_LPW + 1)>();
+      else wait_vm<2 * KV_LPW>();
+    } else if (i + 1 < total) {
+      if (wave == 0) wait_vm<KV_LPW + 1>();
+      else wait_vm<KV_LPW>();
+    } else {
+      wait_vm<0>();
+    }
+    lds_barrier();
+    if (i + NR - 1 < total) issue_next((i + NR - 1) & (NR - 1));
+    const uint32_t base = (uint32_t)((i & (NR - 1)) * KV_ITEM);
+    int lc = threadIdx.x & 63;
+    asm volatile("" : "+v"(lc));
+    const int l16 = lc & 15, kb = lc >> 4;
+    kaddr = (uint32_t)(lc * 16);
+    vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
+    // queries [32 u, 32 u + 32) against keys [kbase, kbase + 16 NKB), both relative to c0: nothing to do if
+    // every query is before every key or past the window of every key
+    const bool none = (32 * u + 31 < kbase) || (p.wl >= 0 && 32 * u > kbase + 16 * NKB - 1 + p.wl);
+    if (!none) {
+      const bool edge = (32 * u < kbase + 16 * NKB - 1) || (p.wl >= 0 && 32 * u + 31 > kbase + p.wl) || (c0 + 32 * u + 32 > eos);
+      // ---- phase 1: S = Q K^T and dP = dO V^T, one 16-key block at a time (two blocks of scores beside both
+      //      gradient accumulators do not fit the register file, so the q / do row fragments are read once per
+      //      block); step i = (contraction step i / 2, 16-query block i % 2).  PD1 / PD2: how many steps ahead
+      //      of its product a fragment is requested from LDS; what the register file allows here (as two
+      //      launches, one gradient each, there is room for 2-3 steps and both blocks of scores: 873 + 709 us
+      //      against 1178 us for this kernel) ----
+      constexpr int N1 = 2 * KS;
+      constexpr int GS = 1;
+      constexpr int PD1 = 0;
+      constexpr int PD2 = 1;
+      bf16x8 Pb[NKB], dSb[NKB];
+      bf16x8 ot[DB], qt[DB];
+#pragma unroll
+      for (int g0 = 0; g0 < NKB; g0 += GS) {
+        f32x4 S[2][GS], dP[2][GS];
+        bf16x8 qa[N1], oa[N1];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < PD1; ++i) {
+          qa[i] = rfrag(base + KV_QR, i & 1, i >> 1);
+          oa[i] = rfrag(base + KV_OR, i & 1, i >> 1);
+        }
+        // rows of the accumulators are the queries 16 qb + 4 kb + r, the column is this lane's key of block
+        // g0 + j; they start from (-lse / scale, -delta) of their rows
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          const NHA_LDS f32x4* lp = reinterpret_cast<const NHA_LDS f32x4*>(lds + base + KV_LD + (16 * qb + 4 * kb) * 8);
+          const f32x4 a0 = lp[0], a1 = lp[1];   // the pairs of rows r = 0, 1 and r = 2, 3
+#pragma unroll
+          for (int j = 0; j < GS; ++j) {
+            S[qb][j] = (f32x4){a0[0], a0[2], a1[0], a1[2]};
+            dP[qb][j] = (f32x4){a0[1], a0[3], a1[1], a1[3]};
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < N1; ++i) {
+          const int qb = i & 1, ks = i >> 1;
+          if (i + PD1 < N1) {
+            qa[i + PD1] = rfrag(base + KV_QR, (i + PD1) & 1, (i + PD1) >> 1);
+            oa[i + PD1] = rfrag(base + KV_OR, (i + PD1) & 1, (i + PD1) >> 1);
+          }
+#pragma unroll
+          for (int j = 0; j < GS; ++j) {
+            S[qb][j] = mfma16(qa[i], kfr[g0 + j][ks], S[qb][j]);
+            dP[qb][j] = mfma16(oa[i], vfr[g0 + j][ks], dP[qb][j]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // the first transposed fragments of phase 2 are requested before the last exponentials
+        if (g0 + GS == NKB) {
+#pragma unroll
+          for (int i = 0; i < PD2; ++i) {
+            ot[i] = tfrag(base + KV_OT, i);
+            qt[i] = tfrag(base + KV_QT, i);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < GS; ++j) {
+          const int kk = g0 + j;
+          f32x4 P[2], dS[2];
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float x = S[qb][j][r] * cs;
+              if (edge) {
+                const int y = 32 * u + 16 * qb + 4 * kb + r, xk = kbase + 16 * kk + l16;
+                const bool ok = (xk <= y) && (p.wl < 0 || y - xk <= p.wl) && (c0 + y < eos);
+                if (!ok) x = -INFINITY;
+              }
+              const float pr = fexp2(x);
+              P[qb][r] = pr;
+              dS[qb][r] = pr * dP[qb][j][r];
+            }
+          Pb[kk] = pack8(P[0], P[1]);
+          dSb[kk] = pack8(dS[0], dS[1]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- phase 2: dV^T[d][key] += dO^T[d][q] P[q][key];  dK^T[d][key] += Q^T[d][q] dS[q][key] ----
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        if (db + PD2 < DB) {
+          ot[db + PD2] = tfrag(base + KV_OT, db + PD2);
+          qt[db + PD2] = tfrag(base + KV_QT, db + PD2);
+        }
+#pragma unroll
+        for (int kk = 0; kk < NKB; ++kk) {
+          dV[db][kk] = mfma16(ot[db], Pb[kk], dV[db][kk]);
+          dK[db][kk] = mfma16(qt[db], dSb[kk], dK[db][kk]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if (++u == nun) u = 0;
+  }
+#pragma unroll
+  for (int kk = 0; kk < NKB; ++kk) {
+    const int tk = c0 + kbase + 16 * kk + l16;
+    if (tk >= eos) continue;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int64_t off = ((int64_t)tk * H + h) * D + 16 * db + 4 * kb;
+      bf16x4 pk;
+      {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pk[r] = (__bf16)(dK[db][kk][r] * p.scale);
+        *reinterpret_cast<bf16x4*>(p.dk + off) = pk;
+      }
+      {
+        const float4 sv = *reinterpret_cast<const float4*>(p.dvs + off);
+        pk[0] = (__bf16)(dV[db][kk][0] + sv.x);
+        pk[1] = (__bf16)(dV[db][kk][1] + sv.y);
+        pk[2] = (__bf16)(dV[db][kk][2] + sv.z);
+        pk[3] = (__bf16)(dV[db][kk][3] + sv.w);
+        *reinterpret_cast<bf16x4*>(p.dv + off) = pk;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 // Served: four (or a multiple of four) query heads per kv-head at D = 128, tensors of one call below 4 GiB
 // (32-bit lane offsets of the LDS-direct loads).
-bool bwd_ring_dq_supported(const NhaPrefillBwdArgs* a) {
+bool bwd_ring_supported(const NhaPrefillBwdArgs* a) {
   static const bool off = getenv("NHA_BWD_NO_RING") != nullptr;   // A/B switch for measurements
   if (off || a->K != 128 || a->V != 128 || a->HQ % a->H != 0 || (a->HQ / a->H) % 4 != 0) return false;
-  return (int64_t)a->T_tot * a->H * 128 * 2 < ((int64_t)1 << 32);
+  return (int64_t)a->T_tot * a->HQ * 128 * 2 < ((int64_t)1 << 32);
 }
 
-int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta) {
+int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta, float2* ld) {
   DqP p;
   p.q = (const bf16_t*)a->q_swa; p.k = (const bf16_t*)a->k_swa; p.v = (const bf16_t*)a->v; p.dout = (const bf16_t*)a->dout;
   p.lse_swa = a->lse_swa; p.lse_gsa = a->lse_gsa; p.delta = delta;
-  p.dq = (bf16_t*)a->dq_swa;
+  p.dq = (bf16_t*)a->dq_swa; p.ld = ld;
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
   p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.NT = a->NT; p.wl = a->wl; p.scale = a->scale;
   static std::once_flag once;
@@ -258,6 +554,28 @@ int bwd_ring_dq(const NhaPrefillBwdArgs* a, const float* delta) {
   }
   hipLaunchKernelGGL(ring_dq_kernel, dim3(p.H * (p.NG / 4), p.NT), dim3(512), BYTES, (hipStream_t)a->stream, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(window dq, ring)");
+  return NHA_OK;
+}
+
+int bwd_ring_dkv(const NhaPrefillBwdArgs* a, const float2* ld, const float* dvs) {
+  DkvP p;
+  p.q = (const bf16_t*)a->q_swa; p.k = (const bf16_t*)a->k_swa; p.v = (const bf16_t*)a->v; p.dout = (const bf16_t*)a->dout;
+  p.ld = ld; p.dvs = dvs;
+  p.dk = (bf16_t*)a->dk_swa; p.dv = (bf16_t*)a->dv;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices;
+  p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H; p.NT = a->NT; p.wl = a->wl; p.scale = a->scale;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)ring_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, KV_BYTES);
+  });
+  if (attr_err != hipSuccess) {
+    set_error("nha_prefill_bwd: cannot reserve %d bytes of LDS: %s", KV_BYTES, hipGetErrorString(attr_err));
+    return NHA_ERR_LAUNCH;
+  }
+  const int ny = 4 * ((p.NT + 3) / 4);
+  hipLaunchKernelGGL(ring_dkv_kernel, dim3(p.H, ny), dim3(512), KV_BYTES, (hipStream_t)a->stream, p);
+  NHA_CHECK_LAUNCH("nha_prefill_bwd(window dk, dv, ring)");
   return NHA_OK;
 }
 

@@ -92,11 +92,16 @@ def test_bwd_all_cotangents_and_varlen(dtype):
 
 
 def test_bwd_head_dims_of_the_models():
-    """D = 128 (hybrid LLM heads, 4 query heads per kv-head) and D = 256 (the 340M layer)."""
+    """D = 128 (hybrid LLM heads, 4 and 8 query heads per kv-head) and D = 256 (the 340M layer)."""
     d = prefill_inputs(7200, 1, 200, 8, 2, 128, 128, 64, dtype=BF, qk_scale=128 ** -0.5, gate_div=1.0, gate_mean=-1.0)
     run_bwd_case("D128 GQA", d, wl=63, shift=64, dtype=BF, impl="mfma")
     d = prefill_inputs(7201, 2, 150, 2, 2, 256, 256, 64, dtype=BF, qk_scale=256 ** -0.5)
     run_bwd_case("D256", d, wl=64, shift=0, dtype=BF, impl="mfma")
+    # eight query heads per kv-head (the MoE hybrid's grouping), packed sequences that end inside a group of four
+    # chunks, inside a chunk and on a chunk boundary: the window gradients come from the LDS-direct kernels
+    cu = [0, 300, 364, 900]
+    d = prefill_inputs(7202, 1, cu[-1], 16, 2, 128, 128, 64, dtype=BF, qk_scale=128 ** -0.5, gate_div=1.0, gate_mean=-1.0, N=3)
+    run_bwd_case("D128 NG8 varlen", d, wl=200, shift=0, dtype=BF, impl="mfma", cu=cu)
 
 
 @pytest.mark.parametrize("HQ,D,M", [(4, 64, 16), (8, 128, 64)])
