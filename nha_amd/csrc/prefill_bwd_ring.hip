@@ -326,11 +326,19 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
       g2l4(p.ld, (uint32_t)(((int64_t)r * HQ + hq) * 2 + (ln & 1)) * 4u, lds0 + slot * KV_ITEM + KV_LD);
     }
   };
-  int ig = 0, iu = 0;   // next item to request
+  // The workgroups of neighbouring key groups of a sequence run at the same time on one XCD, and their
+  // query ranges overlap by all but 8 units.  Each walks the units of a head cyclically, starting where
+  // the walk of the sequence's first key group would be at that moment: neighbours then request the same
+  // q / do rows at about the same time and the second request finds them in L2.
+  const int rot = (nun - (8 * (it >> 2)) % nun) % nun;
+  int ig = 0, iu = rot;   // next item to request
+  int nreq = 0;           // items of the current head requested so far
   auto issue_next = [&](int slot) {
     issue_item(ig, iu, slot);
-    if (++iu == nun) {
-      iu = 0;
+    if (++iu == nun) iu = 0;
+    if (++nreq == nun) {
+      nreq = 0;
+      iu = rot;
       ++ig;
     }
   };
@@ -380,7 +388,7 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
     return __builtin_bit_cast(bf16x8, t);
   };
 
-  int u = 0;   // unit of the item being worked on
+  int u = rot, ndone = 0;   // unit of the item being worked on, items of its head done so far
   for (int i = 0; i < total; ++i) {
     // item i has landed (this wave's part; wave 0 carries one more load per item), then everybody's
     if (i + 2 < total) {
@@ -502,6 +510,10 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
       }
     }
     if (++u == nun) u = 0;
+    if (++ndone == nun) {
+      ndone = 0;
+      u = rot;
+    }
   }
 #pragma unroll
   for (int kk = 0; kk < NKB; ++kk) {
