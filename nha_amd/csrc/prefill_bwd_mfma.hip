@@ -66,6 +66,10 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a
   t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pb);
   return __builtin_bit_cast(bf16x8, t);
 }
+// Query head of workgroup x in a launch whose rows hold one workgroup per query head.  Workgroups are dealt
+// to the 8 XCDs in launch order, so x runs on XCD x % 8: the heads are numbered so that an XCD gets
+// consecutive heads, and the query heads of one kv-head fetch its states and rows through one L2.
+__device__ __forceinline__ int head_of_workgroup(int x, int HQ) { return (HQ & 7) == 0 ? (x & 7) * (HQ >> 3) + (x >> 3) : x; }
 __device__ __forceinline__ float logaddexp_f(float a, float b) {
   const float mx = fmaxf(a, b);
   return mx + logf(expf(a - mx) + expf(b - mx));
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const WP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
-  const int hq = blockIdx.x, h = hq / p.NG;
+  const int hq = head_of_workgroup(blockIdx.x, p.HQ), h = hq / p.NG;
   // last chunk first: the chunks at the start of a sequence see the fewest keys, and short
   // workgroups at the end of the launch leave the smallest tail
   const int chunk = gridDim.y - 1 - blockIdx.y;
@@ -567,7 +571,7 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
-  const int hq = blockIdx.x, h = hq / p.NG, chunk = blockIdx.y;
+  const int hq = head_of_workgroup(blockIdx.x, p.HQ), h = hq / p.NG, chunk = blockIdx.y;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
@@ -911,7 +915,7 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
-  const int hq = blockIdx.x, h = hq / p.NG, chunk = blockIdx.y;
+  const int hq = head_of_workgroup(blockIdx.x, p.HQ), h = hq / p.NG, chunk = blockIdx.y;
   if (p.big[(int64_t)chunk * H + h]) return;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
@@ -970,7 +974,7 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
-  const int hq = blockIdx.x, h = hq / p.NG;
+  const int hq = head_of_workgroup(blockIdx.x, p.HQ), h = hq / p.NG;
   const int chunk = blockIdx.y;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
