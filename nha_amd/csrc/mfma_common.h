@@ -74,6 +74,25 @@ __device__ __forceinline__ bf16x8 pack8(f32x4 a, f32x4 b) {
 
 // workgroup barrier that orders LDS traffic only: outstanding global loads (tile prefetches) stay
 // in flight across it
+// Tile of a workgroup in a launch of (kv-heads x groups-per-kv-head, chunks) tiles.  Workgroups are dispatched
+// in the order L = y * gridDim.x + x and workgroup L runs on XCD L % 8, each XCD with its own L2: XCD k takes
+// the k-th eighth of the tile sequence (kv-head, chunk, group of the kv-head), fastest last, so that what an
+// XCD works on at one time is a run of neighbouring chunks of one kv-head, whose windows overlap.  Returns the
+// tile's x (kv-head * ngrp + group) and y (chunk slot); the launch order itself when the grid is not a
+// multiple of 8.
+__device__ __forceinline__ void xcd_tile(int ngrp, int nchunks, int& vx, int& vy) {
+  vx = blockIdx.x;
+  vy = blockIdx.y;
+  const int total = gridDim.x * gridDim.y;
+  if ((total & 7) == 0) {
+    const int L = blockIdx.y * gridDim.x + blockIdx.x;
+    const int v = (L & 7) * (total >> 3) + (L >> 3);
+    const int g = v % ngrp, rest = v / ngrp;
+    vy = rest % nchunks;
+    vx = (rest / nchunks) * ngrp + g;
+  }
+}
+
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // max over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), VALU only

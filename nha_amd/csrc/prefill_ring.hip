@@ -96,9 +96,11 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
   // grid = (kv-head x group of four q-heads, chunk), chunks from the last to the first (prefill_mfma.hip)
-  const int chunk = p.NT - 1 - blockIdx.y;
   const int ngrp = NG / 4;
-  const int h = blockIdx.x / ngrp, grp = blockIdx.x % ngrp;
+  int vx, vy;
+  xcd_tile(ngrp, p.NT, vx, vy);   // with 8 (kv-head, group) pairs this is the launch order itself
+  const int chunk = p.NT - 1 - vy;
+  const int h = vx / ngrp, grp = vx % ngrp;
   const int hq = h * NG + grp * 4 + wave / 2;
   const int qb0 = (wave % 2) * RQB;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];

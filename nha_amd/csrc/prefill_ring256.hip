@@ -77,21 +77,10 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
-  // grid = (query head, chunk).  Workgroups are dispatched in the order L = y * gridDim.x + x and workgroup
-  // L runs on XCD L % 8, each with its own L2: XCD k takes the k-th eighth of the tile sequence
-  // (kv-head, chunk, query head of the kv-head), fastest last, so that what an XCD works on at one time
-  // is a run of neighbouring chunks of one kv-head, whose windows overlap.  Chunks from the last to the first.
-  int vx = blockIdx.x, vy = blockIdx.y;
-  {
-    const int total = gridDim.x * gridDim.y;
-    if ((total & 7) == 0) {
-      const int L = blockIdx.y * gridDim.x + blockIdx.x;
-      const int v = (L & 7) * (total >> 3) + (L >> 3);
-      const int g = v % NG, rest = v / NG;
-      vy = rest % p.NT;
-      vx = (rest / p.NT) * NG + g;
-    }
-  }
+  // grid = (query head, chunk), tiles dealt so that an XCD works on neighbouring chunks of one kv-head
+  // (xcd_tile); chunks from the last to the first
+  int vx, vy;
+  xcd_tile(NG, p.NT, vx, vy);
   const int chunk = p.NT - 1 - vy;
   const int hq = vx, h = hq / NG;
   const int Q = wave;                          // this wave's 16-row sub-block of the chunk
