@@ -191,20 +191,19 @@ def bench_prefill(torch, steps, warmup, cfg=PREFILL):
         run(0)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    # per-kernel durations with events on the launch stream: state pass alone, output pass alone
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
-    t_state = t_out = 0.0
-    for _ in range(steps):
+    # per-kernel durations with events on the launch stream: state pass alone, output pass alone.  The
+    # events of all steps are recorded before the host waits once, so the launches follow each other as
+    # they do in the timed loop above
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for ev in evs:
         ev[0].record(stream)
         run(1)
         ev[1].record(stream)
         run(2)
         ev[2].record(stream)
-        torch.cuda.synchronize()
-        t_state += ev[0].elapsed_time(ev[1]) * 1e-3
-        t_out += ev[1].elapsed_time(ev[2]) * 1e-3
-    t_state /= steps
-    t_out /= steps
+    torch.cuda.synchronize()
+    t_state = sum(ev[0].elapsed_time(ev[1]) for ev in evs) * 1e-3 / steps
+    t_out = sum(ev[1].elapsed_time(ev[2]) for ev in evs) * 1e-3 / steps
     flops = sum(prefill_flops(1, L, HQ, H, D, M, wl + 1) for L in lens)
     # the output pass carries everything but the slot write (the state pass's flops)
     flops_out = flops - B * T * H * 2 * (D * M + M * D)
