@@ -531,8 +531,8 @@ def main():
     global CLOCK_WARM_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARM_S,
                     help="seconds of untimed back-to-back launches before each timed region (the shader clock of an "
