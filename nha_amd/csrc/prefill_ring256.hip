@@ -14,8 +14,14 @@
 //    and sixteen V fragments held at once (128 registers) would push the accumulators out of the
 //    register file.
 //  * The slot-branch operands (four 64 x 256 tiles, 128 KB) do not fit beside the rings: they pass
-//    through the ring buffers after the window loop, three tiles at once (their latency is covered by
-//    building the decay tables) and the fourth while the first three are worked on.
+//    through the ring buffers.  The two halves of the chunk-start k-state and the first half of the
+//    chunk's k_gsa rows are requested into the K buffers the last iterations of the loop retire, the
+//    second half of the rows into the V buffer the last iteration retires, the halves of the v-state after
+//    the loop; the chunk's v rows replace the k-state once the slot logits are formed.
+//  * The softmax reference of a row is fixed by the prologue (the chunk's own keys): rescaling 64
+//    accumulator registers inside the loop costs the loop its registers whether or not the branch is
+//    taken.  A unit whose maximum tops the reference by 2^96 hands the wave's 16 rows to the exact pass
+//    (mfma_repair_kernel) and is clamped.
 #include "mfma_common.h"
 
 #include <mutex>
