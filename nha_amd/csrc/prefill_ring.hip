@@ -80,7 +80,9 @@ struct RingCfg {
   static constexpr int BYTES = SS + 8192;
   static constexpr int ETAB = 0;               // decay tables (6 units of 4 KB), over the ring once the window is done
   static constexpr int NSLOT_LOADS = 4 * LPW + 3;   // per wave: four tiles, two gate blocks, one s block
-  static_assert(6 * 4096 <= 2 * NR * UB, "decay tables must fit the ring");
+  static constexpr int EGI = ETAB + 6 * 4096;  // exp(gc_i[m]) fp32 [64][64], laid out like GC
+  static constexpr int EGR = EGI + 16384;      // exp(gc_i[m] - gr[m]) fp32 [64][64], gr = gate cumsum before the row's 16-row block
+  static_assert(6 * 4096 + 2 * 16384 <= 2 * NR * UB, "decay tables must fit the ring");
 };
 
 template <int D>
@@ -510,6 +512,23 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     }
     *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
   }
+  // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) of the chunk's rows: the same for the four query heads of the
+  // workgroup, so they are formed once here instead of by every wave for its own rows
+  for (int item = tid; item < 64 * 16; item += 512) {
+    const int j = item >> 4, m = 4 * (item & 15);
+    const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m));
+    f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (j >= 16) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at((j & ~15) - 1, m));
+    f32x4 ei, er;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      ei[r] = fexp(gi[r]);
+      er[r] = fexp(gi[r] - gr4[r]);
+    }
+    const uint32_t off = (uint32_t)(j * 256 + (((m >> 2) ^ (j & 15)) * 16));
+    *reinterpret_cast<NHA_LDS f32x4*>(lds + C::EGI + off) = ei;
+    *reinterpret_cast<NHA_LDS f32x4*>(lds + C::EGR + off) = er;
+  }
   __syncthreads();
 
   // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
@@ -578,18 +597,15 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
         }
     }
     // combine; the slot logits join the running softmax as one more set of keys
-    const int rref = 16 * Q - 1;
     f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
     float xmax = -INFINITY;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
-      const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(irow, 16 * mb + 4 * kb));
-      f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
-      if (Q > 0) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(rref, 16 * mb + 4 * kb));
+      const uint32_t off = (uint32_t)(irow * 256 + (((4 * mb + kb) ^ (irow & 15)) * 16));
+      egi[mb] = *reinterpret_cast<const NHA_LDS f32x4*>(lds + C::EGI + off);
+      egr[mb] = *reinterpret_cast<const NHA_LDS f32x4*>(lds + C::EGR + off);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        egi[mb][r] = fexp(gi[r]);
-        egr[mb][r] = fexp(gi[r] - gr4[r]);
         ok[mb][r] = (ok[mb][r] * egi[mb][r] + oki[mb][r] * egr[mb][r]) * cs;   // slot logit, log2 units
         xmax = fmaxf(xmax, ok[mb][r]);
       }
