@@ -72,6 +72,9 @@ WORKLOADS = dict(
     cfg2_shifted=dict(B=8, T=2048, HQ=4, H=4, D=256, M=64, W=512, gate_mean=0.0),
     cfg3=dict(B=1, T=32768, HQ=4, H=4, D=256, M=64, W=512, wl=512, shift=0, varlen=True, gate_mean=0.0, h0_std=0.1),
     cfg5=dict(B=2, T=16384, HQ=32, H=8, D=128, M=64, W=2048),
+    # the headline heads with the 64-token window of the hybrid models' NHA layers (the only regime of the
+    # reference's fused inference prefill, which is limited to W <= 64)
+    w64=dict(B=2, T=8192, HQ=32, H=8, D=128, M=64, W=64),
 )
 
 
@@ -583,7 +586,7 @@ def main():
     gl = bench_glue(torch, args.steps, args.warmup)
     api = bench_api(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     others = {}
-    for name in ("cfg2", "cfg3", "cfg5"):
+    for name in ("cfg2", "cfg3", "cfg5", "w64"):
         cfg = WORKLOADS[name]
         r = bench_prefill(torch, max(args.steps // 2, 1), min(args.warmup, 2), cfg)
         mb = min_prefill_bytes(cfg, len(workload_lengths(torch, cfg)))
