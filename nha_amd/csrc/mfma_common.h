@@ -123,7 +123,7 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a
 }
 
 // the slot recurrence is cut into segments of SEG chunks (two-level state pass)
-constexpr int SEG = 4;
+constexpr int SEG = 8;
 
 __device__ __forceinline__ int seg_slot(const int32_t* coff, int n, int it) { return coff[n] / SEG + it / SEG + n; }
 
