@@ -832,35 +832,66 @@ __device__ __forceinline__ float ref_of(const SP3& p, int c0, int h, int r, int 
 // The decay-scaled tables enter the gate gradient through a difference of nearly equal sums (dg is
 // a telescoping sum), so they are bf16 pairs (split_bf16) and their products hi*hi + hi*lo + lo*hi.
 // rows of Y = s_j[m] e^(ref - gc_j[m]) (zero for rows without a source token)
-__device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int c0, int h, int R, int vlo, int tid) {
+struct StageY {
   // 16-byte reads, all issued before the first conversion waits for one
-  constexpr int NS = BT * BT / 4 / 256;
+  static constexpr int NS = BT * BT / 4 / 256;
   float4 gj[NS], gr[NS];
   uint2 sr[NS];
+  __device__ __forceinline__ void load(const SP3& p, int c0, int h, int R, int vlo, int tid) {
 #pragma unroll
-  for (int u = 0; u < NS; ++u) {
-    const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
-    gj[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-    sr[u] = make_uint2(0, 0);
-    if (j >= vlo && j < R) {
-      sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + j - p.shift) * p.H + h) * BT + m);
-      gj[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + j) * p.H + h) * BT + m);
-      if (j >= 32) gr[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * p.H + h) * BT + m);
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
+      gj[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      sr[u] = make_uint2(0, 0);
+      if (j >= vlo && j < R) {
+        sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + j - p.shift) * p.H + h) * BT + m);
+        gj[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + j) * p.H + h) * BT + m);
+        if (j >= 32) gr[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * p.H + h) * BT + m);
+      }
     }
   }
+  __device__ __forceinline__ void store(lbf16* Yh, lbf16* Yl, int R, int vlo, int tid) const {
 #pragma unroll
-  for (int u = 0; u < NS; ++u) {
-    const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (j >= vlo && j < R) {
-      v.x = __uint_as_float(sr[u].x << 16) * __expf(gr[u].x - gj[u].x);
-      v.y = __uint_as_float(sr[u].x & 0xffff0000u) * __expf(gr[u].y - gj[u].y);
-      v.z = __uint_as_float(sr[u].y << 16) * __expf(gr[u].z - gj[u].z);
-      v.w = __uint_as_float(sr[u].y & 0xffff0000u) * __expf(gr[u].w - gj[u].w);
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), j = e >> 6, m = e & 63;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j >= vlo && j < R) {
+        v.x = __uint_as_float(sr[u].x << 16) * __expf(gr[u].x - gj[u].x);
+        v.y = __uint_as_float(sr[u].x & 0xffff0000u) * __expf(gr[u].y - gj[u].y);
+        v.z = __uint_as_float(sr[u].y << 16) * __expf(gr[u].z - gj[u].z);
+        v.w = __uint_as_float(sr[u].y & 0xffff0000u) * __expf(gr[u].w - gj[u].w);
+      }
+      split4_bf16(v, Yh, Yl, j * TLD + m);
     }
-    split4_bf16(v, Yh, Yl, j * TLD + m);
   }
+};
+__device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int c0, int h, int R, int vlo, int tid) {
+  StageY y;
+  y.load(p, c0, h, R, vlo, tid);
+  y.store(Yh, Yl, R, vlo, tid);
 }
+
+// per-row operands of the per-token stage for the rows 16 blk + 4 kb + q of a lane (slot m): requested
+// together, ahead of the stage, so that no block of rows waits out a memory latency of its own
+struct RowOps {
+  float gi[4][4], ls[4][4], lg[4][4], g31;
+  __device__ __forceinline__ void load(const SP3& p, int c0, int R, int h, int hq, int m, int kb) {
+    g31 = R > 32 ? p.gc[((int64_t)(c0 + 31) * p.H + h) * BT + m] : 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = 16 * blk + 4 * kb + q;
+        gi[blk][q] = ls[blk][q] = lg[blk][q] = 0.f;
+        if (i < R) {
+          const int64_t tq = (int64_t)(c0 + i) * p.HQ + hq;
+          gi[blk][q] = p.gc[((int64_t)(c0 + i) * p.H + h) * BT + m];
+          ls[blk][q] = p.lse_swa[tq];
+          lg[blk][q] = p.lse_gsa[tq];
+        }
+      }
+  }
+};
 
 // u, dp, p and du of the chunk's rows from the tables in LDS (A, B masked to j <= i; Y high and low
 // parts); the lane's values of q.hk0 and do.hv0 come either from the products kernel's accumulators
@@ -868,11 +899,11 @@ __device__ __forceinline__ void stage_y(lbf16* Yh, lbf16* Yl, const SP3& p, int 
 template <bool FROM_REGS>
 __device__ __forceinline__ void slot_q_rows(const SP3& p, const lbf16* At, const lbf16* Bt, const lbf16* Yh, const lbf16* Yl,
                                             int c0, int R, int h, int hq, int wave, int lane, const f32x4* cU,
-                                            const f32x4* cP, const lfloat* dl) {
+                                            const f32x4* cP, const lfloat* dl, const RowOps& ro) {
   const int l16 = lane & 15, kb = lane >> 4;
   const int HQ = p.HQ;
   const int m = 16 * wave + l16;
-  const float g31 = R > 32 ? gc_at(p, c0, h, 31, m) : 0.f;
+  const float g31 = ro.g31;
 #pragma unroll
   for (int blk = 0; blk < 4; ++blk) {
     f32x4 cu_[2], cd_[2];   // one accumulator per half of the contraction (= per reference)
@@ -889,12 +920,12 @@ __device__ __forceinline__ void slot_q_rows(const SP3& p, const lbf16* At, const
       const int i = 16 * blk + 4 * kb + q;
       if (i >= R) continue;
       const int64_t tq = (int64_t)(c0 + i) * HQ + hq;
-      const float gi = gc_at(p, c0, h, i, m);
+      const float gi = ro.gi[blk][q];
       const float e0 = __expf(gi);
       const float e1 = blk >= 2 ? __expf(gi - g31) : 0.f;   // rows before the second half see none of it
       const float au = p.scale * (e0 * ((FROM_REGS ? cU[blk][q] : p.ust[tq * BT + m]) + cu_[0][q]) + e1 * cu_[1][q]);
       const float ad = e0 * ((FROM_REGS ? cP[blk][q] : p.dpst[tq * BT + m]) + cd_[0][q]) + e1 * cd_[1][q];
-      const float ls = p.lse_swa[tq], lg = p.lse_gsa[tq];
+      const float ls = ro.ls[blk][q], lg = ro.lg[blk][q];
       const float lt = logaddexp_f(ls, lg);
       const float pm = __expf(au - lt);
       float du = pm * (ad - (FROM_REGS ? dl[i] : p.delta[tq]));
@@ -952,9 +983,11 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
       *reinterpret_cast<NHA_LDS bf16x4*>(Bt + i * TLD + j) = pb;
     }
   }
+  RowOps rops;
+  rops.load(p, c0, R, h, hq, 16 * wave + l16, kb);
   stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
   lds_barrier();
-  slot_q_rows<false>(p, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, nullptr, nullptr, nullptr);
+  slot_q_rows<false>(p, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, nullptr, nullptr, nullptr, rops);
 }
 
 // FUSE: the per-token stage of bwd_slot_q_kernel runs in the same workgroup (same grid, same
@@ -980,10 +1013,20 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
-  {
-    Tile<BT, D> rq, ro;
-    rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
-    ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+  // Every global read of the workgroup is requested ahead of the stage that consumes it, in the order
+  // of use, so that the stages do not each wait out a memory latency: q / do tiles, the Y rows, the o
+  // rows of delta and the rows of the Y table here; the per-row operands of the per-token stage before
+  // the products.
+  const bool fused = FUSE && !pq.big[(int64_t)chunk * H + h];
+  int vlo = pq.shift - it * BT;
+  vlo = vlo < 0 ? 0 : vlo;
+  // (at head size 256 the Y rows alone are 192 registers: there the tiles are stored before the Y rows
+  // are requested and the o rows are requested last)
+  constexpr bool EARLY = D <= 128;
+  Tile<BT, D> rq, ro;
+  rq.load(p.q + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+  ro.load(p.dout + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+  if (!EARLY) {
     rq.store(Qt, tid);
     ro.store(Ot, tid);
   }
@@ -1008,19 +1051,37 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
     yhkl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hkl + cg * D + 32 * ks + 8 * kb));
     yhvl[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p.hvl + cg * D + 32 * ks + 8 * kb));
   }
+  // o rows of delta: row i = 16 wave + l16, the four lanes sharing l16 split the columns
+  uint4 ov[KS];
+  auto load_o = [&]() {
+    const int i = 16 * wave + l16;
+    const bf16_t* orow = p.o + ((int64_t)(c0 + (i < R ? i : 0)) * HQ + hq) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      ov[ks] = make_uint4(0, 0, 0, 0);
+      if (i < R) ov[ks] = *reinterpret_cast<const uint4*>(orow + 32 * ks + 8 * kb);
+    }
+  };
+  if (EARLY) load_o();
+  StageY sy;
+  if (fused) sy.load(pq, c0, h, R, vlo, tid);
+  if (EARLY) {
+    rq.store(Qt, tid);
+    ro.store(Ot, tid);
+  } else {
+    load_o();
+  }
   lds_barrier();
   {
-    // delta_i = do_i . o_i: row i = 16 wave + l16, the four lanes sharing l16 split the columns
+    // delta_i = do_i . o_i
     const int i = 16 * wave + l16;
     float acc = 0.f;
-    if (i < R) {
-      const bf16_t* orow = p.o + ((int64_t)(c0 + i) * HQ + hq) * D;
-      for (int c = 8 * kb; c < D; c += 32) {
-        const bf16x8 ov = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(orow + c));
-        const bf16x8 dv = lds_frag(Ot, LDT, i, c);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 o8 = __builtin_bit_cast(bf16x8, ov[ks]);
+      const bf16x8 dv = lds_frag(Ot, LDT, i, 32 * ks + 8 * kb);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)dv[e];
     }
     acc += __shfl_xor(acc, 16, 64);
     acc += __shfl_xor(acc, 32, 64);
@@ -1029,7 +1090,8 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
   }
   float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
   float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
-  const bool fused = FUSE && !pq.big[(int64_t)chunk * H + h];
+  RowOps rops;
+  if (fused) rops.load(pq, c0, R, h, hq, 16 * wave + l16, kb);
   f32x4 cUr[FUSE ? 4 : 1], cPr[FUSE ? 4 : 1];
 #pragma unroll
   for (int blk = 0; blk < 4; ++blk) {
@@ -1066,11 +1128,9 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
   }
   if constexpr (FUSE) {
     if (!fused) return;   // uniform over the workgroup
-    int vlo = p.shift - it * BT;
-    vlo = vlo < 0 ? 0 : vlo;
-    stage_y(Yh, Yl, pq, c0, h, R, vlo, tid);
+    sy.store(Yh, Yl, R, vlo, tid);
     lds_barrier();
-    slot_q_rows<true>(pq, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, cUr, cPr, dlt);
+    slot_q_rows<true>(pq, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, cUr, cPr, dlt, rops);
   }
 }
 
@@ -1097,7 +1157,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
-  stage_y(Yh, Yl, p, c0, h, R, vlo, tid);
+  StageY sy;
+  sy.load(p, c0, h, R, vlo, tid);
   const int col = 16 * wave + l16;
   // columns r of ck / cv in the first half take the tables with ref 0, the others ref gc_31
   const lbf16* const Xch = wave < 2 ? X0h : X1h;
@@ -1107,56 +1168,69 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   f32x4 accS[4];
 #pragma unroll
   for (int rb = 0; rb < 4; ++rb) accS[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int a = 0; a < NG; ++a) {
-    const int hq = h * NG + a;
-    if (a > 0) lds_barrier();
+  // two 4-element groups per thread at a time: their twelve 16-byte reads are in flight together.  The
+  // first pair of a q-head is requested before the products of the head before it, the second pair
+  // before the first is converted: a head waits out one partly hidden memory latency instead of two.
+  struct Pair {
+    float4 gi[2], g31[2], du[2], pv[2], av[2], bv[2];
+  };
+  auto load_pair = [&](Pair& t, int hq, int u0) {
     const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
     const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
-    for (int u0 = 0; u0 < BT * BT / 4 / 256; u0 += 2) {
-      // two 4-element groups per thread at a time: their twelve 16-byte reads are in flight together
-      float4 gi[2], g31[2], du[2], pv[2], av[2], bv[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-        gi[u] = g31[u] = du[u] = pv[u] = av[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < R) {
-          gi[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
-          du[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
-          pv[u] = *reinterpret_cast<const float4*>(p.pp + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
-          if (i >= 32) g31[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
-          if (c <= i) {
-            av[u] = *reinterpret_cast<const float4*>(ap + e);
-            bv[u] = *reinterpret_cast<const float4*>(bp + e);
-          }
+    for (int u = 0; u < 2; ++u) {
+      const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
+      t.gi[u] = t.g31[u] = t.du[u] = t.pv[u] = t.av[u] = t.bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < R) {
+        t.gi[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+        t.du[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+        t.pv[u] = *reinterpret_cast<const float4*>(p.pp + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+        if (i >= 32) t.g31[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
+        if (c <= i) {
+          t.av[u] = *reinterpret_cast<const float4*>(ap + e);
+          t.bv[u] = *reinterpret_cast<const float4*>(bp + e);
         }
-      }
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-        const float g4[4] = {gi[u].x, gi[u].y, gi[u].z, gi[u].w}, r4[4] = {g31[u].x, g31[u].y, g31[u].z, g31[u].w};
-        const float d4[4] = {du[u].x, du[u].y, du[u].z, du[u].w}, q4[4] = {pv[u].x, pv[u].y, pv[u].z, pv[u].w};
-        const float a4[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, b4[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
-        float x0[4], x1[4], p0[4], p1[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float e0 = i < R ? __expf(g4[q]) : 0.f;
-          const float e1 = (i < R && i >= 32) ? __expf(g4[q] - r4[q]) : 0.f;
-          x0[q] = d4[q] * e0;
-          p0[q] = q4[q] * e0;
-          x1[q] = d4[q] * e1;
-          p1[q] = q4[q] * e1;
-          const bool in = i < R && c + q <= i;
-          AT[(c + q) * TLD + i] = f32_to_bf16(in ? a4[q] : 0.f);
-          BT_[(c + q) * TLD + i] = f32_to_bf16(in ? b4[q] : 0.f);
-        }
-        split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
-        split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
-        split4_bf16(make_float4(p0[0], p0[1], p0[2], p0[3]), P0h, P0l, i * TLD + c);
-        split4_bf16(make_float4(p1[0], p1[1], p1[2], p1[3]), P1h, P1l, i * TLD + c);
       }
     }
+  };
+  auto store_pair = [&](const Pair& t, int u0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
+      const float g4[4] = {t.gi[u].x, t.gi[u].y, t.gi[u].z, t.gi[u].w}, r4[4] = {t.g31[u].x, t.g31[u].y, t.g31[u].z, t.g31[u].w};
+      const float d4[4] = {t.du[u].x, t.du[u].y, t.du[u].z, t.du[u].w}, q4[4] = {t.pv[u].x, t.pv[u].y, t.pv[u].z, t.pv[u].w};
+      const float a4[4] = {t.av[u].x, t.av[u].y, t.av[u].z, t.av[u].w}, b4[4] = {t.bv[u].x, t.bv[u].y, t.bv[u].z, t.bv[u].w};
+      float x0[4], x1[4], p0[4], p1[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float e0 = i < R ? __expf(g4[q]) : 0.f;
+        const float e1 = (i < R && i >= 32) ? __expf(g4[q] - r4[q]) : 0.f;
+        x0[q] = d4[q] * e0;
+        p0[q] = q4[q] * e0;
+        x1[q] = d4[q] * e1;
+        p1[q] = q4[q] * e1;
+        const bool in = i < R && c + q <= i;
+        AT[(c + q) * TLD + i] = f32_to_bf16(in ? a4[q] : 0.f);
+        BT_[(c + q) * TLD + i] = f32_to_bf16(in ? b4[q] : 0.f);
+      }
+      split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
+      split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
+      split4_bf16(make_float4(p0[0], p0[1], p0[2], p0[3]), P0h, P0l, i * TLD + c);
+      split4_bf16(make_float4(p1[0], p1[1], p1[2], p1[3]), P1h, P1l, i * TLD + c);
+    }
+  };
+  static_assert(BT * BT / 4 / 256 == 4, "two pairs of element groups per thread");
+  Pair t0, t1;
+  load_pair(t0, h * NG, 0);
+  sy.store(Yh, Yl, R, vlo, tid);
+  for (int a = 0; a < NG; ++a) {
+    const int hq = h * NG + a;
+    load_pair(t1, hq, 2);
+    if (a > 0) lds_barrier();
+    store_pair(t0, 0);
+    store_pair(t1, 2);
     lds_barrier();
+    if (a + 1 < NG) load_pair(t0, hq + 1, 0);
     // ck[i][r = col] = sum_m X[i][m] Y[r][m], cv with Xp
     float* ckp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
     float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
