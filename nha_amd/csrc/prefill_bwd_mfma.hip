@@ -590,11 +590,8 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
       if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(p.kg + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
       rk.r[u] = x;
     }
-    rh.store(Ht, tid);
-    rk.store(Kt, tid);
-  }
-  const float* cp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
-  {
+    // the tables are requested before the tiles are stored: one memory latency for both
+    const float* cp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
     constexpr int NS = BT * BT / 4 / 256;
     float4 wv[NS], gv[NS], cv[NS];
 #pragma unroll
@@ -607,6 +604,8 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
         if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
       }
     }
+    rh.store(Ht, tid);
+    rk.store(Kt, tid);
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
@@ -678,47 +677,48 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   const bf16_t* ysrc = isv ? p.v : p.kg;
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
-  {
-    Tile<BT, D> ry;
+  Tile<BT, D> ry;
 #pragma unroll
-    for (int u = 0; u < Tile<BT, D>::NPC; ++u) {
-      const int c = tid + 256 * u;
-      const int row = c / (D / 8), cc = (c % (D / 8)) * 8;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(ysrc + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
-      ry.r[u] = x;
-    }
-    ry.store(Yt, tid);
+  for (int u = 0; u < Tile<BT, D>::NPC; ++u) {
+    const int c = tid + 256 * u;
+    const int row = c / (D / 8), cc = (c % (D / 8)) * 8;
+    uint4 x = make_uint4(0, 0, 0, 0);
+    if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(ysrc + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
+    ry.r[u] = x;
   }
   const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
   const float* gcb = p.gc + ((int64_t)c0 * H + h) * BT;
   {
-    // all global loads of a batch are issued before the first conversion waits for one
+    // all global loads of a batch are issued before the first conversion waits for one; the first batch
+    // of E and the gate rows are requested before the Y tile is stored
     constexpr int NE = D * BT / 4 / 256, EB = NE < 8 ? NE : 8;
     const float4* ep4 = reinterpret_cast<const float4*>(ep);
+    constexpr int NS = BT * BT / 4 / 256;
+    float4 gl[NS], gr[NS];
+    uint2 sr[NS];
 #pragma unroll
     for (int b0 = 0; b0 < NE; b0 += EB) {
       float4 buf[EB];
 #pragma unroll
       for (int u = 0; u < EB; ++u) buf[u] = ep4[tid + 256 * (b0 + u)];
+      if (b0 == 0) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const int e = 4 * (tid + 256 * u), r = e >> 6, m = e & 63;
+          gl[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+          sr[u] = make_uint2(0, 0);
+          if (r >= vlo && r < R) {
+            sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + r - p.shift) * H + h) * BT + m);
+            gl[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)(R - 1) * H * BT + m);
+            gr[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)r * H * BT + m);
+          }
+        }
+        ry.store(Yt, tid);
+      }
 #pragma unroll
       for (int u = 0; u < EB; ++u) {
         const int e = 4 * (tid + 256 * (b0 + u));
         split4_bf16(buf[u], Et, El, (e >> 6) * ELD + (e & 63));
-      }
-    }
-    constexpr int NS = BT * BT / 4 / 256;
-    float4 gl[NS], gr[NS];
-    uint2 sr[NS];
-#pragma unroll
-    for (int u = 0; u < NS; ++u) {
-      const int e = 4 * (tid + 256 * u), r = e >> 6, m = e & 63;
-      gl[u] = gr[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-      sr[u] = make_uint2(0, 0);
-      if (r >= vlo && r < R) {
-        sr[u] = *reinterpret_cast<const uint2*>(p.s + (((int64_t)c0 + r - p.shift) * H + h) * BT + m);
-        gl[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)(R - 1) * H * BT + m);
-        gr[u] = *reinterpret_cast<const float4*>(gcb + (int64_t)r * H * BT + m);
       }
     }
 #pragma unroll
@@ -736,6 +736,27 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   }
   lds_barrier();
   const int col = 16 * wave + l16;
+  // the gate rows of the last products' decay, requested before the products
+  const float glast = gcb[(int64_t)(R - 1) * H * BT + col];
+  float grow[4][4];
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = 16 * rb + 4 * kb + q;
+      grow[rb][q] = r < R ? gcb[(int64_t)r * H * BT + col] : 0.f;
+    }
+  // the partial sums the first products are added to: requested before the products where the registers
+  // allow (head sizes up to 128)
+  const bool has = col >= vlo && col < R;
+  const int64_t oi = (((int64_t)c0 + col - p.shift) * H + h) * D;
+  const float* const part = isv ? p.dvs : p.dks;
+  constexpr bool EARLY = D <= 128;
+  float4 pve[EARLY ? DB : 1];
+  if (EARLY && has) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) pve[EARLY ? db : 0] = *reinterpret_cast<const float4*>(part + oi + 16 * db + 4 * kb);
+  }
   // out^T[x][r = col] = sum_m E[x][m] sE[r][m]: A = E rows (plain), B = sE rows (plain), contraction m in 2 steps
   f32x4 accO[DB];
 #pragma unroll
@@ -749,13 +770,10 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
       accO[db] = mfma16(eh, bs, mfma16(eh, bsl, mfma16(lds_frag(El, ELD, 16 * db + l16, 32 * ks + 8 * kb), bs, accO[db])));
     }
   }
-  const bool has = col >= vlo && col < R;
   if (has) {
-    const int64_t oi = (((int64_t)c0 + col - p.shift) * H + h) * D;
-    float* part = isv ? p.dvs : p.dks;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      const float4 pv = *reinterpret_cast<const float4*>(part + oi + 16 * db + 4 * kb);
+      const float4 pv = EARLY ? pve[EARLY ? db : 0] : *reinterpret_cast<const float4*>(part + oi + 16 * db + 4 * kb);
       const float o0 = accO[db][0] + pv.x, o1 = accO[db][1] + pv.y, o2 = accO[db][2] + pv.z, o3 = accO[db][3] + pv.w;
       if (isv) {
         *reinterpret_cast<float4*>(p.dvs + oi + 16 * db + 4 * kb) = make_float4(o0, o1, o2, o3);
@@ -785,7 +803,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
     for (int q = 0; q < 4; ++q) {
       const int r = 16 * rb + 4 * kb + q;
       if (r < R) {
-        const float dec = __expf(gcb[(int64_t)(R - 1) * H * BT + col] - gcb[(int64_t)r * H * BT + col]);
+        const float dec = __expf(glast - grow[rb][q]);
         p.dsp[(((int64_t)(isv ? 1 : 0) * p.T_tot + c0 + r) * H + h) * BT + col] = acc[q] * dec;
       }
     }
