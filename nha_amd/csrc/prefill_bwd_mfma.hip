@@ -496,29 +496,35 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
     accO[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
   const int col = 16 * wave + l16;   // this lane's column: slot m of N, row r of out
+  // The X tile and the tables of a q-head are requested together (coalesced 16-byte reads over c, all
+  // issued before the first use); at head sizes up to 128 those of the next head are requested before the
+  // products of this one, so that only the first head of a workgroup waits out a memory latency.
+  constexpr int NS = BT * BT / 4 / 256;
+  constexpr bool AHEAD = D <= 128;
+  Tile<BT, D> rx;
+  float4 wv[NS], gv[NS], cv[NS];
+  auto load_head = [&](int hq) {
+    rx.load(xsrc + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+      wv[u] = gv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < R) {
+        wv[u] = *reinterpret_cast<const float4*>(wsrc + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
+        gv[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+        if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
+      }
+    }
+  };
+  if (AHEAD) load_head(h * NG);
   for (int a = 0; a < NG; ++a) {
     const int hq = h * NG + a;
+    if (!AHEAD) load_head(hq);
     if (a > 0) lds_barrier();   // everyone is done with the previous head's tiles
+    rx.store(Xt, tid);
     {
-      Tile<BT, D> rx;
-      rx.load(xsrc + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
-      rx.store(Xt, tid);
-    }
-    const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
-    {
-      // coalesced 16-byte reads over c (all issued before the first use), transposed writes
-      constexpr int NS = BT * BT / 4 / 256;
-      float4 wv[NS], gv[NS], cv[NS];
-#pragma unroll
-      for (int u = 0; u < NS; ++u) {
-        const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-        wv[u] = gv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < R) {
-          wv[u] = *reinterpret_cast<const float4*>(wsrc + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
-          gv[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
-          if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
-        }
-      }
+      // transposed writes
 #pragma unroll
       for (int u = 0; u < NS; ++u) {
         const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
@@ -533,6 +539,7 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
       }
     }
     lds_barrier();
+    if (AHEAD && a + 1 < NG) load_head(hq + 1);
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const bf16x8 bw = table_frag(Wt, col, hf, kb), bwl = table_frag(Wl, col, hf, kb);
