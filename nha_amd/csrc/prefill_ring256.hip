@@ -68,7 +68,6 @@ struct Cfg {
   static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
   static constexpr int ETAB = SS + 8192;       // decay tables, 6 units of 4 KB
   static constexpr int BYTES = ETAB + 6 * 4096;
-  static constexpr int NGS = 16 / NW + 8 / NW; // loads per wave for the gate and s blocks (6)
 };
 
 // LDS layouts as in prefill_ring.hip: a 32-row buffer is cut into 16-row x 32-column blocks of 1 KB
@@ -149,31 +148,6 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     for (int i = 0; i < LPB; ++i) g2l16(src, voff[i], boff[i] + C::RING_V + slot_off);
   };
 
-  // ---- requests: K and V of the first units, then the query fragments ---------------------------------
-  issue_k(0);
-  issue_v(0);
-  issue_k(1);
-  issue_v(1);
-  if (2 < nunits) issue_k_fast(2, 2 * UB);
-  // window-query fragments, pre-scaled by scale * log2(e)
-  bf16x8 qs[KS];
-  {
-    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
-      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
-      bf16x8 r;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float f = __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
-        r[e] = (__bf16)(f * cs);
-      }
-      qs[ks] = r;
-    }
-  }
-
   const int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);   // first row of the chunk whose source token exists
   const int grow_s = c0 - p.shift;                                       // source token of row 0
   auto tok = [&](int r) {   // source token of row r, kept inside the sequence (rows outside [vlo, rows) carry no weight)
@@ -199,6 +173,78 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
       g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok(r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + b * 1024);
     }
   };
+
+  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
+  auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
+  // decay tables E_Q[j][m] = s_j[m] exp(min(gr_Q[m] - gc_j[m], DECAY_CLAMP)) for the rows j of the 16-row
+  // blocks jb <= Q, zero elsewhere (gr_Q: gate cumsum of the row before sub-block Q, 0 for Q = 0); rows
+  // whose source token does not exist carry no weight.  32-row units in the V layout (64 columns):
+  // E_0 -> unit 0, E_1 -> 1, E_2 -> 2,3, E_3 -> 4,5; a thread makes 8 consecutive slots of a row.
+  auto build_decay_tables = [&]() {
+    for (int item = tid; item < 6 * 256; item += 64 * NW) {
+      const int U = item >> 8, r32 = (item >> 3) & 31, m = (item & 7) * 8;
+      const int Qt = U == 0 ? 0 : U == 1 ? 1 : U < 4 ? 2 : 3;
+      const int pr = (U == 3 || U == 5) ? 1 : 0;
+      const int j = 32 * pr + r32;
+      const bool ok = (j >> 4) <= Qt && j >= vlo && j < rows;
+      bf16x8 out;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = (__bf16)0.f;
+      if (ok) {
+        f32x4 gv[2], gr[2];
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m + 4 * hh));
+          gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          if (Qt > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Qt - 1, m + 4 * hh));
+        }
+        const bf16x8 sv = *reinterpret_cast<const NHA_LDS bf16x8*>(s_at(j, m));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)sv[e] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
+      }
+      *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
+    }
+  };
+  // ---- requests: the gate blocks (the decay tables are built from them while the units are still on their
+  //      way), K and V of the first units, then the query fragments -------------------------------------
+  issue_gates();
+  issue_k(0);
+  issue_v(0);
+  issue_k(1);
+  issue_v(1);
+  if (2 < nunits) issue_k_fast(2, 2 * UB);
+  // window-query fragments, pre-scaled by scale * log2(e)
+  bf16x8 qs[KS];
+  uint4 qraw[KS];
+  {
+    // rows past the end of the sequence read the last row (the number of loads must not depend on the lane:
+    // the wait below counts them) and are zeroed afterwards
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + (irow < rows ? irow : rows - 1)) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qraw[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+  }
+  NHA_FENCE();
+  // the gate blocks were requested first: they have landed once no more than the requests made after them
+  // are outstanding (four or five unit buffers and the query loads)
+  if (2 < nunits) wait_vm<5 * LPB + KS>();
+  else wait_vm<4 * LPB + KS>();
+  lds_barrier();
+  build_decay_tables();
+  NHA_FENCE();
+  {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint4 x = irow < rows ? qraw[ks] : make_uint4(0, 0, 0, 0);
+      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+      bf16x8 r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = __uint_as_float((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+        r[e] = (__bf16)(f * cs);
+      }
+      qs[ks] = r;
+    }
+  }
 
   // ---- window loop state ------------------------------------------------------------------------
   f32x4 O[DB];
@@ -345,12 +391,10 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     const bf16x8 Pq = pack_p();
     NHA_FENCE();
     // K of unit u+2 and V of unit u (requested two iterations ago) have landed for this wave, then for
-    // everybody.  What may stay in flight: the requests of the previous iteration (and, right after the
-    // start, K of unit 3 and the gate blocks).
+    // everybody.  What may stay in flight: the requests of the previous iteration.
     if (u >= 1) {
       if (early) {                    // every iteration requests two buffers' worth, V side first
         if (u + 2 == nunits) wait_vm<LPB>();   // last iteration: also V of the last unit; the tile half behind it may fly
-        else if (u <= 2) wait_vm<2 * LPB + C::NGS>();
         else wait_vm<2 * LPB>();
       } else {
         wait_vm<0>();
@@ -378,7 +422,6 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
         issue_tb(off, 0);
       }
     }
-    if (u == 0) issue_gates();
     NHA_FENCE();
     // ---- phase B: value products of unit u on the matrix core, row maximum of unit u+1 on the VALU;
     //      V fragment db is read PD products ahead ----
@@ -462,36 +505,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   // the window's own log-sum-exp, before the slots join the running softmax
   if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[0]) - nm) * LN2;
 
-  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
-  auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
-  // decay tables E_Q[j][m] = s_j[m] exp(min(gr_Q[m] - gc_j[m], DECAY_CLAMP)) for the rows j of the 16-row
-  // blocks jb <= Q, zero elsewhere (gr_Q: gate cumsum of the row before sub-block Q, 0 for Q = 0); rows
-  // whose source token does not exist carry no weight.  32-row units in the V layout (64 columns):
-  // E_0 -> unit 0, E_1 -> 1, E_2 -> 2,3, E_3 -> 4,5; a thread makes 8 consecutive slots of a row.
-  for (int item = tid; item < 6 * 256; item += 64 * NW) {
-    const int U = item >> 8, r32 = (item >> 3) & 31, m = (item & 7) * 8;
-    const int Qt = U == 0 ? 0 : U == 1 ? 1 : U < 4 ? 2 : 3;
-    const int pr = (U == 3 || U == 5) ? 1 : 0;
-    const int j = 32 * pr + r32;
-    const bool ok = (j >> 4) <= Qt && j >= vlo && j < rows;
-    bf16x8 out;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) out[e] = (__bf16)0.f;
-    if (ok) {
-      f32x4 gv[2], gr[2];
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        gv[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(j, m + 4 * hh));
-        gr[hh] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        if (Qt > 0) gr[hh] = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(16 * Qt - 1, m + 4 * hh));
-      }
-      const bf16x8 sv = *reinterpret_cast<const NHA_LDS bf16x8*>(s_at(j, m));
-#pragma unroll
-      for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)sv[e] * fexp(fminf(gr[e >> 2][e & 3] - gv[e >> 2][e & 3], DECAY_CLAMP)));
-    }
-    *reinterpret_cast<NHA_LDS bf16x8*>(lds + C::ETAB + U * 4096 + (r32 >> 4) * 2048 + (m >> 5) * 1024 + ((m >> 4) & 1) * 512 + (r32 & 15) * 32 + (m & 15) * 2) = out;
-  }
-  // k-state and k_gsa rows have landed (the two v-state halves may still fly), the tables are written
+  // k-state and k_gsa rows have landed (the two v-state halves may still fly)
   wait_vm<2 * LPB>();
   __syncthreads();
 
