@@ -104,7 +104,9 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   const int chunk = p.NT - 1 - vy;
   const int h = vx / ngrp, grp = vx % ngrp;
   const int hq = h * NG + grp * 4 + wave / 2;
-  const int qb0 = (wave % 2) * RQB;
+  // rows 0..31 or 32..63 of the chunk: the later rows have more intra-chunk work in the slot branch, so the two
+  // waves that share a SIMD (w and w + 4) take one half each
+  const int qb0 = ((wave ^ (wave >> 2)) & 1) * RQB;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
