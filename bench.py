@@ -328,9 +328,12 @@ def bench_layer(torch, steps, warmup):
     return out
 
 
-def bench_decode(torch, warmup):
+# the decode step at the 340M layers' heads (one query head per kv-head, head size 256, window 512)
+DECODE_D256 = dict(B=128, HQ=4, H=4, D=256, M=64, W=512, steps=128)
+
+
+def bench_decode(torch, warmup, cfg=DECODE):
     from nha_amd import NHARingState, ring_decode_step
-    cfg = DECODE
     dev = torch.device("cuda:0")
     B, HQ, H, D, M, W, steps = (cfg[k] for k in ("B", "HQ", "H", "D", "M", "W", "steps"))
     gen = torch.Generator().manual_seed(0)
@@ -583,6 +586,7 @@ def main():
     pf = bench_prefill(torch, args.steps, args.warmup)
     bw = bench_backward(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     dc = bench_decode(torch, args.warmup)
+    dc256 = bench_decode(torch, args.warmup, DECODE_D256)
     gl = bench_glue(torch, args.steps, args.warmup)
     api = bench_api(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     others = {}
@@ -625,7 +629,12 @@ def main():
                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dc["achieved_gbs"] / PEAK_HBM_GBS,
                                 "traffic": TRAFFIC_BYTES["decode_mfma_kernel<128,4,2>"],
                                 "traffic_source": TRAFFIC_SOURCE["decode_mfma_kernel<128,4,2>"],
-                                "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]}},
+                                "kernel_us": dc["us_kernel"], "algorithmic_bytes": dc["bytes"]},
+                   "other_shapes": {"d256": {"shape": {k: v for k, v in DECODE_D256.items() if k != "steps"},
+                                             "us_per_step": dc256["us_per_step"], "kernel_us": dc256["us_kernel"],
+                                             "kernel": "decode_mfma_kernel<256,1,4>", "algorithmic_bytes": dc256["bytes"],
+                                             "achieved_gbs": dc256["achieved_gbs"],
+                                             "hbm_frac": dc256["achieved_gbs"] / PEAK_HBM_GBS}}},
         "backward": {"metric": "backward of the same prefill call", "ms_per_call": bw["bwd_ms"], "unit": "ms",
                      "tokens_per_s": bw["bwd_tokens_per_s"], "tflops": bw["bwd_tflops"],
                      "flop": bw["bwd_flops"], "note": "2.5 x the forward's algorithmic flop"},

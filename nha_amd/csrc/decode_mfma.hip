@@ -1,4 +1,4 @@
-// Matrix-core decode step for gfx950: bf16, K == V == D in {64,128}, M == 64 slots, up to 8 query
+// Matrix-core decode step for gfx950: bf16, K == V == D in {64,128,256}, M == 64 slots, up to 8 query
 // heads per kv-head; window or ring mode with a pre-rotated window query, or window mode with
 // in-kernel rotate-half RoPE of the raw query and window keys (cos / sin tables,
 // nha_fla/ops/nha/fused_recurrent.py:309-329).
@@ -454,15 +454,20 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
 #pragma unroll
       for (int j = 0; j < KS; ++j) qf[j] = as_bf16x8(qx[j]);
     }
-    uint4 kr0[2 * KS], vr0[NVT], kr1[2 * KS], vr1[NVT];
+    // register buffers of 32-key blocks per wave: two at head sizes up to 128 (32 KB in flight), one at 256
+    // (a block is 32 KB there, and twice the waves per workgroup keep as many bytes in flight per CU)
+    constexpr int NBUF = D > 128 ? 1 : 2;
+    uint4 kr0[2 * KS], vr0[NVT], kr1[NBUF == 2 ? 2 * KS : 1], vr1[NBUF == 2 ? NVT : 1];
     // issue order is the consumption order (the waits count loads still in flight)
     __builtin_amdgcn_sched_barrier(0);
     if (ROT) request_cs(wave);
     __builtin_amdgcn_sched_barrier(0);
     load_block(kr0, vr0, wave);
     __builtin_amdgcn_sched_barrier(0);
-    load_block(kr1, vr1, wave + NW);
-    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NBUF == 2) {
+      load_block(reinterpret_cast<uint4(&)[2 * KS]>(kr1), reinterpret_cast<uint4(&)[NVT]>(vr1), wave + NW);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     f32x4 O[NVT];
 #pragma unroll
     for (int vt = 0; vt < NVT; ++vt) O[vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -494,9 +499,9 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
         const u32x4 x = {vr[u].x, vr[u].y, vr[u].z, vr[u].w};
         *reinterpret_cast<NHA_LDS u32x4*>(X + (u * RV + lane / LV) * LDT + 8 * (lane % LV)) = x;
       }
-      // pin the refill here: right after its registers are free, two blocks ahead of its use
+      // pin the refill here: right after its registers are free, NBUF blocks ahead of its use
       __builtin_amdgcn_sched_barrier(0);
-      load_block(kr, vr, blk + 2 * NW);
+      load_block(kr, vr, blk + NBUF * NW);
       __builtin_amdgcn_sched_barrier(0);
       // S^T rows of this lane: keys 32*blk + 4*qd + r (S0) and + 16 (S1), head l16
       const int wb = 32 * blk + 4 * qd;
@@ -528,9 +533,13 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    for (int blk = wave; blk < nblk; blk += 2 * NW) {
-      process(kr0, vr0, blk);
-      process(kr1, vr1, blk + NW);   // past the end: a fully masked block, contributes nothing
+    if constexpr (NBUF == 2) {
+      for (int blk = wave; blk < nblk; blk += 2 * NW) {
+        process(kr0, vr0, blk);
+        process(reinterpret_cast<uint4(&)[2 * KS]>(kr1), reinterpret_cast<uint4(&)[NVT]>(vr1), blk + NW);   // past the end: a fully masked block, contributes nothing
+      }
+    } else {
+      for (int blk = wave; blk < nblk; blk += NW) process(kr0, vr0, blk);
     }
     lsum = sum_over_rows(lsum);
     if (qd == 0) {
@@ -582,7 +591,7 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
 
 template <int D, int G, bool ROT>
 int launch(const NhaDecodeArgs* a) {
-  constexpr int NW = NHA_DEC_NW;
+  constexpr int NW = D > 128 ? 4 : NHA_DEC_NW;
   const size_t lds = lds_bytes_for(D, G, NW, ROT);
   static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured && lds > 48 * 1024) {
@@ -611,7 +620,8 @@ int dispatch(const NhaDecodeArgs* a, int G) {
 }  // namespace
 
 bool decode_mfma_supported(const NhaDecodeArgs* a) {
-  if (a->dtype != NHA_DTYPE_BF16 || a->K != a->V || (a->K != 64 && a->K != 128)) return false;
+  if (a->dtype != NHA_DTYPE_BF16 || a->K != a->V || (a->K != 64 && a->K != 128 && a->K != 256)) return false;
+  if (a->K == 256 && a->cos) return false;   // the rotary tables of a block do not fit beside the V tiles at this head size
   if (a->mode != NHA_DECODE_WINDOW && a->mode != NHA_DECODE_RING) return false;
   // either a pre-rotated query, or (window mode) cos / sin tables whose rows are 16-byte aligned pieces
   const bool rot = a->cos != nullptr;
@@ -632,6 +642,7 @@ int decode_mfma_impl(const NhaDecodeArgs* a) {
   int G = 1;
   while (G < NG) G <<= 1;
   if (a->cos) return a->K == 64 ? dispatch<64, true>(a, G) : dispatch<128, true>(a, G);
+  if (a->K == 256) return dispatch<256, false>(a, G);
   return a->K == 64 ? dispatch<64, false>(a, G) : dispatch<128, false>(a, G);
 }
 

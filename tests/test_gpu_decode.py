@@ -99,6 +99,24 @@ def test_decode_long_window_streaming_kernel():
         assert_close("long-window hv", hvt, rhv, dtype)
 
 
+@pytest.mark.parametrize("NG,W,B", [(1, 512, 3), (1, 31, 2), (2, 100, 2), (8, 64, 1)])
+def test_decode_head_size_256(NG, W, B):
+    """Head size 256 (the 340M layers: one query head per kv-head) in the window form with a pre-rotated query:
+    served by the matrix-core kernel with one block of loads per wave and four waves per workgroup."""
+    from nha_amd import fused_recurrent_nha_decode
+    dtype, K, M = torch.bfloat16, 256, 64
+    d = decode_inputs(4100 + NG + W, B, 2, NG, K, K, M, W, dtype)
+    c = {k: v.cuda() for k, v in d.items()}
+    o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], s=c["s"], sw_k=c["sk"],
+                                               sw_v=c["vw"], initial_state=(c["hk0"].clone(), c["hv0"].clone()),
+                                               output_final_state=True)
+    ro, rhk, rhv, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sk"], d["vw"], sq=d["sq"], s=d["s"],
+                                      initial_state=(d["hk0"], d["hv0"]))
+    assert_close("d256 o", o, ro, dtype)
+    assert_close("d256 hk", hkt, rhk, dtype)
+    assert_close("d256 hv", hvt, rhv, dtype)
+
+
 def test_decode_state_aliasing_and_errors():
     from nha_amd import fused_recurrent_nha, fused_recurrent_nha_decode
     d = decode_inputs(7, 2, 2, 1, 64, 64, 16, 32, torch.bfloat16)
@@ -119,7 +137,7 @@ def test_decode_state_aliasing_and_errors():
 
 
 @pytest.mark.parametrize("NG,K,M,W", [(4, 128, 64, 48), (1, 64, 16, 8), (8, 64, 80, 33), (2, 64, 64, 300), (8, 128, 64, 130),
-                                      (1, 128, 64, 1)])
+                                      (1, 128, 64, 1), (1, 256, 64, 200), (4, 256, 64, 70), (8, 256, 64, 33)])
 def test_ring_decode_steps(NG, K, M, W):
     """Consecutive ring-buffer steps from random fill levels == the oracle's ring recurrence."""
     from nha_amd import NHARingState, ring_decode_step
