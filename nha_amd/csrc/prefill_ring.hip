@@ -550,8 +550,13 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     return __builtin_bit_cast(bf16x8, t);
   };
   float lg[RQB];
+  // No barrier holds the two waves of a SIMD together from here on, and the older one (w < 4) is served
+  // first: left alone it ends about 5 k cycles before the younger, which then has the SIMD to itself.  The
+  // younger wave gets the higher priority for the first of the two query blocks, so that both end together.
+  if (wave >= 4) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
+    if (qb == RQB - 1) __builtin_amdgcn_s_setprio(0);
     const int Q = qb0 + qb;                // sub-block index inside the chunk
     const int irow = 16 * Q + l16;         // this lane's query row inside the chunk
     // the window's own log-sum-exp, taken before the slots join: afterwards the window sum is only known
