@@ -457,8 +457,14 @@ def chunk_nha(
         if h0[0] is not None:
             h0 = (h0[0][keep], h0[1][keep])
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (*args, *h0)):
-        o, lse_swa, lse_gsa, hkt, hvt = _ChunkNHAFunction.apply(
-            *args, h0[0], h0[1], cu_host, window_size_left, gsa_kv_shift, scale, output_final_state, impl)
+        if impl is None:
+            # the registered operator (nha_amd/custom_ops.py): schema, fake-tensor shapes and autograd formula
+            o, lse_swa, lse_gsa, hkt, hvt = torch.ops.nha_amd.prefill_fwd(
+                *args, torch.from_numpy(np.ascontiguousarray(cu_host, dtype=np.int32)), int(window_size_left),
+                int(gsa_kv_shift), float(scale), h0[0], h0[1], bool(output_final_state))
+        else:
+            o, lse_swa, lse_gsa, hkt, hvt = _ChunkNHAFunction.apply(
+                *args, h0[0], h0[1], cu_host, window_size_left, gsa_kv_shift, scale, output_final_state, impl)
     else:
         o, lse_swa, lse_gsa, hkt, hvt = nha_prefill(
             *args, cu_host, wl=window_size_left, shift=gsa_kv_shift, scale=scale,
