@@ -546,7 +546,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--only", choices=["prefill", "decode", "glue", "layer"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_d256", "glue", "layer"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
     ap.add_argument("--backward", action="store_true",
                     help="with --workload: also time the backward of the prefill op")
@@ -580,7 +580,8 @@ def main():
     if args.only:
         res = (bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else
                bench_glue(torch, args.steps, args.warmup) if args.only == "glue" else
-               bench_layer(torch, args.steps, args.warmup) if args.only == "layer" else bench_decode(torch, args.warmup))
+               bench_layer(torch, args.steps, args.warmup) if args.only == "layer" else
+               bench_decode(torch, args.warmup, DECODE_D256) if args.only == "decode_d256" else bench_decode(torch, args.warmup))
         print(json.dumps(res))
         return
     pf = bench_prefill(torch, args.steps, args.warmup)
