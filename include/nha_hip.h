@@ -361,6 +361,49 @@ int nha_layer_prologue_bwd(const NhaLayerPrologueBwdArgs* a);
 int32_t nha_layer_epilogue_bwd_parts(int32_t rows);
 int nha_layer_epilogue_bwd(const NhaLayerEpilogueBwdArgs* a);
 
+/* Depthwise causal short convolution with optional SiLU over packed tokens: what the layer applies to its
+ * q / k / v projections when use_short_conv is set (nha_fla/layers/nha.py:121-140, :186-206; the module
+ * itself, fla.modules.ShortConvolution, is a dependency outside the reference tree):
+ *   y[t][c] = act(bias[c] + sum_{j < KS} weight[c][j] * x[t - (KS-1) + j][c])
+ * with the taps that would reach before the first token of t's sequence taken as zero.  x, y [T_tot, C];
+ * weight [C, KS] (the module's [C, 1, KS] parameter) and bias [C] (or NULL) in the dtype of x; cu_seqlens
+ * [N+1] on the device, or NULL for N sequences of T_tot / N tokens.  KS in {2, 3, 4}, C a multiple of 8,
+ * activation 0 (none) or 1 (SiLU).  fp32 arithmetic, rounded once.
+ *
+ * nha_short_conv_bwd: dx, and the weight / bias gradients as partial sums dweight_partial [parts, C, KS],
+ * dbias_partial [parts, C] fp32 with parts = nha_short_conv_bwd_parts(T_tot), which the caller adds up over
+ * the first axis (fixed order: run-to-run identical).  Either may be NULL. */
+typedef struct NhaShortConvArgs {
+  const void* x;
+  const void* weight;
+  const void* bias;
+  void* y;
+  const int32_t* cu_seqlens;
+  int32_t T_tot, N, C, KS;
+  int32_t activation;
+  int32_t dtype;
+  void* stream;
+} NhaShortConvArgs;
+
+typedef struct NhaShortConvBwdArgs {
+  const void* x;
+  const void* weight;
+  const void* bias;
+  const void* dy;
+  void* dx;
+  float* dweight_partial;
+  float* dbias_partial;
+  const int32_t* cu_seqlens;
+  int32_t T_tot, N, C, KS;
+  int32_t activation;
+  int32_t dtype;
+  void* stream;
+} NhaShortConvBwdArgs;
+
+int nha_short_conv(const NhaShortConvArgs* a);
+int32_t nha_short_conv_bwd_parts(int32_t T_tot);
+int nha_short_conv_bwd(const NhaShortConvBwdArgs* a);
+
 const char* nha_last_error(void);
 int nha_abi_version(void);
 

@@ -22,6 +22,7 @@ EXPORTS = (
     "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_fwd_noalloc", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
     "nha_decode_step", "nha_decode_advance", "nha_layer_prologue", "nha_layer_epilogue",
     "nha_layer_prologue_bwd", "nha_layer_epilogue_bwd", "nha_layer_epilogue_bwd_parts",
+    "nha_short_conv", "nha_short_conv_bwd", "nha_short_conv_bwd_parts",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
 )
 
@@ -121,6 +122,23 @@ class NhaLayerEpilogueBwdArgs(C.Structure):
     ]
 
 
+class NhaShortConvArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("weight", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("cu_seqlens", C.c_void_p),
+        ("T_tot", C.c_int32), ("N", C.c_int32), ("C", C.c_int32), ("KS", C.c_int32),
+        ("activation", C.c_int32), ("dtype", C.c_int32), ("stream", C.c_void_p),
+    ]
+
+
+class NhaShortConvBwdArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("weight", C.c_void_p), ("bias", C.c_void_p), ("dy", C.c_void_p), ("dx", C.c_void_p),
+        ("dweight_partial", C.c_void_p), ("dbias_partial", C.c_void_p), ("cu_seqlens", C.c_void_p),
+        ("T_tot", C.c_int32), ("N", C.c_int32), ("C", C.c_int32), ("KS", C.c_int32),
+        ("activation", C.c_int32), ("dtype", C.c_int32), ("stream", C.c_void_p),
+    ]
+
+
 class NhaError(RuntimeError):
     def __init__(self, code: int, msg: str):
         super().__init__(f"libnha_hip error {code}: {msg}")
@@ -163,6 +181,12 @@ def load() -> C.CDLL:
     lib.nha_layer_epilogue_bwd.argtypes = [C.POINTER(NhaLayerEpilogueBwdArgs)]
     lib.nha_layer_epilogue_bwd_parts.restype = C.c_int32
     lib.nha_layer_epilogue_bwd_parts.argtypes = [C.c_int32]
+    lib.nha_short_conv.restype = C.c_int
+    lib.nha_short_conv.argtypes = [C.POINTER(NhaShortConvArgs)]
+    lib.nha_short_conv_bwd.restype = C.c_int
+    lib.nha_short_conv_bwd.argtypes = [C.POINTER(NhaShortConvBwdArgs)]
+    lib.nha_short_conv_bwd_parts.restype = C.c_int32
+    lib.nha_short_conv_bwd_parts.argtypes = [C.c_int32]
     lib.nha_varlen_num_chunks.restype = C.c_int32
     lib.nha_varlen_num_chunks.argtypes = [C.c_void_p, C.c_int32, C.c_int32]
     lib.nha_varlen_indices.restype = C.c_int

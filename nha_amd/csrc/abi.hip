@@ -242,6 +242,41 @@ int nha_layer_epilogue_bwd(const NhaLayerEpilogueBwdArgs* a) {
   return layer_epilogue_bwd_impl(a);
 }
 
+static int check_short_conv(const char* who, const void* x, const void* w, int T_tot, int N, int C, int KS, int act, int dtype) {
+  NHA_CHECK_ARG(T_tot > 0 && N > 0 && C > 0, "%s: non-positive dimension", who);
+  NHA_CHECK_ARG(dtype == NHA_DTYPE_F32 || dtype == NHA_DTYPE_BF16, "%s: bad dtype %d", who, dtype);
+  NHA_CHECK_ARG(x && w, "%s: x and weight are required", who);
+  NHA_CHECK_ARG(act == 0 || act == 1, "%s: activation must be 0 (none) or 1 (SiLU), got %d", who, act);
+  if (KS < 2 || KS > 4 || C % 8 != 0) {
+    nha::set_error("%s: kernel size must be 2, 3 or 4 and C a multiple of 8 (got KS = %d, C = %d)", who, KS, C);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(x) & 15) == 0, "%s: tensors must be 16-byte aligned", who);
+  return NHA_OK;
+}
+
+int nha_short_conv(const NhaShortConvArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_short_conv: null args");
+  const int rc = check_short_conv("nha_short_conv", a->x, a->weight, a->T_tot, a->N, a->C, a->KS, a->activation, a->dtype);
+  if (rc != NHA_OK) return rc;
+  NHA_CHECK_ARG(a->y != nullptr && (reinterpret_cast<uintptr_t>(a->y) & 15) == 0, "nha_short_conv: y is required, 16-byte aligned");
+  NHA_CHECK_ARG(a->cu_seqlens || a->T_tot % a->N == 0, "nha_short_conv: T_tot must be a multiple of N without cu_seqlens");
+  return short_conv_impl(a);
+}
+
+int32_t nha_short_conv_bwd_parts(int32_t T_tot) { return T_tot > 0 ? short_conv_bwd_parts(T_tot) : 0; }
+
+int nha_short_conv_bwd(const NhaShortConvBwdArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_short_conv_bwd: null args");
+  const int rc = check_short_conv("nha_short_conv_bwd", a->x, a->weight, a->T_tot, a->N, a->C, a->KS, a->activation, a->dtype);
+  if (rc != NHA_OK) return rc;
+  NHA_CHECK_ARG(a->dy && a->dx, "nha_short_conv_bwd: dy and dx are required");
+  NHA_CHECK_ARG(((reinterpret_cast<uintptr_t>(a->dy) | reinterpret_cast<uintptr_t>(a->dx)) & 15) == 0,
+                "nha_short_conv_bwd: tensors must be 16-byte aligned");
+  NHA_CHECK_ARG(a->cu_seqlens || a->T_tot % a->N == 0, "nha_short_conv_bwd: T_tot must be a multiple of N without cu_seqlens");
+  return short_conv_bwd_impl(a);
+}
+
 int32_t nha_varlen_num_chunks(const int32_t* cu, int32_t N, int32_t BT) {
   if (!cu || N <= 0 || BT <= 0) {
     set_error("nha_varlen_num_chunks: bad arguments");

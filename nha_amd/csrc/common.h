@@ -132,6 +132,9 @@ int layer_epilogue_impl(const NhaLayerEpilogueArgs* a);
 int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a);
 int layer_epilogue_bwd_parts(int rows);
 int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a);
+int short_conv_impl(const NhaShortConvArgs* a);
+int short_conv_bwd_parts(int T_tot);
+int short_conv_bwd_impl(const NhaShortConvBwdArgs* a);
 int decode_step_impl(const NhaDecodeArgs* a);
 int decode_advance_impl(int32_t* count, int32_t B, void* stream);
 bool decode_mfma_supported(const NhaDecodeArgs* a);

@@ -503,6 +503,247 @@ int launch_epilogue(const EP& p, hipStream_t st) {
   return 0;
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Depthwise causal short convolution (+ SiLU) over packed tokens, the layer's use_short_conv option
+// (nha_fla/layers/nha.py:186-206):  y[t][c] = act(b[c] + sum_j w[c][j] x[t - (KS-1) + j][c]), taps that
+// would reach before the start of t's sequence are zero.  fp32 arithmetic, rounded once.
+// ------------------------------------------------------------------------------------------
+struct SC {
+  const void *x, *w, *b, *dy;
+  void *y, *dx;
+  float *dw_part, *db_part;
+  const int32_t* cu;
+  int T_tot, N, T, C, act;
+};
+
+constexpr int SC_RUN = 32;    // tokens a thread of the backward walks (one partial weight gradient per run)
+
+// the 8 x KS weights of 8 consecutive channels: contiguous in [C][KS], read as KS 8-element pieces
+template <typename T, int KS>
+__device__ __forceinline__ void load_taps(const T* w, int c, float (&wt)[KS][8]) {
+  float wv[8 * KS];
+#pragma unroll
+  for (int i = 0; i < KS; ++i) Elem<T>::ld8(w + (int64_t)c * KS + 8 * i, wv + 8 * i);
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int j = 0; j < KS; ++j) wt[j][e] = wv[e * KS + j];
+}
+
+// [bos, eos) of the sequence that holds token t0, and the index of the boundary after eos (varlen)
+__device__ __forceinline__ void seq_of(const SC& p, int t0, int& bos, int& eos, int& seq_next) {
+  seq_next = 0;
+  if (!p.cu) {
+    bos = (t0 / p.T) * p.T;
+    eos = bos + p.T;
+    return;
+  }
+  int lo = 0, hi = p.N - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu[mid] <= t0) lo = mid; else hi = mid - 1;
+  }
+  bos = p.cu[lo];
+  eos = p.cu[lo + 1];
+  seq_next = lo + 1;
+}
+
+constexpr int SCF_RUN = 16;   // tokens a thread of the forward walks
+constexpr int SC_GRP = 4;     // tokens whose rows are requested together
+
+// one thread: 8 channels of a run of SCF_RUN tokens, the last KS inputs in registers (every input row is
+// read once); the rows of SC_GRP tokens are requested together
+template <typename T, int KS>
+__global__ __launch_bounds__(256) void short_conv_kernel(const SC p) {
+  const int c8n = p.C / 8;
+  const int cg = blockIdx.y * 256 + threadIdx.x;
+  if (cg >= c8n) return;
+  const int c = cg * 8;
+  const int t0 = blockIdx.x * SCF_RUN;
+  const int t1 = (t0 + SCF_RUN) < p.T_tot ? (t0 + SCF_RUN) : p.T_tot;
+  const T* __restrict__ xp = (const T*)p.x;
+  T* __restrict__ yp = (T*)p.y;
+  float w[KS][8], bias[8];
+  load_taps<T, KS>((const T*)p.w, c, w);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bias[e] = p.b ? Elem<T>::ld((const T*)p.b + c + e) : 0.f;
+  float xh[KS][8];   // xh[d] = x[t - d]
+#pragma unroll
+  for (int d = 0; d < KS; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xh[d][e] = 0.f;
+#pragma unroll
+  for (int d = 1; d < KS; ++d)
+    if (t0 - d >= 0) Elem<T>::ld8(xp + (int64_t)(t0 - d) * p.C + c, xh[d - 1]);
+  int bos, eos, seq_next;
+  seq_of(p, t0, bos, eos, seq_next);
+  for (int tb = t0; tb < t1; tb += SC_GRP) {
+    float xin[SC_GRP][8];
+#pragma unroll
+    for (int i = 0; i < SC_GRP; ++i)
+      if (tb + i < t1) Elem<T>::ld8(xp + (int64_t)(tb + i) * p.C + c, xin[i]);
+#pragma unroll
+    for (int i = 0; i < SC_GRP; ++i) {
+      const int t = tb + i;
+      if (t >= t1) break;
+      while (t >= eos) {   // the walk enters the next sequence
+        bos = eos;
+        if (p.cu) { ++seq_next; eos = p.cu[seq_next]; } else eos = bos + p.T;
+      }
+#pragma unroll
+      for (int d = KS - 1; d >= 1; --d)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xh[d][e] = xh[d - 1][e];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xh[0][e] = xin[i][e];
+      const int reach = t - bos;   // taps d <= reach lie inside the sequence
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float pre = bias[e];
+#pragma unroll
+        for (int d = 0; d < KS; ++d)
+          if (d <= reach) pre += w[KS - 1 - d][e] * xh[d][e];
+        acc[e] = p.act ? silu_f(pre) : pre;
+      }
+      Elem<T>::st8(yp + (int64_t)t * p.C + c, acc);
+    }
+  }
+}
+
+// one thread: 8 channels of a run of SC_RUN tokens, walked in order with the last KS inputs and the KS
+// unfinished input gradients in registers; the KS - 1 tokens after the run are walked too (their
+// pre-activation gradients reach back into the run).  Weight / bias gradients of the run leave as one
+// partial sum per run: [runs][C][KS] and [runs][C], added up by the caller in a fixed order.
+template <typename T, int KS>
+__global__ __launch_bounds__(256) void short_conv_bwd_kernel(const SC p) {
+  const int c8n = p.C / 8;
+  const int run = blockIdx.x;
+  const int cg = blockIdx.y * 256 + threadIdx.x;
+  if (cg >= c8n) return;
+  const int c = cg * 8;
+  const int t0 = run * SC_RUN;
+  const int t1 = (t0 + SC_RUN) < p.T_tot ? (t0 + SC_RUN) : p.T_tot;            // end of the run
+  const int t2 = (t1 + KS - 1) < p.T_tot ? (t1 + KS - 1) : p.T_tot;            // end of the walk
+  const T* __restrict__ xp = (const T*)p.x;
+  const T* __restrict__ dyp = (const T*)p.dy;
+  T* __restrict__ dxp = (T*)p.dx;
+  float w[KS][8], bias[8];
+  load_taps<T, KS>((const T*)p.w, c, w);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bias[e] = p.b ? Elem<T>::ld((const T*)p.b + c + e) : 0.f;
+  float xh[KS][8], dxr[KS][8], dw[KS][8], db[8];   // xh[d] = x[t - d], dxr[d] = unfinished dx[t - d]
+#pragma unroll
+  for (int d = 0; d < KS; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xh[d][e] = dxr[d][e] = dw[d][e] = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) db[e] = 0.f;
+  // inputs before the run (the walk shifts them into place)
+#pragma unroll
+  for (int d = 1; d < KS; ++d)
+    if (t0 - d >= 0) Elem<T>::ld8(xp + (int64_t)(t0 - d) * p.C + c, xh[d - 1]);
+  int bos, eos, seq_next;
+  seq_of(p, t0, bos, eos, seq_next);
+  for (int tb = t0; tb < t2; tb += SC_GRP) {
+    float xin[SC_GRP][8], dyin[SC_GRP][8];
+#pragma unroll
+    for (int i = 0; i < SC_GRP; ++i)
+      if (tb + i < t2) {
+        Elem<T>::ld8(xp + (int64_t)(tb + i) * p.C + c, xin[i]);
+        Elem<T>::ld8(dyp + (int64_t)(tb + i) * p.C + c, dyin[i]);
+      }
+#pragma unroll
+    for (int i = 0; i < SC_GRP; ++i) {
+      const int t = tb + i;
+      if (t >= t2) break;
+      while (t >= eos) {   // the walk enters the next sequence
+        bos = eos;
+        if (p.cu) { ++seq_next; eos = p.cu[seq_next]; } else eos = bos + p.T;
+      }
+      // shift the histories: slot d now belongs to token t - d
+#pragma unroll
+      for (int d = KS - 1; d >= 1; --d)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xh[d][e] = xh[d - 1][e];
+          dxr[d][e] = dxr[d - 1][e];
+        }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xh[0][e] = xin[i][e];
+        dxr[0][e] = 0.f;
+      }
+      const int reach = t - bos;   // taps d <= reach lie inside the sequence
+      float dpre[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float pre = bias[e];
+#pragma unroll
+        for (int d = 0; d < KS; ++d)
+          if (d <= reach) pre += w[KS - 1 - d][e] * xh[d][e];
+        float g = dyin[i][e];
+        if (p.act) {
+          const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-pre));
+          g *= sg * (1.f + pre * (1.f - sg));
+        }
+        dpre[e] = g;
+      }
+      const bool own = t < t1;
+#pragma unroll
+      for (int d = 0; d < KS; ++d) {
+        if (d > reach) continue;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          dxr[d][e] += w[KS - 1 - d][e] * dpre[e];
+          if (own) dw[KS - 1 - d][e] += dpre[e] * xh[d][e];
+        }
+      }
+      if (own) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) db[e] += dpre[e];
+      }
+      // token t - (KS-1) has received its last contribution
+      const int u = t - (KS - 1);
+      if (u >= t0 && u < t1) Elem<T>::st8(dxp + (int64_t)u * p.C + c, dxr[KS - 1]);
+    }
+  }
+  // tokens of the run that the walk could not finish (the tensor ends before their last tap)
+#pragma unroll
+  for (int d = 0; d < KS - 1; ++d) {
+    const int u = t2 - 1 - d;
+    if (u >= t0 && u < t1) Elem<T>::st8(dxp + (int64_t)u * p.C + c, dxr[d]);
+  }
+  if (p.dw_part) {
+    float wv[8 * KS];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+#pragma unroll
+      for (int j = 0; j < KS; ++j) wv[e * KS + j] = dw[j][e];
+#pragma unroll
+    for (int i = 0; i < KS; ++i) Elem<float>::st8(p.dw_part + ((int64_t)run * p.C + c) * KS + 8 * i, wv + 8 * i);
+  }
+  if (p.db_part) Elem<float>::st8(p.db_part + (int64_t)run * p.C + c, db);
+}
+
+template <typename T>
+int launch_short_conv(const SC& p, int KS, bool bwd, hipStream_t st) {
+  const int c8n = p.C / 8;
+  if (!bwd) {
+    const dim3 grid((p.T_tot + SCF_RUN - 1) / SCF_RUN, (c8n + 255) / 256);
+    if (KS == 2) hipLaunchKernelGGL((short_conv_kernel<T, 2>), grid, dim3(256), 0, st, p);
+    else if (KS == 3) hipLaunchKernelGGL((short_conv_kernel<T, 3>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((short_conv_kernel<T, 4>), grid, dim3(256), 0, st, p);
+  } else {
+    const dim3 grid((p.T_tot + SC_RUN - 1) / SC_RUN, (c8n + 255) / 256);
+    if (KS == 2) hipLaunchKernelGGL((short_conv_bwd_kernel<T, 2>), grid, dim3(256), 0, st, p);
+    else if (KS == 3) hipLaunchKernelGGL((short_conv_bwd_kernel<T, 3>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((short_conv_bwd_kernel<T, 4>), grid, dim3(256), 0, st, p);
+  }
+  return 0;
+}
+
 }  // namespace
 
 int layer_prologue_impl(const NhaLayerPrologueArgs* a) {
@@ -555,6 +796,40 @@ int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a) {
 }
 
 int layer_epilogue_bwd_parts(int rows) { return (rows + BWD_ROWS - 1) / BWD_ROWS; }
+
+int short_conv_bwd_parts(int T_tot) { return (T_tot + SC_RUN - 1) / SC_RUN; }
+
+int short_conv_impl(const NhaShortConvArgs* a) {
+  SC p = {};
+  p.x = a->x; p.w = a->weight; p.b = a->bias; p.y = a->y; p.cu = a->cu_seqlens;
+  p.T_tot = a->T_tot; p.N = a->N; p.T = a->T_tot / a->N; p.C = a->C; p.act = a->activation;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->dtype == NHA_DTYPE_BF16) launch_short_conv<bf16_t>(p, a->KS, false, st);
+  else launch_short_conv<float>(p, a->KS, false, st);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("nha_short_conv: launch failed: %s", hipGetErrorString(e));
+    return NHA_ERR_LAUNCH;
+  }
+  return NHA_OK;
+}
+
+int short_conv_bwd_impl(const NhaShortConvBwdArgs* a) {
+  SC p = {};
+  p.x = a->x; p.w = a->weight; p.b = a->bias; p.dy = a->dy; p.dx = a->dx;
+  p.dw_part = a->dweight_partial; p.db_part = a->dbias_partial; p.cu = a->cu_seqlens;
+  p.T_tot = a->T_tot; p.N = a->N; p.T = a->T_tot / a->N; p.C = a->C; p.act = a->activation;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->dtype == NHA_DTYPE_BF16) launch_short_conv<bf16_t>(p, a->KS, true, st);
+  else launch_short_conv<float>(p, a->KS, true, st);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("nha_short_conv_bwd: launch failed: %s", hipGetErrorString(e));
+    return NHA_ERR_LAUNCH;
+  }
+  return NHA_OK;
+}
+
 
 int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a) {
   if (a->dim % 8 != 0 || a->dim > 8192) {

@@ -21,6 +21,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops as _ops
 from .ops import chunk_nha, nha_layer_epilogue, nha_layer_prologue
 
 
@@ -110,8 +111,16 @@ class ShortConvolution(nn.Module):
         self.weight = nn.Parameter(torch.empty(hidden_size, 1, kernel_size).uniform_(-kernel_size ** -0.5, kernel_size ** -0.5))
         self.bias = nn.Parameter(torch.zeros(hidden_size)) if bias else None
 
+    def _final_state(self, x, cu_seqlens):
+        return _short_conv_final_state(x, cu_seqlens, self.kernel_size)
+
     def forward(self, x, cache=None, output_final_state=False, cu_seqlens=None):
         B, T, Dm = x.shape
+        if cache is None and _ops.short_conv_supported(x, self.weight):
+            # a fresh sequence on the GPU: one HIP launch (taps, sequence restarts and SiLU fused)
+            y = _ops.nha_short_conv(x, self.weight, self.bias, cu_seqlens=cu_seqlens,
+                                    activation=self.activation if self.activation in ("silu", "swish") else None)
+            return y, (self._final_state(x, cu_seqlens) if output_final_state else None)
         xs = x.transpose(1, 2)
         if cache is not None:
             xs = torch.cat([cache.to(xs.dtype), xs], dim=-1)
@@ -148,6 +157,20 @@ class ShortConvolution(nn.Module):
         if self.activation in ("silu", "swish"):
             y = F.silu(y)
         return y.transpose(1, 2), final
+
+
+def _short_conv_final_state(x, cu_seqlens, kernel_size):
+    """The last kernel_size - 1 inputs of every sequence as [N, C, kernel_size - 1], zeros where it is shorter."""
+    B, T, Dm = x.shape
+    if cu_seqlens is None:
+        xs = F.pad(x.transpose(1, 2), (kernel_size - 1, 0))
+        return xs[..., -(kernel_size - 1):].contiguous()
+    cu = cu_seqlens.to(x.device).long()
+    back = torch.arange(kernel_size - 1, 0, -1, device=x.device)
+    idx = cu[1:, None] - back[None, :]
+    ok = idx >= cu[:-1, None]
+    gathered = x[0][idx.clamp(min=0)]
+    return (gathered * ok[..., None].to(x.dtype)).transpose(1, 2).contiguous()
 
 
 def get_unpad_data(attention_mask: torch.Tensor):

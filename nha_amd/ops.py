@@ -350,6 +350,74 @@ def nha_layer_epilogue(o, weight: Optional[torch.Tensor], bias: Optional[torch.T
     return _epilogue_fwd(o, w, b, float(eps))
 
 
+def _short_conv_args(x, cu):
+    T_tot = x.shape[0] * x.shape[1]
+    N = (cu.numel() - 1) if cu is not None else x.shape[0]
+    return T_tot, N
+
+
+class _ShortConvFunction(torch.autograd.Function):
+    """Autograd node of the short convolution: one launch per direction; the weight / bias gradients are
+    reduced from the kernel's per-run partial sums in a fixed order."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, cu, act):
+        lib = _lib.load()
+        Cn, KS = weight.shape[0], weight.shape[-1]
+        w = weight.detach().to(x.dtype).reshape(Cn, KS).contiguous()
+        b = None if bias is None else bias.detach().to(x.dtype).contiguous()
+        T_tot, N = _short_conv_args(x, cu)
+        y = torch.empty_like(x)
+        a = _lib.NhaShortConvArgs(x=_ptr(x), weight=_ptr(w), bias=_ptr(b), y=_ptr(y), cu_seqlens=_ptr(cu), T_tot=T_tot, N=N,
+                                  C=Cn, KS=KS, activation=int(act), dtype=_dtype_code(x), stream=_stream(x.device))
+        _lib.check(lib.nha_short_conv(C.byref(a)))
+        ctx.save_for_backward(x, w, b, cu)
+        ctx.act = int(act)
+        ctx.wb = (weight.dtype, weight.shape, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        x, w, b, cu = ctx.saved_tensors
+        dy = dy.contiguous()
+        Cn, KS = w.shape
+        T_tot, N = _short_conv_args(x, cu)
+        parts = lib.nha_short_conv_bwd_parts(T_tot)
+        wdt, wshape, bdt = ctx.wb
+        need_w = ctx.needs_input_grad[1]
+        need_b = bdt is not None and ctx.needs_input_grad[2]
+        dwp = torch.empty(parts, Cn, KS, dtype=torch.float32, device=x.device) if need_w else None
+        dbp = torch.empty(parts, Cn, dtype=torch.float32, device=x.device) if need_b else None
+        dx = torch.empty_like(x)
+        a = _lib.NhaShortConvBwdArgs(x=_ptr(x), weight=_ptr(w), bias=_ptr(b), dy=_ptr(dy), dx=_ptr(dx), dweight_partial=_ptr(dwp),
+                                     dbias_partial=_ptr(dbp), cu_seqlens=_ptr(cu), T_tot=T_tot, N=N, C=Cn, KS=KS,
+                                     activation=ctx.act, dtype=_dtype_code(x), stream=_stream(x.device))
+        _lib.check(lib.nha_short_conv_bwd(C.byref(a)))
+        return (dx, dwp.sum(0).to(wdt).reshape(wshape) if need_w else None, dbp.sum(0).to(bdt) if need_b else None, None, None)
+
+
+def short_conv_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether nha_short_conv serves this call: GPU tensors in bf16 / fp32, 2 to 4 taps, channels a multiple of 8."""
+    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float32) and 2 <= weight.shape[-1] <= 4
+            and weight.shape[0] % 8 == 0)
+
+
+def nha_short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], *,
+                   cu_seqlens: Optional[torch.Tensor] = None, activation: Optional[str] = "silu") -> torch.Tensor:
+    """Depthwise causal convolution over ``x [B, T, C]`` with ``weight [C, 1, KS]`` (+ ``bias [C]``) and optional
+    SiLU in one launch, restarting at ``cu_seqlens`` boundaries (then ``B == 1``): what the layer's
+    ``ShortConvolution`` modules compute on a fresh sequence (nha_fla/layers/nha.py:186-206).  Differentiable with
+    respect to x, weight and bias."""
+    _need_cuda(x, weight, bias)
+    if activation not in (None, "silu", "swish"):
+        raise ValueError(f"activation must be None, 'silu' or 'swish', got {activation!r}")
+    if cu_seqlens is not None and x.shape[0] != 1:
+        raise ValueError("cu_seqlens needs the packed layout [1, T_tot, C]")
+    cu = None if cu_seqlens is None else cu_seqlens.to(device=x.device, dtype=torch.int32).contiguous()
+    return _ShortConvFunction.apply(x.contiguous(), weight, bias, cu, 0 if activation is None else 1)
+
+
 class _ChunkNHAFunction(torch.autograd.Function):
     """Autograd node of chunk_nha on packed tensors: same outputs and gradient set as
     ChunkNativeHybridAttentionFunction (nha_fla/ops/nha/chunk.py:364-564)."""

@@ -40,10 +40,15 @@ def test_struct_sizes_match_the_header(tmp_path):
                                                         "feature_map", "dtype", "gate_logit_normalizer", "stream")]
     probes += [("NhaLayerEpilogueBwdArgs", f) for f in ("o", "dy", "dout", "weight", "dweight_partial", "dbias_partial",
                                                         "rows", "dim", "dtype", "eps", "stream")]
+    probes += [("NhaShortConvArgs", f) for f in ("x", "weight", "bias", "y", "cu_seqlens", "T_tot", "KS", "activation", "dtype",
+                                                 "stream")]
+    probes += [("NhaShortConvBwdArgs", f) for f in ("x", "dy", "dx", "dweight_partial", "dbias_partial", "cu_seqlens", "T_tot",
+                                                    "KS", "activation", "dtype", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
            'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));',
            'printf("%zu %zu\\n", sizeof(NhaLayerPrologueArgs), sizeof(NhaLayerEpilogueArgs));',
-           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueBwdArgs), sizeof(NhaLayerEpilogueBwdArgs));']
+           'printf("%zu %zu\\n", sizeof(NhaLayerPrologueBwdArgs), sizeof(NhaLayerEpilogueBwdArgs));',
+           'printf("%zu %zu\\n", sizeof(NhaShortConvArgs), sizeof(NhaShortConvBwdArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
     src += ['return 0; }']
     cfile = tmp_path / "probe.c"
@@ -55,7 +60,8 @@ def test_struct_sizes_match_the_header(tmp_path):
     assert int(out[2]) == C.sizeof(_lib.NhaPrefillBwdArgs)
     assert int(out[3]) == C.sizeof(_lib.NhaLayerPrologueArgs) and int(out[4]) == C.sizeof(_lib.NhaLayerEpilogueArgs)
     assert int(out[5]) == C.sizeof(_lib.NhaLayerPrologueBwdArgs) and int(out[6]) == C.sizeof(_lib.NhaLayerEpilogueBwdArgs)
-    for (t, f), off in zip(probes, out[7:]):
+    assert int(out[7]) == C.sizeof(_lib.NhaShortConvArgs) and int(out[8]) == C.sizeof(_lib.NhaShortConvBwdArgs)
+    for (t, f), off in zip(probes, out[9:]):
         assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 
@@ -95,6 +101,14 @@ def test_argument_validation_without_gpu():
     leb.rows, leb.dim = 4, 64
     assert lib.nha_layer_epilogue_bwd(C.byref(leb)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
     assert lib.nha_layer_epilogue_bwd_parts(0) == 0 and lib.nha_layer_epilogue_bwd_parts(33) == 2
+    sc = _lib.NhaShortConvArgs()
+    assert lib.nha_short_conv(C.byref(sc)) == _lib.NHA_ERR_INVALID and b"non-positive" in lib.nha_last_error()
+    sc.T_tot, sc.N, sc.C, sc.KS = 16, 1, 64, 4
+    assert lib.nha_short_conv(C.byref(sc)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    scb = _lib.NhaShortConvBwdArgs()
+    scb.T_tot, scb.N, scb.C, scb.KS = 16, 1, 60, 4
+    assert lib.nha_short_conv_bwd(C.byref(scb)) == _lib.NHA_ERR_INVALID and b"required" in lib.nha_last_error()
+    assert lib.nha_short_conv_bwd_parts(0) == 0 and lib.nha_short_conv_bwd_parts(33) == 2
     with pytest.raises(_lib.NhaError):
         chunk_tables([0, 5, 5])          # zero-length sequence
     with pytest.raises(_lib.NhaError):
