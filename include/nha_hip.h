@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 6
+#define NHA_ABI_VERSION 7
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {

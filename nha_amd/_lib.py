@@ -14,7 +14,7 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 6
+ABI_VERSION = 7
 NHA_NOALLOC_SCRATCH_BYTES = 32 << 20   # workspace of nha_prefill_fwd_noalloc (include/nha_hip.h)
 NHA_FMAP_NONE, NHA_FMAP_SWISH, NHA_FMAP_RELU = 0, 1, 2
 
