@@ -1059,8 +1059,8 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   }
   hipLaunchKernelGGL(bwd_state_scan_kernel, dim3(a->N * a->H, ((K + V) * M + 255) / 256), dim3(256), 0, st, p);
   if (sp.use_mfma) {
-    // one partial-ds slab per state instead of one per 32-column block
-    p.nbk = p.nbv = 1;
+    // one partial-ds slab per state and column range of a workgroup instead of one per 32-column block
+    p.nbk = p.nbv = bwd_slot_inter_slabs(a);
     rc = bwd_slot_products2(a, 2, sc + sp.hkb, p.dus, p.pp, p.ck, p.cv, p.gc, p.ek, p.ev, p.dks, p.dvs, p.dsp);
     if (rc != NHA_OK) return rc;
   } else {

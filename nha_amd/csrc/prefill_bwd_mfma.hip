@@ -408,7 +408,7 @@ struct SP1 {
 // ------------------------------------------------------------------------------------------
 // Slot branch, products over the rows of a chunk (bf16 operands, fp32 accumulation).
 //
-// bwd_slot_state_kernel, grid (H, NT, 2): per (chunk, kv-head) and state (z = 0: k-state with
+// bwd_slot_state_kernel, grid (H, NT, 2 D / DW): per (chunk, kv-head), state and column range (z even: k-state with
 // X = q_gsa, weights scale*du, matrix ck; z = 1: v-state with X = do, weights p, matrix cv), summed
 // over the q-heads of the group:
 //   N[x][m]  = sum_i X_i[x] w_i[m] e^(gc_i[m])        inhomogeneous term of the state-gradient recurrence
@@ -429,7 +429,7 @@ struct SP2 {
   const float* gc;                   // [T][H][64]
   float *ek, *ev;                    // [NT][H][D][64] x2
   float *dks, *dvs;                  // [T][H][D] x2 (source-token index)
-  float* dsp;                        // [2][T][H][64] inter-chunk part of ds per state
+  float* dsp;                        // [2 * slabs][T][H][64] inter-chunk part of ds per state and column range
   const bf16_t* v;                   // [T,H,D]
   bf16_t* dkg;                       // dk_gsa [T,H,D]
   int T_tot;
@@ -468,11 +468,12 @@ __device__ __forceinline__ void split4_bf16(const float4 x, lbf16* hi, lbf16* lo
   *reinterpret_cast<NHA_LDS bf16x4*>(lo + idx) = l;
 }
 
-template <int D>
+// DW: the columns x a workgroup takes (blockIdx.z / 2 picks them); launched with DW = D
+template <int D, int DW>
 __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
-  constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
+  constexpr int DB = DW / 16, LDT = DW + 16, TILE = BT * LDT;
   extern __shared__ __align__(16) unsigned char smem[];
-  lbf16* const Xt = (lbf16*)smem;        // [64 rows i][D]
+  lbf16* const Xt = (lbf16*)smem;        // [64 rows i][DW]
   lbf16* const Wt = Xt + TILE;           // [64 m][TLD]  (w_i[m] e^(gc_i[m]))^T, high part
   lbf16* const Wl = Wt + BT * TLD;       //              low part
   lbf16* const Ct = Wl + BT * TLD;       // [64 r][TLD]  c[i][r]^T, zero for i < r, high part
@@ -481,7 +482,8 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
   const int h = blockIdx.x, chunk = blockIdx.y;
-  const bool isv = blockIdx.z != 0;
+  const bool isv = (blockIdx.z & 1) != 0;
+  const int x0 = (blockIdx.z >> 1) * DW;   // this workgroup's columns
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
@@ -500,11 +502,11 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   // issued before the first use); at head sizes up to 128 those of the next head are requested before the
   // products of this one, so that only the first head of a workgroup waits out a memory latency.
   constexpr int NS = BT * BT / 4 / 256;
-  constexpr bool AHEAD = D <= 128;
-  Tile<BT, D> rx;
+  constexpr bool AHEAD = DW <= 128;
+  Tile<BT, DW> rx;
   float4 wv[NS], gv[NS], cv[NS];
   auto load_head = [&](int hq) {
-    rx.load(xsrc + (int64_t)hq * D, (int64_t)HQ * D, c0, R, tid);
+    rx.load(xsrc + (int64_t)hq * D + x0, (int64_t)HQ * D, c0, R, tid);
     const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
@@ -553,10 +555,10 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
     }
   }
   // N[x = 16 db + 4 kb + r][m = col];  out^T[x][row = col]
-  float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
+  float* ep = (isv ? p.ev : p.ek) + (((int64_t)chunk * H + h) * D + x0) * BT;
   const int tl = it * BT + col - p.shift;
   const bool has = col < R && tl >= 0;
-  float* op = (isv ? p.dvs : p.dks) + (((int64_t)bos + (has ? tl : 0)) * H + h) * D;
+  float* op = (isv ? p.dvs : p.dks) + (((int64_t)bos + (has ? tl : 0)) * H + h) * D + x0;
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
 #pragma unroll
@@ -658,25 +660,29 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   }
 }
 
-// bwd_slot_inter_kernel, grid (H, NT, 2): the parts that involve E_c, the state gradient carried
-// into the END of chunk c (z = 0: k-state, rows k', output dk_gsa; z = 1: v-state, rows v', output
+// bwd_slot_inter_kernel, grid (H, NT, 2 D / DW): the parts that involve E_c, the state gradient carried
+// into the END of chunk c (z even: k-state, rows k', output dk_gsa; z odd: v-state, rows v', output
 // dvs), with dec_r[m] = e^(gl[m] - gc_r[m]):
 //   out[r][x] = intra part + sum_m (s_r[m] dec_r[m]) E[x][m]         as out^T = E sE^T
 //   dsp[r][m] = dec_r[m] sum_x y_r[x] E[x][m]                         as Y E
-template <int D>
+// A workgroup takes DW of the D columns x (z / 2 picks them): at head size 256 two workgroups of half the
+// columns fit a CU where one of all columns does not, and each writes its own partial of dsp (one slab per
+// state and column range; the gate kernel adds the slabs).
+template <int D, int DW>
 __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
-  constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT, ELD = BT + 8;
+  constexpr int DB = DW / 16, LDT = DW + 16, TILE = BT * LDT, ELD = BT + 8, NH = D / DW;
   extern __shared__ __align__(16) unsigned char smem[];
-  lbf16* const Yt = (lbf16*)smem;        // [64 rows r][D]   k' / v'
-  lbf16* const Et = Yt + TILE;           // [D x][ELD]       E[x][m], high part
-  lbf16* const El = Et + D * ELD;        //                  low part
-  lbf16* const St = El + D * ELD;        // [64 r][TLD]      s_r[m] dec_r[m], high part
+  lbf16* const Yt = (lbf16*)smem;        // [64 rows r][DW]  k' / v'
+  lbf16* const Et = Yt + TILE;           // [DW x][ELD]      E[x][m], high part
+  lbf16* const El = Et + DW * ELD;       //                  low part
+  lbf16* const St = El + DW * ELD;        // [64 r][TLD]      s_r[m] dec_r[m], high part
   lbf16* const Sl = St + BT * TLD;       //                  low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
   const int h = blockIdx.x, chunk = blockIdx.y;
-  const bool isv = blockIdx.z != 0;
+  const bool isv = (blockIdx.z & 1) != 0;
+  const int xh = blockIdx.z >> 1, x0 = xh * DW;   // this workgroup's columns
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
@@ -684,21 +690,21 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   const bf16_t* ysrc = isv ? p.v : p.kg;
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
-  Tile<BT, D> ry;
+  Tile<BT, DW> ry;
 #pragma unroll
-  for (int u = 0; u < Tile<BT, D>::NPC; ++u) {
+  for (int u = 0; u < Tile<BT, DW>::NPC; ++u) {
     const int c = tid + 256 * u;
-    const int row = c / (D / 8), cc = (c % (D / 8)) * 8;
+    const int row = c / (DW / 8), cc = (c % (DW / 8)) * 8;
     uint4 x = make_uint4(0, 0, 0, 0);
-    if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(ysrc + (((int64_t)c0 + row - p.shift) * H + h) * D + cc);
+    if (row >= vlo && row < R) x = *reinterpret_cast<const uint4*>(ysrc + (((int64_t)c0 + row - p.shift) * H + h) * D + x0 + cc);
     ry.r[u] = x;
   }
-  const float* ep = (isv ? p.ev : p.ek) + ((int64_t)chunk * H + h) * D * BT;
+  const float* ep = (isv ? p.ev : p.ek) + (((int64_t)chunk * H + h) * D + x0) * BT;
   const float* gcb = p.gc + ((int64_t)c0 * H + h) * BT;
   {
     // all global loads of a batch are issued before the first conversion waits for one; the first batch
     // of E and the gate rows are requested before the Y tile is stored
-    constexpr int NE = D * BT / 4 / 256, EB = NE < 8 ? NE : 8;
+    constexpr int NE = DW * BT / 4 / 256, EB = NE < 8 ? NE : 8;
     const float4* ep4 = reinterpret_cast<const float4*>(ep);
     constexpr int NS = BT * BT / 4 / 256;
     float4 gl[NS], gr[NS];
@@ -756,9 +762,9 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   // the partial sums the first products are added to: requested before the products where the registers
   // allow (head sizes up to 128)
   const bool has = col >= vlo && col < R;
-  const int64_t oi = (((int64_t)c0 + col - p.shift) * H + h) * D;
+  const int64_t oi = (((int64_t)c0 + col - p.shift) * H + h) * D + x0;
   const float* const part = isv ? p.dvs : p.dks;
-  constexpr bool EARLY = D <= 128;
+  constexpr bool EARLY = DW <= 128;
   float4 pve[EARLY ? DB : 1];
   if (EARLY && has) {
 #pragma unroll
@@ -797,7 +803,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
   for (int rb = 0; rb < 4; ++rb) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int xs = 0; xs < D / 32; ++xs) {
+    for (int xs = 0; xs < DW / 32; ++xs) {
       struct { bf16x4 a, b; } t;
       t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 4 * kb);
       t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(Yt + (16 * rb + l16) * LDT + 32 * xs + 16 + 4 * kb);
@@ -811,7 +817,7 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
       const int r = 16 * rb + 4 * kb + q;
       if (r < R) {
         const float dec = __expf(glast - grow[rb][q]);
-        p.dsp[(((int64_t)(isv ? 1 : 0) * p.T_tot + c0 + r) * H + h) * BT + col] = acc[q] * dec;
+        p.dsp[(((int64_t)((isv ? NH : 0) + xh) * p.T_tot + c0 + r) * H + h) * BT + col] = acc[q] * dec;
       }
     }
   }
@@ -1444,14 +1450,17 @@ int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* h
 
 template <int D>
 static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
+  // (the state kernel takes all columns in one workgroup: split in two at head size 256 it stages its tables twice
+  // and was measured slower, 110 against 103 us)
   const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
   const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
-  const size_t lds_i = (size_t)BT * (D + 16) * 2 + (size_t)2 * D * (BT + 8) * 2 + (size_t)2 * BT * TLD * 2;
+  constexpr int DWI = D > 128 ? 128 : D;   // columns per workgroup of the inter kernel
+  const size_t lds_i = (size_t)BT * (DWI + 16) * 2 + (size_t)2 * DWI * (BT + 8) * 2 + (size_t)2 * BT * TLD * 2;
   static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
   if (!configured) {
-    hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
+    hipError_t e1 = hipFuncSetAttribute((const void*)bwd_slot_state_kernel<D, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
     hipError_t e2 = hipFuncSetAttribute((const void*)bwd_slot_dq_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_q);
-    hipError_t e3 = hipFuncSetAttribute((const void*)bwd_slot_inter_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_i);
+    hipError_t e3 = hipFuncSetAttribute((const void*)bwd_slot_inter_kernel<D, DWI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_i);
     if (e1 == hipSuccess) e1 = e3;
     if (e1 != hipSuccess || e2 != hipSuccess) {
       set_error("nha_prefill_bwd: cannot reserve LDS: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
@@ -1459,8 +1468,8 @@ static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
     }
     configured = true;
   }
-  if (which == 1) hipLaunchKernelGGL((bwd_slot_state_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_s, st, p);
-  else if (which == 2) hipLaunchKernelGGL((bwd_slot_inter_kernel<D>), dim3(p.H, NT, 2), dim3(256), lds_i, st, p);
+  if (which == 1) hipLaunchKernelGGL((bwd_slot_state_kernel<D, D>), dim3(p.H, NT, 2), dim3(256), lds_s, st, p);
+  else if (which == 2) hipLaunchKernelGGL((bwd_slot_inter_kernel<D, DWI>), dim3(p.H, NT, 2 * (D / DWI)), dim3(256), lds_i, st, p);
   else hipLaunchKernelGGL((bwd_slot_dq_kernel<D>), dim3(p.HQ, NT), dim3(256), lds_q, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(slot products, second stage)");
   return NHA_OK;
@@ -1469,6 +1478,9 @@ static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
 // which = 0: dq_gsa (bwd_slot_dq_kernel); 1: N_c and the intra-chunk parts of dk' / dv'
 // (bwd_slot_state_kernel); 2: the parts that involve the scanned E_c (bwd_slot_inter_kernel).
 // Same shapes as bwd_slot_products.
+// partial-ds slabs per state that bwd_slot_inter_kernel writes: one per column range of a workgroup
+int bwd_slot_inter_slabs(const NhaPrefillBwdArgs* a) { return a->K > 128 ? a->K / 128 : 1; }
+
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
                        const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs,
                        float* dsp) {
