@@ -1088,35 +1088,60 @@ __global__ __launch_bounds__(256) void export_states_kernel(const MP p, float* g
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   const int64_t cg = (int64_t)chunk * H + h;
   const int64_t sl = (int64_t)seg_slot(p.coff, n, it) * H + h;
-  for (int e = tid; e < MS * D; e += 256) {
-    const int m = e / D, d = e % D;
+  // eight consecutive d of one slot per thread and trip: 16-byte reads of the bf16 local states, 32-byte
+  // reads of the fp32 segment states, 16-byte writes of the four bf16 copies
+  for (int e8 = tid; e8 < MS * D / 8; e8 += 256) {
+    const int m = e8 / (D / 8), d = (e8 % (D / 8)) * 8;
     const float dc = p.dcum[cg * MS + m];
-    const float hk = bf16_to_f32(p.hkT[(cg * MS + m) * D + d]) + p.hseg_k[(sl * MS + m) * D + d] * dc;
-    const float hv = bf16_to_f32(p.hvc[(cg * MS + m) * D + d]) + p.hseg_v[(sl * MS + m) * D + d] * dc;
-    if (hkc) {   // fp32 copies: only the VALU kernels of the backward read them
-      hkc[(cg * D + d) * MS + m] = hk;
-      hkct[(cg * MS + m) * D + d] = hk;
-      hvct[(cg * D + d) * MS + m] = hv;
+    const int64_t li = (cg * MS + m) * D + d, si = (sl * MS + m) * D + d;
+    float lk[8], lv[8], sk[8], sv[8], hk[8], hv[8];
+    Elem<bf16_t>::ld8(p.hkT + li, lk);
+    Elem<bf16_t>::ld8(p.hvc + li, lv);
+    Elem<float>::ld8(p.hseg_k + si, sk);
+    Elem<float>::ld8(p.hseg_v + si, sv);
+    uint32_t kh[4], vh[4], kl[4], vl[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      hk[j] = lk[j] + sk[j] * dc;
+      hv[j] = lv[j] + sv[j] * dc;
     }
     // bf16 pairs hi + lo: the backward multiplies by hi and by lo
-    const bf16_t hkh = f32_to_bf16(hk), hvh = f32_to_bf16(hv);
-    hkb[(cg * MS + m) * D + d] = hkh;
-    hvb[(cg * MS + m) * D + d] = hvh;
-    hkl[(cg * MS + m) * D + d] = f32_to_bf16(hk - bf16_to_f32(hkh));
-    hvl[(cg * MS + m) * D + d] = f32_to_bf16(hv - bf16_to_f32(hvh));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bf16_t k0 = f32_to_bf16(hk[2 * j]), k1 = f32_to_bf16(hk[2 * j + 1]);
+      const bf16_t v0 = f32_to_bf16(hv[2 * j]), v1 = f32_to_bf16(hv[2 * j + 1]);
+      kh[j] = (uint32_t)k0 | ((uint32_t)k1 << 16);
+      vh[j] = (uint32_t)v0 | ((uint32_t)v1 << 16);
+      kl[j] = (uint32_t)f32_to_bf16(hk[2 * j] - bf16_to_f32(k0)) | ((uint32_t)f32_to_bf16(hk[2 * j + 1] - bf16_to_f32(k1)) << 16);
+      vl[j] = (uint32_t)f32_to_bf16(hv[2 * j] - bf16_to_f32(v0)) | ((uint32_t)f32_to_bf16(hv[2 * j + 1] - bf16_to_f32(v1)) << 16);
+    }
+    *reinterpret_cast<uint4*>(hkb + li) = make_uint4(kh[0], kh[1], kh[2], kh[3]);
+    *reinterpret_cast<uint4*>(hvb + li) = make_uint4(vh[0], vh[1], vh[2], vh[3]);
+    *reinterpret_cast<uint4*>(hkl + li) = make_uint4(kl[0], kl[1], kl[2], kl[3]);
+    *reinterpret_cast<uint4*>(hvl + li) = make_uint4(vl[0], vl[1], vl[2], vl[3]);
+    if (hkc) {   // fp32 copies: only the VALU kernels of the backward read them
+      Elem<float>::st8(hkct + li, hk);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        hkc[(cg * D + d + j) * MS + m] = hk[j];
+        hvct[(cg * D + d + j) * MS + m] = hv[j];
+      }
+    }
   }
-  for (int e = tid; e < R * MS; e += 256) gc[((int64_t)(c0 + e / MS) * H + h) * MS + e % MS] = p.gc[cg * BT * MS + e];
+  for (int e4 = tid; e4 < R * MS / 4; e4 += 256) {
+    const int r = e4 / (MS / 4), m4 = (e4 % (MS / 4)) * 4;
+    *reinterpret_cast<float4*>(gc + ((int64_t)(c0 + r) * H + h) * MS + m4) = *reinterpret_cast<const float4*>(p.gc + cg * BT * MS + r * MS + m4);
+  }
   // chunks in which some slot decays by more than e^-BWD_DECAY_CLAMP over one of the two 32-row halves: the
   // backward's factored products (e^(gc_i - ref) e^(ref - gc_j) as two operands, ref = the start of
-  // j's half) leave the bf16 / fp32 range there
-  if (tid == 0) {
-    int b = 0;
+  // j's half) leave the bf16 / fp32 range there.  One slot per lane of the first wave.
+  if (tid < 64) {
     const float* g = p.gc + cg * BT * MS;
-    for (int m = 0; m < MS; ++m) {
-      const float g31 = g[(R > 32 ? 31 : R - 1) * MS + m];
-      b |= (g31 < -BWD_DECAY_CLAMP) | (g[(R - 1) * MS + m] - g31 < -BWD_DECAY_CLAMP);
-    }
-    big[cg] = b;
+    const int m = tid;
+    const float g31 = g[(R > 32 ? 31 : R - 1) * MS + m];
+    const bool b = (g31 < -BWD_DECAY_CLAMP) | (g[(R - 1) * MS + m] - g31 < -BWD_DECAY_CLAMP);
+    const bool any = __any(b);
+    if (tid == 0) big[cg] = any ? 1 : 0;
   }
 }
 
