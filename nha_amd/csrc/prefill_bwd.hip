@@ -689,19 +689,78 @@ __global__ __launch_bounds__(256) void bwd_state_inter_kernel(const BP p) {
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_gate_local_kernel(const BP p) {
-  // thread = (row group g of 16 rows, slot m): the 16 rows' loads are independent and issued
-  // together; the reverse cumulative sum is a suffix sum in registers plus the sums of the later
-  // groups through LDS
-  __shared__ float gs[4][BT];
+  // M == 64 (the matrix-core path): thread = (group rg of 4 consecutive rows, 4 consecutive slots), 16-byte
+  // reads, all of a thread's rows requested together; the reverse cumulative sum is a suffix sum over the
+  // thread's rows plus the sums of the later groups through LDS.  Other M: thread = (group of 16 rows, slot).
+  __shared__ float gs[16][BT];
   const int M = p.M, H = p.H, HQ = p.HQ;
   const int NG = HQ / H;
   const int chunk = blockIdx.x, h = blockIdx.y;
-  const int m = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   const int nslab = p.nbk + p.nbv;
+  if (M == BT) {
+    const int rg = threadIdx.x >> 4, m = (threadIdx.x & 15) * 4;
+    float z[4][4], dst[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = 4 * rg + q, t = c0 + r, sj = t - p.shift;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) z[q][e] = dst[q][e] = 0.f;
+      if (r < R && sj >= bos) {
+        const int64_t rt = ((int64_t)t * H + h) * M + m;
+        float4 ds4 = *reinterpret_cast<const float4*>(p.dsi + rt);
+        for (int b = 0; b < nslab; ++b) {
+          const float4 a = *reinterpret_cast<const float4*>(p.dsp + (int64_t)b * p.T_tot * H * M + rt);
+          ds4.x += a.x; ds4.y += a.y; ds4.z += a.z; ds4.w += a.w;
+        }
+        float4 x4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int a = 0; a < NG; ++a) {
+          const float4 v = *reinterpret_cast<const float4*>(p.xg + ((int64_t)t * HQ + h * NG + a) * M + m);
+          x4.x += v.x; x4.y += v.y; x4.z += v.z; x4.w += v.w;
+        }
+        float sv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sv[e] = Elem<T>::ld((const T*)p.s + ((int64_t)sj * H + h) * M + m + e);
+        const float d4[4] = {ds4.x, ds4.y, ds4.z, ds4.w}, xx[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          z[q][e] = xx[e] - sv[e] * d4[e];
+          dst[q][e] = d4[e];
+        }
+      }
+    }
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 3; q >= 0; --q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        run[e] += z[q][e];
+        z[q][e] = run[e];   // suffix sum inside the group
+      }
+    *reinterpret_cast<float4*>(&gs[rg][m]) = make_float4(run[0], run[1], run[2], run[3]);
+    __syncthreads();
+    float later[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int g2 = 15; g2 > rg; --g2) {
+      const float4 a = *reinterpret_cast<const float4*>(&gs[g2][m]);
+      later[0] += a.x; later[1] += a.y; later[2] += a.z; later[3] += a.w;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = 4 * rg + q, t = c0 + r, sj = t - p.shift;
+      if (r < R && sj >= bos) {
+        const int64_t rt = ((int64_t)t * H + h) * M + m;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) Elem<T>::st((T*)p.ds + ((int64_t)sj * H + h) * M + m + e, dst[q][e]);
+        *reinterpret_cast<float4*>(p.dsi + rt) = make_float4(z[q][0] + later[0], z[q][1] + later[1], z[q][2] + later[2], z[q][3] + later[3]);   // chunk-local reverse cumulative sum
+      }
+    }
+    if (rg == 0) *reinterpret_cast<float4*>(p.gtot + ((int64_t)chunk * H + h) * M + m) = make_float4(run[0] + later[0], run[1] + later[1], run[2] + later[2], run[3] + later[3]);
+    return;
+  }
+  const int m = threadIdx.x & 63, g = threadIdx.x >> 6;
   float z[16], dst[16];
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
