@@ -849,17 +849,63 @@ __global__ __launch_bounds__(256) void bwd_gate_final_kernel(const BP p) {
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
-  for (int e = threadIdx.x; e < R * M; e += 256) {
-    const int r = e / M, m = e - r * M;
-    const int t = c0 + r, sj = t - p.shift;
-    if (sj < bos) continue;
-    const float val = p.dsi[((int64_t)t * H + h) * M + m] + p.gtot[((int64_t)chunk * H + h) * M + m];
-    Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, val);
+  if (M == BT) {
+    // four consecutive slots of four rows per thread, their 16-byte reads requested together
+    const int m = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;
+    const float4 gt = *reinterpret_cast<const float4*>(p.gtot + ((int64_t)chunk * H + h) * M + m);
+    float4 v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = r0 + 16 * q, t = c0 + r;
+      v[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (r < R && t - p.shift >= bos) v[q] = *reinterpret_cast<const float4*>(p.dsi + ((int64_t)t * H + h) * M + m);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = r0 + 16 * q, sj = c0 + r - p.shift;
+      if (r < R && sj >= bos) {
+        T* dst = (T*)p.dg + ((int64_t)sj * H + h) * M + m;
+        Elem<T>::st(dst, v[q].x + gt.x);
+        Elem<T>::st(dst + 1, v[q].y + gt.y);
+        Elem<T>::st(dst + 2, v[q].z + gt.z);
+        Elem<T>::st(dst + 3, v[q].w + gt.w);
+      }
+    }
+  } else {
+    for (int e = threadIdx.x; e < R * M; e += 256) {
+      const int r = e / M, m = e - r * M;
+      const int t = c0 + r, sj = t - p.shift;
+      if (sj < bos) continue;
+      const float val = p.dsi[((int64_t)t * H + h) * M + m] + p.gtot[((int64_t)chunk * H + h) * M + m];
+      Elem<T>::st((T*)p.dg + ((int64_t)sj * H + h) * M + m, val);
+    }
   }
   // tokens of this chunk that never reach the slots (the last `shift` of the sequence): zero gradients
   const int K = p.K, V = p.V;
   int r0 = eos - p.shift - c0;
   r0 = r0 < 0 ? 0 : r0;
+  if (r0 >= R) return;
+  const int nr = R - r0;
+  if (M % 8 == 0 && K % 8 == 0 && V % 8 == 0) {
+    // 16-byte stores, the rows of the chunk side by side (M, K, V multiples of 8: every row start is 16-byte aligned)
+    constexpr int EPV = 16 / (int)sizeof(T);   // elements of T per 16 bytes
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    for (int i = threadIdx.x; i < nr * (M / EPV); i += 256) {
+      const int r = r0 + i / (M / EPV), e = (i % (M / EPV)) * EPV;
+      const int64_t jh = (int64_t)(c0 + r) * H + h;
+      *reinterpret_cast<uint4*>((T*)p.ds + jh * M + e) = zero;
+      *reinterpret_cast<uint4*>((T*)p.dg + jh * M + e) = zero;
+    }
+    for (int i = threadIdx.x; i < nr * (K / EPV); i += 256) {
+      const int r = r0 + i / (K / EPV), e = (i % (K / EPV)) * EPV;
+      *reinterpret_cast<uint4*>((T*)p.dk_gsa + ((int64_t)(c0 + r) * H + h) * K + e) = zero;
+    }
+    for (int i = threadIdx.x; i < nr * (V / 4); i += 256) {
+      const int r = r0 + i / (V / 4), e = (i % (V / 4)) * 4;
+      *reinterpret_cast<uint4*>(p.dvs + ((int64_t)(c0 + r) * H + h) * V + e) = zero;
+    }
+    return;
+  }
   for (int r = r0; r < R; ++r) {
     const int64_t jh = (int64_t)(c0 + r) * H + h;
     for (int e = threadIdx.x; e < M; e += 256) {
