@@ -19,6 +19,8 @@
 //   K and V rows in registers); the q / do rows of every query head of the group stream through the ring
 //   in items of 32 queries: four tiles (q and do as row fragments for S = Q K^T and dP = dO V^T, and once
 //   more for the transposing read: dV^T += dO^T P, dK^T += Q^T dS) plus the 32 (lse, delta) pairs.
+//   The first and the last units of a head are triangles over the waves (causal edge, window edge) that
+//   complement each other: such units are held in LDS two at a time and every wave works on its own.
 #include "common.h"
 #include "mfma_common.h"
 
@@ -333,20 +335,52 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
   // the walk of the sequence's first key group would be at that moment: neighbours then request the same
   // q / do rows at about the same time and the second request finds them in L2.
   const int rot = (nun - (8 * (it >> 2)) % nun) % nun;
-  int ig = 0, iu = rot;   // next item to request
-  int nreq = 0;           // items of the current head requested so far
-  auto issue_next = [&](int slot) {
-    issue_item(ig, iu, slot);
-    if (++iu == nun) iu = 0;
-    if (++nreq == nun) {
-      nreq = 0;
-      iu = rot;
-      ++ig;
+  // Complementary units.  Against the 256 keys of the workgroup the first units of a head are triangles (wave w has
+  // work in unit u only if w <= u: the queries of a unit must not all lie before the wave's keys) and so are the last
+  // ones (the keys must not all have left the window: unit a + K0 has work only for the waves w >= a + 1), and a
+  // workgroup takes as long over a unit as its busiest wave.  Units a < npair are therefore worked on together with
+  // unit a + K0: both are in LDS at once and every wave takes the one it has work in, never both.
+  const int K0 = p.wl >= 0 ? (p.wl + 63) / 32 : 0;
+  int npair = 0;
+  if (p.wl >= 0 && K0 >= 7 && nun > K0) npair = (nun - K0) < 7 ? (nun - K0) : 7;
+  // the walk of a head: its units in cyclic order from rot, the second units of the pairs left out
+  auto walk_skip = [&](int x) {
+    if (x >= nun) x -= nun;
+    if (x >= K0 && x < K0 + npair) {   // empty range without pairs
+      x = K0 + npair;
+      if (x >= nun) x -= nun;
+    }
+    return x;
+  };
+  const int rot0 = walk_skip(rot);
+  struct Walk { int g, u, cnt; };
+  auto advance = [&](Walk& w) {
+    w.cnt += (w.u < npair) ? 2 : 1;
+    w.u = walk_skip(w.u + 1);
+    if (w.cnt == nun) {
+      w.cnt = 0;
+      w.u = rot0;
+      ++w.g;
     }
   };
-#pragma unroll
-  for (int i = 0; i < NR - 1; ++i)
-    if (i < total) issue_next(i);
+  // requests, in the order the loop below consumes the items: the unit of a step, then the unit paired with it
+  Walk pw = {0, rot0, 0};
+  int pend_u = -1, pend_g = 0;
+  auto issue_next = [&](int slot) {
+    if (pend_u >= 0) {
+      issue_item(pend_g, pend_u, slot);
+      pend_u = -1;
+      return;
+    }
+    issue_item(pw.g, pw.u, slot);
+    if (pw.u < npair) {
+      pend_u = pw.u + K0;
+      pend_g = pw.g;
+    }
+    advance(pw);
+  };
+  int issued = 0;
+  for (; issued < NR - 1 && issued < total; ++issued) issue_next(issued);
 
   // this lane's keys (one per 16-key block of the wave) and their K / V rows (B operands: K[key][32 ks + 8 kb ..])
   const int kbase = 16 * NKB * wave;               // first key of the wave, relative to c0
@@ -390,30 +424,42 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
     return __builtin_bit_cast(bf16x8, t);
   };
 
-  int u = rot, ndone = 0;   // unit of the item being worked on, items of its head done so far
-  for (int i = 0; i < total; ++i) {
-    // item i has landed (this wave's part; wave 0 carries one more load per item), then everybody's
-    if (i + 2 < total) {
+  // queries [32 u, 32 u + 32) against keys [kbase, kbase + 16 NKB), both relative to c0: nothing to do if
+  // every query is before every key or past the window of every key
+  auto no_work = [&](int u) { return (32 * u + 31 < kbase) || (p.wl >= 0 && 32 * u > kbase + 16 * NKB - 1 + p.wl); };
+  Walk cw = {0, rot0, 0};
+  for (int k = 0; k < total;) {
+    const int prim = cw.u;
+    const int need = prim < npair ? 2 : 1;   // items of this step: k .. k + need - 1
+    advance(cw);
+    // they have landed (this wave's part; wave 0 carries one more load per item), then everybody's; the
+    // requests after them stay in flight
+    const int younger = issued - (k + need);
+    if (younger >= 2) {
       if (wave == 0) wait_vm<2 * (KV_LPW + 1)>();
       else wait_vm<2 * KV_LPW>();
-    } else if (i + 1 < total) {
+    } else if (younger == 1) {
       if (wave == 0) wait_vm<KV_LPW + 1>();
       else wait_vm<KV_LPW>();
     } else {
       wait_vm<0>();
     }
     lds_barrier();
-    if (i + NR - 1 < total) issue_next((i + NR - 1) & (NR - 1));
-    const uint32_t base = (uint32_t)((i & (NR - 1)) * KV_ITEM);
+    // every wave is past the items before k: their slots take the next requests
+    for (; issued < total && issued < k + NR; ++issued) issue_next(issued & (NR - 1));
+    int u = prim;
+    uint32_t base = (uint32_t)((k & (NR - 1)) * KV_ITEM);
+    if (need == 2 && no_work(prim)) {
+      u = prim + K0;
+      base = (uint32_t)(((k + 1) & (NR - 1)) * KV_ITEM);
+    }
+    k += need;
     int lc = threadIdx.x & 63;
     asm volatile("" : "+v"(lc));
     const int l16 = lc & 15, kb = lc >> 4;
     kaddr = (uint32_t)(lc * 16);
     vaddr = (uint32_t)((4 * kb + (l16 >> 2)) * 32 + 8 * (l16 & 3));
-    // queries [32 u, 32 u + 32) against keys [kbase, kbase + 16 NKB), both relative to c0: nothing to do if
-    // every query is before every key or past the window of every key
-    const bool none = (32 * u + 31 < kbase) || (p.wl >= 0 && 32 * u > kbase + 16 * NKB - 1 + p.wl);
-    if (!none) {
+    if (!no_work(u)) {
       const bool edge = (32 * u < kbase + 16 * NKB - 1) || (p.wl >= 0 && 32 * u + 31 > kbase + p.wl) || (c0 + 32 * u + 32 > eos);
       // ---- phase 1: S = Q K^T and dP = dO V^T, one 16-key block at a time (two blocks of scores beside both
       //      gradient accumulators do not fit the register file, so the q / do row fragments are read once per
@@ -510,11 +556,6 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-    }
-    if (++u == nun) u = 0;
-    if (++ndone == nun) {
-      ndone = 0;
-      u = rot;
     }
   }
 #pragma unroll
