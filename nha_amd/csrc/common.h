@@ -146,13 +146,13 @@ size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
 int prefill_mfma_impl(const NhaPrefillArgs* a);
 int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb,
                                void* hkl, void* hvl, int* big);
-int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const float* ap, const float* bp, const float* ust,
+int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const bf16_t* ap, const bf16_t* bp, const float* ust,
                        const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
                        float* cv, float* dsi);
 int bwd_slot_inter_slabs(const NhaPrefillBwdArgs* a);
 int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, const float* dus, const float* pp,
                        const float* ck, const float* cv, const float* gc, float* ek, float* ev, float* dks, float* dvs, float* dsp);
-int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap, float* bp, float* ust, float* dpst,
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, bf16_t* ap, bf16_t* bp, float* ust, float* dpst,
                       float* delta, const int* big, const float* gc, float* dus, float* pp, float* xg);
 bool bwd_slot_products_fuses_q(const NhaPrefillBwdArgs* a);
 bool prefill_bwd_supported(const NhaPrefillBwdArgs* a);

@@ -48,7 +48,7 @@ struct BP {
   float *dsi;             // [T_tot][H][M]     intra-chunk part of ds, indexed by row token
   float *dsp;             // [nbk+nbv][T_tot][H][M]  inter-chunk part of ds per column block
   float *dvs;             // [T_tot][H][V]     slot-branch dv, indexed by SOURCE token
-  const float *ap, *bp;   // [NT][HQ][BT][BT]  q_gsa_i . k'_j and do_i . v'_j from the matrix cores, or NULL
+  const bf16_t *ap, *bp;  // [NT][HQ][BT][BT]  q_gsa_i . k'_j and do_i . v'_j from the matrix cores (bf16), or NULL
   const float *ust, *dpst; // [T_tot][HQ][M]    q_gsa_t . hk0[:,m] and do_t . hv0[m,:] (chunk-start states), or NULL
   const int* big;         // [NT][H] chunks the matrix-core slot kernels leave to the VALU kernels, or NULL (all)
   float *gtot;            // [NT][H][M]        chunk sums of the dg summand, then sums of all later chunks
@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256) void bwd_q_kernel(const BP p) {
     const int64_t sj = (int64_t)bos + tl0 + j;
     if (p.ap) {
       const int64_t pi = (((int64_t)chunk * HQ + hq) * BT + rr) * BT + j;
-      Aj[j] = has ? p.ap[pi] * p.scale : 0.f;
-      Bj[j] = has ? p.bp[pi] : 0.f;
+      Aj[j] = has ? bf16_to_f32(p.ap[pi]) * p.scale : 0.f;
+      Bj[j] = has ? bf16_to_f32(p.bp[pi]) : 0.f;
     } else {
       Aj[j] = has ? dot_row<T>(qg, kgs + (sj * H + h) * K, K) : 0.f;
       Bj[j] = has ? dot_row<T>(dov, vv_ + (sj * H + h) * V, V) : 0.f;
@@ -337,8 +337,8 @@ __global__ __launch_bounds__(512) void bwd_intra_kernel(const BP p) {
       const int sj = src[r];
       float av = 0.f, bv = 0.f;
       if (sj >= 0 && p.ap) {
-        av = p.ap[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r];
-        bv = p.bp[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r];
+        av = bf16_to_f32(p.ap[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r]);
+        bv = bf16_to_f32(p.bp[(((int64_t)chunk * HQ + hq) * BT + i) * BT + r]);
       } else if (sj >= 0) {
         const T* qrow = (const T*)p.q_gsa + ((int64_t)(c0 + i) * HQ + hq) * K;
         const T* krow = (const T*)p.k_gsa + ((int64_t)sj * H + h) * K;
@@ -1006,8 +1006,8 @@ BwdPlan plan_bwd(const NhaPrefillBwdArgs* a, const NhaPrefillArgs& f) {
     s.hvb = off; off += aligned((size_t)a->NT * a->H * a->M * a->V * 2);
     s.hkl = off; off += aligned((size_t)a->NT * a->H * a->M * a->K * 2);
     s.hvl = off; off += aligned((size_t)a->NT * a->H * a->M * a->V * 2);
-    s.ap = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
-    s.bp = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 4);
+    s.ap = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 2);
+    s.bp = off; off += aligned((size_t)a->NT * a->HQ * BT * BT * 2);
     s.ust = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
     s.dpst = off; off += aligned((size_t)a->T_tot * a->HQ * a->M * 4);
     s.big = off; off += aligned((size_t)a->NT * a->H * 4);
@@ -1072,7 +1072,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
     rc = prefill_mfma_export_states(&f, gc, nullptr, nullptr, nullptr, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (int*)(sc + sp.big));
     // the decay-free products of the slot branch on the matrix cores
     // (with the decay-coupled terms on the matrix cores too, the per-token stage rides along)
-    if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (float*)(sc + sp.ap), (float*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst),
+    if (rc == NHA_OK) rc = bwd_slot_products(a, sc + sp.hkb, sc + sp.hvb, sc + sp.hkl, sc + sp.hvl, (bf16_t*)(sc + sp.ap), (bf16_t*)(sc + sp.bp), (float*)(sc + sp.ust), (float*)(sc + sp.dpst),
                                              (float*)(sc + sp.delta), intra_mfma ? (const int*)(sc + sp.big) : nullptr, gc,
                                              (float*)(sc + sp.dus), (float*)(sc + sp.pp), (float*)(sc + sp.xg));
   } else {
@@ -1092,11 +1092,12 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
   p.gc = gc; p.hkc = hkc; p.hvc = hvc;
   p.hkct = (float*)(sc + sp.hkct); p.hvct = (float*)(sc + sp.hvct);
-  p.ap = p.bp = p.ust = p.dpst = nullptr;
+  p.ap = p.bp = nullptr;
+  p.ust = p.dpst = nullptr;
   p.big = nullptr;
   if (sp.use_mfma) {
     if (intra_mfma) p.big = (const int*)(sc + sp.big);
-    p.ap = (float*)(sc + sp.ap); p.bp = (float*)(sc + sp.bp);
+    p.ap = (const bf16_t*)(sc + sp.ap); p.bp = (const bf16_t*)(sc + sp.bp);
     p.ust = (float*)(sc + sp.ust); p.dpst = (float*)(sc + sp.dpst);
   }
   p.hkT = (float*)(sc + sp.hkT); p.hvT = (float*)(sc + sp.hvT);

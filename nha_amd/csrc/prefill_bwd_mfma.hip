@@ -397,7 +397,7 @@ struct SP1 {
   const bf16_t *q, *dout, *kg, *v;   // q_gsa [T,HQ,D], dout [T,HQ,D], k_gsa [T,H,D], v [T,H,D]
   const bf16_t *hkb, *hvb;           // [NT][H][64][D] chunk-start states, hk transposed (high parts)
   const bf16_t *hkl, *hvl;           // their low parts
-  float *ap, *bp;                    // [NT][HQ][64][64]
+  bf16_t *ap, *bp;                   // [NT][HQ][64][64] bf16: every consumer takes them as matrix-core operands
   float *ust, *dpst;                 // [T][HQ][64]
   const bf16_t* o;                   // [T,HQ,D]
   float* delta;                      // [T][HQ]  do . o
@@ -841,7 +841,8 @@ __global__ __launch_bounds__(256) void bwd_slot_inter_kernel(const SP2 p) {
 // ------------------------------------------------------------------------------------------
 struct SP3 {
   const bf16_t* s;                                 // [T,H,64]
-  const float *ap, *bp, *ust, *dpst, *gc, *delta;  // see bwd_slot_products
+  const bf16_t *ap, *bp;                           // see bwd_slot_products
+  const float *ust, *dpst, *gc, *delta;
   const float *lse_swa, *lse_gsa, *dlse_gsa;
   float *dus, *pp, *xg;                            // [T][HQ][64]
   float *ck, *cv;                                  // [NT][HQ][64][64]
@@ -985,33 +986,34 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
   int vlo = p.shift - it * BT;
   vlo = vlo < 0 ? 0 : vlo;
-  const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
-  const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+  const bf16_t* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+  const bf16_t* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
   {
     constexpr int NS = BT * BT / 4 / 256;
-    float4 av[NS], bv[NS];
+    uint2 av[NS], bv[NS];
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, j = e & 63;
-      av[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      av[u] = bv[u] = make_uint2(0, 0);
       if (j <= i && i < R) {
-        av[u] = *reinterpret_cast<const float4*>(ap + e);
-        bv[u] = *reinterpret_cast<const float4*>(bp + e);
+        av[u] = *reinterpret_cast<const uint2*>(ap + e);
+        bv[u] = *reinterpret_cast<const uint2*>(bp + e);
       }
     }
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, j = e & 63;
-      const float a4[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, b4[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
-      bf16x4 pa, pb;
+      const uint16_t a4[4] = {(uint16_t)av[u].x, (uint16_t)(av[u].x >> 16), (uint16_t)av[u].y, (uint16_t)(av[u].y >> 16)};
+      const uint16_t b4[4] = {(uint16_t)bv[u].x, (uint16_t)(bv[u].x >> 16), (uint16_t)bv[u].y, (uint16_t)(bv[u].y >> 16)};
+      uint16_t pa[4], pb[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const bool in = j + q <= i && i < R;
-        pa[q] = (__bf16)(in ? a4[q] : 0.f);
-        pb[q] = (__bf16)(in ? b4[q] : 0.f);
+        pa[q] = in ? a4[q] : (uint16_t)0;
+        pb[q] = in ? b4[q] : (uint16_t)0;
       }
-      *reinterpret_cast<NHA_LDS bf16x4*>(At + i * TLD + j) = pa;
-      *reinterpret_cast<NHA_LDS bf16x4*>(Bt + i * TLD + j) = pb;
+      *reinterpret_cast<NHA_LDS uint2*>(At + i * TLD + j) = make_uint2(pa[0] | ((uint32_t)pa[1] << 16), pa[2] | ((uint32_t)pa[3] << 16));
+      *reinterpret_cast<NHA_LDS uint2*>(Bt + i * TLD + j) = make_uint2(pb[0] | ((uint32_t)pb[1] << 16), pb[2] | ((uint32_t)pb[3] << 16));
     }
   }
   RowOps rops;
@@ -1119,8 +1121,8 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
     if (kb == 0 && i < R) p.delta[(int64_t)(c0 + i) * HQ + hq] = acc;
     if (FUSE && kb == 0) dlt[i] = acc;
   }
-  float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
-  float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+  bf16_t* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+  bf16_t* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
   RowOps rops;
   if (fused) rops.load(pq, c0, R, h, hq, 16 * wave + l16, kb);
   f32x4 cUr[FUSE ? 4 : 1], cPr[FUSE ? 4 : 1];
@@ -1144,13 +1146,15 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i = 16 * blk + 4 * kb + r;
-      ap[i * BT + j] = cA[r];
-      bp[i * BT + j] = cB[r];
-      if (fused) {
+      if (fused) {   // the tables go to LDS; their global copies are written from there in 16-byte pieces below
         const bool in = j <= i && i < R;
         At[i * TLD + j] = f32_to_bf16(in ? cA[r] : 0.f);
         Bt[i * TLD + j] = f32_to_bf16(in ? cB[r] : 0.f);
-      } else if (i < R) {
+      } else {
+        ap[i * BT + j] = f32_to_bf16(cA[r]);
+        bp[i * BT + j] = f32_to_bf16(cB[r]);
+      }
+      if (!fused && i < R) {
         const int64_t tq = ((int64_t)(c0 + i) * HQ + hq) * BT + j;
         p.ust[tq] = cU[r];
         p.dpst[tq] = cP[r];
@@ -1161,6 +1165,14 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
     if (!fused) return;   // uniform over the workgroup
     sy.store(Yh, Yl, R, vlo, tid);
     lds_barrier();
+    // global copies of the two score tables for the intra-chunk kernel (masked like the LDS tables: above the
+    // diagonal and past the last row they are zero, and every reader masks those elements itself)
+#pragma unroll
+    for (int u = 0; u < BT * BT / 8 / 256; ++u) {
+      const int e = tid + 256 * u, i = e >> 3, c8 = (e & 7) * 8;
+      *reinterpret_cast<uint4*>(ap + i * BT + c8) = *reinterpret_cast<const NHA_LDS uint4*>(At + i * TLD + c8);
+      *reinterpret_cast<uint4*>(bp + i * BT + c8) = *reinterpret_cast<const NHA_LDS uint4*>(Bt + i * TLD + c8);
+    }
     slot_q_rows<true>(pq, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, cUr, cPr, dlt, rops);
   }
 }
@@ -1203,23 +1215,25 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   // first pair of a q-head is requested before the products of the head before it, the second pair
   // before the first is converted: a head waits out one partly hidden memory latency instead of two.
   struct Pair {
-    float4 gi[2], g31[2], du[2], pv[2], av[2], bv[2];
+    float4 gi[2], g31[2], du[2], pv[2];
+    uint2 av[2], bv[2];   // four bf16 each
   };
   auto load_pair = [&](Pair& t, int hq, int u0) {
-    const float* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
-    const float* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
+    const bf16_t* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
+    const bf16_t* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-      t.gi[u] = t.g31[u] = t.du[u] = t.pv[u] = t.av[u] = t.bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      t.gi[u] = t.g31[u] = t.du[u] = t.pv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      t.av[u] = t.bv[u] = make_uint2(0, 0);
       if (i < R) {
         t.gi[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
         t.du[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
         t.pv[u] = *reinterpret_cast<const float4*>(p.pp + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
         if (i >= 32) t.g31[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
         if (c <= i) {
-          t.av[u] = *reinterpret_cast<const float4*>(ap + e);
-          t.bv[u] = *reinterpret_cast<const float4*>(bp + e);
+          t.av[u] = *reinterpret_cast<const uint2*>(ap + e);
+          t.bv[u] = *reinterpret_cast<const uint2*>(bp + e);
         }
       }
     }
@@ -1230,7 +1244,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
       const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
       const float g4[4] = {t.gi[u].x, t.gi[u].y, t.gi[u].z, t.gi[u].w}, r4[4] = {t.g31[u].x, t.g31[u].y, t.g31[u].z, t.g31[u].w};
       const float d4[4] = {t.du[u].x, t.du[u].y, t.du[u].z, t.du[u].w}, q4[4] = {t.pv[u].x, t.pv[u].y, t.pv[u].z, t.pv[u].w};
-      const float a4[4] = {t.av[u].x, t.av[u].y, t.av[u].z, t.av[u].w}, b4[4] = {t.bv[u].x, t.bv[u].y, t.bv[u].z, t.bv[u].w};
+      const bf16_t a4[4] = {(bf16_t)t.av[u].x, (bf16_t)(t.av[u].x >> 16), (bf16_t)t.av[u].y, (bf16_t)(t.av[u].y >> 16)};
+      const bf16_t b4[4] = {(bf16_t)t.bv[u].x, (bf16_t)(t.bv[u].x >> 16), (bf16_t)t.bv[u].y, (bf16_t)(t.bv[u].y >> 16)};
       float x0[4], x1[4], p0[4], p1[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -1241,8 +1256,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
         x1[q] = d4[q] * e1;
         p1[q] = q4[q] * e1;
         const bool in = i < R && c + q <= i;
-        AT[(c + q) * TLD + i] = f32_to_bf16(in ? a4[q] : 0.f);
-        BT_[(c + q) * TLD + i] = f32_to_bf16(in ? b4[q] : 0.f);
+        AT[(c + q) * TLD + i] = in ? a4[q] : (bf16_t)0;
+        BT_[(c + q) * TLD + i] = in ? b4[q] : (bf16_t)0;
       }
       split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
       split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
@@ -1412,7 +1427,7 @@ static int launch_slot_products(const SP1& p, const SP3& pq, int NT, hipStream_t
   return NHA_OK;
 }
 
-static SP3 make_sp3(const NhaPrefillBwdArgs* a, const int* big, const float* ap, const float* bp, const float* ust,
+static SP3 make_sp3(const NhaPrefillBwdArgs* a, const int* big, const bf16_t* ap, const bf16_t* bp, const float* ust,
                     const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
                     float* cv, float* dsi) {
   SP3 p;
@@ -1429,8 +1444,8 @@ static SP3 make_sp3(const NhaPrefillBwdArgs* a, const int* big, const float* ap,
 // bwd_slot_products_fuses_q() tells the caller to skip bwd_slot_products3(which = 0).
 bool bwd_slot_products_fuses_q(const NhaPrefillBwdArgs* a) { return a->K <= 128; }
 
-int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, float* ap,
-                      float* bp, float* ust, float* dpst, float* delta, const int* big, const float* gc, float* dus, float* pp,
+int bwd_slot_products(const NhaPrefillBwdArgs* a, const void* hkb, const void* hvb, const void* hkl, const void* hvl, bf16_t* ap,
+                      bf16_t* bp, float* ust, float* dpst, float* delta, const int* big, const float* gc, float* dus, float* pp,
                       float* xg) {
   SP1 p;
   p.q = (const bf16_t*)a->q_gsa; p.dout = (const bf16_t*)a->dout; p.kg = (const bf16_t*)a->k_gsa; p.v = (const bf16_t*)a->v;
@@ -1501,7 +1516,7 @@ int bwd_slot_products2(const NhaPrefillBwdArgs* a, int which, const void* hkb, c
 
 // which = 0: bwd_slot_q_kernel (per-token vectors); 1: bwd_slot_intra_kernel (ck, cv, intra part of
 // ds).  Chunks flagged in `big` are left to the fp32 VALU kernels.
-int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const float* ap, const float* bp, const float* ust,
+int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const bf16_t* ap, const bf16_t* bp, const float* ust,
                        const float* dpst, const float* gc, const float* delta, float* dus, float* pp, float* xg, float* ck,
                        float* cv, float* dsi) {
   const SP3 p = make_sp3(a, big, ap, bp, ust, dpst, gc, delta, dus, pp, xg, ck, cv, dsi);
