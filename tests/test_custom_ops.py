@@ -86,3 +86,33 @@ def test_full_graph_trace():
     assert torch.allclose(out, ref)
     for a, x in zip(gref, xs):
         assert torch.equal(a, x.grad)
+
+
+@pytest.mark.gpu
+def test_operator_carries_initial_and_final_states():
+    """Initial states in, final states out, cotangents on both: the operator's autograd formula against chunk_nha's."""
+    from nha_amd import chunk_nha, chunk_nha_packed
+    T, HQ, H, D, M = 260, 4, 2, 64, 64
+    cu = torch.tensor([0, 100, 260], dtype=torch.int32)
+    xs = _inputs(13, T, HQ, H, D, M, "cuda")
+    gen = torch.Generator().manual_seed(14)
+    h0k = (torch.randn(2, H, D, M, generator=gen) * 0.1).cuda().requires_grad_(True)
+    h0v = (torch.randn(2, H, M, D, generator=gen) * 0.1).cuda().requires_grad_(True)
+    do = torch.randn(T, HQ, D, generator=gen).cuda().to(torch.bfloat16)
+    dk, dv = torch.randn(2, H, D, M, generator=gen).cuda(), torch.randn(2, H, M, D, generator=gen).cuda()
+
+    def run(fn, packed):
+        for x in (*xs, h0k, h0v):
+            x.grad = None
+        if packed:
+            o, ls, lg, (hk, hv) = fn(*xs, cu, window_size_left=40, gsa_kv_shift=0, initial_state=(h0k, h0v), output_final_state=True)
+        else:
+            o, ls, lg, (hk, hv) = fn(*[x[None] for x in xs], cu_seqlens=cu.cuda(), window_size_left=40, gsa_kv_shift=0,
+                                     initial_state=(h0k, h0v), output_final_state=True)
+            o, ls, lg = o[0], ls[0], lg[0]
+        ((o.float() * do.float()).sum() + (hk * dk).sum() + (hv * dv).sum() + 0.3 * ls.sum() - 0.2 * lg.sum()).backward()
+        return [o, ls, lg, hk, hv] + [x.grad.clone() for x in (*xs, h0k, h0v)]
+
+    a, b = run(chunk_nha_packed, True), run(chunk_nha, False)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
