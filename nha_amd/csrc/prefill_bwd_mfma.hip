@@ -504,22 +504,32 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   constexpr int NS = BT * BT / 4 / 256;
   constexpr bool AHEAD = DW <= 128;
   Tile<BT, DW> rx;
-  float4 wv[NS], gv[NS], cv[NS];
+  float4 wv[NS], cv[NS];
   auto load_head = [&](int hq) {
     rx.load(xsrc + (int64_t)hq * D + x0, (int64_t)HQ * D, c0, R, tid);
     const float* cp = csrc + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-      wv[u] = gv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      wv[u] = cv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
       if (i < R) {
         wv[u] = *reinterpret_cast<const float4*>(wsrc + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
-        gv[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
         if (c <= i) cv[u] = *reinterpret_cast<const float4*>(cp + i * BT + c);
       }
     }
   };
   if (AHEAD) load_head(h * NG);
+  // e^(gc) of this thread's elements: the same for every q-head of the group, read and formed once
+  float4 eg[NS];
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+    eg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < R) {
+      const float4 g = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+      eg[u] = make_float4(__expf(g.x), __expf(g.y), __expf(g.z), __expf(g.w));
+    }
+  }
   for (int a = 0; a < NG; ++a) {
     const int hq = h * NG + a;
     if (!AHEAD) load_head(hq);
@@ -530,8 +540,7 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
 #pragma unroll
       for (int u = 0; u < NS; ++u) {
         const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-        const float w4[4] = {wv[u].x * __expf(gv[u].x), wv[u].y * __expf(gv[u].y), wv[u].z * __expf(gv[u].z),
-                             wv[u].w * __expf(gv[u].w)};
+        const float w4[4] = {wv[u].x * eg[u].x, wv[u].y * eg[u].y, wv[u].z * eg[u].z, wv[u].w * eg[u].w};
         const float c4[4] = {cv[u].x, cv[u].y, cv[u].z, cv[u].w};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -1215,22 +1224,36 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   // first pair of a q-head is requested before the products of the head before it, the second pair
   // before the first is converted: a head waits out one partly hidden memory latency instead of two.
   struct Pair {
-    float4 gi[2], g31[2], du[2], pv[2];
+    float4 du[2], pv[2];
     uint2 av[2], bv[2];   // four bf16 each
   };
+  // e^(gc_i) and e^(gc_i - gc_31) (rows of the second half) of this thread's sixteen elements: the same for every
+  // q-head of the group, read and formed once
+  float4 e0v[4], e1v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+    e0v[u] = e1v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < R) {
+      const float4 g = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
+      e0v[u] = make_float4(__expf(g.x), __expf(g.y), __expf(g.z), __expf(g.w));
+      if (i >= 32) {
+        const float4 r = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
+        e1v[u] = make_float4(__expf(g.x - r.x), __expf(g.y - r.y), __expf(g.z - r.z), __expf(g.w - r.w));
+      }
+    }
+  }
   auto load_pair = [&](Pair& t, int hq, int u0) {
     const bf16_t* ap = p.ap + ((int64_t)chunk * HQ + hq) * BT * BT;
     const bf16_t* bp = p.bp + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-      t.gi[u] = t.g31[u] = t.du[u] = t.pv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      t.du[u] = t.pv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
       t.av[u] = t.bv[u] = make_uint2(0, 0);
       if (i < R) {
-        t.gi[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
         t.du[u] = *reinterpret_cast<const float4*>(p.dus + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
         t.pv[u] = *reinterpret_cast<const float4*>(p.pp + ((int64_t)(c0 + i) * HQ + hq) * BT + c);
-        if (i >= 32) t.g31[u] = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
         if (c <= i) {
           t.av[u] = *reinterpret_cast<const uint2*>(ap + e);
           t.bv[u] = *reinterpret_cast<const uint2*>(bp + e);
@@ -1242,15 +1265,15 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-      const float g4[4] = {t.gi[u].x, t.gi[u].y, t.gi[u].z, t.gi[u].w}, r4[4] = {t.g31[u].x, t.g31[u].y, t.g31[u].z, t.g31[u].w};
+      const float4 ev0 = e0v[u0 + u], ev1 = e1v[u0 + u];
+      const float e0q[4] = {ev0.x, ev0.y, ev0.z, ev0.w}, e1q[4] = {ev1.x, ev1.y, ev1.z, ev1.w};
       const float d4[4] = {t.du[u].x, t.du[u].y, t.du[u].z, t.du[u].w}, q4[4] = {t.pv[u].x, t.pv[u].y, t.pv[u].z, t.pv[u].w};
       const bf16_t a4[4] = {(bf16_t)t.av[u].x, (bf16_t)(t.av[u].x >> 16), (bf16_t)t.av[u].y, (bf16_t)(t.av[u].y >> 16)};
       const bf16_t b4[4] = {(bf16_t)t.bv[u].x, (bf16_t)(t.bv[u].x >> 16), (bf16_t)t.bv[u].y, (bf16_t)(t.bv[u].y >> 16)};
       float x0[4], x1[4], p0[4], p1[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const float e0 = i < R ? __expf(g4[q]) : 0.f;
-        const float e1 = (i < R && i >= 32) ? __expf(g4[q] - r4[q]) : 0.f;
+        const float e0 = e0q[q], e1 = e1q[q];
         x0[q] = d4[q] * e0;
         p0[q] = q4[q] * e0;
         x1[q] = d4[q] * e1;
