@@ -1021,8 +1021,9 @@ __global__ __launch_bounds__(256) void bwd_slot_q_kernel(const SP3 p) {
         pa[q] = in ? a4[q] : (uint16_t)0;
         pb[q] = in ? b4[q] : (uint16_t)0;
       }
-      *reinterpret_cast<NHA_LDS uint2*>(At + i * TLD + j) = make_uint2(pa[0] | ((uint32_t)pa[1] << 16), pa[2] | ((uint32_t)pa[3] << 16));
-      *reinterpret_cast<NHA_LDS uint2*>(Bt + i * TLD + j) = make_uint2(pb[0] | ((uint32_t)pb[1] << 16), pb[2] | ((uint32_t)pb[3] << 16));
+      typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+      *reinterpret_cast<NHA_LDS u32x2_t*>(At + i * TLD + j) = (u32x2_t){pa[0] | ((uint32_t)pa[1] << 16), pa[2] | ((uint32_t)pa[3] << 16)};
+      *reinterpret_cast<NHA_LDS u32x2_t*>(Bt + i * TLD + j) = (u32x2_t){pb[0] | ((uint32_t)pb[1] << 16), pb[2] | ((uint32_t)pb[3] << 16)};
     }
   }
   RowOps rops;
@@ -1179,8 +1180,10 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
 #pragma unroll
     for (int u = 0; u < BT * BT / 8 / 256; ++u) {
       const int e = tid + 256 * u, i = e >> 3, c8 = (e & 7) * 8;
-      *reinterpret_cast<uint4*>(ap + i * BT + c8) = *reinterpret_cast<const NHA_LDS uint4*>(At + i * TLD + c8);
-      *reinterpret_cast<uint4*>(bp + i * BT + c8) = *reinterpret_cast<const NHA_LDS uint4*>(Bt + i * TLD + c8);
+      const nha_u32x4 ta = *reinterpret_cast<const NHA_LDS nha_u32x4*>(At + i * TLD + c8);
+      const nha_u32x4 tb = *reinterpret_cast<const NHA_LDS nha_u32x4*>(Bt + i * TLD + c8);
+      *reinterpret_cast<nha_u32x4*>(ap + i * BT + c8) = ta;
+      *reinterpret_cast<nha_u32x4*>(bp + i * BT + c8) = tb;
     }
     slot_q_rows<true>(pq, At, Bt, Yh, Yl, c0, R, h, hq, wave, lane, cUr, cPr, dlt, rops);
   }
