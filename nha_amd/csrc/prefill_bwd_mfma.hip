@@ -1193,14 +1193,18 @@ __global__ __launch_bounds__(256) void bwd_slot_products_kernel(const SP1 p, con
 __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   extern __shared__ __align__(16) unsigned char smem[];
   // tables [64 rows][TLD]; X0 = scale du_i[m] e^(gc_i[m]), X1 = scale du_i[m] e^(gc_i[m] - gc_31[m])
-  // (rows >= 32), P0 / P1 the same with p; each as a high and a low part
+  // (rows >= 32 only: 32-row tables whose pointers are set back by 32 rows, so that row i is indexed as in the
+  // others), P0 / P1 the same with p; each as a high and a low part.  Y is the same for every q-head and each
+  // lane needs the same four fragments of it throughout: they are read into registers once and the transposed
+  // A / B tables of the heads then use Y's place.  Eight tables = 72 KB: two workgroups per CU.
   lbf16* const T0 = (lbf16*)smem;
-  lbf16* const X0h = T0, * const X0l = T0 + BT * TLD, * const X1h = T0 + 2 * BT * TLD, * const X1l = T0 + 3 * BT * TLD;
-  lbf16* const P0h = T0 + 4 * BT * TLD, * const P0l = T0 + 5 * BT * TLD, * const P1h = T0 + 6 * BT * TLD, * const P1l = T0 + 7 * BT * TLD;
-  lbf16* const Yh = T0 + 8 * BT * TLD;   // [64 r][TLD]
-  lbf16* const Yl = T0 + 9 * BT * TLD;
-  lbf16* const AT = T0 + 10 * BT * TLD;  // [64 r][TLD]  A[i][r] transposed, zero for i < r
-  lbf16* const BT_ = T0 + 11 * BT * TLD; // [64 r][TLD]  B[i][r] transposed
+  lbf16* const X0h = T0, * const X0l = T0 + BT * TLD, * const P0h = T0 + 2 * BT * TLD, * const P0l = T0 + 3 * BT * TLD;
+  lbf16* const Yh = T0 + 4 * BT * TLD;   // [64 r][TLD]
+  lbf16* const Yl = T0 + 5 * BT * TLD;
+  lbf16* const AT = Yh;                  // [64 r][TLD]  A[i][r] transposed, zero for i < r
+  lbf16* const BT_ = Yl;                 // [64 r][TLD]  B[i][r] transposed
+  lbf16* const X1h = T0 + (6 * BT - 32) * TLD, * const X1l = T0 + 6 * BT * TLD;
+  lbf16* const P1h = T0 + (7 * BT - 32) * TLD, * const P1l = T0 + 7 * BT * TLD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
@@ -1232,17 +1236,18 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   };
   // e^(gc_i) and e^(gc_i - gc_31) (rows of the second half) of this thread's sixteen elements: the same for every
   // q-head of the group, read and formed once
-  float4 e0v[4], e1v[4];
+  float4 e0v[4], e1v[2];   // groups 2 and 3 of a thread are the rows >= 32
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-    e0v[u] = e1v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    e0v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (u >= 2) e1v[u - 2] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < R) {
       const float4 g = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + i) * H + h) * BT + c);
       e0v[u] = make_float4(__expf(g.x), __expf(g.y), __expf(g.z), __expf(g.w));
-      if (i >= 32) {
+      if (u >= 2) {
         const float4 r = *reinterpret_cast<const float4*>(p.gc + ((int64_t)(c0 + 31) * H + h) * BT + c);
-        e1v[u] = make_float4(__expf(g.x - r.x), __expf(g.y - r.y), __expf(g.z - r.z), __expf(g.w - r.w));
+        e1v[u - 2] = make_float4(__expf(g.x - r.x), __expf(g.y - r.y), __expf(g.z - r.z), __expf(g.w - r.w));
       }
     }
   }
@@ -1268,7 +1273,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int e = 4 * (tid + 256 * (u0 + u)), i = e >> 6, c = e & 63;
-      const float4 ev0 = e0v[u0 + u], ev1 = e1v[u0 + u];
+      const bool second = u0 >= 2;   // rows >= 32: the only ones the ref-gc_31 tables hold
+      const float4 ev0 = e0v[u0 + u], ev1 = second ? e1v[u0 + u - 2] : make_float4(0.f, 0.f, 0.f, 0.f);
       const float e0q[4] = {ev0.x, ev0.y, ev0.z, ev0.w}, e1q[4] = {ev1.x, ev1.y, ev1.z, ev1.w};
       const float d4[4] = {t.du[u].x, t.du[u].y, t.du[u].z, t.du[u].w}, q4[4] = {t.pv[u].x, t.pv[u].y, t.pv[u].z, t.pv[u].w};
       const bf16_t a4[4] = {(bf16_t)t.av[u].x, (bf16_t)(t.av[u].x >> 16), (bf16_t)t.av[u].y, (bf16_t)(t.av[u].y >> 16)};
@@ -1286,19 +1292,28 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
         BT_[(c + q) * TLD + i] = in ? b4[q] : (bf16_t)0;
       }
       split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
-      split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
       split4_bf16(make_float4(p0[0], p0[1], p0[2], p0[3]), P0h, P0l, i * TLD + c);
-      split4_bf16(make_float4(p1[0], p1[1], p1[2], p1[3]), P1h, P1l, i * TLD + c);
+      if (second) {
+        split4_bf16(make_float4(x1[0], x1[1], x1[2], x1[3]), X1h, X1l, i * TLD + c);
+        split4_bf16(make_float4(p1[0], p1[1], p1[2], p1[3]), P1h, P1l, i * TLD + c);
+      }
     }
   };
   static_assert(BT * BT / 4 / 256 == 4, "two pairs of element groups per thread");
   Pair t0, t1;
   load_pair(t0, h * NG, 0);
   sy.store(Yh, Yl, R, vlo, tid);
+  lds_barrier();
+  bf16x8 yfh[2], yfl[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    yfh[ks] = lds_frag(Yh, TLD, col, 32 * ks + 8 * kb);
+    yfl[ks] = lds_frag(Yl, TLD, col, 32 * ks + 8 * kb);
+  }
   for (int a = 0; a < NG; ++a) {
     const int hq = h * NG + a;
     load_pair(t1, hq, 2);
-    if (a > 0) lds_barrier();
+    lds_barrier();   // the Y fragments are read (first head) / the head before is done with the tables
     store_pair(t0, 0);
     store_pair(t1, 2);
     lds_barrier();
@@ -1308,10 +1323,11 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
     float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
+      if (wave >= 2 && blk < 2) continue;   // rows above this wave's columns: nothing to store, and no X1 / P1 rows
       f32x4 c1 = {0.f, 0.f, 0.f, 0.f}, c2 = c1;
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8 yh = lds_frag(Yh, TLD, col, 32 * ks + 8 * kb), yl = lds_frag(Yl, TLD, col, 32 * ks + 8 * kb);
+        const bf16x8 yh = yfh[ks], yl = yfl[ks];
         const bf16x8 xh = lds_frag(Xch, TLD, 16 * blk + l16, 32 * ks + 8 * kb);
         const bf16x8 ph = lds_frag(Pch, TLD, 16 * blk + l16, 32 * ks + 8 * kb);
         c1 = mfma16(xh, yh, mfma16(xh, yl, mfma16(lds_frag(Xcl, TLD, 16 * blk + l16, 32 * ks + 8 * kb), yh, c1)));
@@ -1549,7 +1565,7 @@ int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, co
   hipStream_t st = (hipStream_t)a->stream;
   if (which == 0) hipLaunchKernelGGL(bwd_slot_q_kernel, dim3(a->HQ, a->NT), dim3(256), 0, st, p);
   else {
-    const size_t lds = (size_t)12 * BT * TLD * 2;
+    const size_t lds = (size_t)8 * BT * TLD * 2;
     static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
     if (!configured) {
       hipError_t e = hipFuncSetAttribute((const void*)bwd_slot_intra_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
