@@ -474,9 +474,11 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
   constexpr int DB = DW / 16, LDT = DW + 16, TILE = BT * LDT;
   extern __shared__ __align__(16) unsigned char smem[];
   lbf16* const Xt = (lbf16*)smem;        // [64 rows i][DW]
-  lbf16* const Wt = Xt + TILE;           // [64 m][TLD]  (w_i[m] e^(gc_i[m]))^T, high part
+  // the two tables lie as they are read from memory, row i by row i (8-byte LDS writes); the transposing LDS
+  // read turns them into B operands (2-byte writes of the transposed tables cost four times the instructions)
+  lbf16* const Wt = Xt + TILE;           // [64 i][TLD]  w_i[m] e^(gc_i[m]), high part
   lbf16* const Wl = Wt + BT * TLD;       //              low part
-  lbf16* const Ct = Wl + BT * TLD;       // [64 r][TLD]  c[i][r]^T, zero for i < r, high part
+  lbf16* const Ct = Wl + BT * TLD;       // [64 i][TLD]  c[i][r], zero for i < r, high part
   lbf16* const Cl = Ct + BT * TLD;       //              low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
@@ -535,26 +537,22 @@ __global__ __launch_bounds__(256) void bwd_slot_state_kernel(const SP2 p) {
     if (!AHEAD) load_head(hq);
     if (a > 0) lds_barrier();   // everyone is done with the previous head's tiles
     rx.store(Xt, tid);
-    {
-      // transposed writes
 #pragma unroll
-      for (int u = 0; u < NS; ++u) {
-        const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-        const float w4[4] = {wv[u].x * eg[u].x, wv[u].y * eg[u].y, wv[u].z * eg[u].z, wv[u].w * eg[u].w};
-        const float c4[4] = {cv[u].x, cv[u].y, cv[u].z, cv[u].w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          split_bf16(i < R ? w4[q] : 0.f, Wt, Wl, (c + q) * TLD + i);
-          split_bf16(c + q <= i ? c4[q] : 0.f, Ct, Cl, (c + q) * TLD + i);
-        }
-      }
+    for (int u = 0; u < NS; ++u) {
+      const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
+      // rows i >= R were not read: wv, cv and eg are zero there
+      split4_bf16(make_float4(wv[u].x * eg[u].x, wv[u].y * eg[u].y, wv[u].z * eg[u].z, wv[u].w * eg[u].w), Wt, Wl, i * TLD + c);
+      split4_bf16(make_float4(c <= i ? cv[u].x : 0.f, c + 1 <= i ? cv[u].y : 0.f, c + 2 <= i ? cv[u].z : 0.f,
+                              c + 3 <= i ? cv[u].w : 0.f), Ct, Cl, i * TLD + c);
     }
     lds_barrier();
     if (AHEAD && a + 1 < NG) load_head(hq + 1);
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      const bf16x8 bw = table_frag(Wt, col, hf, kb), bwl = table_frag(Wl, col, hf, kb);
-      const bf16x8 bc = table_frag(Ct, col, hf, kb), bcl = table_frag(Cl, col, hf, kb);
+      const bf16x8 bw = lds_frag_tr(Wt, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 bwl = lds_frag_tr(Wl, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 bc = lds_frag_tr(Ct, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
+      const bf16x8 bcl = lds_frag_tr(Cl, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const bf16x8 xa = lds_frag_tr(Xt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // X^T[x][i]
@@ -1201,8 +1199,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
   lbf16* const X0h = T0, * const X0l = T0 + BT * TLD, * const P0h = T0 + 2 * BT * TLD, * const P0l = T0 + 3 * BT * TLD;
   lbf16* const Yh = T0 + 4 * BT * TLD;   // [64 r][TLD]
   lbf16* const Yl = T0 + 5 * BT * TLD;
-  lbf16* const AT = Yh;                  // [64 r][TLD]  A[i][r] transposed, zero for i < r
-  lbf16* const BT_ = Yl;                 // [64 r][TLD]  B[i][r] transposed
+  lbf16* const AT = Yh;                  // [64 i][TLD]  A[i][r], zero for i < r; read with the transposing LDS read
+  lbf16* const BT_ = Yl;                 // [64 i][TLD]  B[i][r]
   lbf16* const X1h = T0 + (6 * BT - 32) * TLD, * const X1l = T0 + 6 * BT * TLD;
   lbf16* const P1h = T0 + (7 * BT - 32) * TLD, * const P1l = T0 + 7 * BT * TLD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1277,8 +1275,15 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
       const float4 ev0 = e0v[u0 + u], ev1 = second ? e1v[u0 + u - 2] : make_float4(0.f, 0.f, 0.f, 0.f);
       const float e0q[4] = {ev0.x, ev0.y, ev0.z, ev0.w}, e1q[4] = {ev1.x, ev1.y, ev1.z, ev1.w};
       const float d4[4] = {t.du[u].x, t.du[u].y, t.du[u].z, t.du[u].w}, q4[4] = {t.pv[u].x, t.pv[u].y, t.pv[u].z, t.pv[u].w};
-      const bf16_t a4[4] = {(bf16_t)t.av[u].x, (bf16_t)(t.av[u].x >> 16), (bf16_t)t.av[u].y, (bf16_t)(t.av[u].y >> 16)};
-      const bf16_t b4[4] = {(bf16_t)t.bv[u].x, (bf16_t)(t.bv[u].x >> 16), (bf16_t)t.bv[u].y, (bf16_t)(t.bv[u].y >> 16)};
+      {
+        // elements c + q > i (and rows i >= R, which were not read) are zero
+        typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+        const int d = i < R ? i - c : -1;
+        const uint32_t m0 = (d >= 0 ? 0xffffu : 0u) | (d >= 1 ? 0xffff0000u : 0u);
+        const uint32_t m1 = (d >= 2 ? 0xffffu : 0u) | (d >= 3 ? 0xffff0000u : 0u);
+        *reinterpret_cast<NHA_LDS u32x2_t*>(AT + i * TLD + c) = (u32x2_t){t.av[u].x & m0, t.av[u].y & m1};
+        *reinterpret_cast<NHA_LDS u32x2_t*>(BT_ + i * TLD + c) = (u32x2_t){t.bv[u].x & m0, t.bv[u].y & m1};
+      }
       float x0[4], x1[4], p0[4], p1[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -1287,9 +1292,6 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
         p0[q] = q4[q] * e0;
         x1[q] = d4[q] * e1;
         p1[q] = q4[q] * e1;
-        const bool in = i < R && c + q <= i;
-        AT[(c + q) * TLD + i] = in ? a4[q] : (bf16_t)0;
-        BT_[(c + q) * TLD + i] = in ? b4[q] : (bf16_t)0;
       }
       split4_bf16(make_float4(x0[0], x0[1], x0[2], x0[3]), X0h, X0l, i * TLD + c);
       split4_bf16(make_float4(p0[0], p0[1], p0[2], p0[3]), P0h, P0l, i * TLD + c);
@@ -1351,7 +1353,8 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
       const bf16x8 p0l = lds_frag_tr(P0l, TLD, 32 * hf, 32 * hf + 16, 16 * wave, lane);
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
-        const bf16x8 af = table_frag(AT, 16 * rb + l16, hf, kb), bf = table_frag(BT_, 16 * rb + l16, hf, kb);
+        const bf16x8 af = lds_frag_tr(AT, TLD, 32 * hf, 32 * hf + 16, 16 * rb, lane);
+        const bf16x8 bf = lds_frag_tr(BT_, TLD, 32 * hf, 32 * hf + 16, 16 * rb, lane);
         accS[rb] = mfma16(af, x0h, mfma16(af, x0l, accS[rb]));
         accS[rb] = mfma16(bf, p0h, mfma16(bf, p0l, accS[rb]));
       }
@@ -1362,7 +1365,7 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
       const bf16x8 p1h = lds_frag_tr(P1h, TLD, 32, 48, 16 * wave, lane), p1l = lds_frag_tr(P1l, TLD, 32, 48, 16 * wave, lane);
 #pragma unroll
       for (int rb = 2; rb < 4; ++rb) {
-        const bf16x8 af = table_frag(AT, 16 * rb + l16, 1, kb), bf = table_frag(BT_, 16 * rb + l16, 1, kb);
+        const bf16x8 af = lds_frag_tr(AT, TLD, 32, 48, 16 * rb, lane), bf = lds_frag_tr(BT_, TLD, 32, 48, 16 * rb, lane);
         accS[rb] = mfma16(af, x1h, mfma16(af, x1l, accS[rb]));
         accS[rb] = mfma16(bf, p1h, mfma16(bf, p1l, accS[rb]));
       }
