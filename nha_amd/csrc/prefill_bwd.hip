@@ -818,21 +818,21 @@ __global__ void bwd_gate_scan_kernel(const BP p) {
     const float* b = p.hvT + (((int64_t)n * H + h) * M + m) * V;
     for (int c = 0; c < V; ++c) run += a[c] * b[c];
   }
-  // four chunk sums are fetched before the first is consumed, so the loads overlap
+  // sixteen chunk sums are fetched before the first is consumed, so the loads overlap
   const int nchunks = (eos - bos + BT - 1) / BT;
   float* gt = p.gtot + ((int64_t)p.coff[n] * H + h) * M + m;
   const int64_t cs = (int64_t)H * M;
   int it = nchunks - 1;
-  for (; it >= 3; it -= 4) {
-    const float t0 = gt[it * cs], t1 = gt[(it - 1) * cs], t2 = gt[(it - 2) * cs], t3 = gt[(it - 3) * cs];
-    gt[it * cs] = run;
-    run += t0;
-    gt[(it - 1) * cs] = run;
-    run += t1;
-    gt[(it - 2) * cs] = run;
-    run += t2;
-    gt[(it - 3) * cs] = run;
-    run += t3;
+  constexpr int NB = 16;
+  for (; it >= NB - 1; it -= NB) {
+    float t[NB];
+#pragma unroll
+    for (int u = 0; u < NB; ++u) t[u] = gt[(it - u) * cs];
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      gt[(it - u) * cs] = run;
+      run += t[u];
+    }
   }
   for (; it >= 0; --it) {
     const float tot = gt[it * cs];
