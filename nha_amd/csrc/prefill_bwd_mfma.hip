@@ -578,12 +578,15 @@ template <int D>
 __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   constexpr int DB = D / 16, LDT = D + 16, TILE = BT * LDT;
   extern __shared__ __align__(16) unsigned char smem[];
+  // The two products run one after the other through the same LDS (a tile and one table as a high and a low
+  // part: 36 KB, four workgroups per CU; with both sets resident, 72 KB, two); the operands of the second are
+  // requested with those of the first and wait in registers.
   lbf16* const Ht = (lbf16*)smem;        // [64 m][D]  hk0^T
-  lbf16* const Kt = Ht + TILE;           // [64 j][D]  k' rows
-  lbf16* const Wt = Kt + TILE;           // [64 i][TLD]  scale du_i[m] e^(gc_i[m]), high part
+  lbf16* const Kt = Ht;                  // [64 j][D]  k' rows (second product)
+  lbf16* const Wt = Ht + TILE;           // [64 i][TLD]  scale du_i[m] e^(gc_i[m]), high part
   lbf16* const Wl = Wt + BT * TLD;       //              low part
-  lbf16* const Ct = Wl + BT * TLD;       // [64 i][TLD]  ck[i][j], zero for j > i, high part
-  lbf16* const Cl = Ct + BT * TLD;       //              low part
+  lbf16* const Ct = Wt;                  // [64 i][TLD]  ck[i][j], zero for j > i, high part (second product)
+  lbf16* const Cl = Wl;                  //              low part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
@@ -592,8 +595,11 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int R = (eos - c0) < BT ? (eos - c0) : BT;
+  Tile<BT, D> rk;
+  constexpr int NS = BT * BT / 4 / 256;
+  float4 cv[NS];
   {
-    Tile<BT, D> rh, rk;
+    Tile<BT, D> rh;
     rh.load(p.hkb + ((int64_t)chunk * H + h) * BT * D, D, 0, BT, tid);
     // k' row j is the k_gsa row of source token c0 + j - shift: rows before the sequence are zero
     int vlo = p.shift - it * BT;
@@ -608,8 +614,7 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
     }
     // the tables are requested before the tiles are stored: one memory latency for both
     const float* cp = p.ck + ((int64_t)chunk * HQ + hq) * BT * BT;
-    constexpr int NS = BT * BT / 4 / 256;
-    float4 wv[NS], gv[NS], cv[NS];
+    float4 wv[NS], gv[NS];
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
@@ -621,21 +626,15 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
       }
     }
     rh.store(Ht, tid);
-    rk.store(Kt, tid);
 #pragma unroll
     for (int u = 0; u < NS; ++u) {
       const int e = 4 * (tid + 256 * u), i = e >> 6, c = e & 63;
-      float4 w, cc;
+      float4 w;
       w.x = i < R ? wv[u].x * __expf(gv[u].x) : 0.f;
       w.y = i < R ? wv[u].y * __expf(gv[u].y) : 0.f;
       w.z = i < R ? wv[u].z * __expf(gv[u].z) : 0.f;
       w.w = i < R ? wv[u].w * __expf(gv[u].w) : 0.f;
-      cc.x = c <= i ? cv[u].x : 0.f;
-      cc.y = c + 1 <= i ? cv[u].y : 0.f;
-      cc.z = c + 2 <= i ? cv[u].z : 0.f;
-      cc.w = c + 3 <= i ? cv[u].w : 0.f;
       split4_bf16(w, Wt, Wl, i * TLD + c);
-      split4_bf16(cc, Ct, Cl, i * TLD + c);
     }
   }
   lds_barrier();
@@ -646,12 +645,31 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
     const bf16x8 bw = table_frag(Wt, i, hf, kb), bwl = table_frag(Wl, i, hf, kb);   // contraction over m
-    const bf16x8 bc = table_frag(Ct, i, hf, kb), bcl = table_frag(Cl, i, hf, kb);   // contraction over j
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       const bf16x8 ha = lds_frag_tr(Ht, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // hk0[d][m]
-      const bf16x8 ka = lds_frag_tr(Kt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // k'_j[d]
       acc[db] = mfma16(ha, bw, mfma16(ha, bwl, acc[db]));
+    }
+  }
+  lds_barrier();   // everyone has read the first product's operands
+  rk.store(Kt, tid);
+#pragma unroll
+  for (int u = 0; u < NS; ++u) {
+    const int e = 4 * (tid + 256 * u), i2 = e >> 6, c = e & 63;
+    float4 cc;
+    cc.x = c <= i2 ? cv[u].x : 0.f;
+    cc.y = c + 1 <= i2 ? cv[u].y : 0.f;
+    cc.z = c + 2 <= i2 ? cv[u].z : 0.f;
+    cc.w = c + 3 <= i2 ? cv[u].w : 0.f;
+    split4_bf16(cc, Ct, Cl, i2 * TLD + c);
+  }
+  lds_barrier();
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    const bf16x8 bc = table_frag(Ct, i, hf, kb), bcl = table_frag(Cl, i, hf, kb);   // contraction over j
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const bf16x8 ka = lds_frag_tr(Kt, LDT, 32 * hf, 32 * hf + 16, 16 * db, lane);   // k'_j[d]
       acc[db] = mfma16(ka, bc, mfma16(ka, bcl, acc[db]));
     }
   }
@@ -1513,7 +1531,7 @@ static int launch_slot_stage2(const SP2& p, int NT, int which, hipStream_t st) {
   // (the state kernel takes all columns in one workgroup: split in two at head size 256 it stages its tables twice
   // and was measured slower, 110 against 103 us)
   const size_t lds_s = (size_t)BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
-  const size_t lds_q = (size_t)2 * BT * (D + 16) * 2 + (size_t)4 * BT * TLD * 2;
+  const size_t lds_q = (size_t)BT * (D + 16) * 2 + (size_t)2 * BT * TLD * 2;
   constexpr int DWI = D > 128 ? 128 : D;   // columns per workgroup of the inter kernel
   const size_t lds_i = (size_t)BT * (DWI + 16) * 2 + (size_t)2 * DWI * (BT + 8) * 2 + (size_t)2 * BT * TLD * 2;
   static std::atomic<bool> configured{false};   // the attribute call is idempotent: a second thread may repeat it
