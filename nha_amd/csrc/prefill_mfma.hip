@@ -159,7 +159,11 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
     if (jc + 1 < nloc) issue(it + 1);
     __syncthreads();
     // this lane's rows: element e = 4*q + r is row t = 16*q + 4*kb + r
+    // (the sixteen gate and s values of a lane are a column of their tiles: four transposing reads each
+    // instead of sixteen 2-byte reads)
     float gcv[16], sg[16];
+    const bf16x8 gq01 = lds_frag_tr(Gt, SLD, 0, 16, 16 * wave, lane), gq23 = lds_frag_tr(Gt, SLD, 32, 48, 16 * wave, lane);
+    const bf16x8 sq01 = lds_frag_tr(St, SLD, 0, 16, 16 * wave, lane), sq23 = lds_frag_tr(St, SLD, 32, 48, 16 * wave, lane);
     {
       float run[4], base = 0.f;
 #pragma unroll
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
         float a = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          a += bf16_to_f32(Gt[(16 * q + 4 * kb + r) * SLD + m]);
+          a += (float)(q < 2 ? gq01[4 * q + r] : gq23[4 * (q - 2) + r]);
           gcv[4 * q + r] = a;
         }
         run[q] = a;
@@ -218,7 +222,7 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int t = 16 * (e >> 2) + 4 * kb + (e & 3);
-      sg[e] = (t < rows) ? bf16_to_f32(St[t * SLD + m]) * fexp(glast - gcv[e]) : 0.f;
+      sg[e] = (t < rows) ? (float)(e < 8 ? sq01[e] : sq23[e - 8]) * fexp(glast - gcv[e]) : 0.f;
     }
     bf16x8 sg0, sg1;   // contraction steps over rows [0,32) and [32,64)
 #pragma unroll
