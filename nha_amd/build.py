@@ -25,7 +25,28 @@ EXTRA = {"prefill_mfma.hip": ["-fno-honor-nans"], "prefill_ring.hip": ["-fno-hon
          "prefill_bwd_mfma.hip": ["-fno-honor-nans"], "prefill_bwd_ring.hip": ["-fno-honor-nans"]}
 
 
+STAMP = os.path.join(HERE, "build", "sources.sha256")
+
+
+def sources_digest() -> str:
+    """sha256 over the library's sources (csrc/ and the C header), in name order.  The build writes it beside the
+    objects after a successful link; a test compares, so a library older than its sources does not pass for current."""
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    files += sorted(os.path.join(inc, f) for f in os.listdir(inc) if f.endswith(".h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
 def build_library(verbose: bool = False, jobs: int = 4) -> str:
+    digest = sources_digest()
+    if os.path.exists(STAMP):
+        os.remove(STAMP)
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
@@ -46,6 +67,8 @@ def build_library(verbose: bool = False, jobs: int = 4) -> str:
     out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if out.returncode != 0:
         raise RuntimeError("link failed:\n" + out.stdout)
+    with open(STAMP, "w") as fh:
+        fh.write(digest + "\n")
     return LIB
 
 

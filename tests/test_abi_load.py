@@ -25,6 +25,16 @@ def test_library_loads_and_exports_header_symbols():
     assert lib.nha_abi_version() == _lib.ABI_VERSION
 
 
+def test_library_is_built_from_the_current_sources():
+    """The build records a digest of csrc/ and the header after a successful link: a compile error that leaves the
+    previous library in place (or an edit without a rebuild) must not pass for the current code."""
+    from nha_amd import build
+    _lib.load()
+    assert os.path.exists(build.STAMP), "no build stamp: run python -m nha_amd.build"
+    with open(build.STAMP) as fh:
+        assert fh.read().strip() == build.sources_digest(), "libnha_hip.so is older than its sources: run python -m nha_amd.build"
+
+
 def test_struct_sizes_match_the_header(tmp_path):
     """sizeof and the offsets of the ctypes mirrors against the C compiler's view of the header."""
     import subprocess
