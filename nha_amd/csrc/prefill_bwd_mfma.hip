@@ -666,6 +666,7 @@ __global__ __launch_bounds__(256) void bwd_slot_dq_kernel(const SP2 p) {
   lds_barrier();
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
+    if (hf == 1 && wave < 2) continue;   // ck[i][j] is zero for j > i: rows below 32 have no second half
     const bf16x8 bc = table_frag(Ct, i, hf, kb), bcl = table_frag(Cl, i, hf, kb);   // contraction over j
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
@@ -1343,7 +1344,7 @@ __global__ __launch_bounds__(256) void bwd_slot_intra_kernel(const SP3 p) {
     float* cvp = p.cv + ((int64_t)chunk * HQ + hq) * BT * BT;
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
-      if (wave >= 2 && blk < 2) continue;   // rows above this wave's columns: nothing to store, and no X1 / P1 rows
+      if (blk < wave) continue;   // rows above this wave's columns: nothing to store (and no X1 / P1 rows below 32)
       f32x4 c1 = {0.f, 0.f, 0.f, 0.f}, c2 = c1;
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
