@@ -6,10 +6,10 @@ from ._lib import NhaError
 from .ops import chunk_nha, fused_chunk_nha_prefill, fused_recurrent_nha, fused_recurrent_nha_decode
 from .custom_ops import chunk_nha_packed      # also registers torch.ops.nha_amd.prefill_fwd / prefill_bwd
 from .ring import NHARingState, ring_decode_step
-from .cache import NHARingCache
+from .cache import NHACache, NHARingCache
 from .hybrid import (HybridNHAConfig, LlamaNativeHybridAttention, Qwen3MoeNativeHybridAttention, init_gates_from_keys,
                      pool_k_to_g)
 
 __all__ = ["chunk_nha", "chunk_nha_packed", "fused_chunk_nha_prefill", "fused_recurrent_nha", "fused_recurrent_nha_decode",
-           "NHARingState", "ring_decode_step", "NHARingCache", "NhaError", "HybridNHAConfig",
+           "NHARingState", "ring_decode_step", "NHARingCache", "NHACache", "NhaError", "HybridNHAConfig",
            "LlamaNativeHybridAttention", "Qwen3MoeNativeHybridAttention", "init_gates_from_keys", "pool_k_to_g"]

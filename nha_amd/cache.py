@@ -26,8 +26,8 @@ from .ring import NHARingState, ring_decode_step
 class NHARingCache:
     """Decode cache for a stack of NHA layers with window `window_size`."""
 
-    def __init__(self, window_size: int, seen_tokens: int = 0):
-        self.window_size = int(window_size)
+    def __init__(self, window_size: Optional[int] = None, seen_tokens: int = 0):
+        self.window_size = None if window_size is None else int(window_size)
         self.states: List[Optional[NHARingState]] = []     # ring-buffer form of a layer's window + slot state
         self.extra: List[Dict[str, object]] = []           # what `update` was given: recurrent / conv / ffn / attn state
         self.former_tokens = seen_tokens
@@ -98,9 +98,10 @@ class NHARingCache:
         return out
 
     @classmethod
-    def from_legacy_cache(cls, past_key_values=None, seen_tokens: int = 0, window_size: int = 0) -> "NHARingCache":
+    def from_legacy_cache(cls, past_key_values=None, seen_tokens: int = 0,
+                          window_size: Optional[int] = None) -> "NHARingCache":
         """A cache holding the per-layer dicts of `to_legacy_cache()` (nha_fla/models/nha_cache.py:167-182)."""
-        cache = cls(window_size, seen_tokens)
+        cache = cls(window_size=window_size, seen_tokens=seen_tokens)
         if isinstance(past_key_values, (list, tuple)):
             for i, st in enumerate(past_key_values):
                 cache._grow(i)
@@ -140,7 +141,7 @@ class NHARingCache:
         with (window_size_left, gsa_kv_shift) = (W-1, W)) over to the ring buffers of `layer_idx`.
         `window_size` overrides the cache's window for this layer (models mix short-window layers with
         2048-token ones)."""
-        W = self.window_size if window_size is None else int(window_size)
+        W = self._window(window_size)
         st = NHARingState.from_prefill(k_swa, k_gsa, v, g, final_state, W, cu_seqlens=cu_seqlens)
         self._grow(layer_idx)
         self.states[layer_idx] = st
@@ -148,6 +149,14 @@ class NHARingCache:
         self._layer_tokens[layer_idx] = longest
         self._count_tokens(layer_idx, longest, whole_step=True)
         return st
+
+    def _window(self, window_size: Optional[int]) -> int:
+        """The window of a call: its own `window_size`, else the one the cache was built with."""
+        W = self.window_size if window_size is None else int(window_size)
+        if W is None:
+            raise ValueError("this cache was built without a window size: pass `window_size` with the call "
+                             "(the attention modules do) or to the constructor")
+        return W
 
     def has_ring(self, layer_idx: int) -> bool:
         """Whether `layer_idx` holds ring buffers (a prompt was handed over with `prefill`)."""
@@ -189,8 +198,10 @@ class NHARingCache:
         st = self._ring(layer_idx)
         if st is None:
             held = self.extra[layer_idx]["attn_state"] if layer_idx < len(self.extra) else None
-            W = self.window_size if window_size is None else window_size
-            if held is not None and held[0].shape[-2] >= W:
+            if held is None:
+                return (None, None, None)
+            W = self._window(window_size)
+            if held[0].shape[-2] >= W:
                 return tuple(x[..., 0:1, :] for x in held)
             return (None, None, None)
         W = st.window
@@ -213,3 +224,13 @@ class NHARingCache:
 
     def to_legacy_cache(self) -> Tuple:
         return tuple(self[i] for i in range(len(self)))
+
+
+class NHACache(NHARingCache):
+    """`NHARingCache` under the reference cache's name and constructor (`NHACache(seen_tokens=0)`,
+    nha_fla/models/nha_cache.py:20-29; built without arguments at scripts/verify_opt_parity.py:671): the
+    window size is not a property of the reference's cache -- its callers pass it with every `update`
+    and `get_pop_kvf`, as the attention modules here pass it to `prefill` -- so it is an optional keyword."""
+
+    def __init__(self, seen_tokens: int = 0, window_size: Optional[int] = None):
+        super().__init__(window_size=window_size, seen_tokens=seen_tokens)

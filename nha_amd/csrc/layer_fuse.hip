@@ -589,7 +589,9 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const SC p) {
       if (t >= t1) break;
       while (t >= eos) {   // the walk enters the next sequence
         bos = eos;
-        if (p.cu) { ++seq_next; eos = p.cu[seq_next]; } else eos = bos + p.T;
+        if (!p.cu) eos = bos + p.T;
+        else if (seq_next < p.N) { ++seq_next; eos = p.cu[seq_next]; }
+        else eos = p.T_tot;   // boundaries that end before the last token: the rest is one more sequence
       }
 #pragma unroll
       for (int d = KS - 1; d >= 1; --d)
@@ -660,7 +662,9 @@ __global__ __launch_bounds__(256) void short_conv_bwd_kernel(const SC p) {
       if (t >= t2) break;
       while (t >= eos) {   // the walk enters the next sequence
         bos = eos;
-        if (p.cu) { ++seq_next; eos = p.cu[seq_next]; } else eos = bos + p.T;
+        if (!p.cu) eos = bos + p.T;
+        else if (seq_next < p.N) { ++seq_next; eos = p.cu[seq_next]; }
+        else eos = p.T_tot;   // boundaries that end before the last token: the rest is one more sequence
       }
       // shift the histories: slot d now belongs to token t - d
 #pragma unroll

@@ -25,6 +25,7 @@ The cache is `NHARingCache`; a layer hands its prompt over with `cache.prefill` 
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -106,6 +107,17 @@ def zero_sink_count(T: int, window: int, num_sinks: int, device) -> torch.Tensor
     covers: positions are shifted by num_sinks, the window spans [t + num_sinks - W + 1, t + num_sinks]."""
     t = torch.arange(T, device=device)
     return (window - 1 - t).clamp(0, num_sinks)
+
+
+def zero_sink_rescale(lse_swa: torch.Tensor, num_sinks: int, sinks_seen: torch.Tensor) -> torch.Tensor:
+    """(e^lse + num_sinks) / (e^lse + sinks_seen), formed in log space so that a window whose scores are all
+    strongly negative (lse < -88, where e^-lse leaves fp32) still gives the finite ratio num_sinks / sinks_seen
+    (with no sink seen the ratio is 1 + num_sinks e^-lse, capped at the largest fp32 so that a row whose
+    output has underflowed to zero stays zero instead of becoming 0 * inf)."""
+    lse = lse_swa.to(torch.float32)
+    log_seen = torch.log(sinks_seen.to(torch.float32))          # -inf where the window covers no sink
+    return torch.exp(torch.logaddexp(lse, torch.full_like(lse, math.log(num_sinks)))
+                     - torch.logaddexp(lse, log_seen.expand_as(lse))).clamp(max=torch.finfo(torch.float32).max)
 
 
 def pool_k_to_g(k_weight: torch.Tensor, target_rows: int) -> torch.Tensor:
@@ -213,9 +225,16 @@ class HybridNHAAttention(nn.Module):
         decode_step = (not self.training) and T == 1 and has_state
         mask_t = None
         if attention_mask is not None:         # left padding: a padded token writes nothing into the slots
-            if attention_mask.dim() != 2:
-                raise ValueError(f"attention_mask must be the [batch, tokens] padding mask, got {tuple(attention_mask.shape)}")
-            mask_t = attention_mask[:, -T:].to(v.dtype)[:, :, None, None]
+            if attention_mask.dim() == 2:      # [batch, tokens]
+                mask_t = attention_mask[:, -T:].to(v.dtype)[:, :, None, None]
+            elif attention_mask.dim() == 4:
+                # [batch, 1, queries, tokens]: the reference multiplies its head-first [B, heads, T, dim] tensors by
+                # mask[:, :, :, -T:] (qwennha.py:133-136), so the last T columns broadcast over (token, dim);
+                # the same product on the token-major layout here
+                mask_t = attention_mask[:, :, :, -T:].to(v.dtype).transpose(1, 2)
+            else:
+                raise ValueError("attention_mask must be [batch, tokens] or [batch, 1, queries, tokens], got "
+                                 f"{tuple(attention_mask.shape)}")
             v = v * mask_t
         cos, sin = self._tables(v, position_ids, position_embeddings, past_key_value, T)
         sq, sk = rotate_half_apply(q, cos, sin), rotate_half_apply(k, cos, sin)
@@ -249,9 +268,8 @@ class HybridNHAAttention(nn.Module):
                 if not nha:
                     # M zero-logit sinks were in the softmax at every t; the reference's window covers
                     # zero_sink_count(t) of them
-                    e = torch.exp(-lse_swa)                                         # [B,T,HQ] fp32
-                    n0 = zero_sink_count(T, W, M, e.device).to(e.dtype)[None, :, None]
-                    o = (o.to(torch.float32) * ((1 + M * e) / (1 + n0 * e))[..., None]).to(o.dtype)
+                    n0 = zero_sink_count(T, W, M, lse_swa.device)[None, :, None]
+                    o = (o.to(torch.float32) * zero_sink_rescale(lse_swa, M, n0)[..., None]).to(o.dtype)
             if past_key_value is not None:
                 past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W)
         o = self.o_proj(o.reshape(B, T, HQ * D))

@@ -78,15 +78,28 @@ def prefill_tables(cu_host: np.ndarray, device) -> Tuple[torch.Tensor, torch.Ten
 # stream are ordered by the stream, so they can share it; another stream gets its own.
 # ---------------------------------------------------------------------------------------------
 _WORKSPACE: dict = {}
+_WORKSPACE_MAX_STREAMS = 16      # entries kept; the one used longest ago leaves first (streams come and go)
 
 
 def _workspace(nbytes: int, dev, stream: int) -> torch.Tensor:
     key = (str(dev), stream)
-    ws = _WORKSPACE.get(key)
+    ws = _WORKSPACE.pop(key, None)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _WORKSPACE[key] = ws
+    _WORKSPACE[key] = ws             # re-inserted: the dict's order is the order of last use
+    while len(_WORKSPACE) > _WORKSPACE_MAX_STREAMS:
+        _WORKSPACE.pop(next(iter(_WORKSPACE)))
     return ws
+
+
+def release_workspaces() -> int:
+    """Drop the cached prefill workspaces (forward and backward) of every device and stream and return
+    the bytes they held.  The buffers are grow-only: one large prefill otherwise keeps its scratch for the life of the
+    process, out of reach of `torch.cuda.empty_cache()`.  Work already queued keeps its buffer alive through the
+    caching allocator's stream ordering, so this is safe to call between steps."""
+    held = sum(ws.numel() for ws in _WORKSPACE.values())
+    _WORKSPACE.clear()
+    return held
 
 
 # host copies of cu_seqlens tensors, keyed by the tensor OBJECT (weakly) and its version counter, so that
@@ -188,7 +201,7 @@ def nha_prefill_bwd(q_swa, k_swa, q_gsa, k_gsa, v, s, g, o, lse_swa, lse_gsa, do
     nbytes = lib.nha_prefill_bwd_scratch_bytes(C.byref(a))
     if nbytes == 0:
         _lib.check(_lib.NHA_ERR_INVALID)
-    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    scratch = _workspace(nbytes, dev, a.stream or 0)     # shared with the forward: calls on one stream are ordered
     a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
     _lib.check(lib.nha_prefill_bwd(C.byref(a)))
     return (*outs, dh0k, dh0v)
@@ -412,8 +425,22 @@ def nha_short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     _need_cuda(x, weight, bias)
     if activation not in (None, "silu", "swish"):
         raise ValueError(f"activation must be None, 'silu' or 'swish', got {activation!r}")
+    if x.dim() != 3:
+        raise ValueError(f"x must be [batch, tokens, channels], got {tuple(x.shape)}")
+    Cn = x.shape[-1]
+    if weight.shape[0] != Cn or weight.numel() != Cn * weight.shape[-1]:
+        raise ValueError(f"weight must be [{Cn}, 1, taps] for x with {Cn} channels, got {tuple(weight.shape)}")
+    if bias is not None and bias.numel() != Cn:
+        raise ValueError(f"bias must have {Cn} entries, got {tuple(bias.shape)}")
     if cu_seqlens is not None and x.shape[0] != 1:
         raise ValueError("cu_seqlens needs the packed layout [1, T_tot, C]")
+    if cu_seqlens is not None:
+        # the kernels walk the boundaries: they must start at 0, not decrease and end at the token count
+        cu_host = _cu_to_host(cu_seqlens)
+        if cu_host.ndim != 1 or cu_host.size < 2 or cu_host[0] != 0 or cu_host[-1] != x.shape[1] \
+                or (np.diff(cu_host) < 0).any():
+            raise ValueError(f"cu_seqlens must rise from 0 to the token count {x.shape[1]}, got {cu_host.tolist()[:8]}"
+                             f"{'...' if cu_host.size > 8 else ''}")
     cu = None if cu_seqlens is None else cu_seqlens.to(device=x.device, dtype=torch.int32).contiguous()
     return _ShortConvFunction.apply(x.contiguous(), weight, bias, cu, 0 if activation is None else 1)
 

@@ -1,3 +1,3 @@
-from nha_amd.cache import NHARingCache as NHACache
+from nha_amd.cache import NHACache
 
 __all__ = ["NHACache"]

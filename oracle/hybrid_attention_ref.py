@@ -100,7 +100,10 @@ class HybridAttentionRef:
         decode = T == 1 and had_content
         s = None if decode else self._r(1 - self._r(torch.exp(g)))  # qwennha.py:126-130
         if attention_mask is not None:                              # qwennha.py:133-144
-            m = attention_mask.to(F64)[:, -T:, None, None]
+            if attention_mask.dim() == 4:                           # [B,1,Q,T'] against head-first tensors (:134-136)
+                m = attention_mask.to(F64)[:, :, :, -T:].transpose(1, 2)
+            else:
+                m = attention_mask.to(F64)[:, -T:, None, None]
             v = v * m
             if s is not None:
                 s = s * m

@@ -152,6 +152,35 @@ def test_bwd_matrix_core_path_matches_fp32_path_at_size():
             check_grad(f"size wl={wl} d{k}", gb, gf.double().cpu(), BF)
 
 
+def test_bwd_window_longer_than_64_key_units_against_the_oracle():
+    """wl = 2047 on a 2300-token sequence at head size 128 with four query heads per kv-head, against reverse-mode
+    differentiation of the fp64 recurrence: the LDS-direct window-gradient kernels with a window of more than 64
+    units of 32 keys (a workgroup of the key-side kernel owns four chunks and pairs the first and last query units
+    of its range), rows with a full window and rows that still see the start of the sequence, a ragged last chunk."""
+    T, W = 2300, 2048
+    d = prefill_inputs(7700, 1, T, 4, 1, 128, 128, 64, dtype=BF, qk_scale=128 ** -0.5, gate_div=1.0, gate_mean=-1.0)
+    run_bwd_case("wl 2047 shifted", d, wl=W - 1, shift=W, dtype=BF)
+
+
+def test_bwd_long_context_heads_with_the_real_window_against_the_fp32_call():
+    """The long-context head shape with its own window (32 / 8 heads, D = 128, M = 64, W = 2048, shifted convention,
+    gate logits N(-1, 1), one 4096-token sequence): every gradient of the bf16 call (matrix-core kernels) against
+    the fp32 call (generic fp32 kernels only) on the same bf16-rounded inputs and cotangent."""
+    from nha_amd import chunk_nha
+    B, T, HQ, H, D, M, W = 1, 4096, 32, 8, 128, 64, 2048
+    d = prefill_inputs(7800, B, T, HQ, H, D, D, M, dtype=BF, qk_scale=D ** -0.5, gate_div=1.0, gate_mean=-1.0)
+    do = torch.randn(B, T, HQ, D, generator=torch.Generator().manual_seed(4)).to(BF)
+    grads = []
+    for dt in (BF, torch.float32):
+        x = [d[k].cuda().to(dt).requires_grad_(True) for k in KEYS]
+        o = chunk_nha(*x, window_size_left=W - 1, gsa_kv_shift=W)[0]
+        o.backward(do.cuda().to(dt))
+        grads.append([t.grad for t in x])
+        del x, o
+    for k, gb, gf in zip(KEYS, *grads):
+        check_grad(f"long context d{k}", gb, gf.double().cpu(), BF)
+
+
 def test_bwd_rejects_unsupported_shapes():
     from nha_amd import NhaError, chunk_nha
     d = prefill_inputs(7300, 1, 64, 2, 2, 64, 64, 128, dtype=torch.float32)

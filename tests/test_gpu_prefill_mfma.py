@@ -215,5 +215,9 @@ def test_mfma_layer_workloads_match_c_oracle(name):
     assert_close("lse_gsa", got[2], ref[2].double(), BF)
     assert_close("hk", got[3][0], ref[3].double(), BF)
     assert_close("hv", got[3][1], ref[4].double(), BF)
-    rel = ((got[0].double().cpu() - ref[0].double()).norm() / ref[0].double().norm()).item()
-    assert rel <= 5e-3, f"o: relative L2 error {rel:.3e}"
+    # the absolute bar says little where a tensor's values are small (final states of about 0.05 at these input
+    # scales): relative L2 error of every output as well (bf16 output rounding alone is 2^-9)
+    for nm, a, b in (("o", got[0], ref[0]), ("lse_swa", got[1], ref[1]), ("lse_gsa", got[2], ref[2]),
+                     ("hk", got[3][0], ref[3]), ("hv", got[3][1], ref[4])):
+        rel = ((a.double().cpu() - b.double()).norm() / b.double().norm()).item()
+        assert rel <= 5e-3, f"{nm}: relative L2 error {rel:.3e}"

@@ -81,3 +81,20 @@ def test_short_conv_fixed_length_batch():
     yr.sum().backward()
     assert_close("batch y", y.reshape(B * T, Cn), yr.detach(), torch.bfloat16)
     assert_close("batch dx", xd.grad.reshape(B * T, Cn), xr.grad, torch.bfloat16)
+
+
+def test_short_conv_rejects_operands_the_kernel_would_misread():
+    """Boundaries that do not end at the token count, a weight or bias of another channel count: refused on the host,
+    before any launch (the kernels index weight and bias by x's channels and walk cu_seqlens up to its last entry)."""
+    from nha_amd.ops import nha_short_conv
+    x = torch.zeros(1, 64, 32, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(32, 1, 4, dtype=torch.bfloat16, device="cuda")
+    good = torch.tensor([0, 20, 64], dtype=torch.int32, device="cuda")
+    assert nha_short_conv(x, w, None, cu_seqlens=good).shape == x.shape
+    for bad in ([0, 20, 60], [0, 20, 70], [4, 20, 64], [0, 40, 30, 64], [64]):
+        with pytest.raises(ValueError, match="cu_seqlens must rise"):
+            nha_short_conv(x, w, None, cu_seqlens=torch.tensor(bad, dtype=torch.int32, device="cuda"))
+    with pytest.raises(ValueError, match="weight must be"):
+        nha_short_conv(x, torch.zeros(16, 1, 4, dtype=torch.bfloat16, device="cuda"), None)
+    with pytest.raises(ValueError, match="bias must have"):
+        nha_short_conv(x, w, torch.zeros(16, dtype=torch.bfloat16, device="cuda"))

@@ -90,6 +90,46 @@ def test_ring_cache_counts_layers_and_windows_per_layer():
     assert not c.has_ring(0) and c.layer_tokens(0) == 0 and c.get_seq_length(0) == 0
 
 
+def test_cache_under_the_reference_name_takes_the_reference_constructor():
+    """`NHACache()` / `NHACache(seen_tokens)` / `NHACache.from_legacy_cache(None)` as the reference's callers build it
+    (scripts/verify_opt_parity.py:671; nha_cache.py:20-29, :167-182), then the window rule through `update` and
+    `get_pop_kvf` with the window size passed per call, as qwennha.py:151-176 does."""
+    from nha_fla.models.nha_cache import NHACache
+    W, H, D, M = 4, 2, 3, 5
+    for cache in (NHACache(), NHACache.from_legacy_cache(None), NHACache(0)):
+        assert cache.window_size is None and cache.seen_tokens == 0 and len(cache) == 0
+        gen = torch.Generator().manual_seed(0)
+        rows = [tuple(torch.randn(1, 1, H * d, generator=gen) for d in (D, D, M)) for _ in range(7)]
+        for t, row in enumerate(rows):
+            pop = cache.get_pop_kvf(0, W)
+            if t < W:
+                assert pop == (None, None, None)
+            else:                                     # the entry that leaves is the oldest one held
+                assert all(torch.equal(a, b) for a, b in zip(pop, rows[t - W]))
+            held = cache.update(attn_state=row, layer_idx=0, offset=1, cache_kwargs=dict(window_size=W))["attn_state"]
+            assert held[0].shape[-2] == min(t + 1, W) and torch.equal(held[0][..., -1:, :], row[0])
+        assert cache.seen_tokens == 7 and cache.get_seq_length(0) == 6
+    assert NHACache(5).seen_tokens == 5 and NHACache(5).window_size is None
+    with pytest.raises(ValueError, match="window size"):
+        c = NHACache()
+        c.update(attn_state=rows[0], layer_idx=0)
+        c.get_pop_kvf(0)
+
+
+def test_zero_sink_rescale_stays_finite_for_strongly_negative_window_scores():
+    """(e^lse + M) / (e^lse + n0) against float64 at lse = +-100, where e^-lse is outside fp32."""
+    from nha_amd.hybrid import zero_sink_rescale
+    lse = torch.tensor([-100.0, -100.0, -88.5, -30.0, 0.0, 3.0, 100.0, 100.0])
+    n0 = torch.tensor([3.0, 64.0, 1.0, 0.0, 7.0, 0.0, 0.0, 64.0])
+    got = zero_sink_rescale(lse, 64, n0)
+    ref = (torch.exp(lse.double()) + 64) / (torch.exp(lse.double()) + n0.double())
+    assert torch.isfinite(got).all()
+    assert torch.allclose(got.double(), ref, rtol=1e-5), (got, ref)
+    # no sink in view and a window weight below fp32: the ratio is capped, and a zero output row stays zero
+    capped = zero_sink_rescale(torch.tensor([-100.0]), 64, torch.tensor([0.0]))
+    assert torch.isfinite(capped).all() and float(capped * 0.0) == 0.0
+
+
 def test_reference_import_paths_resolve_to_these_modules():
     from nha_fla.models.qwen3_moe_nha.qwennha import Qwen3MoeNativeHybridAttention as A
     from nha_fla.models.llama3_nha.llamanha import LlamaNativeHybridAttention as B_
@@ -97,7 +137,7 @@ def test_reference_import_paths_resolve_to_these_modules():
     from nha_fla.ops.nha.chunk_fused import fused_chunk_nha_prefill as f
     import nha_amd
     assert A is nha_amd.Qwen3MoeNativeHybridAttention and B_ is nha_amd.LlamaNativeHybridAttention
-    assert NHACache is nha_amd.NHARingCache and f is nha_amd.fused_chunk_nha_prefill
+    assert NHACache is nha_amd.NHACache and issubclass(NHACache, nha_amd.NHARingCache) and f is nha_amd.fused_chunk_nha_prefill
     m = A(nha_amd.HybridNHAConfig(hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16, num_slots=8,
                                   block_size=2, transformer_idx=1), layer_idx=3)
     assert m.window_size == 2048 and not m.is_nha_layer and sorted(n for n, _ in m.named_parameters()) == [
@@ -107,20 +147,28 @@ def test_reference_import_paths_resolve_to_these_modules():
 
 
 # ----------------------------------------------------------------------------- GPU: the end-to-end case
-def _stack(tag, flavour, dev):
+# (q heads, kv heads, head size, slots, window of the NHA layers).  "small" runs the generic kernels; the other two are
+# head shapes of the converted models (eight / four query heads per kv-head at head size 128, 64 slots, window 64:
+# qwen3_moe_nha and llama3_nha), which the LDS-direct prefill, the matrix-core decode step and the hand-over of that
+# prefill's final state to the ring buffers serve.
+SHAPES = {"small": (8, 2, 32, 16, 32), "moe_heads": (32, 4, 128, 64, 64), "dense_heads": (8, 2, 128, 64, 64)}
+
+
+def _stack(tag, flavour, dev, shape="small"):
     from nha_amd.hybrid import HybridNHAConfig, Qwen3MoeNativeHybridAttention, LlamaNativeHybridAttention
-    cfg = HybridNHAConfig(hidden_size=256, num_attention_heads=8, num_key_value_heads=2, head_dim=32, num_slots=16,
-                          window_size=32, max_position_embeddings=4096,
+    HQ, H, D, M, W = SHAPES[shape]
+    cfg = HybridNHAConfig(hidden_size=256, num_attention_heads=HQ, num_key_value_heads=H, head_dim=D, num_slots=M,
+                          window_size=W, max_position_embeddings=4096,
                           block_size=2 if tag == "mixed" else None, transformer_idx=1 if tag == "mixed" else None)
     cls = Qwen3MoeNativeHybridAttention if flavour == "moe" else LlamaNativeHybridAttention
     gen = torch.Generator().manual_seed(1234)
     layers, refs = [], []
     for i in range(4):
-        w = _weights(gen, 256, 8, 2, 32, 16, flavour == "moe")
+        w = _weights(gen, 256, HQ, H, D, M, flavour == "moe")
         m = cls(cfg, layer_idx=i).to(torch.bfloat16)
         m.load_state_dict(w, strict=True)
         layers.append(m.to(dev).eval())
-        refs.append(HybridAttentionRef(w, num_heads=8, num_kv_heads=2, head_dim=32, num_slots=16, window_size=m.window_size,
+        refs.append(HybridAttentionRef(w, num_heads=HQ, num_kv_heads=H, head_dim=D, num_slots=M, window_size=m.window_size,
                                        qk_norm=flavour == "moe", round_to=torch.bfloat16))
     return cfg, layers, refs
 
@@ -157,16 +205,20 @@ def _close(name, got, ref, tol=2.5e-2):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("tag,flavour,B", [("nha", "moe", 1), ("nha", "moe", 4), ("mixed", "moe", 1), ("mixed", "moe", 4),
-                                           ("nha", "dense", 4), ("mixed", "dense", 1)])
-def test_stack_prompt_128_then_16_steps_matches_restated_modules(tag, flavour, B):
-    from nha_amd import NHARingCache
+@pytest.mark.parametrize("tag,flavour,B,shape", [
+    ("nha", "moe", 1, "small"), ("nha", "moe", 4, "small"), ("mixed", "moe", 1, "small"), ("mixed", "moe", 4, "small"),
+    ("nha", "dense", 4, "small"), ("mixed", "dense", 1, "small"),
+    ("nha", "moe", 2, "moe_heads"), ("mixed", "moe", 1, "moe_heads"), ("mixed", "dense", 2, "dense_heads")])
+def test_stack_prompt_128_then_16_steps_matches_restated_modules(tag, flavour, B, shape):
+    from nha_amd import NHACache, NHARingCache
     dev = torch.device("cuda:0")
-    cfg, layers, refs = _stack(tag, flavour, dev)
+    cfg, layers, refs = _stack(tag, flavour, dev, shape)
     gen = torch.Generator().manual_seed(99)
     x_pre = torch.randn(B, 128, 256, generator=gen).to(torch.bfloat16)
     x_dec = torch.randn(B, 16, 256, generator=gen).to(torch.bfloat16)
-    cache, ref_caches = NHARingCache(cfg.window_size), [{} for _ in refs]
+    # the cache under the reference's name and constructor for the model head shapes, the ring cache's own otherwise
+    cache = NHACache() if shape != "small" else NHARingCache(cfg.window_size)
+    ref_caches = [{} for _ in refs]
     with torch.no_grad():
         pos = torch.arange(128)[None].expand(B, -1)
         got = _run_stack(layers, x_pre.to(dev), pos.to(dev), cache)
@@ -184,7 +236,7 @@ def test_stack_prompt_128_then_16_steps_matches_restated_modules(tag, flavour, B
         k, v, g = cache.window(i)
         n = min(144, m.window_size)
         pos = torch.arange(144 - n, 144)[None].expand(B, -1)
-        cos, sin = (t.to(torch.bfloat16).to(F64) for t in _rope_tables(pos, 32, 10000.0))
+        cos, sin = (t.to(torch.bfloat16).to(F64) for t in _rope_tables(pos, cfg.head_dim, 10000.0))
         _close(f"layer {i} window keys", k, _rotate_half(ref_caches[i]["k"], cos, sin))
         _close(f"layer {i} window values", v, ref_caches[i]["v"])
         if m.is_nha_layer:
@@ -196,21 +248,23 @@ def test_stack_prompt_128_then_16_steps_matches_restated_modules(tag, flavour, B
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("grad", [False, True])
-def test_zero_sink_layer_prompt_longer_than_its_window(grad):
+@pytest.mark.parametrize("HQ,H,D", [(4, 2, 64), (8, 2, 128)])
+def test_zero_sink_layer_prompt_longer_than_its_window(grad, HQ, H, D):
     """A layer of the zero-sink kind whose window (96) the prompt (300 tokens) outgrows: the number of
     visible sinks falls from M to 0 along the prompt, which the per-query rescaling has to follow.  With
-    gradients enabled the same numbers come out of the differentiable op."""
+    gradients enabled the same numbers come out of the differentiable op.  The second head shape (four query
+    heads per kv-head at head size 128) is served by the LDS-direct prefill kernel."""
     from nha_amd.hybrid import HybridNHAConfig, Qwen3MoeNativeHybridAttention
     dev = torch.device("cuda:0")
-    cfg = HybridNHAConfig(hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=64, num_slots=64, window_size=32)
+    cfg = HybridNHAConfig(hidden_size=128, num_attention_heads=HQ, num_key_value_heads=H, head_dim=D, num_slots=64, window_size=32)
     gen = torch.Generator().manual_seed(5)
-    w = _weights(gen, 128, 4, 2, 64, 64, True, bias=True)
+    w = _weights(gen, 128, HQ, H, D, 64, True, bias=True)
     cfg.attention_bias = True
     m = Qwen3MoeNativeHybridAttention(cfg, 0).to(torch.bfloat16)
     m.load_state_dict(w)
     m = m.to(dev).eval()
     m.window_size = 96
-    ref = HybridAttentionRef(w, num_heads=4, num_kv_heads=2, head_dim=64, num_slots=64, window_size=96, qk_norm=True,
+    ref = HybridAttentionRef(w, num_heads=HQ, num_kv_heads=H, head_dim=D, num_slots=64, window_size=96, qk_norm=True,
                              round_to=torch.bfloat16)
     x = (torch.randn(2, 300, 128, generator=gen) * 2).to(torch.bfloat16)
     pos = torch.arange(300)[None].expand(2, -1)
@@ -250,7 +304,9 @@ def test_left_padded_prompt_and_steps():
         _close("prompt without padding", got[0], want[0])
         _close("padded prompt", got[1, 9:], want[1, 9:])
         for t in range(70, 74):
-            got, _ = m(x[:, t:t + 1].to(dev), attention_mask=mask[:, :t + 1].to(dev), position_ids=pos[:, t:t + 1].to(dev),
+            # steps 70 and 72 pass the mask in its four-dimensional form [batch, 1, queries, tokens] (qwennha.py:133-136)
+            mk = mask[:, :t + 1] if t % 2 else mask[:, None, None, :t + 1]
+            got, _ = m(x[:, t:t + 1].to(dev), attention_mask=mk.to(dev), position_ids=pos[:, t:t + 1].to(dev),
                        past_key_value=cache, use_cache=True)
             _close(f"padded step {t}", got, ref.forward(x[:, t:t + 1], pos[:, t:t + 1], rc, attention_mask=mask[:, :t + 1]))
 
