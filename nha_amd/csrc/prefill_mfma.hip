@@ -65,10 +65,10 @@ __device__ __forceinline__ void tile_r2l(lbf16* lds, const TileRegs<ROWS, D, NTH
 // segment and stores, per chunk, the local chunk-start states, the gate cumsum table and the
 // decay accumulated since the segment start; per segment, the local end state and total decay.
 // Level 2 carries the true state across segments element-wise, h_seg[s+1] = h_seg[s] * dtot[s] + hend[s],
-// in one of two forms.  The forward (state_final_kernel) turns every chunk-start state of the
-// segment into the true one on the way, h_loc + h_seg * dcum, rounded to bf16 in place, so that the
-// output pass reads plain operand tiles.  The backward (state_scan_kernel) keeps the segment-local
-// states and writes the segment-start states h_seg beside them: it needs the sum in fp32.
+// in one of two forms.  The forward turns every chunk-start state into the true one, h_loc + h_seg * dcum,
+// rounded to bf16 in place, so that the output pass reads plain operand tiles (state_final_kernel inside the
+// scan, or state_scan_kernel followed by state_apply_kernel).  The backward (state_scan_kernel) keeps the
+// segment-local states and writes the segment-start states h_seg beside them: it needs the sum in fp32.
 // Both states are kept as C[d][m] accumulators (slot m = lane % 16).
 
 // DW: columns of the state one workgroup carries (D, or D/2: twice the workgroups with half the
@@ -257,37 +257,97 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   if (kb == 0 && !isv && lead) p.dtot[sl * MS + m] = fexp(gsum);
 }
 
-// Level 2: one thread per state element, sequential over the segments of its sequence.
-// grid (N*H, 2*MS*D/256): the first MS*D elements are the k-state ([m][d]), the rest the v-state.
+// Level 2, the scan: four consecutive d of one slot per thread, sequential over the segments of its sequence;
+// writes the true segment-start states h_seg and the final states.  The loads do not depend on the chain, so the
+// end states and decays of SCAN_AHEAD segments are requested together, one group ahead of the group that is
+// being combined: a thread waits for memory once per group, not once per segment.
+// grid (N*H, 2*MS*D/1024): the first MS*D/4 groups are the k-state ([m][d]), the rest the v-state.
+constexpr int SCAN_AHEAD = 4;
+
 template <int D>
 __global__ __launch_bounds__(256) void state_scan_kernel(const MP p) {
   const int H = p.H;
   const int n = blockIdx.x / H, h = blockIdx.x % H;
-  const int e = blockIdx.y * 256 + threadIdx.x;
-  const bool isv = e >= MS * D;
-  const int em = isv ? e - MS * D : e;
+  const int e4 = blockIdx.y * 256 + threadIdx.x;
+  const bool isv = e4 >= MS * D / 4;
+  const int em = (isv ? e4 - MS * D / 4 : e4) * 4;
   const int m = em / D, d = em % D;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int nchunks = (eos - bos + BT - 1) / BT;
   const int nseg = (nchunks + SEG - 1) / SEG;
-  float hcur = 0.f;
-  if (p.h0k) hcur = isv ? p.h0v[(((int64_t)n * H + h) * MS + m) * D + d] : p.h0k[(((int64_t)n * H + h) * D + d) * MS + m];
-  const float* hend = isv ? p.hend_v : p.hend_k;
-  float* hseg = isv ? p.hseg_v : p.hseg_k;
+  float4 hcur = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (p.h0k) {
+    if (isv) {
+      hcur = *reinterpret_cast<const float4*>(p.h0v + (((int64_t)n * H + h) * MS + m) * D + d);
+    } else {
+      const float* src = p.h0k + (((int64_t)n * H + h) * D + d) * MS + m;
+      hcur = make_float4(src[0], src[MS], src[2 * MS], src[3 * MS]);
+    }
+  }
+  const float* __restrict__ hend = isv ? p.hend_v : p.hend_k;
+  float* __restrict__ hseg = isv ? p.hseg_v : p.hseg_k;
+  const float* __restrict__ dtot = p.dtot;
   const int slot0 = p.coff[n] / SEG + n;
-  for (int sg = 0; sg < nseg; ++sg) {
-    const int64_t sl = (int64_t)(slot0 + sg) * H + h;
-    hseg[(sl * MS + m) * D + d] = hcur;
-    hcur = hcur * p.dtot[sl * MS + m] + hend[(sl * MS + m) * D + d];
+  struct Grp {
+    float4 he[SCAN_AHEAD];
+    float dt[SCAN_AHEAD];
+  };
+  auto request = [&](Grp& g, int sg0) {
+#pragma unroll
+    for (int i = 0; i < SCAN_AHEAD; ++i) {
+      g.he[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      g.dt[i] = 0.f;
+      if (sg0 + i < nseg) {
+        const int64_t sl = (int64_t)(slot0 + sg0 + i) * H + h;
+        g.he[i] = *reinterpret_cast<const float4*>(hend + (sl * MS + m) * D + d);
+        g.dt[i] = dtot[sl * MS + m];
+      }
+    }
+  };
+  Grp cur, nxt;
+  request(cur, 0);
+  for (int sg0 = 0; sg0 < nseg; sg0 += SCAN_AHEAD) {
+    if (sg0 + SCAN_AHEAD < nseg) request(nxt, sg0 + SCAN_AHEAD);
+#pragma unroll
+    for (int i = 0; i < SCAN_AHEAD; ++i) {
+      if (sg0 + i < nseg) {
+        const int64_t sl = (int64_t)(slot0 + sg0 + i) * H + h;
+        *reinterpret_cast<float4*>(hseg + (sl * MS + m) * D + d) = hcur;
+        hcur.x = hcur.x * cur.dt[i] + cur.he[i].x;
+        hcur.y = hcur.y * cur.dt[i] + cur.he[i].y;
+        hcur.z = hcur.z * cur.dt[i] + cur.he[i].z;
+        hcur.w = hcur.w * cur.dt[i] + cur.he[i].w;
+      }
+    }
+    cur = nxt;
   }
   if (p.hkt) {
-    if (isv) p.hvt[(((int64_t)n * H + h) * MS + m) * D + d] = hcur;
-    else p.hkt[(((int64_t)n * H + h) * D + d) * MS + m] = hcur;
+    if (isv) {
+      *reinterpret_cast<float4*>(p.hvt + (((int64_t)n * H + h) * MS + m) * D + d) = hcur;
+    } else {
+      float* dst = p.hkt + (((int64_t)n * H + h) * D + d) * MS + m;
+      dst[0] = hcur.x; dst[MS] = hcur.y; dst[2 * MS] = hcur.z; dst[3 * MS] = hcur.w;
+    }
   }
 }
 
-// Level 2, forward form: four consecutive d of one slot per thread, sequential over the segments
-// of its sequence; the loads of the next segment are requested before the current one is combined.
+// Level 2, forward form: every chunk-start state becomes the true one, h_loc + h_seg * dcum, rounded to bf16 in
+// place, so that the output pass reads plain operand tiles.
+//
+// Where the carried part h_seg * dcum is below CARRY_FLOOR in absolute value for all four elements of a thread,
+// the local state is left as it is -- neither read nor written: the sum would be the local state again to within
+// 2^-100, fifty binary orders below anything bf16 tensors of representable magnitude can show.  Gates that forget
+// quickly (log-gates of about -1 per token: e^-80 per chunk) leave only the first chunk of a segment to rewrite;
+// with slow gates (the layers' logsigmoid / 8: e^-5 per chunk) every chunk is rewritten.
+//
+// Two forms.  state_final_kernel does it inside the scan (no h_seg round trip through memory; a thread's chain
+// costs about a memory latency per segment): for sequences of a few segments.  state_apply_kernel runs after
+// state_scan_kernel, one thread per (segment, slot, four d) with no chain: for long sequences.
+constexpr float CARRY_FLOOR = 0x1p-100f;
+
+// Four consecutive d of one slot per thread, sequential over the segments of its sequence; the small loads of
+// segment sg + 2 (decays, end state) and the local states of segment sg + 1 that need rewriting are requested
+// before segment sg is combined.
 // grid (N*H, 2*MS*D/1024): the first MS*D/4 groups are the k-state ([m][d]), the rest the v-state.
 template <int D>
 __global__ __launch_bounds__(256) void state_final_kernel(const MP p) {
@@ -314,50 +374,70 @@ __global__ __launch_bounds__(256) void state_final_kernel(const MP p) {
   bf16_t* hloc = isv ? p.hvc : p.hkT;
   const int chunk0 = p.coff[n];
   const int slot0 = chunk0 / SEG + n;
-  struct SegRegs {
-    uint2 loc[SEG];
+  struct Small {      // what the chain itself needs of a segment
     float dc[SEG];
     float dt;
     float4 he;
   };
-  auto request = [&](SegRegs& r, int sg) {
+  struct Loc {        // local chunk-start states of a segment (those that are rewritten)
+    uint2 v[SEG];
+    unsigned need;
+  };
+  auto request_small = [&](Small& r, int sg) {
     const int64_t sl = (int64_t)(slot0 + sg) * H + h;
 #pragma unroll
     for (int jc = 0; jc < SEG; ++jc) {
-      r.loc[jc] = make_uint2(0, 0);
       r.dc[jc] = 0.f;
-      if (sg * SEG + jc < nchunks) {
-        const int64_t cg = (int64_t)(chunk0 + sg * SEG + jc) * H + h;
-        r.loc[jc] = *reinterpret_cast<const uint2*>(hloc + (cg * MS + m) * D + d);
-        r.dc[jc] = p.dcum[cg * MS + m];
-      }
+      if (sg * SEG + jc < nchunks) r.dc[jc] = p.dcum[((int64_t)(chunk0 + sg * SEG + jc) * H + h) * MS + m];
     }
     r.dt = p.dtot[sl * MS + m];
     r.he = *reinterpret_cast<const float4*>(hend + (sl * MS + m) * D + d);
   };
-  SegRegs cur, nxt;
-  request(cur, 0);
-  for (int sg = 0; sg < nseg; ++sg) {
-    if (sg + 1 < nseg) request(nxt, sg + 1);
+  // hs: the state that enters segment sg
+  auto request_loc = [&](Loc& r, const Small& sm, int sg, const float (&hs)[4]) {
+    const float amax = fmaxf(fmaxf(fabsf(hs[0]), fabsf(hs[1])), fmaxf(fabsf(hs[2]), fabsf(hs[3])));
+    r.need = 0;
 #pragma unroll
     for (int jc = 0; jc < SEG; ++jc) {
-      if (sg * SEG + jc < nchunks) {
+      r.v[jc] = make_uint2(0, 0);
+      if (sg * SEG + jc < nchunks && amax * sm.dc[jc] >= CARRY_FLOOR) {
+        r.need |= 1u << jc;
+        r.v[jc] = *reinterpret_cast<const uint2*>(hloc + (((int64_t)(chunk0 + sg * SEG + jc) * H + h) * MS + m) * D + d);
+      }
+    }
+  };
+  Small s_cur, s_nxt, s_nn;
+  Loc l_cur, l_nxt;
+  request_small(s_cur, 0);
+  if (nseg > 1) request_small(s_nxt, 1);
+  request_loc(l_cur, s_cur, 0, hcur);
+  for (int sg = 0; sg < nseg; ++sg) {
+    float hn[4];
+    hn[0] = hcur[0] * s_cur.dt + s_cur.he.x;
+    hn[1] = hcur[1] * s_cur.dt + s_cur.he.y;
+    hn[2] = hcur[2] * s_cur.dt + s_cur.he.z;
+    hn[3] = hcur[3] * s_cur.dt + s_cur.he.w;
+    if (sg + 2 < nseg) request_small(s_nn, sg + 2);
+    if (sg + 1 < nseg) request_loc(l_nxt, s_nxt, sg + 1, hn);
+#pragma unroll
+    for (int jc = 0; jc < SEG; ++jc) {
+      if (l_cur.need & (1u << jc)) {
         const int64_t cg = (int64_t)(chunk0 + sg * SEG + jc) * H + h;
-        const uint32_t w[2] = {cur.loc[jc].x, cur.loc[jc].y};
+        const uint32_t w[2] = {l_cur.v[jc].x, l_cur.v[jc].y};
         bf16x4 o4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float a0 = __uint_as_float((i & 1) ? (w[i >> 1] & 0xffff0000u) : (w[i >> 1] << 16));
-          o4[i] = (__bf16)(a0 + hcur[i] * cur.dc[jc]);
+          o4[i] = (__bf16)(a0 + hcur[i] * s_cur.dc[jc]);
         }
         *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + d) = o4;
       }
     }
-    hcur[0] = hcur[0] * cur.dt + cur.he.x;
-    hcur[1] = hcur[1] * cur.dt + cur.he.y;
-    hcur[2] = hcur[2] * cur.dt + cur.he.z;
-    hcur[3] = hcur[3] * cur.dt + cur.he.w;
-    cur = nxt;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hcur[i] = hn[i];
+    s_cur = s_nxt;
+    s_nxt = s_nn;
+    l_cur = l_nxt;
   }
   if (p.hkt) {
     if (isv) {
@@ -365,6 +445,64 @@ __global__ __launch_bounds__(256) void state_final_kernel(const MP p) {
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) p.hkt[(((int64_t)n * H + h) * D + d + i) * MS + m] = hcur[i];
+    }
+  }
+}
+
+// After state_scan_kernel: one thread per (segment, kv-head, slot, four consecutive d), every segment at once.
+// grid (segment slots, H, 2*MS*D/1024): the first MS*D/4 groups of z are the k-state ([m][d]), the rest the v-state.
+template <int D>
+__global__ __launch_bounds__(256) void state_apply_kernel(const MP p) {
+  const int H = p.H;
+  const int slot = blockIdx.x, h = blockIdx.y;
+  int n = 0;
+  {
+    int lo = 0, hi = p.N - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.coff[mid] / SEG + mid <= slot) lo = mid; else hi = mid - 1;
+    }
+    n = lo;
+  }
+  const int it0 = (slot - (p.coff[n] / SEG + n)) * SEG;
+  const int nchunks = p.coff[n + 1] - p.coff[n];
+  if (it0 >= nchunks) return;
+  const int nloc = (nchunks - it0) < SEG ? (nchunks - it0) : SEG;
+  const int e4 = blockIdx.z * 256 + threadIdx.x;
+  const bool isv = e4 >= MS * D / 4;
+  const int em = (isv ? e4 - MS * D / 4 : e4) * 4;
+  const int m = em / D, d = em % D;
+  const int64_t sl = (int64_t)slot * H + h;
+  const float4 hs = *reinterpret_cast<const float4*>((isv ? p.hseg_v : p.hseg_k) + (sl * MS + m) * D + d);
+  const float amax = fmaxf(fmaxf(fabsf(hs.x), fabsf(hs.y)), fmaxf(fabsf(hs.z), fabsf(hs.w)));
+  if (!(amax >= CARRY_FLOOR)) return;      // nothing is carried into this segment (its first, without initial state)
+  bf16_t* hloc = isv ? p.hvc : p.hkT;
+  const int64_t cg0 = (int64_t)(p.coff[n] + it0) * H + h;
+  float dc[SEG];
+#pragma unroll
+  for (int jc = 0; jc < SEG; ++jc) dc[jc] = jc < nloc ? p.dcum[(cg0 + (int64_t)jc * H) * MS + m] : 0.f;
+  uint2 loc[SEG];
+  unsigned need = 0;
+#pragma unroll
+  for (int jc = 0; jc < SEG; ++jc) {
+    loc[jc] = make_uint2(0, 0);
+    if (amax * dc[jc] >= CARRY_FLOOR) {
+      need |= 1u << jc;
+      loc[jc] = *reinterpret_cast<const uint2*>(hloc + ((cg0 + (int64_t)jc * H) * MS + m) * D + d);
+    }
+  }
+  const float hv4[4] = {hs.x, hs.y, hs.z, hs.w};
+#pragma unroll
+  for (int jc = 0; jc < SEG; ++jc) {
+    if (need & (1u << jc)) {
+      const uint32_t w[2] = {loc[jc].x, loc[jc].y};
+      bf16x4 o4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = __uint_as_float((i & 1) ? (w[i >> 1] & 0xffff0000u) : (w[i >> 1] << 16));
+        o4[i] = (__bf16)(a0 + hv4[i] * dc[jc]);
+      }
+      *reinterpret_cast<bf16x4*>(hloc + ((cg0 + (int64_t)jc * H) * MS + m) * D + d) = o4;
     }
   }
 }
@@ -1179,8 +1317,16 @@ int run_state_pass(const MP& p, bool segment_form, hipStream_t st) {
   }
   hipLaunchKernelGGL((mfma_state_local_kernel<D, DW>), dim3(p.NT / SEG + p.N + 1, p.H, 2 * (D / DW)), dim3(256), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
-  if (segment_form) hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 256), dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((state_final_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);
+  // the forward's chunk states: inside the scan while a sequence has about eight segments or fewer (a thread's
+  // chain there costs a memory latency per segment: 15 us at 4 segments, 21 us at 16 on one box), after it beyond
+  // (two launches without a chain: 16-18 us whatever the length)
+  const bool in_scan = !segment_form && (int64_t)p.NT <= (int64_t)8 * SEG * p.N;
+  if (in_scan) {
+    hipLaunchKernelGGL((state_final_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);
+  } else {
+    hipLaunchKernelGGL((state_scan_kernel<D>), dim3(p.N * p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);
+    if (!segment_form) hipLaunchKernelGGL((state_apply_kernel<D>), dim3(p.NT / SEG + p.N + 1, p.H, 2 * MS * D / 1024), dim3(256), 0, st, p);
+  }
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 2)");
   return NHA_OK;
 }

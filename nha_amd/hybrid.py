@@ -83,12 +83,20 @@ class RotaryTables(nn.Module):
 
     def __init__(self, head_dim: int, base: float = 10000.0):
         super().__init__()
-        inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
-        self.register_buffer("inv_freq", inv_freq, persistent=False)
+        self.head_dim, self.base = head_dim, base
+        self._inv_freq = {}          # per device; not a buffer: `module.to(torch.bfloat16)` would round a buffer, and
+                                     # frequencies rounded to 8 bits put position 100 off by a quarter of a radian
+
+    def inv_freq(self, device) -> torch.Tensor:
+        f = self._inv_freq.get(device)
+        if f is None:
+            f = 1.0 / (self.base ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim))
+            f = self._inv_freq[device] = f.to(device)
+        return f
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor, position_ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-        ang = position_ids.to(self.inv_freq.device, torch.float32)[..., None] * self.inv_freq
+        ang = position_ids.to(x.device, torch.float32)[..., None] * self.inv_freq(x.device)
         emb = torch.cat([ang, ang], -1)
         return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
 
