@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 7
+#define NHA_ABI_VERSION 8
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -83,8 +83,6 @@ typedef struct NhaPrefillArgs {
   int32_t shift;  /* gsa_kv_shift */
   int32_t dtype;  /* NHA_DTYPE_* of q/k/v/s/g/o */
   int32_t impl;   /* NHA_IMPL_* */
-  int32_t phases; /* 0 or 3 = whole op; 1 = state pass only (fills scratch, final states);
-                     2 = output pass only (scratch must hold a prior state pass of the same inputs) */
   float scale;
   void* stream;
 } NhaPrefillArgs;

@@ -14,7 +14,7 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 7
+ABI_VERSION = 8
 NHA_NOALLOC_SCRATCH_BYTES = 32 << 20   # workspace of nha_prefill_fwd_noalloc (include/nha_hip.h)
 NHA_FMAP_NONE, NHA_FMAP_SWISH, NHA_FMAP_RELU = 0, 1, 2
 
@@ -37,7 +37,7 @@ class NhaPrefillArgs(C.Structure):
         ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t),
         ("T_tot", C.c_int32), ("N", C.c_int32), ("NT", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32),
         ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
-        ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32), ("impl", C.c_int32), ("phases", C.c_int32),
+        ("wl", C.c_int32), ("shift", C.c_int32), ("dtype", C.c_int32), ("impl", C.c_int32),
         ("scale", C.c_float), ("stream", C.c_void_p),
     ]
 

@@ -25,7 +25,6 @@ static int check_prefill(const NhaPrefillArgs* a, bool pointers, bool own_scratc
   NHA_CHECK_ARG(a->shift >= 0, "nha_prefill: gsa_kv_shift must be >= 0, got %d", a->shift);
   NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_prefill: bad dtype %d", a->dtype);
   NHA_CHECK_ARG(a->impl >= NHA_IMPL_AUTO && a->impl <= NHA_IMPL_MFMA, "nha_prefill: bad impl %d", a->impl);
-  NHA_CHECK_ARG(a->phases >= 0 && a->phases <= 3, "nha_prefill: bad phases %d", a->phases);
   if (pointers) {
     NHA_CHECK_ARG(a->q_swa && a->k_swa && a->q_gsa && a->k_gsa && a->v && a->s && a->g && a->o,
                   "nha_prefill_fwd: q_swa, k_swa, q_gsa, k_gsa, v, s, g, o are required");
@@ -108,7 +107,23 @@ size_t nha_prefill_scratch_bytes(const NhaPrefillArgs* a) {
   return use_mfma(a) ? prefill_mfma_scratch_bytes(a) : prefill_simple_scratch_bytes(a);
 }
 
-int nha_prefill_fwd(const NhaPrefillArgs* a) {
+// The forward in parts, for measurements (bench.py times the state pass and the output pass apart): phase 1 = the
+// state pass only (fills the scratch, writes the final states), 2 = the output pass only (the scratch must hold a
+// state pass of the same inputs), 0 = the whole op.  Exported, but no part of the public header: a user's call is
+// nha_prefill_fwd.
+static int prefill_fwd_phase(const NhaPrefillArgs* a, int phase);
+
+int nha_internal_prefill_fwd_phase(const NhaPrefillArgs* a, int phase) {
+  if (phase < 0 || phase > 2) {
+    set_error("nha_internal_prefill_fwd_phase: bad phase %d", phase);
+    return NHA_ERR_INVALID;
+  }
+  return prefill_fwd_phase(a, phase);
+}
+
+int nha_prefill_fwd(const NhaPrefillArgs* a) { return prefill_fwd_phase(a, 0); }
+
+static int prefill_fwd_phase(const NhaPrefillArgs* a, int phase) {
   int rc = check_prefill(a, true);
   if (rc != NHA_OK) return rc;
   const bool mfma = use_mfma(a);
@@ -122,7 +137,7 @@ int nha_prefill_fwd(const NhaPrefillArgs* a) {
     set_error("nha_prefill_fwd: scratch has %zu bytes, %zu needed", a->scratch_bytes, need);
     return NHA_ERR_SCRATCH;
   }
-  return mfma ? prefill_mfma_impl(a) : prefill_simple_impl(a);
+  return mfma ? prefill_mfma_impl(a, phase) : prefill_simple_impl(a, phase);
 }
 
 int nha_prefill_fwd_noalloc(const NhaPrefillArgs* a) {
@@ -148,7 +163,7 @@ int nha_prefill_fwd_noalloc(const NhaPrefillArgs* a) {
   NhaPrefillArgs b = *a;
   b.scratch = ptr;
   b.scratch_bytes = (size_t)NHA_NOALLOC_SCRATCH_BYTES;
-  return mfma ? prefill_mfma_impl(&b) : prefill_simple_impl(&b);
+  return mfma ? prefill_mfma_impl(&b, 0) : prefill_simple_impl(&b, 0);
 }
 
 size_t nha_prefill_bwd_scratch_bytes(const NhaPrefillBwdArgs* a) {

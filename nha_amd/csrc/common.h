@@ -140,10 +140,11 @@ int decode_advance_impl(int32_t* count, int32_t B, void* stream);
 bool decode_mfma_supported(const NhaDecodeArgs* a);
 int decode_mfma_impl(const NhaDecodeArgs* a);
 size_t prefill_simple_scratch_bytes(const NhaPrefillArgs* a);
-int prefill_simple_impl(const NhaPrefillArgs* a);
+// phase: 0 = whole op, 1 = state pass only, 2 = output pass only (scratch filled by an earlier state pass)
+int prefill_simple_impl(const NhaPrefillArgs* a, int phase);
 bool prefill_mfma_supported(const NhaPrefillArgs* a);
 size_t prefill_mfma_scratch_bytes(const NhaPrefillArgs* a);
-int prefill_mfma_impl(const NhaPrefillArgs* a);
+int prefill_mfma_impl(const NhaPrefillArgs* a, int phase);
 int prefill_mfma_export_states(const NhaPrefillArgs* a, float* gc, float* hkc, float* hkct, float* hvct, void* hkb, void* hvb,
                                void* hkl, void* hvl, int* big);
 int bwd_slot_products3(const NhaPrefillBwdArgs* a, int which, const int* big, const bf16_t* ap, const bf16_t* bp, const float* ust,

@@ -686,9 +686,12 @@ int decode_step_impl(const NhaDecodeArgs* a) {
     set_error("nha_decode_step: cos/sin strides must be multiples of 8 elements");
     return NHA_ERR_UNSUPPORTED;
   }
-  // matrix-core kernel for the common bf16 shapes (NHA_DECODE_VALU=1 keeps the VALU kernels, for
-  // comparisons)
+  // matrix-core kernel for the common bf16 shapes
+#ifdef NHA_AB_SWITCHES   // measurement builds only (-DNHA_AB_SWITCHES): NHA_DECODE_VALU=1 keeps the VALU kernels
   static const bool valu_only = getenv("NHA_DECODE_VALU") != nullptr;
+#else
+  constexpr bool valu_only = false;
+#endif
   if (!valu_only && decode_mfma_supported(a)) return decode_mfma_impl(a);
   int G = 1;
   while (G < NG) G <<= 1;

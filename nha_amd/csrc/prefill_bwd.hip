@@ -1042,7 +1042,7 @@ NhaPrefillArgs forward_args(const NhaPrefillBwdArgs* a) {
   f.h0k = a->h0k; f.h0v = a->h0v;
   f.cu_seqlens = a->cu_seqlens; f.chunk_indices = a->chunk_indices; f.chunk_offsets = a->chunk_offsets;
   f.T_tot = a->T_tot; f.N = a->N; f.NT = a->NT; f.HQ = a->HQ; f.H = a->H; f.K = a->K; f.V = a->V; f.M = a->M;
-  f.wl = a->wl; f.shift = a->shift; f.dtype = a->dtype; f.impl = NHA_IMPL_SIMPLE; f.phases = 1;
+  f.wl = a->wl; f.shift = a->shift; f.dtype = a->dtype; f.impl = NHA_IMPL_SIMPLE;
   f.scale = a->scale; f.stream = a->stream;
   return f;
 }
@@ -1061,7 +1061,11 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   float* hkc = (float*)fs;
   fs += aligned((size_t)a->NT * a->H * a->K * a->M * 4);
   float* hvc = (float*)fs;
+#ifdef NHA_AB_SWITCHES   // measurement builds only (-DNHA_AB_SWITCHES)
   static const bool intra_mfma = getenv("NHA_BWD_INTRA_VALU") == nullptr;
+#else
+  constexpr bool intra_mfma = true;
+#endif
   int rc;
   if (sp.use_mfma) {
     f.impl = NHA_IMPL_MFMA;
@@ -1078,7 +1082,7 @@ int run_bwd(const NhaPrefillBwdArgs* a) {
   } else {
     f.scratch = sc + sp.fwd;
     f.scratch_bytes = prefill_simple_scratch_bytes(&f);
-    rc = prefill_simple_impl(&f);
+    rc = prefill_simple_impl(&f, 1);   // the state pass only
   }
   if (rc != NHA_OK) return rc;
 

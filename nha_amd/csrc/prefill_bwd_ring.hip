@@ -588,7 +588,11 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
 // Served: four (or a multiple of four) query heads per kv-head at D = 128, tensors of one call below 4 GiB
 // (32-bit lane offsets of the LDS-direct loads).
 bool bwd_ring_supported(const NhaPrefillBwdArgs* a) {
-  static const bool off = getenv("NHA_BWD_NO_RING") != nullptr;   // A/B switch for measurements
+#ifdef NHA_AB_SWITCHES   // measurement builds only (-DNHA_AB_SWITCHES)
+  static const bool off = getenv("NHA_BWD_NO_RING") != nullptr;
+#else
+  constexpr bool off = false;
+#endif
   if (off || a->K != 128 || a->V != 128 || a->HQ % a->H != 0 || (a->HQ / a->H) % 4 != 0) return false;
   return (int64_t)a->T_tot * a->HQ * 128 * 2 < ((int64_t)1 << 32);
 }

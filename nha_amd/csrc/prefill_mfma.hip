@@ -1346,7 +1346,11 @@ int run_mfma(const MP& p, int phases, hipStream_t st) {
     // or 16 (G = 2) query rows, two per SIMD; D = 256: 32-key tiles and 16-row waves to fit the
     // register file and LDS
     int rc;
-    static const bool ring_off = getenv("NHA_PREFILL_NO_RING") != nullptr;   // A/B switch for measurements
+#ifdef NHA_AB_SWITCHES   // measurement builds only (-DNHA_AB_SWITCHES): run the kernels the LDS-direct ones replaced
+    static const bool ring_off = getenv("NHA_PREFILL_NO_RING") != nullptr;
+#else
+    constexpr bool ring_off = false;
+#endif
     if (!ring_off && prefill_ring_supported(p, D)) {
       rc = prefill_ring_launch(p, D, st);
     } else if (!ring_off && prefill_ring256_supported(p, D)) {
@@ -1428,12 +1432,12 @@ MP make_mp(const NhaPrefillArgs* a) {
 }
 }  // namespace
 
-int prefill_mfma_impl(const NhaPrefillArgs* a) {
+int prefill_mfma_impl(const NhaPrefillArgs* a, int phase) {
   const MP p = make_mp(a);
   hipStream_t st = (hipStream_t)a->stream;
-  if (a->K == 64) return run_mfma<64>(p, a->phases, st);
-  if (a->K == 128) return run_mfma<128>(p, a->phases, st);
-  return run_mfma<256>(p, a->phases, st);
+  if (a->K == 64) return run_mfma<64>(p, phase, st);
+  if (a->K == 128) return run_mfma<128>(p, phase, st);
+  return run_mfma<256>(p, phase, st);
 }
 
 // Runs the state pass of `a` in the segment form and exports it; gc [T_tot][H][M], hkc

@@ -279,7 +279,7 @@ size_t prefill_simple_scratch_bytes(const NhaPrefillArgs* a) {
 }
 
 template <typename T>
-static int run_simple(const NhaPrefillArgs* a) {
+static int run_simple(const NhaPrefillArgs* a, int phase) {
   SP p;
   p.q_swa = a->q_swa; p.k_swa = a->k_swa; p.q_gsa = a->q_gsa; p.k_gsa = a->k_gsa;
   p.v = a->v; p.s = a->s; p.g = a->g; p.o = a->o;
@@ -302,24 +302,24 @@ static int run_simple(const NhaPrefillArgs* a) {
     set_error("nha_prefill_fwd(simple): head dims too large for the generic kernels (K=%d V=%d M=%d)", a->K, a->V, a->M);
     return NHA_ERR_UNSUPPORTED;
   }
-  if (a->phases != 2) {
+  if (phase != 2) {
     hipLaunchKernelGGL((simple_state_kernel<T>), dim3(a->N * a->H, (a->M + BMS - 1) / BMS), dim3(256), lds1, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(simple state pass)");
   }
-  if (a->phases != 1) {
+  if (phase != 1) {
     hipLaunchKernelGGL((simple_out_kernel<T>), dim3(a->NT * BT, a->HQ), dim3(256), lds2, st, p);
     NHA_CHECK_LAUNCH("nha_prefill_fwd(simple output pass)");
   }
   return NHA_OK;
 }
 
-int prefill_simple_impl(const NhaPrefillArgs* a) {
+int prefill_simple_impl(const NhaPrefillArgs* a, int phase) {
   if (a->V > 1024 * 64) {
     set_error("nha_prefill_fwd(simple): V too large");
     return NHA_ERR_UNSUPPORTED;
   }
-  if (a->dtype == NHA_DTYPE_BF16) return run_simple<bf16_t>(a);
-  return run_simple<float>(a);
+  if (a->dtype == NHA_DTYPE_BF16) return run_simple<bf16_t>(a, phase);
+  return run_simple<float>(a, phase);
 }
 
 }  // namespace nha

@@ -39,7 +39,7 @@ def test_struct_sizes_match_the_header(tmp_path):
     """sizeof and the offsets of the ctypes mirrors against the C compiler's view of the header."""
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    probes = [("NhaPrefillArgs", f) for f in ("q_swa", "scratch_bytes", "T_tot", "phases", "scale", "stream")]
+    probes = [("NhaPrefillArgs", f) for f in ("q_swa", "scratch_bytes", "T_tot", "impl", "scale", "stream")]
     probes += [("NhaDecodeArgs", f) for f in ("mode", "scale", "q", "cos_sb", "count", "o", "stream", "count_next")]
     probes += [("NhaPrefillBwdArgs", f) for f in ("q_swa", "o", "dout", "dhvt", "dq_swa", "dg", "dh0v", "cu_seqlens",
                                                   "scratch_bytes", "T_tot", "dtype", "scale", "stream")]
