@@ -342,6 +342,109 @@ def bench_layer(torch, steps, warmup):
     return out
 
 
+def bench_hybrid(torch, steps, warmup):
+    """One attention block of the MoE-flavour hybrid decoder (hidden 2048, 32 query / 4 kv heads of 128, 64 slots),
+    bf16, autograd off: the prompt (B=2, T=8192) through an NHA layer (window 64) and through a zero-sink layer
+    (window 2048), and single-token steps at B=128 on the ring cache after a 256-token prompt -- each as the whole
+    block (projection GEMMs, the glue launch, the attention kernels, the output projection) next to its parts timed
+    alone, with the fused glue and with the tensor-op chain."""
+    from nha_amd import NHACache, fused_chunk_nha_prefill
+    from nha_amd.hybrid import HybridNHAConfig, Qwen3MoeNativeHybridAttention
+    from nha_amd.ops import nha_hybrid_prologue
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+    hidden, HQ, H, D, M = 2048, 32, 4, 128, 64
+
+    def timed(fn, n=steps, busy=0.5):
+        keep_busy(torch, fn, seconds=min(busy, CLOCK_WARM_S))
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record(stream)
+        for _ in range(n):
+            fn()
+        ev[1].record(stream)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / n
+
+    out = {"shape": {"hidden": hidden, "HQ": HQ, "H": H, "D": D, "M": M, "prefill": "B=2 T=8192", "decode": "B=128"}}
+    torch.manual_seed(0)
+    for W, tag in ((64, "w64"), (2048, "w2048")):
+        cfg = HybridNHAConfig(hidden_size=hidden, num_attention_heads=HQ, num_key_value_heads=H, head_dim=D, num_slots=M,
+                              window_size=64, block_size=1 if W == 2048 else None, transformer_idx=0 if W == 2048 else None)
+        blk = Qwen3MoeNativeHybridAttention(cfg, 0).to(torch.bfloat16).to(dev).eval()
+        assert blk.window_size == W
+        x = (torch.randn(2, 8192, hidden, device=dev) * 0.5).to(torch.bfloat16)
+        pos = torch.arange(8192, device=dev)[None].expand(2, -1)
+        res = {}
+        with torch.no_grad():
+            for fuse in (True, False):
+                blk.fuse_glue = fuse
+                ms = timed(lambda: blk(x, position_ids=pos), n=max(steps // 2, 4))
+                res["block_ms" if fuse else "block_chain_ms"] = ms
+            res["tokens_per_s"] = 2 * 8192 / (res["block_ms"] * 1e-3)
+            # the parts of the fused block, each alone
+            blk.fuse_glue = True
+            nha = blk.is_nha_layer
+            y = blk._fused_projection(x, nha)
+            res["projection_ms"] = timed(lambda: blk._fused_projection(x, nha), n=max(steps // 2, 4))
+            cos, sin = blk._tables(x, pos, None, None, 8192)
+            o0, o1, o2 = HQ * D, HQ * D + H * D, HQ * D + 2 * H * D
+            glue = lambda: nha_hybrid_prologue(y[..., :o0], y[..., o0:o1], y[..., o1:o2], y[..., o2:] if nha else None, cos, sin,
+                                               num_heads=HQ, num_kv_heads=H, head_dim=D, num_slots=M,
+                                               q_weight=blk.q_norm.weight, k_weight=blk.k_norm.weight, eps=1e-6)
+            q, sq, k, sk, v, g, s_ = glue()
+            res["glue_ms"] = timed(glue, n=max(steps // 2, 4))
+            moved = 2 * 8192 * 2 * (3 * HQ * D + 3 * H * D + 2 * H * D + (3 if nha else 2) * H * M + 2 * D)
+            res["glue_gbs"] = moved / (res["glue_ms"] * 1e-3) / 1e9
+            if nha:
+                op = lambda: fused_chunk_nha_prefill(q=q, k=k, v=v, rotary_q=sq, rotary_k=sk, s=s_, g=g, window_size=W,
+                                                     scale=D ** -0.5)
+            else:
+                from nha_amd import chunk_nha
+                op = lambda: chunk_nha(sq, sk, q, k, v, s_, g, window_size_left=W - 1, gsa_kv_shift=W, scale=D ** -0.5)
+            o = op()[0]
+            res["attention_op_ms"] = timed(op, n=max(steps // 2, 4))
+            res["o_proj_ms"] = timed(lambda: blk.o_proj(o.reshape(2, 8192, HQ * D)), n=max(steps // 2, 4))
+            res["parts_sum_ms"] = res["projection_ms"] + res["glue_ms"] + res["attention_op_ms"] + res["o_proj_ms"]
+        out["prefill_" + tag] = res
+        # decode: B = 128 after a 256-token prompt (the NHA layer's window is full; the zero-sink layer holds 256 of 2048)
+        B = 128
+        xp = (torch.randn(B, 256, hidden, device=dev) * 0.5).to(torch.bfloat16)
+        xs = (torch.randn(B, 1, hidden, device=dev) * 0.5).to(torch.bfloat16)
+        dres = {}
+        with torch.no_grad():
+            for fuse in (True, False):
+                blk.fuse_glue = fuse
+                cache = NHACache()
+                blk(xp, position_ids=torch.arange(256, device=dev)[None].expand(B, -1), past_key_value=cache, use_cache=True)
+                pos1 = torch.full((B, 1), 256, device=dev)
+                step = lambda: blk(xs, position_ids=pos1, past_key_value=cache, use_cache=True)
+                dres["block_us" if fuse else "block_chain_us"] = timed(step, n=128, busy=0.2) * 1e3
+            # the bare kernel step on the same cache, and the glue and GEMMs of a step alone
+            from nha_amd import ring_decode_step
+            blk.fuse_glue = True
+            st = cache.states[0]
+            y1 = blk._fused_projection(xs, nha)
+            cos1, sin1 = blk._tables(xs, pos1, None, None, 1)
+            glue1 = lambda: nha_hybrid_prologue(y1[..., :o0], y1[..., o0:o1], y1[..., o1:o2], y1[..., o2:] if nha else None, cos1,
+                                                sin1, num_heads=HQ, num_kv_heads=H, head_dim=D, num_slots=M,
+                                                q_weight=blk.q_norm.weight, k_weight=blk.k_norm.weight, eps=1e-6, want_s=False)
+            q1, sq1, k1, sk1, v1, g1, _ = glue1()
+            dres["ring_decode_step_us"] = timed(lambda: ring_decode_step(st, q1[:, 0], sq1[:, 0], sk1[:, 0], k1[:, 0], v1[:, 0],
+                                                                         g1[:, 0], scale=D ** -0.5), n=128, busy=0.2) * 1e3
+            dres["glue_us"] = timed(glue1, n=128, busy=0.2) * 1e3
+            dres["projection_us"] = timed(lambda: blk._fused_projection(xs, nha), n=128, busy=0.2) * 1e3
+            o1_ = torch.empty(B, 1, HQ * D, dtype=torch.bfloat16, device=dev)
+            dres["o_proj_us"] = timed(lambda: blk.o_proj(o1_), n=128, busy=0.2) * 1e3
+            dres["parts_sum_us"] = dres["ring_decode_step_us"] + dres["glue_us"] + dres["projection_us"] + dres["o_proj_us"]
+            dres["block_over_bare_step"] = dres["block_us"] / dres["ring_decode_step_us"]
+        out["decode_" + tag] = dres
+        del blk, cache
+    return out
+
+
 # the decode step at the 340M layers' heads (one query head per kv-head, head size 256, window 512)
 DECODE_D256 = dict(B=128, HQ=4, H=4, D=256, M=64, W=512, steps=128)
 
@@ -560,7 +663,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--only", choices=["prefill", "decode", "decode_d256", "glue", "layer"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "decode_d256", "glue", "layer", "hybrid"], default=None,
                     help="development aid: time one leg only and print its raw numbers")
     ap.add_argument("--backward", action="store_true",
                     help="with --workload: also time the backward of the prefill op")
@@ -595,6 +698,7 @@ def main():
         res = (bench_prefill(torch, args.steps, args.warmup) if args.only == "prefill" else
                bench_glue(torch, args.steps, args.warmup) if args.only == "glue" else
                bench_layer(torch, args.steps, args.warmup) if args.only == "layer" else
+               bench_hybrid(torch, args.steps, args.warmup) if args.only == "hybrid" else
                bench_decode(torch, args.warmup, DECODE_D256) if args.only == "decode_d256" else bench_decode(torch, args.warmup))
         print(json.dumps(res))
         return
@@ -605,6 +709,7 @@ def main():
     dc256 = bench_decode(torch, args.warmup, DECODE_D256)
     gl = bench_glue(torch, args.steps, args.warmup)
     api = bench_api(torch, max(args.steps // 2, 1), min(args.warmup, 2))
+    hyb = bench_hybrid(torch, max(args.steps // 2, 1), min(args.warmup, 2))
     others = {}
     for name in ("cfg2", "cfg3", "cfg5", "w64"):
         cfg = WORKLOADS[name]
@@ -673,6 +778,7 @@ def main():
                 "chunk_nha_varlen_cfg3_ms": api["chunk_nha_varlen_cfg3_ms"],
                 "fused_recurrent_nha_decode_window_eager_us": api["decode_window_eager_us"],
                 "fused_recurrent_nha_decode_window_rotary_us": api["decode_window_rotary_us"]},
+        "hybrid": hyb,
         "workloads": others,
         "cpu_baseline": cpu,
     }

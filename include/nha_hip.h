@@ -304,6 +304,59 @@ typedef struct NhaLayerEpilogueArgs {
 int nha_layer_prologue(const NhaLayerPrologueArgs* a);
 int nha_layer_epilogue(const NhaLayerEpilogueArgs* a);
 
+/* ------------------------------------------------------------------------------------------
+ * Glue of the hybrid decoder models' attention blocks in one launch (inference): from the raw
+ * projections of a block -- which may be column slices of one fused projection output: `*_stride`
+ * is the number of elements between the rows of two tokens -- it writes the contiguous operands of
+ * the prefill op and of the decode step.  Replaces the tensor-op chain of
+ * nha_fla/models/qwen3_moe_nha/qwennha.py:103-106 (per-head RMSNorm of q and k: x * rsqrt(mean(x^2) +
+ * eps) in fp32, rounded, times `q_weight` / `k_weight` [D]; NULL weights = the dense flavour,
+ * nha_fla/models/llama3_nha/llamanha.py:79-81), :117-128 (g = logsigmoid(f) / normalizer,
+ * s = 1 - exp(g), each step rounded to the tensor dtype), :133-144 (v and s times the padding mask
+ * of the token, `mask` [B*T] in the tensor dtype or NULL), :240-247 (rotate-half rotary embedding with
+ * cos / sin [B or 1, T, D] in the tensor dtype, `cs_batch_stride` = T*D or 0; evaluated in fp32, rounded
+ * once).  Outputs: q_out / sq_out [B,T,HQ,D] (normed, and normed + rotated), k_out / sk_out [B,T,H,D],
+ * v_out [B,T,H,D], g_out and s_out [B,T,H,M] (s_out may be NULL: a decode step does not read it).
+ * f == NULL writes g = s = 0 (the layers whose slots never absorb anything).  D in {64, 128, 256},
+ * M a multiple of 8, every pointer and stride 16-byte aligned. */
+typedef struct NhaHybridPrologueArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* f;
+  int64_t q_stride, k_stride, v_stride, f_stride;
+  const void* q_weight;
+  const void* k_weight;
+  const void* cos;
+  const void* sin;
+  int64_t cs_batch_stride;
+  const void* mask;
+  void* q_out;
+  void* sq_out;
+  void* k_out;
+  void* sk_out;
+  void* v_out;
+  void* g_out;
+  void* s_out;
+  int32_t B, T, HQ, H, D, M;
+  int32_t dtype;
+  float eps;
+  float gate_logit_normalizer;
+  void* stream;
+} NhaHybridPrologueArgs;
+
+int nha_hybrid_prologue(const NhaHybridPrologueArgs* a);
+
+/* The "full attention" layers of the hybrid models (window 2048: a sliding-window softmax preceded by M all-zero
+ * key / value rows, nha_fla/models/qwen3_moe_nha/qwennha.py:323-336, :400-413;
+ * nha_fla/models/llama3_nha/llamanha.py:204-216) run through nha_prefill_fwd with slot states that stay zero, which
+ * puts M zero-logit, zero-value keys into every query's softmax; the reference's window still covers
+ * n0(t) = clamp(W - 1 - t, 0, M) of them at position t of its sequence.  This call multiplies row (b, t, head) of
+ * o [B,T,HQ,D] in place by (e^lse + M) / (e^lse + n0(t)), lse = lse_swa [B,T,HQ] of that prefill call.
+ * D in {64, 128, 256}; o 16-byte aligned. */
+int nha_zero_sink_rescale(void* o, const float* lse_swa, int32_t B, int32_t T, int32_t HQ, int32_t D, int32_t W, int32_t M,
+                          int32_t dtype, void* stream);
+
 /* Backward of the two launches above (what autograd derives from the tensor-op chain of
  * nha_fla/layers/nha.py:214-237, :278; the reference has no hand-written counterpart).
  *

@@ -22,7 +22,7 @@ EXPORTS = (
     "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_fwd_noalloc", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
     "nha_decode_step", "nha_decode_advance", "nha_layer_prologue", "nha_layer_epilogue",
     "nha_layer_prologue_bwd", "nha_layer_epilogue_bwd", "nha_layer_epilogue_bwd_parts",
-    "nha_short_conv", "nha_short_conv_bwd", "nha_short_conv_bwd_parts",
+    "nha_short_conv", "nha_short_conv_bwd", "nha_short_conv_bwd_parts", "nha_hybrid_prologue", "nha_zero_sink_rescale",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
 )
 
@@ -90,6 +90,19 @@ class NhaLayerPrologueArgs(C.Structure):
         ("K", C.c_int32), ("V", C.c_int32), ("M", C.c_int32),
         ("feature_map", C.c_int32), ("seqlen_offset", C.c_int32), ("dtype", C.c_int32),
         ("gate_logit_normalizer", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
+class NhaHybridPrologueArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("f", C.c_void_p),
+        ("q_stride", C.c_int64), ("k_stride", C.c_int64), ("v_stride", C.c_int64), ("f_stride", C.c_int64),
+        ("q_weight", C.c_void_p), ("k_weight", C.c_void_p), ("cos", C.c_void_p), ("sin", C.c_void_p),
+        ("cs_batch_stride", C.c_int64), ("mask", C.c_void_p),
+        ("q_out", C.c_void_p), ("sq_out", C.c_void_p), ("k_out", C.c_void_p), ("sk_out", C.c_void_p),
+        ("v_out", C.c_void_p), ("g_out", C.c_void_p), ("s_out", C.c_void_p),
+        ("B", C.c_int32), ("T", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32), ("D", C.c_int32), ("M", C.c_int32),
+        ("dtype", C.c_int32), ("eps", C.c_float), ("gate_logit_normalizer", C.c_float), ("stream", C.c_void_p),
     ]
 
 
@@ -181,6 +194,10 @@ def load() -> C.CDLL:
     lib.nha_layer_epilogue_bwd.argtypes = [C.POINTER(NhaLayerEpilogueBwdArgs)]
     lib.nha_layer_epilogue_bwd_parts.restype = C.c_int32
     lib.nha_layer_epilogue_bwd_parts.argtypes = [C.c_int32]
+    lib.nha_hybrid_prologue.restype = C.c_int
+    lib.nha_hybrid_prologue.argtypes = [C.POINTER(NhaHybridPrologueArgs)]
+    lib.nha_zero_sink_rescale.restype = C.c_int
+    lib.nha_zero_sink_rescale.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int32] * 7 + [C.c_void_p]
     lib.nha_short_conv.restype = C.c_int
     lib.nha_short_conv.argtypes = [C.POINTER(NhaShortConvArgs)]
     lib.nha_short_conv_bwd.restype = C.c_int

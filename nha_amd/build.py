@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnha_hip.so")
 SOURCES = ["abi.hip", "decode.hip", "decode_mfma.hip", "prefill_simple.hip", "prefill_mfma.hip", "prefill_ring.hip", "prefill_ring256.hip", "prefill_bwd.hip", "prefill_bwd_mfma.hip", "prefill_bwd_ring.hip",
-           "layer_fuse.hip"]
+           "layer_fuse.hip", "hybrid_fuse.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math" if False else "-fno-fast-math",

@@ -211,6 +211,42 @@ int nha_layer_prologue(const NhaLayerPrologueArgs* a) {
   return layer_prologue_impl(a);
 }
 
+int nha_hybrid_prologue(const NhaHybridPrologueArgs* a) {
+  NHA_CHECK_ARG(a != nullptr, "nha_hybrid_prologue: null args");
+  NHA_CHECK_ARG(a->B > 0 && a->T > 0 && a->HQ > 0 && a->H > 0 && a->M > 0, "nha_hybrid_prologue: non-positive dimension");
+  NHA_CHECK_ARG(a->D == 64 || a->D == 128 || a->D == 256, "nha_hybrid_prologue: head size must be 64, 128 or 256, got %d", a->D);
+  NHA_CHECK_ARG(a->M % 8 == 0, "nha_hybrid_prologue: M must be a multiple of 8, got %d", a->M);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_hybrid_prologue: bad dtype %d", a->dtype);
+  NHA_CHECK_ARG(a->q && a->k && a->v && a->cos && a->sin, "nha_hybrid_prologue: q, k, v, cos, sin are required");
+  NHA_CHECK_ARG(a->q_out && a->sq_out && a->k_out && a->sk_out && a->v_out && a->g_out,
+                "nha_hybrid_prologue: q_out, sq_out, k_out, sk_out, v_out, g_out are required");
+  NHA_CHECK_ARG((a->q_weight == nullptr) == (a->k_weight == nullptr), "nha_hybrid_prologue: pass both norm weights or neither");
+  NHA_CHECK_ARG(a->gate_logit_normalizer != 0.f, "nha_hybrid_prologue: gate_logit_normalizer must not be 0");
+  const int64_t esz = a->dtype == NHA_DTYPE_BF16 ? 2 : 4;
+  NHA_CHECK_ARG(a->q_stride >= (int64_t)a->HQ * a->D && a->k_stride >= (int64_t)a->H * a->D && a->v_stride >= (int64_t)a->H * a->D &&
+                    (a->f == nullptr || a->f_stride >= (int64_t)a->H * a->M),
+                "nha_hybrid_prologue: a row stride is shorter than its row");
+  NHA_CHECK_ARG(a->cs_batch_stride == 0 || a->cs_batch_stride >= (int64_t)a->T * a->D, "nha_hybrid_prologue: bad cos / sin batch stride");
+  const int64_t strides[] = {a->q_stride, a->k_stride, a->v_stride, a->f ? a->f_stride : 0, a->cs_batch_stride};
+  for (int64_t s : strides) NHA_CHECK_ARG((s * esz) % 16 == 0, "nha_hybrid_prologue: strides must be multiples of 16 bytes");
+  const void* ptrs[] = {a->q, a->k, a->v, a->f, a->q_weight, a->k_weight, a->cos, a->sin, a->q_out, a->sq_out, a->k_out, a->sk_out,
+                        a->v_out, a->g_out, a->s_out};
+  for (const void* p : ptrs)
+    NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(p) & 15) == 0, "nha_hybrid_prologue: tensors must be 16-byte aligned");
+  return hybrid_prologue_impl(a);
+}
+
+int nha_zero_sink_rescale(void* o, const float* lse_swa, int32_t B, int32_t T, int32_t HQ, int32_t D, int32_t W, int32_t M,
+                          int32_t dtype, void* stream) {
+  NHA_CHECK_ARG(o && lse_swa, "nha_zero_sink_rescale: o and lse_swa are required");
+  NHA_CHECK_ARG(B > 0 && T > 0 && HQ > 0 && W > 0 && M >= 0, "nha_zero_sink_rescale: bad dimension");
+  NHA_CHECK_ARG(D == 64 || D == 128 || D == 256, "nha_zero_sink_rescale: head size must be 64, 128 or 256, got %d", D);
+  NHA_CHECK_ARG(dtype == NHA_DTYPE_F32 || dtype == NHA_DTYPE_BF16, "nha_zero_sink_rescale: bad dtype %d", dtype);
+  NHA_CHECK_ARG((reinterpret_cast<uintptr_t>(o) & 15) == 0, "nha_zero_sink_rescale: o must be 16-byte aligned");
+  NHA_CHECK_ARG((int64_t)B * T * HQ < ((int64_t)1 << 31), "nha_zero_sink_rescale: too many rows");
+  return zero_sink_rescale_impl(o, lse_swa, B, T, HQ, D, W, M, dtype, stream);
+}
+
 int nha_layer_epilogue(const NhaLayerEpilogueArgs* a) {
   NHA_CHECK_ARG(a != nullptr, "nha_layer_epilogue: null args");
   NHA_CHECK_ARG(a->rows > 0 && a->dim > 0, "nha_layer_epilogue: non-positive dimension");

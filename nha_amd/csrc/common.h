@@ -132,6 +132,8 @@ int layer_epilogue_impl(const NhaLayerEpilogueArgs* a);
 int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a);
 int layer_epilogue_bwd_parts(int rows);
 int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a);
+int hybrid_prologue_impl(const NhaHybridPrologueArgs* a);
+int zero_sink_rescale_impl(void* o, const float* lse_swa, int B, int T, int HQ, int D, int W, int M, int dtype, void* stream);
 int short_conv_impl(const NhaShortConvArgs* a);
 int short_conv_bwd_parts(int T_tot);
 int short_conv_bwd_impl(const NhaShortConvBwdArgs* a);

@@ -34,7 +34,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .cache import NHARingCache
-from .ops import chunk_nha, fused_chunk_nha_prefill
+from .ops import (chunk_nha, fused_chunk_nha_prefill, hybrid_prologue_supported, nha_hybrid_prologue,
+                  nha_zero_sink_rescale_)
 
 GATE_LOGIT_NORMALIZER = 8          # qwennha.py:62, llamanha.py:96
 FULL_ATTENTION_WINDOW = 2048       # qwennha.py:66, llamanha.py:60
@@ -158,9 +159,11 @@ class HybridNHAAttention(nn.Module):
     `forward` has the reference modules' signature and returns `(output, None)`."""
 
     qk_norm = False
+    fuse_glue = True      # inference: fused projection GEMM + one glue launch (False keeps the tensor-op chain)
 
     def __init__(self, config, layer_idx: int = 0):
         super().__init__()
+        self._fused_key, self._fused_wb = None, None
         self.config = config
         self.layer_idx = layer_idx
         self.hidden_size = config.hidden_size
@@ -187,6 +190,23 @@ class HybridNHAAttention(nn.Module):
             self.q_norm = HeadRMSNorm(D, eps)
             self.k_norm = HeadRMSNorm(D, eps)
         self.rotary_emb = RotaryTables(D, getattr(config, "rope_theta", 10000.0))
+
+    def _fused_projection(self, x: torch.Tensor, with_gates: bool) -> torch.Tensor:
+        """q | k | v | (gate logits) of `x` from ONE GEMM on the concatenated projection weights.  The concatenation is
+        a copy held by the module (rebuilt when a weight's storage or version changes): inference memory for the
+        attention projections doubles, four launches become one."""
+        mods = [self.q_proj, self.k_proj, self.v_proj] + ([self.g_proj] if with_gates else [])
+        key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype, m.weight.device,
+                     None if m.bias is None else (m.bias.data_ptr(), m.bias._version)) for m in mods)
+        if self._fused_key != key:
+            w = torch.cat([m.weight.detach() for m in mods], 0)
+            b = None
+            if any(m.bias is not None for m in mods):
+                b = torch.cat([m.bias.detach() if m.bias is not None else
+                               torch.zeros(m.weight.shape[0], dtype=w.dtype, device=w.device) for m in mods], 0)
+            self._fused_key, self._fused_wb = key, (w, b)
+        w, b = self._fused_wb
+        return F.linear(x, w, b)
 
     @property
     def is_nha_layer(self) -> bool:
@@ -219,37 +239,64 @@ class HybridNHAAttention(nn.Module):
                             f"(NHARingCache.from_legacy_cache converts), got {type(past_key_value).__name__}")
         B, T, _ = hidden_states.shape
         HQ, H, D, M, W = self.num_heads, self.num_key_value_heads, self.head_dim, self.num_slots, self.window_size
-        q = self.q_proj(hidden_states).view(B, T, HQ, D)
-        k = self.k_proj(hidden_states).view(B, T, H, D)
-        v = self.v_proj(hidden_states).view(B, T, H, D)
-        if self.qk_norm:
-            q, k = self.q_norm(q), self.k_norm(k)
         nha = self.is_nha_layer
-        if nha:
-            g = F.logsigmoid(self.g_proj(hidden_states).view(B, T, H, M)) / self.gate_logit_normalizer
-        else:                                  # the slots of a full-attention layer never absorb anything
-            g = torch.zeros(B, T, H, M, dtype=v.dtype, device=v.device)
         has_state = past_key_value is not None and past_key_value.has_ring(self.layer_idx)
         decode_step = (not self.training) and T == 1 and has_state
-        mask_t = None
-        if attention_mask is not None:         # left padding: a padded token writes nothing into the slots
-            if attention_mask.dim() == 2:      # [batch, tokens]
-                mask_t = attention_mask[:, -T:].to(v.dtype)[:, :, None, None]
-            elif attention_mask.dim() == 4:
-                # [batch, 1, queries, tokens]: the reference multiplies its head-first [B, heads, T, dim] tensors by
-                # mask[:, :, :, -T:] (qwennha.py:133-136), so the last T columns broadcast over (token, dim);
-                # the same product on the token-major layout here
-                mask_t = attention_mask[:, :, :, -T:].to(v.dtype).transpose(1, 2)
-            else:
-                raise ValueError("attention_mask must be [batch, tokens] or [batch, 1, queries, tokens], got "
-                                 f"{tuple(attention_mask.shape)}")
-            v = v * mask_t
-        cos, sin = self._tables(v, position_ids, position_embeddings, past_key_value, T)
-        sq, sk = rotate_half_apply(q, cos, sin), rotate_half_apply(k, cos, sin)
-        dt = q.dtype
-        if dt == torch.float32 and torch.is_autocast_enabled():
-            dt = torch.get_autocast_gpu_dtype()
-        q, k, v, g, sq, sk = (x.to(dt).contiguous() for x in (q, k, v, g, sq, sk))
+        mask2d = None
+        if attention_mask is not None and attention_mask.dim() == 2:
+            mask2d = attention_mask[:, -T:]
+        # inference on the GPU: one GEMM for the q / k / v / gate projections and one launch for everything between
+        # them and the attention op (q / k norm, gates, padding mask, rotary, contiguous operands)
+        fused = (self.fuse_glue and not torch.is_grad_enabled() and hybrid_prologue_supported(hidden_states, D, M)
+                 and (attention_mask is None or mask2d is not None)
+                 and not (hidden_states.dtype == torch.float32 and torch.is_autocast_enabled()))
+        if fused:
+            y = self._fused_projection(hidden_states, with_gates=nha)
+            o0, o1, o2 = HQ * D, HQ * D + H * D, HQ * D + 2 * H * D
+            cos, sin = self._tables(hidden_states, position_ids, position_embeddings, past_key_value, T)
+            q, sq, k, sk, v, g, s = nha_hybrid_prologue(
+                y[..., :o0], y[..., o0:o1], y[..., o1:o2], y[..., o2:] if nha else None, cos, sin, num_heads=HQ,
+                num_kv_heads=H, head_dim=D, num_slots=M, q_weight=self.q_norm.weight if self.qk_norm else None,
+                k_weight=self.k_norm.weight if self.qk_norm else None,
+                eps=self.q_norm.variance_epsilon if self.qk_norm else 0.0, mask=mask2d,
+                gate_logit_normalizer=self.gate_logit_normalizer, want_s=not decode_step)
+        else:
+            q = self.q_proj(hidden_states).view(B, T, HQ, D)
+            k = self.k_proj(hidden_states).view(B, T, H, D)
+            v = self.v_proj(hidden_states).view(B, T, H, D)
+            if self.qk_norm:
+                q, k = self.q_norm(q), self.k_norm(k)
+            if nha:
+                g = F.logsigmoid(self.g_proj(hidden_states).view(B, T, H, M)) / self.gate_logit_normalizer
+            else:                                  # the slots of a full-attention layer never absorb anything
+                g = torch.zeros(B, T, H, M, dtype=v.dtype, device=v.device)
+            mask_t = None
+            if attention_mask is not None:         # left padding: a padded token writes nothing into the slots
+                if mask2d is not None:             # [batch, tokens]
+                    mask_t = mask2d.to(v.dtype)[:, :, None, None]
+                elif attention_mask.dim() == 4:
+                    # [batch, 1, queries, tokens]: the reference multiplies its head-first [B, heads, T, dim] tensors by
+                    # mask[:, :, :, -T:] (qwennha.py:133-136), so the last T columns broadcast over (token, dim);
+                    # the same product on the token-major layout here
+                    mask_t = attention_mask[:, :, :, -T:].to(v.dtype).transpose(1, 2)
+                else:
+                    raise ValueError("attention_mask must be [batch, tokens] or [batch, 1, queries, tokens], got "
+                                     f"{tuple(attention_mask.shape)}")
+                v = v * mask_t
+            cos, sin = self._tables(v, position_ids, position_embeddings, past_key_value, T)
+            sq, sk = rotate_half_apply(q, cos, sin), rotate_half_apply(k, cos, sin)
+            dt = q.dtype
+            if dt == torch.float32 and torch.is_autocast_enabled():
+                dt = torch.get_autocast_gpu_dtype()
+            q, k, v, g, sq, sk = (x.to(dt).contiguous() for x in (q, k, v, g, sq, sk))
+            s = None
+            if not decode_step:
+                if nha:
+                    s = 1 - torch.exp(g).to(g.dtype)
+                    if mask_t is not None:
+                        s = s * mask_t
+                else:
+                    s = torch.zeros_like(g)
 
         if decode_step:
             o = past_key_value.decode(self.layer_idx, q[:, 0], sq[:, 0], sk[:, 0], k[:, 0], v[:, 0], g[:, 0],
@@ -258,12 +305,6 @@ class HybridNHAAttention(nn.Module):
             if has_state:
                 raise NotImplementedError("a multi-token step on top of a cached prompt is not supported "
                                           "(the reference's modules do not support it either)")
-            if nha:
-                s = 1 - torch.exp(g).to(g.dtype)
-                if mask_t is not None:
-                    s = s * mask_t
-            else:
-                s = torch.zeros_like(g)
             want_state = use_cache or past_key_value is not None
             if nha and not torch.is_grad_enabled():
                 o, state = fused_chunk_nha_prefill(q=q, k=k, v=v, rotary_q=sq, rotary_k=sk, s=s, g=g, window_size=W,
@@ -276,8 +317,11 @@ class HybridNHAAttention(nn.Module):
                 if not nha:
                     # M zero-logit sinks were in the softmax at every t; the reference's window covers
                     # zero_sink_count(t) of them
-                    n0 = zero_sink_count(T, W, M, lse_swa.device)[None, :, None]
-                    o = (o.to(torch.float32) * zero_sink_rescale(lse_swa, M, n0)[..., None]).to(o.dtype)
+                    if not torch.is_grad_enabled() and D in (64, 128, 256) and o.is_contiguous():
+                        o = nha_zero_sink_rescale_(o, lse_swa.contiguous(), W, M)        # one launch, in place
+                    else:
+                        n0 = zero_sink_count(T, W, M, lse_swa.device)[None, :, None]
+                        o = (o.to(torch.float32) * zero_sink_rescale(lse_swa, M, n0)[..., None]).to(o.dtype)
             if past_key_value is not None:
                 past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W)
         o = self.o_proj(o.reshape(B, T, HQ * D))

@@ -445,6 +445,82 @@ def nha_short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     return _ShortConvFunction.apply(x.contiguous(), weight, bias, cu, 0 if activation is None else 1)
 
 
+def hybrid_prologue_supported(q: torch.Tensor, D: int, M: int) -> bool:
+    """Whether nha_hybrid_prologue serves these tensors: GPU, bf16 / fp32, head size 64 / 128 / 256, M a multiple of 8."""
+    return q.is_cuda and q.dtype in (torch.bfloat16, torch.float32) and D in (64, 128, 256) and M % 8 == 0
+
+
+def _row_view(x: torch.Tensor, width: int, what: str):
+    """(tensor, elements between the rows of two tokens) of a `[B, T, width]` view whose rows are contiguous and
+    whose tokens are evenly spaced (a column slice of a fused projection output, or a contiguous tensor)."""
+    B, T = x.shape[0], x.shape[1]
+    if x.shape[2] != width or (width > 1 and x.stride(2) != 1) or (B > 1 and T > 1 and x.stride(0) != T * x.stride(1)):
+        x = x.contiguous()
+    stride = x.stride(1) if T > 1 else (x.stride(0) if B > 1 else width)
+    esz = x.element_size()
+    if (stride * esz) % 16 or x.data_ptr() % 16:
+        x = x.contiguous()
+        stride = width
+    return x, stride
+
+
+@torch.no_grad()
+def nha_hybrid_prologue(q, k, v, f, cos, sin, *, num_heads: int, num_kv_heads: int, head_dim: int, num_slots: int,
+                        q_weight=None, k_weight=None, eps: float = 1e-6, mask=None, gate_logit_normalizer: float = 8.0,
+                        want_s: bool = True):
+    """One launch for the glue of a hybrid decoder attention block (inference): per-head RMSNorm of q and k (when
+    weights are given), rotary embedding, the gates and the padding mask
+    (nha_fla/models/qwen3_moe_nha/qwennha.py:103-144, :240-247).  q / k / v / f are `[B, T, heads * dim]` views
+    (column slices of one fused projection output are read in place); cos / sin `[B or 1, T, D]`; mask `[B, T]` or
+    None; f None writes g = s = 0.  Returns contiguous q, sq `[B,T,HQ,D]`, k, sk, v `[B,T,H,D]`, g, s `[B,T,H,M]`
+    (s None unless `want_s`)."""
+    _need_cuda(q, k, v, cos, sin)
+    B, T = q.shape[0], q.shape[1]
+    HQ, H, D, M = num_heads, num_kv_heads, head_dim, num_slots
+    dt, dev = q.dtype, q.device
+    q, qs = _row_view(q, HQ * D, "q")
+    k, ks = _row_view(k, H * D, "k")
+    v, vs = _row_view(v, H * D, "v")
+    fs = 0
+    if f is not None:
+        f, fs = _row_view(f, H * M, "f")
+    if cos.shape[-1] != D or cos.shape[-2] != T or cos.shape[0] not in (1, B) or sin.shape != cos.shape:
+        raise ValueError(f"cos / sin must be [{B} or 1, {T}, {D}], got {tuple(cos.shape)} / {tuple(sin.shape)}")
+    cos, sin = cos.to(dt).contiguous(), sin.to(dt).contiguous()
+    for x in (k, v, f, q_weight, k_weight):
+        if x is not None and x.dtype != dt:
+            raise ValueError(f"every tensor must have the dtype of q ({dt}), got {x.dtype}")
+    if mask is not None:
+        mask = mask.reshape(B * T).to(dt).contiguous()
+    new = lambda h, d: torch.empty(B, T, h, d, dtype=dt, device=dev)
+    qo, sqo, ko, sko, vo, go = new(HQ, D), new(HQ, D), new(H, D), new(H, D), new(H, D), new(H, M)
+    so = new(H, M) if want_s else None
+    a = _lib.NhaHybridPrologueArgs(
+        q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), q_stride=qs, k_stride=ks, v_stride=vs, f_stride=fs,
+        q_weight=_ptr(None if q_weight is None else q_weight.contiguous()),
+        k_weight=_ptr(None if k_weight is None else k_weight.contiguous()), cos=_ptr(cos), sin=_ptr(sin),
+        cs_batch_stride=(T * D if cos.shape[0] == B and B > 1 else 0), mask=_ptr(mask), q_out=_ptr(qo), sq_out=_ptr(sqo),
+        k_out=_ptr(ko), sk_out=_ptr(sko), v_out=_ptr(vo), g_out=_ptr(go), s_out=_ptr(so), B=B, T=T, HQ=HQ, H=H, D=D, M=M,
+        dtype=_dtype_code(q), eps=float(eps), gate_logit_normalizer=float(gate_logit_normalizer), stream=_stream(dev))
+    _lib.check(_lib.load().nha_hybrid_prologue(C.byref(a)))
+    return qo, sqo, ko, sko, vo, go, so
+
+
+@torch.no_grad()
+def nha_zero_sink_rescale_(o: torch.Tensor, lse_swa: torch.Tensor, window: int, num_sinks: int) -> torch.Tensor:
+    """In place: row (b, t, head) of ``o [B,T,HQ,D]`` times (e^lse + num_sinks) / (e^lse + clamp(window - 1 - t, 0,
+    num_sinks)) -- takes the zero-logit sinks that the NHA kernel's zero slot states put into every softmax back out
+    where the reference's window no longer covers them (nha_fla/models/qwen3_moe_nha/qwennha.py:323-336)."""
+    _need_cuda(o, lse_swa)
+    B, T, HQ, D = o.shape
+    if not o.is_contiguous() or lse_swa.dtype != torch.float32 or not lse_swa.is_contiguous() or tuple(lse_swa.shape) != (B, T, HQ):
+        raise ValueError("o must be contiguous [B,T,HQ,D] and lse_swa contiguous fp32 [B,T,HQ]")
+    lib = _lib.load()
+    _lib.check(lib.nha_zero_sink_rescale(_ptr(o), _ptr(lse_swa), B, T, HQ, D, int(window), int(num_sinks), _dtype_code(o),
+                                         _stream(o.device)))
+    return o
+
+
 class _ChunkNHAFunction(torch.autograd.Function):
     """Autograd node of chunk_nha on packed tensors: same outputs and gradient set as
     ChunkNativeHybridAttentionFunction (nha_fla/ops/nha/chunk.py:364-564)."""
