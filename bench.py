@@ -561,6 +561,17 @@ def bench_api(torch, steps, warmup):
             q, k, v, g, swk, swv, sq=sq, initial_state=(hk, hv), output_final_state=True), n)
         out["decode_window_rotary_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
             q, k, v, g, swk, swv, cos=cos, sin=sin, initial_state=(hk, hv), output_final_state=True), n)
+        # the call forms that the generic (vector-unit) decode kernels serve: caller-supplied window logits
+        # (fused_recurrent_nha, the dense hybrids' step) and float32 tensors
+        from nha_amd import fused_recurrent_nha
+        logits = (r(B, 1, HQ, Wd)).to(torch.bfloat16).to(dev)
+        s_ = (1 - g.float().exp()).to(torch.bfloat16)
+        out["fused_recurrent_nha_logits_us"] = 1e3 * timed(lambda: fused_recurrent_nha(
+            q, k, v, logits, s_, g, initial_state=(hk, hv), output_final_state=True), n)
+        f32 = lambda x: x.float()
+        q32, sq32, k32, v32, g32, swk32, swv32 = map(f32, (q, sq, k, v, g, swk, swv))
+        out["decode_window_fp32_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
+            q32, k32, v32, g32, swk32, swv32, sq=sq32, initial_state=(hk, hv), output_final_state=True), max(n // 4, 8))
     return out
 
 
@@ -777,7 +788,9 @@ def main():
                 "chunk_nha_vs_abi": api["chunk_nha_ms"] / api["abi_ms_adjacent"],
                 "chunk_nha_varlen_cfg3_ms": api["chunk_nha_varlen_cfg3_ms"],
                 "fused_recurrent_nha_decode_window_eager_us": api["decode_window_eager_us"],
-                "fused_recurrent_nha_decode_window_rotary_us": api["decode_window_rotary_us"]},
+                "fused_recurrent_nha_decode_window_rotary_us": api["decode_window_rotary_us"],
+                "fused_recurrent_nha_logits_mode_us": api["fused_recurrent_nha_logits_us"],
+                "fused_recurrent_nha_decode_window_fp32_us": api["decode_window_fp32_us"]},
         "hybrid": hyb,
         "workloads": others,
         "cpu_baseline": cpu,
