@@ -422,6 +422,11 @@ def bench_hybrid(torch, steps, warmup):
                 pos1 = torch.full((B, 1), 256, device=dev)
                 step = lambda: blk(xs, position_ids=pos1, past_key_value=cache, use_cache=True)
                 dres["block_us" if fuse else "block_chain_us"] = timed(step, n=128, busy=0.2) * 1e3
+                if fuse:
+                    # the same step recorded into a HIP graph (no per-launch host work)
+                    rec = blk.record_decode_step(cache, B)
+                    dres["recorded_block_us"] = timed(lambda: rec.step(xs, pos1), n=128, busy=0.2) * 1e3
+                    del rec
             # the bare kernel step on the same cache, and the glue and GEMMs of a step alone
             from nha_amd import ring_decode_step
             blk.fuse_glue = True
@@ -440,6 +445,7 @@ def bench_hybrid(torch, steps, warmup):
             dres["o_proj_us"] = timed(lambda: blk.o_proj(o1_), n=128, busy=0.2) * 1e3
             dres["parts_sum_us"] = dres["ring_decode_step_us"] + dres["glue_us"] + dres["projection_us"] + dres["o_proj_us"]
             dres["block_over_bare_step"] = dres["block_us"] / dres["ring_decode_step_us"]
+            dres["recorded_block_over_bare_step"] = dres["recorded_block_us"] / dres["ring_decode_step_us"]
         out["decode_" + tag] = dres
         del blk, cache
     return out

@@ -314,8 +314,9 @@ int nha_layer_epilogue(const NhaLayerEpilogueArgs* a);
  * nha_fla/models/llama3_nha/llamanha.py:79-81), :117-128 (g = logsigmoid(f) / normalizer,
  * s = 1 - exp(g), each step rounded to the tensor dtype), :133-144 (v and s times the padding mask
  * of the token, `mask` [B*T] in the tensor dtype or NULL), :240-247 (rotate-half rotary embedding with
- * cos / sin [B or 1, T, D] in the tensor dtype, `cs_batch_stride` = T*D or 0; evaluated in fp32, rounded
- * once).  Outputs: q_out / sq_out [B,T,HQ,D] (normed, and normed + rotated), k_out / sk_out [B,T,H,D],
+ * cos / sin [B or 1, T, D] in the tensor dtype, `cs_batch_stride` = T*D or 0 -- or with `positions` and
+ * `inv_freq`, from which the kernel forms the same table rows itself; the rotation is evaluated in fp32 and
+ * rounded once).  Outputs: q_out / sq_out [B,T,HQ,D] (normed, and normed + rotated), k_out / sk_out [B,T,H,D],
  * v_out [B,T,H,D], g_out and s_out [B,T,H,M] (s_out may be NULL: a decode step does not read it).
  * f == NULL writes g = s = 0 (the layers whose slots never absorb anything).  D in {64, 128, 256},
  * M a multiple of 8, every pointer and stride 16-byte aligned. */
@@ -330,6 +331,8 @@ typedef struct NhaHybridPrologueArgs {
   const void* cos;
   const void* sin;
   int64_t cs_batch_stride;
+  const int64_t* positions; /* [B*T] token positions, with inv_freq [D/2] fp32: cos / sin of position * inv_freq are */
+  const float* inv_freq;    /* formed in the kernel (fp32, rounded to the tensor dtype) and cos / sin are not read   */
   const void* mask;
   void* q_out;
   void* sq_out;

@@ -98,7 +98,7 @@ class NhaHybridPrologueArgs(C.Structure):
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("f", C.c_void_p),
         ("q_stride", C.c_int64), ("k_stride", C.c_int64), ("v_stride", C.c_int64), ("f_stride", C.c_int64),
         ("q_weight", C.c_void_p), ("k_weight", C.c_void_p), ("cos", C.c_void_p), ("sin", C.c_void_p),
-        ("cs_batch_stride", C.c_int64), ("mask", C.c_void_p),
+        ("cs_batch_stride", C.c_int64), ("positions", C.c_void_p), ("inv_freq", C.c_void_p), ("mask", C.c_void_p),
         ("q_out", C.c_void_p), ("sq_out", C.c_void_p), ("k_out", C.c_void_p), ("sk_out", C.c_void_p),
         ("v_out", C.c_void_p), ("g_out", C.c_void_p), ("s_out", C.c_void_p),
         ("B", C.c_int32), ("T", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32), ("D", C.c_int32), ("M", C.c_int32),

@@ -20,7 +20,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from .ring import NHARingState, ring_decode_step
+from .ring import NHARingState, ring_advance, ring_decode_step
 
 
 class NHARingCache:
@@ -166,14 +166,24 @@ class NHARingCache:
         """Tokens the ring of `layer_idx` has taken (its longest sequence): the next token's position."""
         return self._layer_tokens.get(layer_idx, 0)
 
-    def decode(self, layer_idx: int, q_gsa, q_swa, k_swa, k_gsa, v, g, scale: Optional[float] = None) -> torch.Tensor:
+    def decode(self, layer_idx: int, q_gsa, q_swa, k_swa, k_gsa, v, g, scale: Optional[float] = None,
+               in_place_counters: bool = False) -> torch.Tensor:
         """One token per sequence through layer `layer_idx`: pops the entry leaving the window into the
-        slots, stores the new token, attends (one launch).  Tensors `[B, heads, dim]`; returns o."""
+        slots, stores the new token, attends (one launch).  Tensors `[B, heads, dim]`; returns o.
+        `in_place_counters`: advance the ring counters with a second small launch on the same array instead of
+        trading the two counter arrays (what a step recorded into a HIP graph needs: a replay uses fixed pointers)."""
         st = self.states[layer_idx]
-        o = ring_decode_step(st, q_gsa, q_swa, k_swa, k_gsa, v, g, scale=scale)
+        o = ring_decode_step(st, q_gsa, q_swa, k_swa, k_gsa, v, g, scale=scale, advance=not in_place_counters)
+        if in_place_counters:
+            ring_advance(st)
+        self.note_step(layer_idx)
+        return o
+
+    def note_step(self, layer_idx: int) -> None:
+        """Host-side bookkeeping of one decode step of `layer_idx` (token counts; no GPU work): `decode` calls it,
+        and so does every replay of a recorded step."""
         self._layer_tokens[layer_idx] = self._layer_tokens.get(layer_idx, 0) + 1
         self._count_tokens(layer_idx, 1, whole_step=True)
-        return o
 
     def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
         """Tokens cached before the latest update of layer 0 (`former_tokens`,

@@ -217,7 +217,9 @@ int nha_hybrid_prologue(const NhaHybridPrologueArgs* a) {
   NHA_CHECK_ARG(a->D == 64 || a->D == 128 || a->D == 256, "nha_hybrid_prologue: head size must be 64, 128 or 256, got %d", a->D);
   NHA_CHECK_ARG(a->M % 8 == 0, "nha_hybrid_prologue: M must be a multiple of 8, got %d", a->M);
   NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_hybrid_prologue: bad dtype %d", a->dtype);
-  NHA_CHECK_ARG(a->q && a->k && a->v && a->cos && a->sin, "nha_hybrid_prologue: q, k, v, cos, sin are required");
+  NHA_CHECK_ARG(a->q && a->k && a->v, "nha_hybrid_prologue: q, k, v are required");
+  NHA_CHECK_ARG((a->cos && a->sin) || (a->positions && a->inv_freq),
+                "nha_hybrid_prologue: pass cos and sin, or positions and inv_freq");
   NHA_CHECK_ARG(a->q_out && a->sq_out && a->k_out && a->sk_out && a->v_out && a->g_out,
                 "nha_hybrid_prologue: q_out, sq_out, k_out, sk_out, v_out, g_out are required");
   NHA_CHECK_ARG((a->q_weight == nullptr) == (a->k_weight == nullptr), "nha_hybrid_prologue: pass both norm weights or neither");

@@ -23,6 +23,8 @@ struct HP {
   const void *q_weight, *k_weight;                  // [D], or null: no norm
   const void *cos, *sin;                            // [B or 1][T][D]
   int64_t cs_batch_stride;                          // elements; 0 = one table for every sequence
+  const int64_t* positions;                         // [B*T] and inv_freq [D/2]: the tables' rows formed here instead
+  const float* inv_freq;
   const void* mask;                                 // [B*T] in the tensor dtype, or null
   void *q_out, *sq_out, *k_out, *sk_out, *v_out, *g_out, *s_out;
   int B, T, HQ, H, M;
@@ -43,7 +45,16 @@ __global__ __launch_bounds__(256) void hybrid_prologue_kernel(const HP p) {
   const int c = lane % LPR, rsub = lane / LPR;
   const bool first_half = c < LPR / 2;
   float cs[8], sn[8];
-  {
+  if (p.positions) {
+    // cos / sin of position * inv_freq[column % (D / 2)], each rounded to the tensor dtype as a table entry would be
+    const float pos = (float)p.positions[tok];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ang = pos * p.inv_freq[(8 * c + e) % (D / 2)];
+      cs[e] = rnd<T>(cosf(ang));
+      sn[e] = rnd<T>(sinf(ang));
+    }
+  } else {
     const int64_t off = (int64_t)b * p.cs_batch_stride + (int64_t)t * D + 8 * c;
     Elem<T>::ld8((const T*)p.cos + off, cs);
     Elem<T>::ld8((const T*)p.sin + off, sn);
@@ -201,6 +212,7 @@ int hybrid_prologue_impl(const NhaHybridPrologueArgs* a) {
   p.q_stride = a->q_stride; p.k_stride = a->k_stride; p.v_stride = a->v_stride; p.f_stride = a->f_stride;
   p.q_weight = a->q_weight; p.k_weight = a->k_weight;
   p.cos = a->cos; p.sin = a->sin; p.cs_batch_stride = a->cs_batch_stride;
+  p.positions = a->positions; p.inv_freq = a->inv_freq;
   p.mask = a->mask;
   p.q_out = a->q_out; p.sq_out = a->sq_out; p.k_out = a->k_out; p.sk_out = a->sk_out;
   p.v_out = a->v_out; p.g_out = a->g_out; p.s_out = a->s_out;

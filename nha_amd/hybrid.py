@@ -160,6 +160,7 @@ class HybridNHAAttention(nn.Module):
 
     qk_norm = False
     fuse_glue = True      # inference: fused projection GEMM + one glue launch (False keeps the tensor-op chain)
+    _recording = False    # set while a decode step is recorded into a HIP graph (record_decode_step)
 
     def __init__(self, config, layer_idx: int = 0):
         super().__init__()
@@ -208,6 +209,10 @@ class HybridNHAAttention(nn.Module):
         w, b = self._fused_wb
         return F.linear(x, w, b)
 
+    def record_decode_step(self, cache: NHARingCache, batch: int) -> "RecordedDecodeStep":
+        """Record this block's single-token step on `cache` (which holds the prompt) into a HIP graph."""
+        return RecordedDecodeStep(self, cache, batch)
+
     @property
     def is_nha_layer(self) -> bool:
         return self.window_size <= NHA_MAX_WINDOW
@@ -253,9 +258,17 @@ class HybridNHAAttention(nn.Module):
         if fused:
             y = self._fused_projection(hidden_states, with_gates=nha)
             o0, o1, o2 = HQ * D, HQ * D + H * D, HQ * D + 2 * H * D
-            cos, sin = self._tables(hidden_states, position_ids, position_embeddings, past_key_value, T)
+            cos = sin = pos = inv = None
+            if position_embeddings is not None:
+                cos, sin = self._tables(hidden_states, position_ids, position_embeddings, past_key_value, T)
+            else:                                  # the rows of the rotary tables are formed inside the glue launch
+                pos, inv = position_ids, self.rotary_emb.inv_freq(hidden_states.device)
+                if pos is None:
+                    start = past_key_value.layer_tokens(self.layer_idx) if past_key_value is not None else 0
+                    pos = torch.arange(start, start + T, device=hidden_states.device)[None].expand(B, T)
             q, sq, k, sk, v, g, s = nha_hybrid_prologue(
-                y[..., :o0], y[..., o0:o1], y[..., o1:o2], y[..., o2:] if nha else None, cos, sin, num_heads=HQ,
+                y[..., :o0], y[..., o0:o1], y[..., o1:o2], y[..., o2:] if nha else None, cos, sin, positions=pos, inv_freq=inv,
+                num_heads=HQ,
                 num_kv_heads=H, head_dim=D, num_slots=M, q_weight=self.q_norm.weight if self.qk_norm else None,
                 k_weight=self.k_norm.weight if self.qk_norm else None,
                 eps=self.q_norm.variance_epsilon if self.qk_norm else 0.0, mask=mask2d,
@@ -300,7 +313,7 @@ class HybridNHAAttention(nn.Module):
 
         if decode_step:
             o = past_key_value.decode(self.layer_idx, q[:, 0], sq[:, 0], sk[:, 0], k[:, 0], v[:, 0], g[:, 0],
-                                      scale=self.scaling)[:, None]
+                                      scale=self.scaling, in_place_counters=self._recording)[:, None]
         else:
             if has_state:
                 raise NotImplementedError("a multi-token step on top of a cached prompt is not supported "
@@ -326,6 +339,59 @@ class HybridNHAAttention(nn.Module):
                 past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W)
         o = self.o_proj(o.reshape(B, T, HQ * D))
         return o, None
+
+
+class RecordedDecodeStep:
+    """One decode step of an attention block as a HIP graph: `step(hidden [B,1,hidden], position_ids [B,1])` copies
+    its arguments into the graph's input buffers, replays the recorded launches (fused projection, glue, ring decode
+    step, counter advance, output projection) and returns the graph's output buffer `[B,1,hidden]` (overwritten by
+    the next step).  The host does no per-launch work, which is what a step of a few tens of microseconds of GPU
+    time needs: the eager block spends more time issuing its launches than the GPU spends on them."""
+
+    def __init__(self, block: "HybridNHAAttention", cache: NHARingCache, batch: int, mask_len: Optional[int] = None):
+        if not cache.has_ring(block.layer_idx):
+            raise ValueError("record a decode step after the prompt has been handed to the cache")
+        p = block.q_proj.weight
+        self.block, self.cache = block, cache
+        self.x = torch.zeros(batch, 1, block.hidden_size, dtype=p.dtype, device=p.device)
+        self.pos = torch.zeros(batch, 1, dtype=torch.long, device=p.device)
+        st = cache.states[block.layer_idx]
+        count0 = st.count.clone()
+        snap = [t.clone() for t in (st.hk, st.hv, st.ring_k, st.ring_kg, st.ring_v, st.ring_g)]
+        tokens = (cache._layer_tokens.get(block.layer_idx, 0), cache.former_tokens, cache._seen_tokens)
+        # the launches are issued once eagerly on a side stream (lazy kernel set-up happens outside the recording),
+        # then recorded; both runs are steps on the real cache, so its contents are put back afterwards
+        side = torch.cuda.Stream(device=p.device)
+        side.wait_stream(torch.cuda.current_stream(p.device))
+        with torch.cuda.stream(side), torch.no_grad():
+            self._run()
+        torch.cuda.current_stream(p.device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            self.out = self._run()
+        for t, s in zip((st.hk, st.hv, st.ring_k, st.ring_kg, st.ring_v, st.ring_g), snap):
+            t.copy_(s)
+        st.count.copy_(count0)
+        cache._layer_tokens[block.layer_idx], cache.former_tokens, cache._seen_tokens = tokens
+        self._count_ptr = st.count.data_ptr()
+
+    def _run(self):
+        self.block._recording = True
+        try:
+            return self.block(self.x, position_ids=self.pos, past_key_value=self.cache, use_cache=True)[0]
+        finally:
+            self.block._recording = False
+
+    @torch.no_grad()
+    def step(self, hidden_states: torch.Tensor, position_ids: torch.Tensor) -> torch.Tensor:
+        if self.cache.states[self.block.layer_idx].count.data_ptr() != self._count_ptr:
+            raise RuntimeError("the cache took an eager decode step since this step was recorded (the eager step trades "
+                               "the ring's two counter arrays, the recording holds the address of one): record again")
+        self.x.copy_(hidden_states)
+        self.pos.copy_(position_ids)
+        self.graph.replay()
+        self.cache.note_step(self.block.layer_idx)
+        return self.out
 
 
 class Qwen3MoeNativeHybridAttention(HybridNHAAttention):

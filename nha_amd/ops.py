@@ -467,26 +467,38 @@ def _row_view(x: torch.Tensor, width: int, what: str):
 @torch.no_grad()
 def nha_hybrid_prologue(q, k, v, f, cos, sin, *, num_heads: int, num_kv_heads: int, head_dim: int, num_slots: int,
                         q_weight=None, k_weight=None, eps: float = 1e-6, mask=None, gate_logit_normalizer: float = 8.0,
-                        want_s: bool = True):
+                        want_s: bool = True, positions=None, inv_freq=None):
     """One launch for the glue of a hybrid decoder attention block (inference): per-head RMSNorm of q and k (when
     weights are given), rotary embedding, the gates and the padding mask
     (nha_fla/models/qwen3_moe_nha/qwennha.py:103-144, :240-247).  q / k / v / f are `[B, T, heads * dim]` views
-    (column slices of one fused projection output are read in place); cos / sin `[B or 1, T, D]`; mask `[B, T]` or
-    None; f None writes g = s = 0.  Returns contiguous q, sq `[B,T,HQ,D]`, k, sk, v `[B,T,H,D]`, g, s `[B,T,H,M]`
+    (column slices of one fused projection output are read in place); cos / sin `[B or 1, T, D]`, or None with
+    `positions [B, T]` (int64) and `inv_freq [D/2]` (fp32), from which the kernel forms the table rows itself; mask
+    `[B, T]` or None; f None writes g = s = 0.  Returns contiguous q, sq `[B,T,HQ,D]`, k, sk, v `[B,T,H,D]`, g, s `[B,T,H,M]`
     (s None unless `want_s`)."""
-    _need_cuda(q, k, v, cos, sin)
+    _need_cuda(q, k, v, cos, sin, positions, inv_freq)
     B, T = q.shape[0], q.shape[1]
     HQ, H, D, M = num_heads, num_kv_heads, head_dim, num_slots
     dt, dev = q.dtype, q.device
+    if (cos is None) == (positions is None):
+        raise ValueError("pass either cos and sin or positions and inv_freq")
     q, qs = _row_view(q, HQ * D, "q")
     k, ks = _row_view(k, H * D, "k")
     v, vs = _row_view(v, H * D, "v")
     fs = 0
     if f is not None:
         f, fs = _row_view(f, H * M, "f")
-    if cos.shape[-1] != D or cos.shape[-2] != T or cos.shape[0] not in (1, B) or sin.shape != cos.shape:
-        raise ValueError(f"cos / sin must be [{B} or 1, {T}, {D}], got {tuple(cos.shape)} / {tuple(sin.shape)}")
-    cos, sin = cos.to(dt).contiguous(), sin.to(dt).contiguous()
+    cs_stride = 0
+    if cos is not None:
+        if cos.shape[-1] != D or cos.shape[-2] != T or cos.shape[0] not in (1, B) or sin.shape != cos.shape:
+            raise ValueError(f"cos / sin must be [{B} or 1, {T}, {D}], got {tuple(cos.shape)} / {tuple(sin.shape)}")
+        cos, sin = cos.to(dt).contiguous(), sin.to(dt).contiguous()
+        cs_stride = T * D if cos.shape[0] == B and B > 1 else 0
+    else:
+        if tuple(positions.shape) != (B, T) or inv_freq.numel() != D // 2:
+            raise ValueError(f"positions must be [{B}, {T}] and inv_freq [{D // 2}], got {tuple(positions.shape)} / "
+                             f"{tuple(inv_freq.shape)}")
+        positions = positions.to(torch.int64).contiguous()
+        inv_freq = inv_freq.to(torch.float32).contiguous()
     for x in (k, v, f, q_weight, k_weight):
         if x is not None and x.dtype != dt:
             raise ValueError(f"every tensor must have the dtype of q ({dt}), got {x.dtype}")
@@ -499,7 +511,7 @@ def nha_hybrid_prologue(q, k, v, f, cos, sin, *, num_heads: int, num_kv_heads: i
         q=_ptr(q), k=_ptr(k), v=_ptr(v), f=_ptr(f), q_stride=qs, k_stride=ks, v_stride=vs, f_stride=fs,
         q_weight=_ptr(None if q_weight is None else q_weight.contiguous()),
         k_weight=_ptr(None if k_weight is None else k_weight.contiguous()), cos=_ptr(cos), sin=_ptr(sin),
-        cs_batch_stride=(T * D if cos.shape[0] == B and B > 1 else 0), mask=_ptr(mask), q_out=_ptr(qo), sq_out=_ptr(sqo),
+        cs_batch_stride=cs_stride, positions=_ptr(positions), inv_freq=_ptr(inv_freq), mask=_ptr(mask), q_out=_ptr(qo), sq_out=_ptr(sqo),
         k_out=_ptr(ko), sk_out=_ptr(sko), v_out=_ptr(vo), g_out=_ptr(go), s_out=_ptr(so), B=B, T=T, HQ=HQ, H=H, D=D, M=M,
         dtype=_dtype_code(q), eps=float(eps), gate_logit_normalizer=float(gate_logit_normalizer), stream=_stream(dev))
     _lib.check(_lib.load().nha_hybrid_prologue(C.byref(a)))

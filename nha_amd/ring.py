@@ -79,6 +79,13 @@ class NHARingState:
         return self.ring_k.shape[1]
 
 
+def ring_advance(state: NHARingState) -> None:
+    """count += 1 for every sequence, in place (one small launch).  For steps taken with ``advance=False``: a
+    captured HIP graph replays fixed pointers, so it cannot trade the two counter arrays as the eager step does;
+    it runs the step on ``count`` and then this launch."""
+    _lib.check(_lib.load().nha_decode_advance(_ptr(state.count), state.count.numel(), _stream(state.count.device)))
+
+
 def ring_decode_step(state: NHARingState, q: torch.Tensor, sq: torch.Tensor, k_new: torch.Tensor,
                      kg_new: torch.Tensor, v_new: torch.Tensor, g_new: torch.Tensor,
                      scale: Optional[float] = None, out: Optional[torch.Tensor] = None,

@@ -54,7 +54,7 @@ def test_struct_sizes_match_the_header(tmp_path):
                                                  "stream")]
     probes += [("NhaShortConvBwdArgs", f) for f in ("x", "dy", "dx", "dweight_partial", "dbias_partial", "cu_seqlens", "T_tot",
                                                     "KS", "activation", "dtype", "stream")]
-    probes += [("NhaHybridPrologueArgs", f) for f in ("q", "f", "q_stride", "f_stride", "q_weight", "cos", "cs_batch_stride", "mask",
+    probes += [("NhaHybridPrologueArgs", f) for f in ("q", "f", "q_stride", "f_stride", "q_weight", "cos", "cs_batch_stride", "positions", "inv_freq", "mask",
                                                       "q_out", "s_out", "B", "M", "dtype", "eps", "gate_logit_normalizer", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
            'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));',

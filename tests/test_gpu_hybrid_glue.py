@@ -88,6 +88,13 @@ def test_hybrid_prologue_matches_the_tensor_op_chain(dt, HQ, H, D, M, norm, gate
                                   eps=1e-6, mask=None if mask is None else mask.cuda())
         for name, a, b in zip(("q", "sq", "k", "sk", "v", "g", "s"), got, ref):
             close(f"{name} B{B} T{T}", a, b, dt)
+        # the same with the table rows formed inside the launch from the positions
+        got_p = nha_hybrid_prologue(dev_parts[0], dev_parts[1], dev_parts[2], dev_parts[3] if gates else None, None, None,
+                                    positions=pos.expand(B, T).cuda(), inv_freq=inv.cuda(), num_heads=HQ, num_kv_heads=H,
+                                    head_dim=D, num_slots=M, q_weight=None if qw is None else qw.cuda(),
+                                    k_weight=None if kw is None else kw.cuda(), eps=1e-6, mask=None if mask is None else mask.cuda())
+        for name, a, b in zip(("q", "sq", "k", "sk", "v", "g", "s"), got_p, ref):
+            close(f"{name} from positions B{B} T{T}", a, b, dt)
         # one table for every sequence ([1, T, D]) and no s (what a decode step asks for)
         if B > 1:
             pos1 = torch.arange(T)[None] + 11
@@ -165,3 +172,47 @@ def test_zero_sink_rescale_matches_the_log_space_formula(dt, D):
     assert float(err.max()) <= tol, float(err.max())
     # rows with every sink still in view are left bit-identical
     assert torch.equal(got[:, : W - 1 - M], o[:, : W - 1 - M])
+
+
+@pytest.mark.parametrize("window", [64, 2048])
+def test_recorded_decode_step_replays_match_eager_steps(window):
+    """A block's decode step recorded into a HIP graph: twelve replays, with eager work of the same program and a
+    synchronisation between them, each against the eager step of a second cache that took the same prompt; the ring
+    contents and counters agree at the end.  An NHA layer (window 64: pops start at once after a 100-token prompt)
+    and a zero-sink layer."""
+    from nha_amd import NHACache
+    from nha_amd.hybrid import HybridNHAConfig, Qwen3MoeNativeHybridAttention
+    cfg = HybridNHAConfig(hidden_size=256, num_attention_heads=8, num_key_value_heads=2, head_dim=128, num_slots=64,
+                          window_size=64, block_size=1 if window == 2048 else None, transformer_idx=0 if window == 2048 else None)
+    torch.manual_seed(11)
+    m = Qwen3MoeNativeHybridAttention(cfg, 0).to(torch.bfloat16).cuda().eval()
+    assert m.window_size == window
+    B, T0 = 3, 100
+    x0 = torch.randn(B, T0, 256, device="cuda").to(torch.bfloat16)
+    pos0 = torch.arange(T0, device="cuda")[None].expand(B, -1)
+    eager, rec = NHACache(), NHACache()
+    with torch.no_grad():
+        m(x0, position_ids=pos0, past_key_value=eager, use_cache=True)
+        m(x0, position_ids=pos0, past_key_value=rec, use_cache=True)
+    step = m.record_decode_step(rec, B)
+    assert rec.layer_tokens(0) == T0 and int(rec.states[0].count[0]) == T0     # recording leaves the cache as it was
+    gen = torch.Generator("cuda").manual_seed(5)
+    for t in range(T0, T0 + 12):
+        xs = torch.randn(B, 1, 256, device="cuda", generator=gen).to(torch.bfloat16)
+        pos = torch.full((B, 1), t, device="cuda")
+        with torch.no_grad():
+            want, _ = m(xs, position_ids=pos, past_key_value=eager, use_cache=True)
+        got = step.step(xs, pos).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (t, float((got.float() - want.float()).abs().max()))
+        _ = (xs.float() @ xs.float().transpose(1, 2)).sum().item()      # eager work and a sync between replays
+    assert rec.layer_tokens(0) == eager.layer_tokens(0) == T0 + 12
+    a, b = eager.states[0], rec.states[0]
+    assert torch.equal(a.count, b.count)
+    for name in ("hk", "hv", "ring_k", "ring_kg", "ring_v", "ring_g"):
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
+    # an eager step on the recorded cache moves its counters to the other array: the recording refuses to go on
+    with torch.no_grad():
+        m(xs, position_ids=pos + 1, past_key_value=rec, use_cache=True)
+    with pytest.raises(RuntimeError, match="record again"):
+        step.step(xs, pos + 2)
