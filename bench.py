@@ -402,8 +402,8 @@ def bench_hybrid(torch, steps, warmup):
                 op = lambda: fused_chunk_nha_prefill(q=q, k=k, v=v, rotary_q=sq, rotary_k=sk, s=s_, g=g, window_size=W,
                                                      scale=D ** -0.5)
             else:
-                from nha_amd import chunk_nha
-                op = lambda: chunk_nha(sq, sk, q, k, v, s_, g, window_size_left=W - 1, gsa_kv_shift=W, scale=D ** -0.5)
+                from nha_amd.ops import zero_sink_attention
+                op = lambda: (zero_sink_attention(sq, sk, v, W, M, scale=D ** -0.5),)
             o = op()[0]
             res["attention_op_ms"] = timed(op, n=max(steps // 2, 4))
             res["o_proj_ms"] = timed(lambda: blk.o_proj(o.reshape(2, 8192, HQ * D)), n=max(steps // 2, 4))

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define NHA_ABI_VERSION 8
+#define NHA_ABI_VERSION 9
 
 enum { NHA_DTYPE_F32 = 0, NHA_DTYPE_BF16 = 1 };
 enum {
@@ -349,6 +349,41 @@ typedef struct NhaHybridPrologueArgs {
 } NhaHybridPrologueArgs;
 
 int nha_hybrid_prologue(const NhaHybridPrologueArgs* a);
+
+/* ------------------------------------------------------------------------------------------
+ * Sliding-window attention with zero sinks: the "full attention" layers of the hybrid models
+ * (nha_fla/models/qwen3_moe_nha/qwennha.py:323-336 with naive_swa, :400-413;
+ * nha_fla/models/llama3_nha/llamanha.py:204-216).  `sinks` all-zero key / value rows precede every
+ * sequence; query t (position in its sequence) attends the keys j with t - window < j <= t and the
+ * clamp(window - 1 - t, 0, sinks) sinks its window still covers, each with logit 0 and value 0:
+ *   o_t = sum_j e^(scale q_t.k_j) v_j / (sum_j e^(scale q_t.k_j) + sinks_in_view(t)).
+ * q [T_tot,HQ,D] and k, v [T_tot,H,D] packed as for nha_prefill_fwd (q and k already rotated), with the
+ * same three index tables; o [T_tot,HQ,D]; lse [T_tot,HQ] fp32 or NULL: the log of the denominator.
+ * One launch of the prefill's window loop (no slot branch, no state pass) + an exact pass for rows whose
+ * sums leave the range of the fixed softmax reference.  Served: bf16, D = 64 or 128, HQ / H a
+ * multiple of four; other shapes return NHA_ERR_UNSUPPORTED (callers then run nha_prefill_fwd with
+ * zero slot writes and nha_zero_sink_rescale).  scratch: nha_sink_window_scratch_bytes(a) bytes. */
+typedef struct NhaSinkWindowArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;
+  const int32_t* cu_seqlens;
+  const int32_t* chunk_indices;
+  const int32_t* chunk_offsets;
+  void* scratch;
+  size_t scratch_bytes;
+  int32_t T_tot, N, NT, HQ, H, D;
+  int32_t window;
+  int32_t sinks;
+  int32_t dtype;
+  float scale;
+  void* stream;
+} NhaSinkWindowArgs;
+
+size_t nha_sink_window_scratch_bytes(const NhaSinkWindowArgs* a);
+int nha_sink_window_fwd(const NhaSinkWindowArgs* a);
 
 /* The "full attention" layers of the hybrid models (window 2048: a sliding-window softmax preceded by M all-zero
  * key / value rows, nha_fla/models/qwen3_moe_nha/qwennha.py:323-336, :400-413;

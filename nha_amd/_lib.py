@@ -14,7 +14,7 @@ NHA_DTYPE_F32, NHA_DTYPE_BF16 = 0, 1
 NHA_IMPL_AUTO, NHA_IMPL_SIMPLE, NHA_IMPL_MFMA = 0, 1, 2
 NHA_DECODE_WINDOW, NHA_DECODE_LOGITS, NHA_DECODE_RING = 0, 1, 2
 NHA_OK, NHA_ERR_INVALID, NHA_ERR_UNSUPPORTED, NHA_ERR_SCRATCH, NHA_ERR_LAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 8
+ABI_VERSION = 9
 NHA_NOALLOC_SCRATCH_BYTES = 32 << 20   # workspace of nha_prefill_fwd_noalloc (include/nha_hip.h)
 NHA_FMAP_NONE, NHA_FMAP_SWISH, NHA_FMAP_RELU = 0, 1, 2
 
@@ -22,7 +22,7 @@ EXPORTS = (
     "nha_prefill_scratch_bytes", "nha_prefill_fwd", "nha_prefill_fwd_noalloc", "nha_prefill_bwd_scratch_bytes", "nha_prefill_bwd",
     "nha_decode_step", "nha_decode_advance", "nha_layer_prologue", "nha_layer_epilogue",
     "nha_layer_prologue_bwd", "nha_layer_epilogue_bwd", "nha_layer_epilogue_bwd_parts",
-    "nha_short_conv", "nha_short_conv_bwd", "nha_short_conv_bwd_parts", "nha_hybrid_prologue", "nha_zero_sink_rescale",
+    "nha_short_conv", "nha_short_conv_bwd", "nha_short_conv_bwd_parts", "nha_hybrid_prologue", "nha_zero_sink_rescale", "nha_sink_window_fwd", "nha_sink_window_scratch_bytes",
     "nha_varlen_num_chunks", "nha_varlen_indices", "nha_last_error", "nha_abi_version",
 )
 
@@ -103,6 +103,16 @@ class NhaHybridPrologueArgs(C.Structure):
         ("v_out", C.c_void_p), ("g_out", C.c_void_p), ("s_out", C.c_void_p),
         ("B", C.c_int32), ("T", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32), ("D", C.c_int32), ("M", C.c_int32),
         ("dtype", C.c_int32), ("eps", C.c_float), ("gate_logit_normalizer", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
+class NhaSinkWindowArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
+        ("cu_seqlens", C.c_void_p), ("chunk_indices", C.c_void_p), ("chunk_offsets", C.c_void_p),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t),
+        ("T_tot", C.c_int32), ("N", C.c_int32), ("NT", C.c_int32), ("HQ", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
+        ("window", C.c_int32), ("sinks", C.c_int32), ("dtype", C.c_int32), ("scale", C.c_float), ("stream", C.c_void_p),
     ]
 
 
@@ -198,6 +208,10 @@ def load() -> C.CDLL:
     lib.nha_hybrid_prologue.argtypes = [C.POINTER(NhaHybridPrologueArgs)]
     lib.nha_zero_sink_rescale.restype = C.c_int
     lib.nha_zero_sink_rescale.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int32] * 7 + [C.c_void_p]
+    lib.nha_sink_window_scratch_bytes.restype = C.c_size_t
+    lib.nha_sink_window_scratch_bytes.argtypes = [C.POINTER(NhaSinkWindowArgs)]
+    lib.nha_sink_window_fwd.restype = C.c_int
+    lib.nha_sink_window_fwd.argtypes = [C.POINTER(NhaSinkWindowArgs)]
     lib.nha_short_conv.restype = C.c_int
     lib.nha_short_conv.argtypes = [C.POINTER(NhaShortConvArgs)]
     lib.nha_short_conv_bwd.restype = C.c_int

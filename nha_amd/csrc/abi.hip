@@ -249,6 +249,37 @@ int nha_zero_sink_rescale(void* o, const float* lse_swa, int32_t B, int32_t T, i
   return zero_sink_rescale_impl(o, lse_swa, B, T, HQ, D, W, M, dtype, stream);
 }
 
+static int check_sink_window(const NhaSinkWindowArgs* a, bool pointers) {
+  NHA_CHECK_ARG(a != nullptr, "nha_sink_window_fwd: null args");
+  NHA_CHECK_ARG(a->T_tot > 0 && a->N > 0 && a->NT > 0 && a->HQ > 0 && a->H > 0 && a->D > 0, "nha_sink_window_fwd: non-positive dimension");
+  NHA_CHECK_ARG(a->HQ % a->H == 0, "nha_sink_window_fwd: HQ (%d) must be a multiple of H (%d)", a->HQ, a->H);
+  NHA_CHECK_ARG(a->window >= 1 && a->sinks >= 0, "nha_sink_window_fwd: window must be >= 1 and sinks >= 0, got %d / %d", a->window, a->sinks);
+  NHA_CHECK_ARG(a->dtype == NHA_DTYPE_F32 || a->dtype == NHA_DTYPE_BF16, "nha_sink_window_fwd: bad dtype %d", a->dtype);
+  if (pointers) {
+    NHA_CHECK_ARG(a->q && a->k && a->v && a->o, "nha_sink_window_fwd: q, k, v, o are required");
+    NHA_CHECK_ARG(a->cu_seqlens && a->chunk_indices && a->chunk_offsets,
+                  "nha_sink_window_fwd: cu_seqlens, chunk_indices and chunk_offsets are required");
+    NHA_CHECK_ARG(a->scratch != nullptr, "nha_sink_window_fwd: scratch is required");
+  }
+  return NHA_OK;
+}
+
+size_t nha_sink_window_scratch_bytes(const NhaSinkWindowArgs* a) {
+  if (check_sink_window(a, false) != NHA_OK) return 0;
+  return sink_window_scratch_bytes(a);
+}
+
+int nha_sink_window_fwd(const NhaSinkWindowArgs* a) {
+  const int rc = check_sink_window(a, true);
+  if (rc != NHA_OK) return rc;
+  const size_t need = sink_window_scratch_bytes(a);
+  if (a->scratch_bytes < need) {
+    set_error("nha_sink_window_fwd: scratch has %zu bytes, %zu needed", a->scratch_bytes, need);
+    return NHA_ERR_SCRATCH;
+  }
+  return sink_window_impl(a);
+}
+
 int nha_layer_epilogue(const NhaLayerEpilogueArgs* a) {
   NHA_CHECK_ARG(a != nullptr, "nha_layer_epilogue: null args");
   NHA_CHECK_ARG(a->rows > 0 && a->dim > 0, "nha_layer_epilogue: non-positive dimension");

@@ -133,6 +133,8 @@ int layer_prologue_bwd_impl(const NhaLayerPrologueBwdArgs* a);
 int layer_epilogue_bwd_parts(int rows);
 int layer_epilogue_bwd_impl(const NhaLayerEpilogueBwdArgs* a);
 int hybrid_prologue_impl(const NhaHybridPrologueArgs* a);
+int sink_window_impl(const NhaSinkWindowArgs* a);
+size_t sink_window_scratch_bytes(const NhaSinkWindowArgs* a);
 int zero_sink_rescale_impl(void* o, const float* lse_swa, int B, int T, int HQ, int D, int W, int M, int dtype, void* stream);
 int short_conv_impl(const NhaShortConvArgs* a);
 int short_conv_bwd_parts(int T_tot);

@@ -55,6 +55,7 @@ struct MP {
   float* dtot;   // [NSLOT][H][MS]   total decay of a segment
   int* flags;    // [NT][H][4]       per 16-slot block: bit q = sub-block q decays past DECAY_CLAMP
   int T_tot, N, NT, HQ, H, NG, wl, shift;
+  int sinks;     // window-only launches (prefill_ring.hip, SINK): zero-logit keys in front of every sequence
   float scale;
 };
 

@@ -85,7 +85,11 @@ struct RingCfg {
   static_assert(6 * 4096 + 2 * 16384 <= 2 * NR * UB, "decay tables must fit the ring");
 };
 
-template <int D>
+// SINK: the window branch alone, with p.sinks zero-logit, zero-value keys in front of every sequence of which query t
+// (position in its sequence) still sees clamp(p.wl - t, 0, p.sinks): the "full attention" layers of the hybrid models
+// (nha_fla/models/qwen3_moe_nha/qwennha.py:323-336, :400-413).  No slot operands are requested, the slot branch and its
+// tables are skipped, and the sinks join the denominator in the epilogue with the weight 2^(-reference) each.
+template <int D, bool SINK = false>
 __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   using C = RingCfg<D>;
   constexpr int KS = C::KS, DB = C::DB, UB = C::UB, HB = C::HB, NR = C::NR, LPW = C::LPW;
@@ -408,7 +412,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     // u+3 .. u+NR-2, and the slot-branch operands while u <= NR-3 (queued behind unit NR-1 in iteration 0)
     if (u + 2 < nunits) {
       if (u + NR - 2 < nunits) {
-        if (u >= 1 && u <= NR - 3) wait_vm<LPW * (NR - 4) + C::NSLOT_LOADS>();
+        if (!SINK && u >= 1 && u <= NR - 3) wait_vm<LPW * (NR - 4) + C::NSLOT_LOADS>();
         else wait_vm<LPW * (NR - 4)>();
       } else {
         wait_vm<0>();
@@ -420,7 +424,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
       for (int i = 0; i < LPW; ++i) g2l16(u_isv[i] ? vreq : kreq, u_off[i], u_lds[i] + slot * UB);
     }
-    if (u == 0) issue_slot_operands();
+    if (!SINK && u == 0) issue_slot_operands();
     kreq -= ustep;
     vreq -= ustep;
     NHA_FENCE();
@@ -455,7 +459,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     const uint32_t v_c = C::RING_V + (u & (NR - 1)) * UB + vaddr;
 #pragma unroll
     for (int db = 0; db < DB; ++db) vf[db] = vfrag(v_c, db);
-    load_qg(qg, 0);
+    if (!SINK) load_qg(qg, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -478,6 +482,19 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     const bool bad = (16 * (qb0 + qb) + l16 < rows) && (Lw[qb][0] >= 0x1p100f || Lw[qb][0] < 0x1p-100f);
     if (__any(bad) && lane == 0) atomicOr(p.flags + cg * 4, 1 << (qb0 + qb));
   }
+  float lg[RQB];
+  if constexpr (SINK) {
+    // the sinks still in view: logit 0, i.e. 2^(0 - reference) each relative to the row's reference; value 0
+#pragma unroll
+    for (int qb = 0; qb < RQB; ++qb) {
+      const int irow = 16 * (qb0 + qb) + l16;
+      int n0 = p.wl - (c0 - bos + irow);
+      n0 = n0 < 0 ? 0 : (n0 > p.sinks ? p.sinks : n0);
+      lg[qb] = (float)n0 * fexp2(nm[qb]);
+      if (p.lse_swa && kb == 0 && irow < rows)
+        p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[qb][0] + lg[qb]) - nm[qb]) * LN2;
+    }
+  } else {
   // ================= slot branch, folded into the running softmax =================================
   // every LDS-direct request of this wave has landed, every wave is done with the ring
   wait_vm<0>();
@@ -549,7 +566,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 512);
     return __builtin_bit_cast(bf16x8, t);
   };
-  float lg[RQB];
   // No barrier holds the two waves of a SIMD together from here on, and the older one (w < 4) is served
   // first: left alone it ends about 5 k cycles before the younger, which then has the SIMD to itself.  The
   // younger wave gets the higher priority for the first of the two query blocks, so that both end together.
@@ -696,6 +712,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
         for (int db = 0; db < DB; ++db) O[db][qb] = mfma16(vfrag(C::TD + pr * UB + vaddr, db), bAv[pr], O[db][qb]);
       }
   }
+  }   // !SINK
 
   // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
   //      row block db + 1, and the two trade their halves) -------------------------------------------
@@ -724,19 +741,84 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   }
 }
 
-template <int D>
+template <int D, bool SINK>
 int launch_ring(const MP& p, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  const size_t lds = RingCfg<D>::BYTES;
-  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring_out_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  // the window-only launch has no slot operands: the ring is all the LDS it uses
+  const size_t lds = SINK ? (size_t)RingCfg<D>::TA : (size_t)RingCfg<D>::BYTES;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring_out_kernel<D, SINK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
   if (attr_err != hipSuccess) {
     set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((ring_out_kernel<D>), dim3(p.H * (p.NG / 4), p.NT), dim3(512), lds, st, p);
+  hipLaunchKernelGGL((ring_out_kernel<D, SINK>), dim3(p.H * (p.NG / 4), p.NT), dim3(512), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass, ring)");
   return NHA_OK;
+}
+
+__global__ __launch_bounds__(256) void zero_flags_kernel(int* flags, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) flags[i] = 0;
+}
+
+// Exact rows for the window-only launch: the rows of 16-row blocks whose window sums left the range of their fixed
+// softmax reference (flags set by ring_out_kernel<D, true>) are recomputed key by key in fp32 with a running maximum,
+// the sinks in view joining as keys of logit 0 and value 0.  grid (chunk, kv-head); workgroups of unflagged chunks
+// read four words and leave.
+template <int D>
+__global__ __launch_bounds__(256) void sink_repair_kernel(const MP p) {
+  const int chunk = blockIdx.x, h = blockIdx.y;
+  const int H = p.H, HQ = p.HQ;
+  const int* fl = p.flags + ((int64_t)chunk * H + h) * 4;
+  const int bits = fl[0] | fl[1] | fl[2] | fl[3];
+  if (bits == 0) return;
+  __shared__ float qs[D];
+  __shared__ float pw[256];
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  const int bos = p.cu[n], eos = p.cu[n + 1];
+  const int c0 = bos + it * BT;
+  const int rows = (eos - c0) < BT ? (eos - c0) : BT;
+  for (int hq = h * p.NG; hq < (h + 1) * p.NG; ++hq)
+    for (int r = 0; r < rows; ++r) {
+      if (!((bits >> (r >> 4)) & 1)) continue;
+      const int t = c0 + r;
+      __syncthreads();   // the previous row is finished
+      const bf16_t* qsw = p.q_swa + ((int64_t)t * HQ + hq) * D;
+      for (int i = tid; i < D; i += 256) qs[i] = bf16_to_f32(qsw[i]) * p.scale;
+      __syncthreads();
+      int n0 = p.wl - (t - bos);
+      n0 = n0 < 0 ? 0 : (n0 > p.sinks ? p.sinks : n0);
+      const int lo = p.wl < 0 ? bos : (t - p.wl > bos ? t - p.wl : bos);
+      float wm = -INFINITY, wsum = 0.f;
+      for (int j = lo + tid; j <= t; j += 256) {
+        const float d = dot_row<bf16_t>(qs, p.k_swa + ((int64_t)j * H + h) * D, D);
+        if (d > wm) {
+          wsum = wsum * expf(wm - d) + 1.f;
+          wm = d;
+        } else {
+          wsum += expf(d - wm);
+        }
+      }
+      float mt = block_max(wm, red);
+      if (n0 > 0) mt = fmaxf(mt, 0.f);
+      const float lw = block_sum(wm == -INFINITY ? 0.f : wsum * expf(wm - mt), red) + (float)n0 * expf(-mt);
+      if (tid == 0 && p.lse_swa) p.lse_swa[(int64_t)t * HQ + hq] = mt + logf(lw);
+      const float inv = 1.f / lw;
+      float acc = 0.f;   // value column tid (D <= 256 == threads)
+      for (int jb = lo; jb <= t; jb += 256) {
+        const int j = jb + tid;
+        __syncthreads();
+        pw[tid] = j <= t ? expf(dot_row<bf16_t>(qs, p.k_swa + ((int64_t)j * H + h) * D, D) - mt) * inv : 0.f;
+        __syncthreads();
+        const int cnt = (t - jb + 1) < 256 ? (t - jb + 1) : 256;
+        if (tid < D)
+          for (int x = 0; x < cnt; ++x) acc += pw[x] * bf16_to_f32(p.v[((int64_t)(jb + x) * H + h) * D + tid]);
+      }
+      if (tid < D) p.o[((int64_t)t * HQ + hq) * D + tid] = f32_to_bf16(acc);
+    }
 }
 
 }  // namespace
@@ -750,7 +832,37 @@ bool prefill_ring_supported(const mf::MP& p, int D) {
 }
 
 int prefill_ring_launch(const mf::MP& p, int D, hipStream_t st) {
-  return D == 64 ? launch_ring<64>(p, st) : launch_ring<128>(p, st);
+  return D == 64 ? launch_ring<64, false>(p, st) : launch_ring<128, false>(p, st);
+}
+
+// Sliding-window attention with zero sinks (nha_sink_window_fwd): the window loop of ring_out_kernel alone.  The scratch
+// holds the flags of the 16-row blocks that go to the exact pass.
+size_t sink_window_scratch_bytes(const NhaSinkWindowArgs* a) { return ((size_t)a->NT * a->H * 4 * sizeof(int) + 255) & ~(size_t)255; }
+
+int sink_window_impl(const NhaSinkWindowArgs* a) {
+  mf::MP p = {};
+  p.q_swa = (const bf16_t*)a->q; p.k_swa = (const bf16_t*)a->k; p.v = (const bf16_t*)a->v;
+  p.o = (bf16_t*)a->o;
+  p.lse_swa = a->lse;
+  p.cu = a->cu_seqlens; p.cidx = a->chunk_indices; p.coff = a->chunk_offsets;
+  p.flags = (int*)a->scratch;
+  p.T_tot = a->T_tot; p.N = a->N; p.NT = a->NT; p.HQ = a->HQ; p.H = a->H; p.NG = a->HQ / a->H;
+  p.wl = a->window - 1; p.shift = 0; p.scale = a->scale; p.sinks = a->sinks;
+  if (a->dtype != NHA_DTYPE_BF16 || !prefill_ring_supported(p, a->D) || p.NT > 65535) {
+    set_error("nha_sink_window_fwd: built for bf16, head size 64 or 128, a multiple of four query heads per kv-head, "
+              "at most 65535 chunks and tensors below 4 GiB (dtype=%d D=%d HQ/H=%d NT=%d)", a->dtype, a->D, p.NG, p.NT);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = (hipStream_t)a->stream;
+  const int nflags = a->NT * a->H * 4;
+  hipLaunchKernelGGL(zero_flags_kernel, dim3((nflags + 255) / 256), dim3(256), 0, st, p.flags, nflags);
+  NHA_CHECK_LAUNCH("nha_sink_window_fwd(flags)");
+  const int rc = a->D == 64 ? launch_ring<64, true>(p, st) : launch_ring<128, true>(p, st);
+  if (rc != NHA_OK) return rc;
+  if (a->D == 64) hipLaunchKernelGGL((sink_repair_kernel<64>), dim3(p.NT, p.H), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((sink_repair_kernel<128>), dim3(p.NT, p.H), dim3(256), 0, st, p);
+  NHA_CHECK_LAUNCH("nha_sink_window_fwd(exact rows)");
+  return NHA_OK;
 }
 
 }  // namespace nha

@@ -35,7 +35,7 @@ import torch.nn.functional as F
 
 from .cache import NHARingCache
 from .ops import (chunk_nha, fused_chunk_nha_prefill, hybrid_prologue_supported, nha_hybrid_prologue,
-                  nha_zero_sink_rescale_)
+                  nha_zero_sink_rescale_, zero_sink_attention, zero_sink_attention_supported)
 
 GATE_LOGIT_NORMALIZER = 8          # qwennha.py:62, llamanha.py:96
 FULL_ATTENTION_WINDOW = 2048       # qwennha.py:66, llamanha.py:60
@@ -319,7 +319,15 @@ class HybridNHAAttention(nn.Module):
                 raise NotImplementedError("a multi-token step on top of a cached prompt is not supported "
                                           "(the reference's modules do not support it either)")
             want_state = use_cache or past_key_value is not None
-            if nha and not torch.is_grad_enabled():
+            if not nha and not torch.is_grad_enabled() and zero_sink_attention_supported(sq, sk):
+                # a full-attention layer at inference: the window loop alone, the sinks in its denominator (no state
+                # pass, no slot branch, nothing to rescale); its slot states are zero by construction
+                o = zero_sink_attention(sq, sk, v, W, M, scale=self.scaling)
+                state = (None, None)
+                if want_state:
+                    state = (torch.zeros(B, H, D, M, dtype=torch.float32, device=o.device),
+                             torch.zeros(B, H, M, D, dtype=torch.float32, device=o.device))
+            elif nha and not torch.is_grad_enabled():
                 o, state = fused_chunk_nha_prefill(q=q, k=k, v=v, rotary_q=sq, rotary_k=sk, s=s, g=g, window_size=W,
                                                    output_final_state=want_state, scale=self.scaling)
             else:

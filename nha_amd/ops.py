@@ -454,7 +454,9 @@ def _row_view(x: torch.Tensor, width: int, what: str):
     """(tensor, elements between the rows of two tokens) of a `[B, T, width]` view whose rows are contiguous and
     whose tokens are evenly spaced (a column slice of a fused projection output, or a contiguous tensor)."""
     B, T = x.shape[0], x.shape[1]
-    if x.shape[2] != width or (width > 1 and x.stride(2) != 1) or (B > 1 and T > 1 and x.stride(0) != T * x.stride(1)):
+    if x.dim() != 3 or x.shape[2] != width:
+        raise ValueError(f"{what} must be [batch, tokens, {width}], got {tuple(x.shape)}")
+    if (width > 1 and x.stride(2) != 1) or (B > 1 and T > 1 and x.stride(0) != T * x.stride(1)):
         x = x.contiguous()
     stride = x.stride(1) if T > 1 else (x.stride(0) if B > 1 else width)
     esz = x.element_size()
@@ -516,6 +518,56 @@ def nha_hybrid_prologue(q, k, v, f, cos, sin, *, num_heads: int, num_kv_heads: i
         dtype=_dtype_code(q), eps=float(eps), gate_logit_normalizer=float(gate_logit_normalizer), stream=_stream(dev))
     _lib.check(_lib.load().nha_hybrid_prologue(C.byref(a)))
     return qo, sqo, ko, sko, vo, go, so
+
+
+def zero_sink_attention_supported(q: torch.Tensor, k: torch.Tensor) -> bool:
+    """Whether nha_sink_window_fwd serves these tensors: GPU, bf16, head size 64 or 128, a multiple of four query heads
+    per kv-head, tensors of one call below 4 GiB."""
+    HQ, H, D = q.shape[-2], k.shape[-2], q.shape[-1]
+    tokens = q.numel() // (HQ * D)
+    return (q.is_cuda and q.dtype == torch.bfloat16 and D in (64, 128) and HQ % H == 0 and (HQ // H) % 4 == 0
+            and tokens * H * D * 2 < (1 << 32) and tokens <= 65535 * CHUNK)
+
+
+@torch.no_grad()
+def zero_sink_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int, num_sinks: int,
+                        scale: Optional[float] = None, cu_seqlens: Optional[torch.Tensor] = None,
+                        output_lse: bool = False):
+    """Sliding-window softmax attention preceded by `num_sinks` all-zero key / value rows per sequence: the "full
+    attention" layers of the hybrid decoder models (nha_fla/models/qwen3_moe_nha/qwennha.py:323-336, :400-413).  q
+    `[B,T,HQ,D]` and k, v `[B,T,H,D]` (rotated q / k; `[1,T_tot,...]` with cu_seqlens); query t of a sequence sees keys
+    t - window < j <= t and clamp(window - 1 - t, 0, num_sinks) sinks of logit 0 and value 0.  One launch of the
+    prefill's window loop.  Returns o `[B,T,HQ,D]` (and the log of the softmax denominator `[B,T,HQ]`)."""
+    _need_cuda(q, k, v)
+    if not zero_sink_attention_supported(q, k):
+        raise _lib.NhaError(_lib.NHA_ERR_UNSUPPORTED, "zero_sink_attention: bf16, head size 64 / 128 and a multiple of four "
+                                                       "query heads per kv-head are served")
+    B, T, HQ, D = q.shape
+    H = k.shape[2]
+    if cu_seqlens is not None:
+        if B != 1:
+            raise ValueError("cu_seqlens needs the packed layout [1, T_tot, ...]")
+        cu_host = _cu_to_host(cu_seqlens)
+    else:
+        cu_host = np.arange(0, (B + 1) * T, T, dtype=np.int32)
+    if scale is None:
+        scale = D ** -0.5
+    dev = q.device
+    q_, k_, v_ = (_flat(x) for x in (q, k, v))
+    cu_d, idx_d, off_d, NT = prefill_tables(cu_host, dev)
+    o = torch.empty(B * T, HQ, D, dtype=q.dtype, device=dev)
+    lse = torch.empty(B * T, HQ, dtype=torch.float32, device=dev) if output_lse else None
+    a = _lib.NhaSinkWindowArgs(q=_ptr(q_), k=_ptr(k_), v=_ptr(v_), o=_ptr(o), lse=_ptr(lse), cu_seqlens=_ptr(cu_d),
+                               chunk_indices=_ptr(idx_d), chunk_offsets=_ptr(off_d), T_tot=B * T, N=cu_host.size - 1, NT=NT,
+                               HQ=HQ, H=H, D=D, window=int(window), sinks=int(num_sinks), dtype=_dtype_code(q),
+                               scale=float(scale), stream=_stream(dev))
+    lib = _lib.load()
+    nbytes = lib.nha_sink_window_scratch_bytes(C.byref(a))
+    scratch = _workspace(nbytes, dev, a.stream or 0)
+    a.scratch, a.scratch_bytes = _ptr(scratch), nbytes
+    _lib.check(lib.nha_sink_window_fwd(C.byref(a)))
+    o = o.view(B, T, HQ, D)
+    return (o, lse.view(B, T, HQ)) if output_lse else o
 
 
 @torch.no_grad()

@@ -56,12 +56,14 @@ def test_struct_sizes_match_the_header(tmp_path):
                                                     "KS", "activation", "dtype", "stream")]
     probes += [("NhaHybridPrologueArgs", f) for f in ("q", "f", "q_stride", "f_stride", "q_weight", "cos", "cs_batch_stride", "positions", "inv_freq", "mask",
                                                       "q_out", "s_out", "B", "M", "dtype", "eps", "gate_logit_normalizer", "stream")]
+    probes += [("NhaSinkWindowArgs", f) for f in ("q", "o", "lse", "cu_seqlens", "scratch", "scratch_bytes", "T_tot", "D", "window",
+                                                  "sinks", "dtype", "scale", "stream")]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "nha_hip.h"', 'int main(void) {',
            'printf("%zu %zu %zu\\n", sizeof(NhaPrefillArgs), sizeof(NhaDecodeArgs), sizeof(NhaPrefillBwdArgs));',
            'printf("%zu %zu\\n", sizeof(NhaLayerPrologueArgs), sizeof(NhaLayerEpilogueArgs));',
            'printf("%zu %zu\\n", sizeof(NhaLayerPrologueBwdArgs), sizeof(NhaLayerEpilogueBwdArgs));',
            'printf("%zu %zu\\n", sizeof(NhaShortConvArgs), sizeof(NhaShortConvBwdArgs));',
-           'printf("%zu\\n", sizeof(NhaHybridPrologueArgs));']
+           'printf("%zu %zu\\n", sizeof(NhaHybridPrologueArgs), sizeof(NhaSinkWindowArgs));']
     src += [f'printf("%zu\\n", offsetof({t}, {f}));' for t, f in probes]
     src += ['return 0; }']
     cfile = tmp_path / "probe.c"
@@ -74,8 +76,8 @@ def test_struct_sizes_match_the_header(tmp_path):
     assert int(out[3]) == C.sizeof(_lib.NhaLayerPrologueArgs) and int(out[4]) == C.sizeof(_lib.NhaLayerEpilogueArgs)
     assert int(out[5]) == C.sizeof(_lib.NhaLayerPrologueBwdArgs) and int(out[6]) == C.sizeof(_lib.NhaLayerEpilogueBwdArgs)
     assert int(out[7]) == C.sizeof(_lib.NhaShortConvArgs) and int(out[8]) == C.sizeof(_lib.NhaShortConvBwdArgs)
-    assert int(out[9]) == C.sizeof(_lib.NhaHybridPrologueArgs)
-    for (t, f), off in zip(probes, out[10:]):
+    assert int(out[9]) == C.sizeof(_lib.NhaHybridPrologueArgs) and int(out[10]) == C.sizeof(_lib.NhaSinkWindowArgs)
+    for (t, f), off in zip(probes, out[11:]):
         assert getattr(getattr(_lib, t), f).offset == int(off), (t, f)
 
 

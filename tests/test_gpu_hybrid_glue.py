@@ -10,6 +10,8 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+from oracle.hybrid_attention_ref import zero_sink_attention_ref
+
 pytestmark = pytest.mark.gpu
 
 
@@ -140,7 +142,13 @@ def test_block_with_fused_glue_matches_block_on_the_tensor_op_chain():
                 b, _ = m(xs, attention_mask=mask[:, :t + 1], position_ids=pos[:, t:t + 1], past_key_value=cache, use_cache=True)
                 steps.append(b)
         outs.append((a, steps))
+    # rotary tables handed in by the caller (`position_embeddings`, as the decoder models do) instead of formed in the launch
+    m.fuse_glue = True
+    with torch.no_grad():
+        tables = m.rotary_emb(x, pos[:, :150])
+        a2, _ = m(x, attention_mask=mask[:, :150], position_embeddings=tables)
     (a1, s1), (a0, s0) = outs
+    assert float((a2[0] - a1[0]).abs().max()) <= 1e-2 * float(a1[0].abs().max())
     scale = float(a0[1, 20:].abs().max())
     assert float((a1[0] - a0[0]).abs().max()) <= 2e-2 * scale and float((a1[1, 20:] - a0[1, 20:]).abs().max()) <= 2e-2 * scale
     for x1, x0 in zip(s1, s0):
@@ -216,3 +224,68 @@ def test_recorded_decode_step_replays_match_eager_steps(window):
         m(xs, position_ids=pos + 1, past_key_value=rec, use_cache=True)
     with pytest.raises(RuntimeError, match="record again"):
         step.step(xs, pos + 2)
+
+
+@pytest.mark.parametrize("HQ,H,D", [(8, 2, 128), (4, 1, 64), (16, 2, 128)])
+def test_zero_sink_attention_matches_the_restated_module_path(HQ, H, D):
+    """nha_sink_window_fwd (the prefill's window loop alone, sinks in the denominator) against the oracle's restatement
+    of the reference's zero-prefix sliding-window attention (pinned by brute force on the CPU), bf16: sequences shorter
+    and longer than the window, windows shorter than a 32-key unit, not a multiple of it, and 2048; packed sequences;
+    the returned log-denominator against the same softmax."""
+    from nha_amd.ops import zero_sink_attention
+    gen = torch.Generator().manual_seed(HQ + D)
+    bf = torch.bfloat16
+    for B, T, W, M in ((2, 300, 96, 64), (1, 700, 256, 64), (2, 130, 2048, 64), (1, 90, 20, 16), (3, 64, 33, 64)):
+        q = (torch.randn(B, T, HQ, D, generator=gen) * D ** -0.25).to(bf)
+        k = (torch.randn(B, T, H, D, generator=gen) * D ** -0.25).to(bf)
+        v = torch.randn(B, T, H, D, generator=gen).to(bf)
+        ref = zero_sink_attention_ref(q.double(), k.double(), v.double(), W, M)
+        got, lse = zero_sink_attention(q.cuda(), k.cuda(), v.cuda(), W, M, output_lse=True)
+        close(f"o B{B} T{T} W{W}", got, ref, bf)
+        # the denominator: log(sum over the window of e^(scale q.k) + sinks in view)
+        G = HQ // H
+        kk = k.double().repeat_interleave(G, 2)
+        sc = torch.einsum("bthd,bnhd->bhtn", q.double(), kk) / D ** 0.5
+        i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+        vis = (j <= i) & (j > i - W)
+        e = torch.exp(sc.masked_fill(~vis[None, None], -1e30)).sum(-1).transpose(1, 2)          # [B, T, HQ]
+        n0 = (W - 1 - torch.arange(T)).clamp(0, M).double()[None, :, None]
+        assert torch.allclose(lse.double().cpu(), torch.log(e + n0), atol=2e-2, rtol=1e-2)
+    # packed sequences (one of a single token, one ending mid-chunk)
+    cu = [0, 1, 130, 451]
+    q = (torch.randn(1, cu[-1], HQ, D, generator=gen) * D ** -0.25).to(bf)
+    k = (torch.randn(1, cu[-1], H, D, generator=gen) * D ** -0.25).to(bf)
+    v = torch.randn(1, cu[-1], H, D, generator=gen).to(bf)
+    got = zero_sink_attention(q.cuda(), k.cuda(), v.cuda(), 100, 64, cu_seqlens=torch.tensor(cu, dtype=torch.int32).cuda())
+    for a, b in zip(cu[:-1], cu[1:]):
+        ref = zero_sink_attention_ref(q[:, a:b].double(), k[:, a:b].double(), v[:, a:b].double(), 100, 64)
+        close(f"packed [{a},{b})", got[:, a:b], ref, bf)
+
+
+def test_zero_sink_attention_rows_far_from_the_fixed_reference_take_the_exact_pass():
+    """Scale 1 with unnormalised q / k: window scores of a few hundred above and below those of a row's nearest keys, so
+    rows whose sums leave the fp32 range around the fixed softmax reference are recomputed by the exact pass.  Finite
+    everywhere, relative L2 within 3e-2 (logits of this size make the softmax one-hot: single outputs move by more than
+    the element-wise bar under bf16 rounding of the scores)."""
+    from nha_amd.ops import zero_sink_attention
+    gen = torch.Generator().manual_seed(9)
+    bf = torch.bfloat16
+    B, T, HQ, H, D, W, M = 2, 200, 8, 2, 128, 100, 64
+    for qk in (1.0, 3.0):
+        q = (torch.randn(B, T, HQ, D, generator=gen) * qk).to(bf)
+        k = (torch.randn(B, T, H, D, generator=gen) * qk).to(bf)
+        v = torch.randn(B, T, H, D, generator=gen).to(bf)
+        got = zero_sink_attention(q.cuda(), k.cuda(), v.cuda(), W, M, scale=1.0).double().cpu()
+        qq, kk, vv = q.double(), k.double().repeat_interleave(HQ // H, 2), v.double().repeat_interleave(HQ // H, 2)
+        sc = torch.einsum("bthd,bnhd->bhtn", qq, kk)
+        i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+        vis = (j <= i) & (j > i - W)
+        sc = sc.masked_fill(~vis[None, None], -float("inf"))
+        n0 = (W - 1 - torch.arange(T)).clamp(0, M).double()
+        mx = torch.maximum(sc.amax(-1), torch.zeros(()).double())
+        e = torch.exp(sc - mx[..., None])
+        den = e.sum(-1) + n0[None, None] * torch.exp(-mx)
+        ref = torch.einsum("bhtn,bnhd->bthd", e / den[..., None], vv)
+        assert torch.isfinite(got).all()
+        rel = ((got - ref).norm() / ref.norm()).item()
+        assert rel <= 3e-2, (qk, rel)
