@@ -136,13 +136,16 @@ class NHARingCache:
         return c[0]
 
     def prefill(self, layer_idx: int, k_swa, k_gsa, v, g, final_state, cu_seqlens=None,
-                window_size: Optional[int] = None) -> NHARingState:
+                window_size: Optional[int] = None, zero_state: bool = False) -> NHARingState:
         """Hand a prompt's prefill (operands and final state of chunk_nha / fused_chunk_nha_prefill
         with (window_size_left, gsa_kv_shift) = (W-1, W)) over to the ring buffers of `layer_idx`.
         `window_size` overrides the cache's window for this layer (models mix short-window layers with
         2048-token ones)."""
         W = self._window(window_size)
         st = NHARingState.from_prefill(k_swa, k_gsa, v, g, final_state, W, cu_seqlens=cu_seqlens)
+        # `zero_state`: a layer whose gates are all 0 and whose write strengths are all 0 (the caller's promise, for
+        # this prompt and every later step): its slot state stays zero and the decode step skips it
+        st.zero_state = bool(zero_state)
         self._grow(layer_idx)
         self.states[layer_idx] = st
         longest = k_swa.shape[1] if cu_seqlens is None else int(st.count.max().item())

@@ -344,7 +344,7 @@ class HybridNHAAttention(nn.Module):
                         n0 = zero_sink_count(T, W, M, lse_swa.device)[None, :, None]
                         o = (o.to(torch.float32) * zero_sink_rescale(lse_swa, M, n0)[..., None]).to(o.dtype)
             if past_key_value is not None:
-                past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W)
+                past_key_value.prefill(self.layer_idx, sk, k, v, g, state, window_size=W, zero_state=not nha)
         o = self.o_proj(o.reshape(B, T, HQ * D))
         return o, None
 

@@ -29,6 +29,9 @@ class NHARingState:
     ring_g: torch.Tensor    # [B,W,H,M]
     count: torch.Tensor     # [B] int32; the tensor bound to this name changes with every step
     count_alt: Optional[torch.Tensor] = None   # the other counter array (the step writes count + 1 there)
+    # the slots never absorb anything (every cached log-gate is 0 and every write strength 0: the zero-sink layers of
+    # the hybrid models): hk and hv stay zero, and the step neither reads nor writes them
+    zero_state: bool = False
 
     @classmethod
     def empty(cls, B, H, K, V, M, W, dtype=torch.bfloat16, device="cuda") -> "NHARingState":
@@ -115,7 +118,8 @@ def ring_decode_step(state: NHARingState, q: torch.Tensor, sq: torch.Tensor, k_n
     a.ring_k, a.ring_kg, a.ring_v, a.ring_g = map(_ptr, (state.ring_k, state.ring_kg, state.ring_v, state.ring_g))
     a.k_new, a.kg_new, a.v_new, a.g_new = _ptr(k_new), _ptr(kg_new), _ptr(v_new), _ptr(g_new)
     a.count = _ptr(state.count)
-    a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(state.hk), _ptr(state.hv), _ptr(state.hk), _ptr(state.hv)
+    if not state.zero_state:      # NULL states: the kernel takes zeros and writes nothing back
+        a.hk_in, a.hv_in, a.hk_out, a.hv_out = _ptr(state.hk), _ptr(state.hv), _ptr(state.hk), _ptr(state.hv)
     a.o, a.stream = _ptr(o), _stream(q.device)
     if advance:
         # the kernel writes count + 1 into the second array; the two arrays then trade places
