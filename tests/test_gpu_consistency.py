@@ -56,3 +56,28 @@ def test_decode_continues_prefill(B, HQ, H, D, M, W, T0, n):
     for name, a, b in (("hk", st.hk, hk_full), ("hv", st.hv, hv_full)):
         err = (a - b).abs().max().item()
         assert err <= 2e-2 * max(b.abs().max().item(), 1.0), f"{name}: {err}"
+
+
+def test_workspace_cache_is_bounded_and_can_be_released():
+    """The prefill workspace is one grow-only buffer per (device, stream): the cache keeps at most sixteen of them (least
+    recently used leaves first) and `release_workspaces()` drops them all and reports what they held."""
+    import nha_amd
+    from nha_amd import ops
+    from tests.util import prefill_inputs
+    nha_amd.release_workspaces()
+    d = prefill_inputs(1, 1, 200, 8, 2, 128, 128, 64, dtype=torch.bfloat16)
+    keys = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+    x = [d[k].cuda() for k in keys]
+    ref = nha_amd.chunk_nha(*x, window_size_left=63, gsa_kv_shift=64)[0]
+    assert len(ops._WORKSPACE) == 1
+    streams = [torch.cuda.Stream() for _ in range(ops._WORKSPACE_MAX_STREAMS + 3)]
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            o = nha_amd.chunk_nha(*x, window_size_left=63, gsa_kv_shift=64)[0]
+        torch.cuda.current_stream().wait_stream(st)
+        assert torch.equal(o, ref)
+    assert len(ops._WORKSPACE) == ops._WORKSPACE_MAX_STREAMS
+    held = nha_amd.release_workspaces()
+    assert held >= ops._WORKSPACE_MAX_STREAMS * (1 << 20) and len(ops._WORKSPACE) == 0
+    assert torch.equal(nha_amd.chunk_nha(*x, window_size_left=63, gsa_kv_shift=64)[0], ref)
