@@ -161,6 +161,30 @@ def test_mfma_matches_simple_kernels_at_size():
     assert_close("hv", a[3][1], b[3][1].double(), BF)
 
 
+@pytest.mark.parametrize("B,T", [(1, 6144), (2, 3072)])
+@pytest.mark.parametrize("gate_div,gate_mean", [(8.0, 0.0), (1.0, -1.0)])
+def test_mfma_long_sequences_both_forms_of_the_state_carry(B, T, gate_div, gate_mean):
+    """Sequences of 12 and 6 segments: the first takes the scan-then-apply form of the state pass's second level, the
+    second the form inside the scan; with the layers' slow gates (logsigmoid / 8: the carried state reaches every chunk
+    of a segment) and with fast ones (everything past a segment's first chunks is left as it is).  Initial states, so
+    that the first segment carries something too.  Against the fp32-math kernels."""
+    from nha_amd import chunk_nha
+    HQ, H, D, W = 8, 2, 128, 256
+    d = prefill_inputs(910 + B, B, T, HQ, H, D, D, 64, dtype=BF, qk_scale=D ** -0.5, gate_div=gate_div, gate_mean=gate_mean,
+                       with_state=True, state_scale=0.5)
+    c = [d[k].cuda() for k in KEYS]
+    h0 = (d["h0"][0].cuda(), d["h0"][1].cuda())
+    a = chunk_nha(*c, window_size_left=W - 1, gsa_kv_shift=W, initial_state=h0, output_final_state=True, impl="mfma")
+    b = chunk_nha(*c, window_size_left=W - 1, gsa_kv_shift=W, initial_state=h0, output_final_state=True, impl="simple")
+    assert_close("o", a[0], b[0].double(), BF)
+    assert_close("lse_gsa", a[2], b[2].double(), BF)
+    assert_close("hk", a[3][0], b[3][0].double(), BF)
+    assert_close("hv", a[3][1], b[3][1].double(), BF)
+    for nm, x, y in (("o", a[0], b[0]), ("hk", a[3][0], b[3][0]), ("hv", a[3][1], b[3][1])):
+        rel = ((x.double() - y.double()).norm() / y.double().norm()).item()
+        assert rel <= 5e-3, f"{nm}: relative L2 error {rel:.3e}"
+
+
 def test_mfma_headline_shape_matches_c_oracle():
     """The benchmark's own shape (T=8192, 32/8 heads, D=128, M=64, W=2048; one of its two sequences)
     element by element against the plain-C restatement of the oracle, which gets through it in
