@@ -476,8 +476,11 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
     // consumes the block held in (kr, vr) and refills the registers as soon as they are free
     auto process = [&](uint4(&kr)[2 * KS], uint4(&vr)[NVT], int blk) {
       if (ROT) {
-        // the block's keys are here (the compiler waits on kr), and with them the cos / sin pieces
-        // requested before them; rotate in place, then ask for the next block's pieces
+        // The pieces of this block were requested after the keys of this block and before the refill of the other
+        // register buffer: waiting for the keys (the compiler's wait on kr) does not cover them.  Everything up to
+        // that refill has landed once at most one block of loads is in flight (the first block's pieces were requested
+        // ahead of both buffers: covered as well).  Then rotate in place and ask for the next block's pieces.
+        if constexpr (NBUF == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * KS + NVT) : "memory");
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
