@@ -160,3 +160,136 @@ def test_prefill_backward_sweep():
         if h0 is not None:
             _grad_close(f"{tag} dh0k", h0c[0].grad, G["dh0k"], 1e-2)
             _grad_close(f"{tag} dh0v", h0c[1].grad, G["dh0v"], 1e-2)
+
+
+def test_ring_decode_sweep():
+    """Ring-buffer steps from drawn fill levels (empty, one short of full, full, wrapped several times), four steps
+    each, every step and the final rings, counters and states against the oracle's ring recurrence."""
+    import torch.nn.functional as F
+    from nha_amd import NHARingState, ring_decode_step
+    from tests.util import randn
+    for i in range(120):
+        rnd = random.Random(i)
+        dtype = rnd.choice([BF, BF, torch.float32])
+        NG, H, K = rnd.choice([1, 2, 3, 4, 8]), rnd.choice([1, 2, 3]), rnd.choice([32, 64, 128, 128, 256])
+        M, B = rnd.choice([16, 64, 64, 64, 80]), rnd.choice([1, 2, 3, 4])
+        W = rnd.choice([1, 2, 16, 31, 32, 33, 63, 64, 65, 128, 256, rnd.randint(1, 700)])
+        HQ, V = H * NG, K
+        gen = torch.Generator().manual_seed(40_000 + i)
+        st = NHARingState.empty(B, H, K, V, M, W, dtype=dtype)
+        st.hk.copy_(randn(gen, B, H, K, M, dtype=torch.float32, scale=0.1))
+        st.hv.copy_(randn(gen, B, H, M, V, dtype=torch.float32, scale=0.1))
+        st.ring_k.copy_(randn(gen, B, W, H, K, dtype=dtype))
+        st.ring_kg.copy_(randn(gen, B, W, H, K, dtype=dtype))
+        st.ring_v.copy_(randn(gen, B, W, H, V, dtype=dtype))
+        st.ring_g.copy_((F.logsigmoid(torch.randn(B, W, H, M, generator=gen)) / 8).to(dtype))
+        counts = torch.tensor([rnd.choice([0, 1, max(W - 2, 0), max(W - 1, 0), W, W + 1, 5 * W + 3, rnd.randint(0, 3 * W)])
+                               for _ in range(B)], dtype=torch.int32)
+        st.count.copy_(counts)
+        tag = f"sweep {i}: {str(dtype)[6:]} NG{NG} H{H} K{K} M{M} B{B} W{W} counts{counts.tolist()}"
+        print("case", tag, flush=True)
+        ref = dict(hk=st.hk.cpu().double(), hv=st.hv.cpu().double(),
+                   rings=tuple(x.cpu().double() for x in (st.ring_k, st.ring_kg, st.ring_v, st.ring_g)), count=counts.clone())
+        for step in range(4):
+            q, sq = randn(gen, B, HQ, K, dtype=dtype), randn(gen, B, HQ, K, dtype=dtype)
+            kn, kgn, vn = randn(gen, B, H, K, dtype=dtype), randn(gen, B, H, K, dtype=dtype), randn(gen, B, H, V, dtype=dtype)
+            gn = (F.logsigmoid(torch.randn(B, H, M, generator=gen)) / 8).to(dtype)
+            o = ring_decode_step(st, q.cuda(), sq.cuda(), kn.cuda(), kgn.cuda(), vn.cuda(), gn.cuda())
+            ro, ref["hk"], ref["hv"], ref["rings"] = R.decode_ring_ref(q, sq, kn, kgn, vn, gn, *ref["rings"], ref["count"],
+                                                                       ref["hk"], ref["hv"])
+            ref["count"] += 1
+            assert_close(f"{tag} step {step} o", o, ro, dtype)
+        assert torch.equal(st.count.cpu(), ref["count"])
+        assert_close(tag + " hk", st.hk, ref["hk"], dtype)
+        assert_close(tag + " hv", st.hv, ref["hv"], dtype)
+        for got, want in zip((st.ring_k, st.ring_kg, st.ring_v, st.ring_g), ref["rings"]):
+            assert torch.equal(got.cpu().double(), want), tag
+
+
+def test_zero_sink_attention_sweep():
+    """nha_sink_window_fwd against the restated zero-prefix window attention: windows of 1 .. 2048 keys, 0 .. 100 sinks,
+    batches and packed sequences, four to twelve query heads per kv-head."""
+    from nha_amd.ops import zero_sink_attention
+    from oracle.hybrid_attention_ref import zero_sink_attention_ref
+    for i in range(150):
+        rnd = random.Random(i)
+        D, H, NG = rnd.choice([64, 128, 128]), rnd.choice([1, 2, 3]), rnd.choice([4, 8, 4, 12])
+        HQ = H * NG
+        nseq = rnd.choice([1, 1, 2, 3, 4])
+        lens = [rnd.choice([1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, rnd.randint(1, 600)]) for _ in range(nseq)]
+        packed = rnd.random() < 0.5
+        W = rnd.choice([1, 2, 20, 31, 32, 33, 63, 64, 65, 96, 100, 128, 255, 256, 257, 2048, rnd.randint(1, 700)])
+        M = rnd.choice([0, 1, 16, 64, 64, 100])
+        gen = torch.Generator().manual_seed(60_000 + i)
+        if packed:
+            cu = [0] + [int(x) for x in np.cumsum(lens)]
+            B, T = 1, cu[-1]
+        else:
+            B, T, cu = rnd.choice([1, 2, 3]), lens[0], None
+        tag = f"sweep {i}: D{D} H{H} NG{NG} B{B} T{T} cu{cu} W{W} sinks{M}"
+        print("case", tag, flush=True)
+        q = (torch.randn(B, T, HQ, D, generator=gen) * D ** -0.25).to(BF)
+        k = (torch.randn(B, T, H, D, generator=gen) * D ** -0.25).to(BF)
+        v = torch.randn(B, T, H, D, generator=gen).to(BF)
+        got = zero_sink_attention(q.cuda(), k.cuda(), v.cuda(), W, M,
+                                  cu_seqlens=None if cu is None else torch.tensor(cu, dtype=torch.int32).cuda())
+        for a, b in [(0, T)] if cu is None else zip(cu[:-1], cu[1:]):
+            ref = zero_sink_attention_ref(q[:, a:b].double(), k[:, a:b].double(), v[:, a:b].double(), W, M)
+            assert_close(f"{tag} [{a},{b})", got[:, a:b], ref, BF)
+
+
+def test_hybrid_block_stack_sweep():
+    """Two-block stacks of the hybrid decoders' attention modules (both flavours; all-NHA and NHA + zero-sink; head shapes
+    on the generic, the matrix-core and the LDS-direct kernels; zero-sink windows shorter than the prompt; left padding):
+    a prompt, then single-token steps on the ring cache, against the restated modules."""
+    from nha_amd import NHARingCache
+    from nha_amd.hybrid import HybridNHAConfig, LlamaNativeHybridAttention, Qwen3MoeNativeHybridAttention
+    from oracle.hybrid_attention_ref import HybridAttentionRef
+    from tests.test_hybrid_modules import F64, _close, _run_ref_stack, _run_stack, _weights
+    dev = torch.device("cuda:0")
+    hidden = 128
+    for i in range(60):
+        rnd = random.Random(i)
+        flavour = rnd.choice(["moe", "dense"])
+        HQ, H, D, M = rnd.choice([(8, 2, 32, 16), (32, 4, 128, 64), (8, 2, 128, 64), (4, 4, 64, 64), (4, 2, 64, 64), (2, 2, 256, 64),
+                                  (6, 2, 64, 64), (16, 2, 128, 64)])
+        W = rnd.choice([16, 32, 64, 64, 48])
+        mixed = rnd.random() < 0.5
+        sink_window = rnd.choice([2048, 96, 40])
+        B, T0, steps = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 17, 63, 64, 65, 128, rnd.randint(1, 300)]), rnd.choice([1, 3, 6])
+        pad = rnd.random() < 0.4 and B > 1 and T0 > 4
+        tag = f"sweep {i}: {flavour} HQ{HQ} H{H} D{D} M{M} W{W} mixed={mixed} sink window {sink_window} B{B} prompt {T0} steps {steps} pad={pad}"
+        print("case", tag, flush=True)
+        cfg = HybridNHAConfig(hidden_size=hidden, num_attention_heads=HQ, num_key_value_heads=H, head_dim=D, num_slots=M, window_size=W,
+                              max_position_embeddings=4096, block_size=2 if mixed else None, transformer_idx=1 if mixed else None)
+        cls = Qwen3MoeNativeHybridAttention if flavour == "moe" else LlamaNativeHybridAttention
+        gen = torch.Generator().manual_seed(100_000 + i)
+        layers, refs = [], []
+        for li in range(2):
+            w = _weights(gen, hidden, HQ, H, D, M, flavour == "moe")
+            m = cls(cfg, layer_idx=li).to(BF)
+            m.load_state_dict(w, strict=True)
+            if not m.is_nha_layer:
+                m.window_size = sink_window
+            layers.append(m.to(dev).eval())
+            refs.append(HybridAttentionRef(w, num_heads=HQ, num_kv_heads=H, head_dim=D, num_slots=M, window_size=m.window_size,
+                                           qk_norm=flavour == "moe", round_to=BF))
+        x = torch.randn(B, T0 + steps, hidden, generator=gen).to(BF)
+        mask = torch.ones(B, T0 + steps, dtype=torch.long)
+        if pad:
+            mask[-1, : rnd.randint(1, T0 // 2)] = 0
+        npad = int((mask[-1] == 0).sum())
+        pos = (mask.cumsum(1) - 1).clamp(min=0)
+        cache, ref_caches = NHARingCache(W), [{} for _ in refs]
+        with torch.no_grad():
+            mk = mask[:, :T0] if pad else None
+            got = _run_stack(layers, x[:, :T0].to(dev), pos[:, :T0].to(dev), cache, None if mk is None else mk.to(dev))
+            ref = _run_ref_stack(refs, x[:, :T0].to(F64), pos[:, :T0], ref_caches, mk)
+            if B > 1:
+                _close(tag + " prompt", got[:-1], ref[:-1])
+            _close(tag + " prompt, last row", got[-1, npad:], ref[-1, npad:])
+            for t in range(T0, T0 + steps):
+                mk = mask[:, :t + 1] if pad else None
+                got = _run_stack(layers, x[:, t:t + 1].to(dev), pos[:, t:t + 1].to(dev), cache, None if mk is None else mk.to(dev))
+                ref = _run_ref_stack(refs, x[:, t:t + 1].to(F64), pos[:, t:t + 1], ref_caches, mk)
+                _close(f"{tag} step {t}", got, ref)
