@@ -88,8 +88,8 @@ static size_t lds_bytes_for(int D, int G, int NW, bool rot) {
 
 // 16 bytes per lane from global memory into LDS at lds_base + 16 * lane (lds_base wave-uniform): the
 // cos / sin pieces of the next block wait there instead of in registers.  Outside the compiler's
-// memory model; it is issued before the register loads that the next wait counts, so that wait
-// covers it.
+// memory model: no wait the compiler places knows of it, so its reader waits by count (s_waitcnt vmcnt)
+// for everything issued up to it.
 __device__ __forceinline__ void g2l16(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
 }
