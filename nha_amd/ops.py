@@ -658,6 +658,12 @@ def chunk_nha(
         )
     assert q_swa.dim() == 4, "Expected [B, T, H, D] for input"
     _need_cuda(q_swa, k_swa, q_gsa, k_gsa, v, s, g)
+    if q_swa.dtype == torch.float16:
+        # float16 tensors: computed in float32 (every float16 value is one) by the generic kernels, o returned in float16
+        out = chunk_nha(*(x.float() for x in (q_swa, k_swa, q_gsa, k_gsa, v, s, g)), cu_seqlens=cu_seqlens, max_seqlen=max_seqlen,
+                        scale=scale, window_size_left=window_size_left, window_size_right=window_size_right, head_first=head_first,
+                        gsa_kv_shift=gsa_kv_shift, initial_state=initial_state, output_final_state=output_final_state, impl=impl)
+        return (out[0].to(torch.float16), *out[1:])
     B, T, HQ, D = q_swa.shape
     H = k_swa.shape[2]
     if scale is None:
@@ -746,6 +752,10 @@ def fused_chunk_nha_prefill(
     assert HQ % H == 0
     assert W >= 1
     _need_cuda(q, k, v, rotary_q, rotary_k, s, g)
+    if q.dtype == torch.float16:   # computed in float32, o returned in float16
+        o, st = fused_chunk_nha_prefill(*(x.float() for x in (q, k, v, rotary_q, rotary_k, s, g)), window_size=window_size,
+                                        initial_state=initial_state, output_final_state=output_final_state, scale=scale, impl=impl)
+        return o.to(torch.float16), st
     if initial_state is not None and initial_state[0] is not None:
         hk0, hv0 = initial_state
         assert tuple(hk0.shape) == (B, H, K, s.shape[-1]) and tuple(hv0.shape) == (B, H, s.shape[-1], v.shape[-1]), \
@@ -816,6 +826,11 @@ def fused_recurrent_nha_decode(
     assert HQ % H == 0
     assert K >= 16 and V >= 16
     _need_cuda(q, k, v, g, sw_k, sw_v, sq, s, cos, sin)
+    if q.dtype == torch.float16:   # computed in float32, o returned in float16
+        f = lambda x: None if x is None else x.float()
+        o, st = fused_recurrent_nha_decode(f(q), f(k), f(v), f(g), f(sw_k), f(sw_v), sq=f(sq), s=f(s), cos=f(cos), sin=f(sin),
+                                           initial_state=initial_state, output_final_state=output_final_state, scale=scale)
+        return o.to(torch.float16), st
     NG = HQ // H
     if scale is None:
         scale = K ** -0.5
@@ -878,6 +893,10 @@ def fused_recurrent_nha(
         )
     assert not q.requires_grad, "fused_recurrent_nha is inference-only (no autograd)"
     _need_cuda(q, k, v, sliding_window, s, g)
+    if q.dtype == torch.float16:   # computed in float32, o returned in float16
+        o, p, st = fused_recurrent_nha(q.float(), k.float(), v.float(), sliding_window.float(), s.float(), g.float(), scale=scale,
+                                       initial_state=initial_state, output_final_state=output_final_state)
+        return o.to(torch.float16), p, st
     if scale is None:
         scale = k.shape[-1] ** -0.5
     B, _, HQ, K = q.shape

@@ -81,3 +81,66 @@ def test_workspace_cache_is_bounded_and_can_be_released():
     held = nha_amd.release_workspaces()
     assert held >= ops._WORKSPACE_MAX_STREAMS * (1 << 20) and len(ops._WORKSPACE) == 0
     assert torch.equal(nha_amd.chunk_nha(*x, window_size_left=63, gsa_kv_shift=64)[0], ref)
+
+
+def test_float16_tensors_are_computed_in_float32():
+    """float16 inputs (the reference's Triton kernels take them like any other dtype): the four stateless ops compute in
+    float32 on the generic kernels and return o in float16.  Against the oracle on the float16 values: 2e-3 abs + 2e-3 rel
+    (one float16 rounding of o), gradients in float16 within 1e-2 relative L2."""
+    from nha_amd import chunk_nha, fused_chunk_nha_prefill, fused_recurrent_nha, fused_recurrent_nha_decode
+    from oracle import nha_ref as R
+    from tests.test_gpu_decode import decode_inputs
+    from tests.util import prefill_inputs
+    keys = ["q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g"]
+    f16 = torch.float16
+
+    def near(name, got, ref, atol=2e-3, rtol=2e-3):
+        got, ref = got.detach().double().cpu(), ref.double()
+        bad = (got - ref).abs() > atol + rtol * ref.abs()
+        assert torch.isfinite(got).all() and not bad.any(), f"{name}: {int(bad.sum())} off, max {(got - ref).abs().max():.2e}"
+
+    d = prefill_inputs(31, 2, 150, 8, 2, 64, 64, 64, dtype=torch.float32, qk_scale=64 ** -0.5, with_state=True)
+    d = {k: (v.to(f16) if k in keys else v) for k, v in d.items()}
+    x = [d[k].cuda().requires_grad_(True) for k in keys]
+    h0 = tuple(t.cuda() for t in d["h0"])
+    o, ls, lg, (hk, hv) = chunk_nha(*x, window_size_left=31, gsa_kv_shift=32, initial_state=h0, output_final_state=True)
+    assert o.dtype == f16 and ls.dtype == torch.float32 and hk.dtype == torch.float32
+    ro, rls, rlg, rhk, rhv = R.prefill_ref(*[d[k] for k in keys], window_size_left=31, gsa_kv_shift=32, initial_state=d["h0"])
+    near("o", o, ro)
+    near("lse_swa", ls, rls)
+    near("lse_gsa", lg, rlg)
+    near("hk", hk, rhk)
+    near("hv", hv, rhv)
+    gen = torch.Generator().manual_seed(1)
+    do = torch.randn(o.shape, generator=gen).to(f16)
+    (o.float() * do.cuda().float()).sum().backward()
+    G = R.prefill_grad_ref(*[d[k] for k in keys], do, window_size_left=31, gsa_kv_shift=32, initial_state=d["h0"])
+    for k, t in zip(keys, x):
+        assert t.grad.dtype == f16
+        rel = ((t.grad.double().cpu() - G["d" + k]).norm() / G["d" + k].norm()).item()
+        assert rel <= 1e-2, (k, rel)
+    with torch.no_grad():
+        o2, (hk2, _) = fused_chunk_nha_prefill(x[2], x[3], x[4], x[0], x[1], x[5], x[6], window_size=32, initial_state=h0,
+                                               output_final_state=True)
+    assert o2.dtype == f16
+    near("fused prefill o", o2, ro)
+    near("fused prefill hk", hk2, rhk)
+    # the single-token ops
+    dd = decode_inputs(5, 2, 2, 4, 64, 64, 64, 40, torch.float32)
+    dd = {k: (v.to(f16) if v.dtype == torch.float32 and k not in ("hk0", "hv0") else v) for k, v in dd.items()}
+    c = {k: v.cuda() for k, v in dd.items()}
+    o3, (hk3, hv3) = fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], s=c["s"], sw_k=c["sk"], sw_v=c["vw"],
+                                                initial_state=(c["hk0"].clone(), c["hv0"].clone()), output_final_state=True)
+    r3, rhk3, rhv3, _, _ = R.decode_ref(dd["q"], dd["k"], dd["v"], dd["g"], dd["sk"], dd["vw"], sq=dd["sq"], s=dd["s"],
+                                        initial_state=(dd["hk0"], dd["hv0"]))
+    assert o3.dtype == f16
+    near("decode o", o3, r3)
+    near("decode hv", hv3, rhv3)
+    o4, p4, (hk4, hv4) = fused_recurrent_nha(c["q"], c["k"], c["v"], c["sliding_window"], c["s"], c["g"],
+                                             initial_state=(c["hk0"].clone(), c["hv0"].clone()), output_final_state=True)
+    r4, rp4, rhk4, rhv4 = R.fused_recurrent_ref(dd["q"], dd["k"], dd["v"], dd["sliding_window"], dd["s"], dd["g"],
+                                                initial_state=(dd["hk0"], dd["hv0"]))
+    assert o4.dtype == f16
+    near("logits-form o", o4, r4)
+    near("logits-form p", p4, rp4)
+    near("logits-form hk", hk4, rhk4)
