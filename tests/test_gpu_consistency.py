@@ -144,3 +144,51 @@ def test_float16_tensors_are_computed_in_float32():
     near("logits-form o", o4, r4)
     near("logits-form p", p4, rp4)
     near("logits-form hk", hk4, rhk4)
+
+
+@pytest.mark.parametrize("NSEQ,HQ,H,D,W,parts,same_kernel", [
+    (128, 32, 8, 128, 2048, 8, True),     # q, o: 8 GiB; k, v: 2 GiB -- the LDS-direct kernels with row addresses past 2^32 bytes
+    (264, 32, 8, 128, 512, 11, False),    # k, v: 4.1 GiB -- past the LDS-direct kernels' 32-bit lane offsets: mfma_out_kernel
+])
+def test_calls_whose_tensors_pass_4_gib(NSEQ, HQ, H, D, W, parts, same_kernel):
+    """Packed sequences of 8192 tokens, 1M and 2.2M tokens in one call, against the same sequences in calls of 16 / 24
+    sequences each (sequences do not interact, so the split calls are the reference): bit-identical while the same
+    kernels serve both, within one bf16 rounding of o where the large call falls back to the kernel with 64-bit
+    offsets.  Inputs are drawn on the device."""
+    from nha_amd import chunk_nha
+    dev, L = "cuda:0", 8192
+    T = NSEQ * L
+    try:
+        gen = torch.Generator(device=dev).manual_seed(NSEQ)
+
+        def draw(width, scale):
+            out = torch.empty(1, T, width[0], width[1], dtype=torch.bfloat16, device=dev)
+            for a in range(0, T, T // 8):
+                out[:, a:a + T // 8] = (torch.randn(1, T // 8, *width, device=dev, generator=gen) * scale).to(torch.bfloat16)
+            return out
+        q_swa, q_gsa = draw((HQ, D), D ** -0.5), draw((HQ, D), D ** -0.5)
+        k_swa, k_gsa, v = draw((H, D), D ** -0.5), draw((H, D), D ** -0.5), draw((H, D), 1.0)
+        g = (torch.nn.functional.logsigmoid(draw((H, 64), 1.0).float()) / 8).to(torch.bfloat16)
+        s = (1 - g.float().exp()).to(torch.bfloat16)
+        xs = (q_swa, k_swa, q_gsa, k_gsa, v, s, g)
+        cu = torch.arange(0, T + 1, L, dtype=torch.int32, device=dev)
+        o, ls, lg, (hk, hv) = chunk_nha(*xs, cu_seqlens=cu, window_size_left=W - 1, gsa_kv_shift=W, output_final_state=True)
+        per = NSEQ // parts
+        cu_p = torch.arange(0, per * L + 1, L, dtype=torch.int32, device=dev)
+        for pi in range(parts):
+            a, b = pi * per * L, (pi + 1) * per * L
+            o2, ls2, lg2, (hk2, hv2) = chunk_nha(*(x[:, a:b] for x in xs), cu_seqlens=cu_p, window_size_left=W - 1, gsa_kv_shift=W,
+                                                 output_final_state=True)
+            assert torch.equal(hk[pi * per:(pi + 1) * per], hk2) and torch.equal(hv[pi * per:(pi + 1) * per], hv2), pi
+            if same_kernel:
+                assert torch.equal(o[:, a:b], o2) and torch.equal(ls[:, a:b], ls2) and torch.equal(lg[:, a:b], lg2), pi
+            else:
+                assert (o[:, a:b].float() - o2.float()).abs().max().item() <= 4e-3, pi
+                assert (ls[:, a:b] - ls2).abs().max().item() <= 2e-2 and (lg[:, a:b] - lg2).abs().max().item() <= 1e-4, pi
+    except torch.cuda.OutOfMemoryError:
+        pytest.skip("not enough free device memory for this case")
+    finally:
+        q_swa = q_gsa = k_swa = k_gsa = v = g = s = xs = o = ls = lg = hk = hv = None
+        from nha_amd import release_workspaces
+        release_workspaces()
+        torch.cuda.empty_cache()
