@@ -426,6 +426,8 @@ def bench_hybrid(torch, steps, warmup):
                     # the same step recorded into a HIP graph (no per-launch host work)
                     rec = blk.record_decode_step(cache, B)
                     dres["recorded_block_us"] = timed(lambda: rec.step(xs, pos1), n=128, busy=0.2) * 1e3
+                    # the caller fills the graph's input buffers itself: the replay alone
+                    dres["recorded_block_replay_only_us"] = timed(lambda: rec.step(rec.x, rec.pos), n=128, busy=0.2) * 1e3
                     del rec
             # the bare kernel step on the same cache, and the glue and GEMMs of a step alone
             from nha_amd import ring_decode_step

@@ -351,7 +351,7 @@ class HybridNHAAttention(nn.Module):
 
 class RecordedDecodeStep:
     """One decode step of an attention block as a HIP graph: `step(hidden [B,1,hidden], position_ids [B,1])` copies
-    its arguments into the graph's input buffers, replays the recorded launches (fused projection, glue, ring decode
+    its arguments into the graph's input buffers `x` and `pos` (not when they are those buffers), replays the recorded launches (fused projection, glue, ring decode
     step, counter advance, output projection) and returns the graph's output buffer `[B,1,hidden]` (overwritten by
     the next step).  The host does no per-launch work, which is what a step of a few tens of microseconds of GPU
     time needs: the eager block spends more time issuing its launches than the GPU spends on them."""
@@ -395,8 +395,11 @@ class RecordedDecodeStep:
         if self.cache.states[self.block.layer_idx].count.data_ptr() != self._count_ptr:
             raise RuntimeError("the cache took an eager decode step since this step was recorded (the eager step trades "
                                "the ring's two counter arrays, the recording holds the address of one): record again")
-        self.x.copy_(hidden_states)
-        self.pos.copy_(position_ids)
+        # a caller that fills the graph's own input buffers (`self.x`, `self.pos`) passes them back and saves the copies
+        if hidden_states is not self.x:
+            self.x.copy_(hidden_states)
+        if position_ids is not self.pos:
+            self.pos.copy_(position_ids)
         self.graph.replay()
         self.cache.note_step(self.block.layer_idx)
         return self.out
