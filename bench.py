@@ -583,6 +583,25 @@ def bench_api(torch, steps, warmup):
     return out
 
 
+def decode_call_forms(api):
+    """The other call forms of the single-token ops at the decode workload's shape (Python ops, outputs allocated per
+    call), each with the bytes its tensors hold and the share of the HBM peak that makes: window rows as a [B,W,H,D]
+    tensor with a pre-rotated query, the same with cos / sin tables (shared [1,W,D] tables: their bytes are not
+    counted), float32 tensors, and caller-supplied window logits (no window rows at all)."""
+    d = DECODE
+    B, HQ, H, D, M, W = (d[k] for k in ("B", "HQ", "H", "D", "M", "W"))
+    state = 2 * 2 * B * H * D * M * 4                      # hk and hv, read and written
+    rows = lambda esz: (2 * B * W * H * D + 2 * B * HQ * D + 2 * B * H * D + B * H * M + B * HQ * D) * esz + state
+    forms = {"window_prerotated": ("decode_window_eager_us", rows(2)), "window_cos_sin_tables": ("decode_window_rotary_us", rows(2)),
+             "window_float32": ("decode_window_fp32_us", rows(4)),
+             "caller_logits": ("fused_recurrent_nha_logits_us", state + B * HQ * W * (2 + 4) + (B * HQ * D * 2 + 2 * B * H * D + 2 * B * H * M) * 2)}
+    out = {}
+    for name, (key, nbytes) in forms.items():
+        us = api[key]
+        out[name] = {"us_per_step": us, "algorithmic_bytes": nbytes, "hbm_frac": nbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
 def cpu_baseline(torch):
     """The oracle on the host cores, bounded sample: the plain-C restatement (oracle/nha_ref_c.c,
     OpenMP over sequences x q-heads, double arithmetic) for the prefill, the torch restatement for a
@@ -777,7 +796,8 @@ def main():
                                              "us_per_step": dc256["us_per_step"], "kernel_us": dc256["us_kernel"],
                                              "kernel": "decode_mfma_kernel<256,1,4>", "algorithmic_bytes": dc256["bytes"],
                                              "achieved_gbs": dc256["achieved_gbs"],
-                                             "hbm_frac": dc256["achieved_gbs"] / PEAK_HBM_GBS}}},
+                                             "hbm_frac": dc256["achieved_gbs"] / PEAK_HBM_GBS},
+                                    "call_forms": decode_call_forms(api)}},
         "backward": {"metric": "backward of the same prefill call", "ms_per_call": bw["bwd_ms"], "unit": "ms",
                      "tokens_per_s": bw["bwd_tokens_per_s"], "tflops": bw["bwd_tflops"],
                      "flop": bw["bwd_flops"], "note": "2.5 x the forward's algorithmic flop"},
