@@ -192,3 +192,67 @@ def test_calls_whose_tensors_pass_4_gib(NSEQ, HQ, H, D, W, parts, same_kernel):
         from nha_amd import release_workspaces
         release_workspaces()
         torch.cuda.empty_cache()
+
+
+def test_ops_recorded_into_a_graph_replay_like_eager_calls():
+    """The library issues kernels only (no allocation, copy, fill or synchronisation of its own), so the ops can be
+    recorded into a HIP graph after one eager call (which builds the index tables and the workspace): a prefill with
+    packed sequences and a decode step, five replays each on fresh input contents, with eager work and a
+    synchronisation between replays, every replay bit-identical to the eager call on the same inputs."""
+    from nha_amd import chunk_nha, fused_recurrent_nha_decode
+    from tests.test_gpu_decode import decode_inputs
+    from tests.util import prefill_inputs
+    keys = ("q_swa", "k_swa", "q_gsa", "k_gsa", "v", "s", "g")
+    cu = torch.tensor([0, 300, 301, 900], dtype=torch.int32, device="cuda")
+
+    def fresh(seed):
+        d = prefill_inputs(seed, 1, 900, 8, 2, 128, 128, 64, dtype=torch.bfloat16, qk_scale=128 ** -0.5, with_state=True, N=3)
+        return [d[k].cuda() for k in keys], tuple(t.cuda() for t in d["h0"])
+
+    def prefill(xs, h0):
+        return chunk_nha(*xs, cu_seqlens=cu, window_size_left=199, gsa_kv_shift=200, initial_state=h0, output_final_state=True)
+
+    xs, h0 = fresh(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        prefill(xs, h0)                                  # tables, workspace and kernel set-up outside the recording
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph):
+        out = prefill(xs, h0)
+    for rep in range(1, 6):
+        ys, g0 = fresh(rep)
+        with torch.no_grad():
+            want = prefill(ys, g0)
+        for a, b in zip(xs + list(h0), ys + list(g0)):
+            a.copy_(b)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (out[0], out[1], out[2], out[3][0], out[3][1])
+        for name, x, y in zip(("o", "lse_swa", "lse_gsa", "hk", "hv"), got, (want[0], want[1], want[2], want[3][0], want[3][1])):
+            assert torch.equal(x, y), (rep, name)
+        _ = (ys[0].float().sum() + ys[4].float().sum()).item()      # eager work and a sync between replays
+
+    def step(c):
+        return fused_recurrent_nha_decode(q=c["q"], sq=c["sq"], k=c["k"], v=c["v"], g=c["g"], s=c["s"], sw_k=c["sk"], sw_v=c["vw"],
+                                          initial_state=(c["hk0"], c["hv0"]), output_final_state=True)
+
+    c = {k: v.cuda() for k, v in decode_inputs(50, 4, 2, 4, 128, 128, 64, 300, torch.bfloat16).items()}
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        step(c)
+    torch.cuda.current_stream().wait_stream(side)
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph2):
+        o, (hk, hv) = step(c)
+    for rep in range(1, 6):
+        d = {k: v.cuda() for k, v in decode_inputs(50 + rep, 4, 2, 4, 128, 128, 64, 300, torch.bfloat16).items()}
+        with torch.no_grad():
+            wo, (whk, whv) = step(d)
+        for k in c:
+            c[k].copy_(d[k])
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, wo) and torch.equal(hk, whk) and torch.equal(hv, whv), rep
+        _ = d["vw"].float().sum().item()
