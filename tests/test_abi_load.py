@@ -158,3 +158,20 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_no_fallback_without_the_library_or_a_gpu(monkeypatch):
+    """The ops have no CPU or eager path: host tensors are refused by name, and a missing library is an error at the
+    first call, not a slower result."""
+    import torch
+    from nha_amd import chunk_nha, fused_recurrent_nha_decode
+    x = torch.zeros(1, 8, 2, 64)
+    g = torch.zeros(1, 8, 2, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        chunk_nha(x, x, x, x, x, g, g)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused_recurrent_nha_decode(q=x[:, :1], k=x[:, :1], v=x[:, :1], g=g[:, :1], sw_k=x, sw_v=x, sq=x[:, :1])
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "nha_amd", "no_such_library.so"))
+    with pytest.raises(RuntimeError, match="no CPU or eager fallback"):
+        _lib.load()
