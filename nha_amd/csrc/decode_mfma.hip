@@ -69,8 +69,6 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int col
   return __builtin_bit_cast(bf16x8, t);
 }
 
-__host__ __device__ constexpr int imax(int a, int b) { return a > b ? a : b; }
-
 // 16 bytes of a window row: read once per step and never again, so the load is marked
 // non-temporal (it does not displace the state lines in L2; measured 145 -> 134 us per step)
 __device__ __forceinline__ uint4 ld16_stream(const bf16_t* p) {

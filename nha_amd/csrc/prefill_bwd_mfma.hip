@@ -448,14 +448,8 @@ __device__ __forceinline__ bf16x8 table_frag(const lbf16* tab, int n, int hf, in
 }
 
 // x as a bf16 pair hi + lo (16 mantissa bits): the tables built from fp32 intermediates are kept
-// this way and multiplied as hi*b + lo*b, so that their rounding stays below that of the bf16 inputs
-__device__ __forceinline__ void split_bf16(float x, lbf16* hi, lbf16* lo, int idx) {
-  const bf16_t h = f32_to_bf16(x);
-  hi[idx] = h;
-  lo[idx] = f32_to_bf16(x - bf16_to_f32(h));
-}
-
-// four consecutive elements at once: two 8-byte LDS writes (idx a multiple of 4)
+// this way and multiplied as hi*b + lo*b, so that their rounding stays below that of the bf16 inputs.
+// Four consecutive elements at once: two 8-byte LDS writes (idx a multiple of 4)
 __device__ __forceinline__ void split4_bf16(const float4 x, lbf16* hi, lbf16* lo, int idx) {
   const float v[4] = {x.x, x.y, x.z, x.w};
   bf16x4 h, l;
@@ -888,7 +882,7 @@ __device__ __forceinline__ float ref_of(const SP3& p, int c0, int h, int r, int 
 }
 
 // The decay-scaled tables enter the gate gradient through a difference of nearly equal sums (dg is
-// a telescoping sum), so they are bf16 pairs (split_bf16) and their products hi*hi + hi*lo + lo*hi.
+// a telescoping sum), so they are bf16 pairs (split4_bf16) and their products hi*hi + hi*lo + lo*hi.
 // rows of Y = s_j[m] e^(ref - gc_j[m]) (zero for rows without a source token)
 struct StageY {
   // 16-byte reads, all issued before the first conversion waits for one
