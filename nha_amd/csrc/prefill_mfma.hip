@@ -84,30 +84,57 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H;
-  // blockIdx.z picks the state: 0 = k-state (rows of k_gsa; it also writes the gate tables),
-  // 1 = v-state (rows of v).  The two recurrences share nothing but the gates, and twice the
-  // workgroups of half the size fill the chip better.
-  const bool isv = (blockIdx.z & 1) != 0;
-  const int dcol0 = (blockIdx.z >> 1) * DW;   // first state column of this workgroup
+  // One-dimensional grid, blockIdx.x = (state and column range z, kv-head h) + H Z k with k counting the segments of
+  // the call one sequence after the other, without gaps: the workgroups that find k past the last segment (the grid
+  // is sized for the most segments NT chunks in N sequences can have) are the last of the launch.  A workgroup
+  // holds its CU slot for the whole chain of its segment and two fit a CU: were workgroups that leave at once
+  // strewn over the launch order, the shader engines' shares of the working ones would differ, some CUs would
+  // get a third one after their first two and others only one -- a second round for a tenth of the chip (49 us
+  // against 32 us per launch at 512 segments x heads x states on 256 CUs).
+  // z picks the state: even = k-state (rows of k_gsa; it also writes the gate tables), odd = v-state (rows of v).
+  // The two recurrences share nothing but the gates, and twice the workgroups of half the size fill the chip better.
+  constexpr int Z = 2 * (D / DW);
+  const int hz = blockIdx.x % (H * Z), k = blockIdx.x / (H * Z);
+  const int h = hz % H, z = hz / H;
+  const bool isv = (z & 1) != 0;
+  const int dcol0 = (z >> 1) * DW;             // first state column of this workgroup
   const bool lead = dcol0 == 0;                // writes what does not depend on the column range
   const bf16_t* xsrc = (isv ? p.v : p.k_gsa) + dcol0;
   bf16_t* hloc = isv ? p.hvc : p.hkT;
   float* hend = isv ? p.hend_v : p.hend_k;
-  // blockIdx.x is a segment slot (seg_slot); slots are dense up to a few gaps per sequence, so
-  // every XCD receives the same share of working workgroups
-  const int slot = blockIdx.x, h = blockIdx.y;
-  int n = 0;
+  // segment k of the call -> (sequence n, segment kseg of it): a running count of ceil(chunks / SEG) over the
+  // sequences, 256 at a time (one per thread, prefix over the workgroup)
+  __shared__ int seg_wave[4], seg_hit[2];
+  int n = 0, kseg = 0;
   {
-    int lo = 0, hi = p.N - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (p.coff[mid] / SEG + mid <= slot) lo = mid; else hi = mid - 1;
+    int base = 0;
+    for (int n0 = 0; n0 < p.N; n0 += 256) {
+      const int i = n0 + tid;
+      const int segs = i < p.N ? (p.coff[i + 1] - p.coff[i] + SEG - 1) / SEG : 0;
+      int incl = segs;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += t;
+      }
+      if (lane == 63) seg_wave[wave] = incl;
+      __syncthreads();
+      int before = base;
+      for (int w = 0; w < wave; ++w) before += seg_wave[w];
+      const int first = before + incl - segs;
+      if (k >= first && k < first + segs) {
+        seg_hit[0] = i;
+        seg_hit[1] = k - first;
+      }
+      base += seg_wave[0] + seg_wave[1] + seg_wave[2] + seg_wave[3];
+      __syncthreads();
+      if (k < base) break;
     }
-    n = lo;
+    if (k >= base) return;   // past the last segment of the call
+    n = seg_hit[0];
+    kseg = seg_hit[1];
   }
-  const int kseg = slot - (p.coff[n] / SEG + n);
   const int it0 = kseg * SEG;
-  if (it0 >= p.coff[n + 1] - p.coff[n]) return;
   const int chunk0 = p.coff[n] + it0;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int L = eos - bos;
@@ -1315,7 +1342,13 @@ int run_state_pass(const MP& p, bool segment_form, hipStream_t st) {
     set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((mfma_state_local_kernel<D, DW>), dim3(p.NT / SEG + p.N + 1, p.H, 2 * (D / DW)), dim3(256), lds, st, p);
+  // at most NT / SEG + N segments: every sequence but for its last segment fills SEG chunks
+  const int64_t l1_grid = (int64_t)(p.NT / SEG + p.N) * p.H * 2 * (D / DW);
+  if (l1_grid > 0x7fffffff) {
+    set_error("nha_prefill_fwd(mfma): too many segments for one launch (%lld workgroups)", (long long)l1_grid);
+    return NHA_ERR_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL((mfma_state_local_kernel<D, DW>), dim3((unsigned)l1_grid), dim3(256), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma state pass, level 1)");
   // the forward's chunk states: inside the scan while a sequence has about eight segments or fewer (a thread's
   // chain there costs a memory latency per segment: 15 us at 4 segments, 21 us at 16 on one box), after it beyond
