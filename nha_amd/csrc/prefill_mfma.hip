@@ -227,10 +227,16 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
       glast = __shfl(cand, l16 + 16 * src_kb, 64);
     }
     const int64_t cg = (int64_t)chunk * H + h;
-    if (!isv && lead) {
+    if (lead) {
+      // the gate table: rows 0..31 from the k-state workgroup, rows 32..63 from the v-state one (both hold it)
       float* gout = p.gc + cg * BT * MS + m;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) gout[(16 * (e >> 2) + 4 * kb + (e & 3)) * MS] = gcv[e];
+      for (int e = 0; e < 8; ++e) {
+        const int ee = isv ? e + 8 : e;
+        gout[(16 * (ee >> 2) + 4 * kb + (ee & 3)) * MS] = isv ? gcv[e + 8] : gcv[e];
+      }
+    }
+    if (!isv && lead) {
       if (kb == 0) p.dcum[cg * MS + m] = fexp(gsum);
       // 16-row sub-blocks over which some slot decays by more than exp(DECAY_CLAMP): the output
       // pass cannot factor their intra-block decay; mfma_repair_kernel recomputes their rows
@@ -257,13 +263,22 @@ __global__ __launch_bounds__(256) void mfma_state_local_kernel(const MP p) {
       sg0[e] = (__bf16)sg[e];
       sg1[e] = (__bf16)sg[8 + e];
     }
-    // local chunk-start states (bf16), before the update: rows m, 4 consecutive d per lane
+    // local chunk-start states (bf16), before the update: rows m.  A lane holds 4 consecutive d of every 16-column
+    // block; the lanes of an even 16-lane row keep block b, those of the odd row block b + 1, and the two trade their
+    // halves, so that a lane stores 16 bytes and a row of the state 64 consecutive bytes per instruction
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      bf16x4 pk;
+    for (int b = 0; b < NB; b += 2) {
+      bf16x4 pa, pb;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) pk[r] = (__bf16)hx[b][r];
-      *reinterpret_cast<bf16x4*>(hloc + (cg * MS + m) * D + dcol0 + 16 * b + 4 * kb) = pk;
+      for (int r = 0; r < 4; ++r) {
+        pa[r] = (__bf16)hx[b][r];
+        pb[r] = (__bf16)hx[b + 1][r];
+      }
+      uint2 ua = __builtin_bit_cast(uint2, pa), ub = __builtin_bit_cast(uint2, pb);
+      const auto s0 = __builtin_amdgcn_permlane16_swap(ua.x, ub.x, false, false);
+      const auto s1 = __builtin_amdgcn_permlane16_swap(ua.y, ub.y, false, false);
+      const int dcol = 16 * (b + (kb & 1)) + 8 * (kb >> 1);
+      *reinterpret_cast<uint4*>(hloc + (cg * MS + m) * D + dcol0 + dcol) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
     }
     const float dk = fexp(glast);
     gsum += glast;
