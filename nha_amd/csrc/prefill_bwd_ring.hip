@@ -261,14 +261,20 @@ struct DkvP {
 constexpr int KV_ITEM = 4 * UB + 1024;   // q rows | do rows | q transposing | do transposing | 32 (lse, delta) pairs
 constexpr int KV_QR = 0, KV_OR = UB, KV_QT = 2 * UB, KV_OT = 3 * UB, KV_LD = 4 * UB;
 constexpr int KV_BYTES = NR * KV_ITEM;
-constexpr int KEYS = 256;                // keys per workgroup
-constexpr int NKB = 2;                   // 16-key blocks per wave
 
 __device__ __forceinline__ void g2l4(const void* gbase, uint32_t voff_bytes, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff_bytes), "s"(gbase), "s"(lds_base) : "memory");
 }
 
+// KEYS: keys per workgroup, 256 or 128 (a wave holds KEYS / 8 of them).  With 256 every q / do fragment read from LDS
+// feeds two matrix products, with 128 one: long windows, which are bound by those reads, take 256 (headline shape:
+// 1.17 ms against 1.5 ms); windows up to 160 keys, where a workgroup's walk is a few items long and the half-size
+// key groups spread more evenly over the CUs, take 128 (window 64: whole backward 1.63 against 1.70 ms).
+template <int KEYS>
 __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
+  constexpr int NKB = KEYS / 16 / 8;       // 16-key blocks per wave
+  constexpr int CPG = KEYS / 64;           // chunks per key group
+  constexpr int UPG = KEYS / 32;           // 32-query units that a key group spans
   constexpr int KV_LPW = 4;   // tile loads per wave and item (32 blocks of 1 KB, 8 waves)
   extern __shared__ __align__(1024) unsigned char smem_[];
   lbyte* const lds = (lbyte*)smem_;
@@ -276,18 +282,18 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
-  // grid = (kv-head, chunk): the workgroup of every fourth chunk of a sequence takes that chunk and the next
-  // three; the others leave at once.  Workgroups are handed to the shader engines in turn, in launch order: were the working ones every
-  // fourth of that order they would all land on the same engine.  The launch order therefore walks the
-  // chunks with stride 4 (chunks 0, 4, 8, ... first, then 1, 5, 9, ...), so that the chunks of a sequence that
-  // start a group of four are neighbours in it; chunks from the last to the first.
-  const int nq = (p.NT + 3) >> 2;
-  const int cperm = 4 * (blockIdx.y % nq) + blockIdx.y / nq;
+  // grid = (kv-head, chunk): the workgroup of every CPG-th chunk of a sequence (every fourth, at 256 keys) takes that
+  // chunk and the next CPG - 1; the others leave at once.  Workgroups are handed to the shader engines in turn, in
+  // launch order: were the working ones every fourth of that order they would all land on the same engine.  The
+  // launch order therefore walks the chunks with stride CPG (chunks 0, 4, 8, ... first, then 1, 5, 9, ...), so that
+  // the chunks of a sequence that start a key group are neighbours in it; chunks from the last to the first.
+  const int nq = (p.NT + CPG - 1) / CPG;
+  const int cperm = CPG * (blockIdx.y % nq) + blockIdx.y / nq;
   if (cperm >= p.NT) return;
   const int chunk = p.NT - 1 - cperm;
   const int h = blockIdx.x;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
-  if (it & 3) return;
+  if (it & (CPG - 1)) return;
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
   const int kspan = (eos - c0) < KEYS ? (eos - c0) : KEYS;
@@ -334,7 +340,7 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
   // query ranges overlap by all but 8 units.  Each walks the units of a head cyclically, starting where
   // the walk of the sequence's first key group would be at that moment: neighbours then request the same
   // q / do rows at about the same time and the second request finds them in L2.
-  const int rot = (nun - (8 * (it >> 2)) % nun) % nun;
+  const int rot = (nun - (UPG * (it / CPG)) % nun) % nun;
   // Complementary units.  Against the 256 keys of the workgroup the first units of a head are triangles (wave w has
   // work in unit u only if w <= u: the queries of a unit must not all lie before the wave's keys) and so are the last
   // ones (the keys must not all have left the window: unit a + K0 has work only for the waves w >= a + 1), and a
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
   // unit a + K0: both are in LDS at once and every wave takes the one it has work in, never both.
   const int K0 = p.wl >= 0 ? (p.wl + 63) / 32 : 0;
   int npair = 0;
-  if (p.wl >= 0 && K0 >= 7 && nun > K0) npair = (nun - K0) < 7 ? (nun - K0) : 7;
+  if (p.wl >= 0 && K0 >= UPG - 1 && nun > K0) npair = (nun - K0) < UPG - 1 ? (nun - K0) : UPG - 1;
   // the walk of a head: its units in cyclic order from rot, the second units of the pairs left out
   auto walk_skip = [&](int x) {
     if (x >= nun) x -= nun;
@@ -469,7 +475,7 @@ __global__ __launch_bounds__(512, 1) void ring_dkv_kernel(const DkvP p) {
       //      against 1178 us for this kernel) ----
       constexpr int N1 = 2 * KS;
       constexpr int GS = 1;
-      constexpr int PD1 = 0;
+      constexpr int PD1 = NKB == 2 ? 0 : 1;
       constexpr int PD2 = 1;
       bf16x8 Pb[NKB], dSb[NKB];
       bf16x8 ot[DB], qt[DB];
@@ -626,14 +632,19 @@ int bwd_ring_dkv(const NhaPrefillBwdArgs* a, const float2* ld, const float* dvs)
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute((const void*)ring_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, KV_BYTES);
+    attr_err = hipFuncSetAttribute((const void*)ring_dkv_kernel<256>, hipFuncAttributeMaxDynamicSharedMemorySize, KV_BYTES);
+    if (attr_err == hipSuccess)
+      attr_err = hipFuncSetAttribute((const void*)ring_dkv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize, KV_BYTES);
   });
   if (attr_err != hipSuccess) {
     set_error("nha_prefill_bwd: cannot reserve %d bytes of LDS: %s", KV_BYTES, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  const int ny = 4 * ((p.NT + 3) / 4);
-  hipLaunchKernelGGL(ring_dkv_kernel, dim3(p.H, ny), dim3(512), KV_BYTES, (hipStream_t)a->stream, p);
+  // one launch row per chunk, rounded up to whole key groups (4 chunks of 256 keys, 2 of 128)
+  if (p.wl >= 0 && p.wl < 160)
+    hipLaunchKernelGGL(ring_dkv_kernel<128>, dim3(p.H, 2 * ((p.NT + 1) / 2)), dim3(512), KV_BYTES, (hipStream_t)a->stream, p);
+  else
+    hipLaunchKernelGGL(ring_dkv_kernel<256>, dim3(p.H, 4 * ((p.NT + 3) / 4)), dim3(512), KV_BYTES, (hipStream_t)a->stream, p);
   NHA_CHECK_LAUNCH("nha_prefill_bwd(window dk, dv, ring)");
   return NHA_OK;
 }
