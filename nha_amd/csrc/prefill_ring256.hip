@@ -53,6 +53,7 @@ __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+template <int NCH>
 struct Cfg {
   static constexpr int D = 256;
   static constexpr int KS = D / 32;            // 32-column blocks per row == contraction steps of q.k
@@ -60,9 +61,9 @@ struct Cfg {
   static constexpr int UB = 32 * D * 2;        // bytes of a 32-row unit buffer (16 KB)
   static constexpr int HB = UB / 2;            // bytes of its 16-row half
   static constexpr int NR = 3;                 // buffers per ring
-  static constexpr int NW = 4;                 // waves
+  static constexpr int NW = 4 * NCH;           // waves: four 16-row sub-blocks per chunk
   static constexpr int BPU = 2 * KS;           // 1 KB blocks of a unit buffer (16)
-  static constexpr int LPB = BPU / NW;         // LDS-direct loads per wave for one buffer (4)
+  static constexpr int LPB = BPU / NW;         // LDS-direct loads per wave for one buffer (4 or 2)
   static constexpr int RING_K = 0, RING_V = NR * UB;
   static constexpr int GC = 2 * NR * UB;       // gate cumsum fp32 [64][64], pieces XORed with row % 16
   static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
@@ -70,11 +71,39 @@ struct Cfg {
   static constexpr int BYTES = ETAB + 6 * 4096;
 };
 
+// Two chunks per workgroup: launch index -> (query head, chunk).  The grid has a workgroup per (query head, chunk);
+// those of a sequence's odd chunks leave at once.  The even chunk indices come first in the launch order (in sequences
+// of even chunk counts they are the working ones), from the last chunk to the first, and as in xcd_tile XCD k (launch
+// index % 8) takes the k-th eighth of each class, so that neighbouring pairs of a kv-head meet in one L2.
+__device__ __forceinline__ void pair_tile(int ngrp, int nchunks, int& vx, int& chunk) {
+  const int nev = (nchunks + 1) >> 1, nod = nchunks >> 1;
+  const int L = blockIdx.y * gridDim.x + blockIdx.x;
+  const int tot_e = gridDim.x * nev, tot_o = gridDim.x * nod;
+  int v, nn, par;
+  if ((tot_e & 7) == 0 && (tot_o & 7) == 0) {
+    const int k = L & 7, w = L >> 3;
+    if (w < (tot_e >> 3)) {
+      v = k * (tot_e >> 3) + w, nn = nev, par = 0;
+    } else {
+      v = k * (tot_o >> 3) + (w - (tot_e >> 3)), nn = nod, par = 1;
+    }
+  } else if (L < tot_e) {
+    v = L, nn = nev, par = 0;
+  } else {
+    v = L - tot_e, nn = nod, par = 1;
+  }
+  const int g = v % ngrp, rest = v / ngrp;
+  vx = (rest / nn) * ngrp + g;
+  chunk = 2 * (nn - 1 - rest % nn) + par;
+}
+
 // LDS layouts as in prefill_ring.hip: a 32-row buffer is cut into 16-row x 32-column blocks of 1 KB
 // (half h, column block c at h * HB + c * 1024).  K layout: 16-byte piece c of row r at 256 c + 16 r (a wave's
 // row fragments are 1 KB of consecutive bytes).  V layout: two planes of 16 rows x 32 bytes (columns 0..15, then 16..31).
-__global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
-  using C = Cfg;
+template <int NCH>
+__global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
+  using C = Cfg<NCH>;
+  constexpr int XB0 = 64 * NCH - 32;           // first key of unit 0, relative to the workgroup's first row
   constexpr int D = C::D, KS = C::KS, DB = C::DB, UB = C::UB, HB = C::HB, NR = C::NR, NW = C::NW, LPB = C::LPB;
   extern __shared__ __align__(1024) unsigned char smem_[];
   lbyte* const lds = (lbyte*)smem_;
@@ -84,26 +113,38 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   const int H = p.H, HQ = p.HQ, NG = p.NG;
   // grid = (query head, chunk), tiles dealt so that an XCD works on neighbouring chunks of one kv-head
   // (xcd_tile); chunks from the last to the first
-  int vx, vy;
-  xcd_tile(NG, p.NT, vx, vy);
-  const int chunk = p.NT - 1 - vy;
+  int vx, chunk;
+  if constexpr (NCH == 1) {
+    int vy;
+    xcd_tile(NG, p.NT, vx, vy);
+    chunk = p.NT - 1 - vy;
+  } else {
+    pair_tile(NG, p.NT, vx, chunk);
+  }
   const int hq = vx, h = hq / NG;
-  const int Q = wave;                          // this wave's 16-row sub-block of the chunk
+  const int ch = wave >> 2;                    // this wave's chunk of the workgroup's NCH
+  const int Q = wave & 3;                      // its 16-row sub-block of that chunk
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
+  // two chunks per workgroup: the workgroup of a sequence's even chunk takes that chunk and the next one of the
+  // same sequence, if there is one; the workgroups of the odd chunks leave at once
+  if (NCH == 2 && (it & 1)) return;
   const int bos = p.cu[n], eos = p.cu[n + 1];
-  const int c0 = bos + it * BT;
-  const int rows = (eos - c0) < BT ? (eos - c0) : BT;
+  const int c0 = bos + it * BT;                // first row of the workgroup (its first chunk)
+  const int rows_wg = (eos - c0) < NCH * BT ? (eos - c0) : NCH * BT;
+  const int rows = rows_wg - BT * ch < 0 ? 0 : (rows_wg - BT * ch < BT ? rows_wg - BT * ch : BT);   // rows of this wave's chunk
   const float cs = p.scale * LOG2E;
-  const int64_t cg = (int64_t)chunk * H + h;
-  const int irow = 16 * Q + l16;               // this lane's query row inside the chunk
+  const int64_t cg = (int64_t)chunk * H + h;   // (chunk, kv-head) of the first chunk; the second one is H further
+  const int irow = 16 * Q + l16;               // this lane's query row inside its chunk
+  const int yrow = BT * ch + irow;             // ... and inside the workgroup's rows
+  const int r0w = BT * ch + 16 * Q;            // first row of this wave
 
-  // window units: unit u covers keys [c0 + 32 - 32 u, c0 + 64 - 32 u); c0 - bos is a multiple of 64, so no
-  // unit starts before its sequence; units 0 and 1 are the chunk's own rows and may run past eos
+  // window units: unit u covers keys [c0 + XB0 - 32 u, c0 + XB0 + 32 - 32 u); c0 - bos is a multiple of 64, so no
+  // unit starts before its sequence; units 0 .. 2 NCH - 1 are the workgroup's own rows and may run past eos
   int lowest = bos;
   if (p.wl >= 0 && c0 - p.wl > bos) lowest = c0 - p.wl;
-  const int nunits = (c0 + 64 - lowest + 31) / 32;   // >= 2
+  const int nunits = (c0 + BT * NCH - lowest + 31) / 32;   // >= 2 NCH
 
-  // ---- LDS-direct loads: block b = wave + 4 i of a buffer; per lane a row of the block and a 16-byte piece
+  // ---- LDS-direct loads: block b = wave + NW i of a buffer; per lane a row of the block and a 16-byte piece
   const int lrow16 = lane & 15, lswz = lane >> 4;          // K layout
   const int lrowv = (lane & 31) >> 1, lpv = 2 * (lane >> 5) + (lane & 1);         // V layout
   // one 32-row buffer from rows of `src` (row stride in elements): row r of the buffer is global row rowmap(r)
@@ -119,15 +160,15 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   };
   const bf16_t* const kbase = p.k_swa + ((int64_t)bos * H + h) * D;
   const bf16_t* const vbase = p.v + ((int64_t)bos * H + h) * D;
-  // rows past eos (units 0 and 1 only) are read from row eos - 1: always masked, always finite
+  // rows past eos (the workgroup's own units only) are read from row eos - 1: always masked, always finite
   auto unit_row = [&](int u) {
-    const int key0 = c0 + 32 - 32 * u - bos;
+    const int key0 = c0 + XB0 - 32 * u - bos;
     const int last = eos - 1 - bos;
     return [=](int r) { return key0 + r < last ? key0 + r : last; };
   };
   auto issue_k = [&](int u) { issue_buffer(C::RING_K + (u % NR) * UB, false, kbase, (uint32_t)(H * D), unit_row(u)); };
   auto issue_v = [&](int u) { issue_buffer(C::RING_V + (u % NR) * UB, true, vbase, (uint32_t)(H * D), unit_row(u)); };
-  // units >= 2 lie wholly before the chunk (never past eos): fixed per-lane offsets from a wave-uniform row pointer
+  // units >= 2 NCH lie wholly before the workgroup's rows (never past eos): fixed per-lane offsets from a wave-uniform row pointer
   uint32_t koff[LPB], voff[LPB], boff[LPB];
 #pragma unroll
   for (int i = 0; i < LPB; ++i) {
@@ -138,32 +179,44 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     boff[i] = lds0 + rh * HB + cq * 1024;
   }
   auto issue_k_fast = [&](int u, uint32_t slot_off) {
-    const bf16_t* src = p.k_swa + (((int64_t)c0 + 32 - 32 * u) * H + h) * D;
+    if (NCH > 1 && u < 2 * NCH) {
+      issue_buffer(C::RING_K + slot_off, false, kbase, (uint32_t)(H * D), unit_row(u));
+      return;
+    }
+    const bf16_t* src = p.k_swa + (((int64_t)c0 + XB0 - 32 * u) * H + h) * D;
 #pragma unroll
     for (int i = 0; i < LPB; ++i) g2l16(src, koff[i], boff[i] + C::RING_K + slot_off);
   };
   auto issue_v_fast = [&](int u, uint32_t slot_off) {
-    const bf16_t* src = p.v + (((int64_t)c0 + 32 - 32 * u) * H + h) * D;
+    if (NCH > 1 && u < 2 * NCH) {
+      issue_buffer(C::RING_V + slot_off, true, vbase, (uint32_t)(H * D), unit_row(u));
+      return;
+    }
+    const bf16_t* src = p.v + (((int64_t)c0 + XB0 - 32 * u) * H + h) * D;
 #pragma unroll
     for (int i = 0; i < LPB; ++i) g2l16(src, voff[i], boff[i] + C::RING_V + slot_off);
   };
 
-  const int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);   // first row of the chunk whose source token exists
-  const int grow_s = c0 - p.shift;                                       // source token of row 0
-  auto tok = [&](int r) {   // source token of row r, kept inside the sequence (rows outside [vlo, rows) carry no weight)
+  // The slot branch runs chunk by chunk (its tables and tiles are one chunk's): cc is the chunk it is at, and these
+  // are that chunk's first row whose source token exists, its number of rows and the source token of its row 0
+  int cc = 0;
+  int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);
+  int rows_c = rows_wg < BT ? rows_wg : BT;
+  int grow_s = c0 - p.shift;
+  auto tok = [&](int r) {   // source token of row r, kept inside the sequence (rows outside [vlo, rows_c) carry no weight)
     int t = grow_s + r;
     t = t < bos ? bos : t;
     t = t < eos ? t : eos - 1;
     return t - bos;
   };
-  // gate cumsums (16 blocks of 4 rows; rows >= `rows` were never written by the state pass and stay unused) and s
+  // gate cumsums (16 blocks of 4 rows; rows >= rows_c were never written by the state pass and stay unused) and s
   auto issue_gates = [&]() {
 #pragma unroll
     for (int i = 0; i < 16 / NW; ++i) {
       const int b = wave + NW * i;
       const int r = 4 * b + (lane >> 4);
       const int c = (lane & 15) ^ (r & 15);
-      g2l16(p.gc + cg * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + C::GC + b * 1024);
+      g2l16(p.gc + (cg + (int64_t)cc * H) * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + C::GC + b * 1024);
     }
 #pragma unroll
     for (int i = 0; i < 8 / NW; ++i) {
@@ -186,7 +239,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
       const int Qt = U == 0 ? 0 : U == 1 ? 1 : U < 4 ? 2 : 3;
       const int pr = (U == 3 || U == 5) ? 1 : 0;
       const int j = 32 * pr + r32;
-      const bool ok = (j >> 4) <= Qt && j >= vlo && j < rows;
+      const bool ok = (j >> 4) <= Qt && j >= vlo && j < rows_c;
       bf16x8 out;
 #pragma unroll
       for (int e = 0; e < 8; ++e) out[e] = (__bf16)0.f;
@@ -219,7 +272,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   {
     // rows past the end of the sequence read the last row (the number of loads must not depend on the lane:
     // the wait below counts them) and are zeroed afterwards
-    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + (irow < rows ? irow : rows - 1)) * HQ + hq) * D + 8 * kb;
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + (yrow < rows_wg ? yrow : rows_wg - 1)) * HQ + hq) * D + 8 * kb;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qraw[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
   }
@@ -276,17 +329,19 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     return __builtin_bit_cast(bf16x8, t);
   };
   auto mask_unit = [&](f32x4 (&S)[2], int u) {
-    const int xbase = 32 - 32 * u;
+    const int xbase = XB0 - 32 * u;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int x = xbase + 16 * kk + 4 * kb + r;
-        const bool ok = (x <= irow) && (p.wl < 0 || x >= irow - p.wl);
+        const bool ok = (x <= yrow) && (p.wl < 0 || x >= yrow - p.wl);
         if (!ok) S[kk][r] = -INFINITY;
       }
   };
-  auto is_edge = [&](int u) -> bool { return (63 - 32 * u > 0) || (p.wl >= 0 && 32 - 32 * u < 63 - p.wl); };
+  // a unit needs the mask when its last key lies after this wave's first row or its first key before the window of
+  // this wave's last row
+  auto is_edge = [&](int u) -> bool { return (XB0 + 31 - 32 * u > r0w) || (p.wl >= 0 && XB0 - 32 * u < r0w + 15 - p.wl); };
   // the reference moves up by delta: everything accumulated so far shrinks by 2^-delta
   auto rescale_acc = [&](float delta) {
     const float alpha = fexp2(-delta);
@@ -336,7 +391,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   // slot-branch query fragments (requested while the last unit is worked on)
   bf16x8 qg[KS];
   auto load_qg = [&]() {
-    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
+    const bf16_t* qp = p.q_gsa + ((int64_t)(c0 + yrow) * HQ + hq) * D + 8 * kb;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       uint4 x = make_uint4(0, 0, 0, 0);
@@ -356,12 +411,10 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   // come free receive four of the six halves while the loop still runs (a half is as many loads as a
   // unit buffer, so the in-flight counts of the loop stay what they are); the two v-state halves follow
   // after the loop, and shorter windows request everything then.
-  const bf16_t* const t_hk = p.hkT + cg * MS * D;
-  const bf16_t* const t_hv = p.hvc + cg * MS * D;
   const bf16_t* const t_kg = p.k_gsa + ((int64_t)bos * H + h) * D;
-  auto issue_ta = [&](uint32_t off, int half) { issue_buffer(off, false, t_hk, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
+  auto issue_ta = [&](uint32_t off, int half) { issue_buffer(off, false, p.hkT + (cg + (int64_t)cc * H) * MS * D, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
   auto issue_tb = [&](uint32_t off, int half) { issue_buffer(off, false, t_kg, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); }); };
-  auto issue_tc = [&](uint32_t off, int half) { issue_buffer(off, true, t_hv, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
+  auto issue_tc = [&](uint32_t off, int half) { issue_buffer(off, true, p.hvc + (cg + (int64_t)cc * H) * MS * D, (uint32_t)D, [=](int r) { return 32 * half + r; }); };
   const bool early = nunits >= 5;
   uint32_t oA0 = C::RING_K, oA1 = C::RING_K + UB, oB0 = C::RING_K + 2 * UB, oB1 = C::RING_V;   // where the halves lie
   uint32_t oC0 = C::RING_V + UB, oC1 = C::RING_V + 2 * UB;
@@ -456,7 +509,7 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
     // is ever taken.  fp32 sums and bf16 probabilities hold 2^BIG above it; a score beyond that sends the
     // wave's 16 rows to the exact pass (mfma_repair_kernel recomputes flagged sub-blocks) and is clamped.
     if (__any(m0 > BIG)) {
-      if (lane == 0) atomicOr(p.flags + cg * 4, 1 << Q);
+      if (lane == 0) atomicOr(p.flags + (cg + (int64_t)ch * H) * 4, 1 << Q);
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
@@ -488,184 +541,217 @@ __global__ __launch_bounds__(256, 1) void ring256_out_kernel(const MP p) {
   }
 
   // ================= slot branch, folded into the running softmax =================================
+  // One chunk at a time: the tables and tiles in LDS are one chunk's.  Every wave requests its share of the loads,
+  // helps with the tables and keeps the barriers; the products are those of the waves whose rows the chunk holds.
   // every request of this wave has landed, every wave is done with the rings
   wait_vm<0>();
   lds_barrier();
-  if (!early) {
-    issue_ta(oA0, 0);
-    issue_ta(oA1, 1);
-    issue_tb(oB0, 0);
-    issue_tb(oB1, 1);
-  } else {   // the V buffers of the last two units (s0, s2 after the loop's last rotation) are the free ones
-    oC0 = C::RING_V + s2;
-    oC1 = C::RING_V + s0;
-  }
-  issue_tc(oC0, 0);
-  issue_tc(oC1, 1);
   // the window's own log-sum-exp, before the slots join the running softmax
-  if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[0]) - nm) * LN2;
-
-  // k-state and k_gsa rows have landed (the two v-state halves may still fly)
-  wait_vm<2 * LPB>();
-  __syncthreads();
-
-  const int etu = Q < 2 ? Q : 2 * Q - 2;   // first table unit of this wave's sub-block
-  // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
-  auto etab_tr = [&](int pr, int mb) -> bf16x8 {
-    const lbyte* pa = lds + C::ETAB + (etu + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 512 + vaddr;
-    struct { s16x4 a, b; } t;
-    t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
-    t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + 2048));
-    return __builtin_bit_cast(bf16x8, t);
-  };
-  // E_Q by rows: row = token 16 jb + l16, contraction over the slots 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
-  auto etab_row = [&](int jb, int pr) -> bf16x8 {
-    const lbyte* pa = lds + C::ETAB + (etu + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 32 + 8 * kb;
-    struct { bf16x4 a, b; } t;
-    t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(pa);
-    t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 512);
-    return __builtin_bit_cast(bf16x8, t);
-  };
-
-  // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
-  f32x4 ok[4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(((mb >> 1) ? oA1 : oA0), mb & 1, ks), qg[ks], ok[mb]);
-  // every wave is done with the k-state tile: the v rows take its buffers and land during what follows
-  lds_barrier();
-#pragma unroll
-  for (int half = 0; half < 2; ++half)
-    issue_buffer(half ? oA1 : oA0, true, vbase, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
-  // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
-  bf16x8 bA[2];
-  {
-    f32x4 at[4];
-#pragma unroll
-    for (int jb = 0; jb < 4; ++jb) at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
-        if (jb <= Q) at[jb] = mfma16(kfrag(((jb >> 1) ? oB1 : oB0), jb & 1, ks), qg[ks], at[jb]);
-#pragma unroll
-    for (int jb = 0; jb < 4; ++jb)
-      if (jb == Q) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (4 * kb + r > l16) at[jb][r] = 0.f;
-      }
-    bA[0] = pack8(at[0], at[1]);
-    bA[1] = pack8(at[2], at[3]);
-  }
-  // okT_intra[m][i] = sum_j s_j[m] exp(gr[m] - gc_j[m]) AT[j][i]
-  f32x4 oki[4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    oki[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
-      if (2 * pr <= Q) oki[mb] = mfma16(etab_tr(pr, mb), bA[pr], oki[mb]);
-  }
-  // combine; the slot logits join the running softmax as one more set of keys
-  const int rref = 16 * Q - 1;
-  f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
-  float xmax = -INFINITY;
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(irow, 16 * mb + 4 * kb));
-    f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
-    if (Q > 0) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(rref, 16 * mb + 4 * kb));
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      egi[mb][r] = fexp(gi[r]);
-      egr[mb][r] = fexp(gi[r] - gr4[r]);
-      ok[mb][r] = (ok[mb][r] * egi[mb][r] + oki[mb][r] * egr[mb][r]) * cs;   // slot logit, log2 units
-      xmax = fmaxf(xmax, ok[mb][r]);
-    }
-  }
-  const float ms = max_over_rows(xmax);   // the slots' own maximum
-  if (__any(ms + nm > THR)) rescale_acc(fmaxf(ms + nm, 0.f));
-  if (p.lse_gsa) {
-    float pown = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) pown += fexp2(ok[mb][r] - ms);
-    pown += __shfl_xor(pown, 16, 64);
-    pown += __shfl_xor(pown, 32, 64);
-    if (kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + irow) * HQ + hq] = (__builtin_amdgcn_logf(pown) + ms) * LN2;
-  }
+  if (p.lse_swa && kb == 0 && irow < rows) p.lse_swa[(int64_t)(c0 + yrow) * HQ + hq] = (__builtin_amdgcn_logf(Lw[0]) - nm) * LN2;
   float psum = 0.f;
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      ok[mb][r] = fexp2(ok[mb][r] + nm);   // unnormalised slot probabilities
-      psum += ok[mb][r];
+#pragma unroll 1
+  for (cc = 0; cc < NCH; ++cc) {
+    if (cc == 0) {
+      if (!early) {
+        issue_ta(oA0, 0);
+        issue_ta(oA1, 1);
+        issue_tb(oB0, 0);
+        issue_tb(oB1, 1);
+      } else {   // the V buffers of the last two units (s0, s2 after the loop's last rotation) are the free ones
+        oC0 = C::RING_V + s2;
+        oC1 = C::RING_V + s0;
+      }
+      issue_tc(oC0, 0);
+      issue_tc(oC1, 1);
+    } else {
+      // the second chunk: its gate blocks and tiles are requested once the first chunk is done with the tables and
+      // the buffers, and its decay tables built when the gate blocks are there
+      if (rows_wg <= BT) break;
+      lds_barrier();
+      vlo = (p.shift - (it + 1) * BT) < 0 ? 0 : (p.shift - (it + 1) * BT);
+      rows_c = rows_wg - BT;
+      grow_s = c0 + BT - p.shift;
+      oA0 = C::RING_K, oA1 = C::RING_K + UB, oB0 = C::RING_K + 2 * UB, oB1 = C::RING_V, oC0 = C::RING_V + UB, oC1 = C::RING_V + 2 * UB;
+      issue_gates();
+      issue_ta(oA0, 0);
+      issue_ta(oA1, 1);
+      issue_tb(oB0, 0);
+      issue_tb(oB1, 1);
+      issue_tc(oC0, 0);
+      issue_tc(oC1, 1);
+      wait_vm<6 * LPB>();
+      lds_barrier();
+      build_decay_tables();
     }
-  psum += __shfl_xor(psum, 16, 64);
-  psum += __shfl_xor(psum, 32, 64);
-  bf16x8 bp[2], bpr[2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
+    const bool mine = ch == cc;
+
+    // k-state and k_gsa rows have landed (the two v-state halves may still fly)
+    wait_vm<2 * LPB>();
+    __syncthreads();
+
+    const int etu = Q < 2 ? Q : 2 * Q - 2;   // first table unit of this wave's sub-block
+    // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+    auto etab_tr = [&](int pr, int mb) -> bf16x8 {
+      const lbyte* pa = lds + C::ETAB + (etu + pr) * 4096 + (mb >> 1) * 1024 + (mb & 1) * 512 + vaddr;
+      struct { s16x4 a, b; } t;
+      t.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)pa);
+      t.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NHA_LDS s16x4*)(pa + 2048));
+      return __builtin_bit_cast(bf16x8, t);
+    };
+    // E_Q by rows: row = token 16 jb + l16, contraction over the slots 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
+    auto etab_row = [&](int jb, int pr) -> bf16x8 {
+      const lbyte* pa = lds + C::ETAB + (etu + (jb >> 1)) * 4096 + (jb & 1) * 2048 + pr * 1024 + l16 * 32 + 8 * kb;
+      struct { bf16x4 a, b; } t;
+      t.a = *reinterpret_cast<const NHA_LDS bf16x4*>(pa);
+      t.b = *reinterpret_cast<const NHA_LDS bf16x4*>(pa + 512);
+      return __builtin_bit_cast(bf16x8, t);
+    };
+
+    // inter-chunk slot logits: okT[m][i] = sum_d hkT[m][d] q[i][d]
+    f32x4 ok[4];
+    if (mine) {
 #pragma unroll
-  for (int pr = 0; pr < 2; ++pr) {
-    f32x4 x0, x1, y0, y1;
+      for (int mb = 0; mb < 4; ++mb) ok[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      x0[r] = ok[2 * pr][r] * egi[2 * pr][r];
-      x1[r] = ok[2 * pr + 1][r] * egi[2 * pr + 1][r];
-      y0[r] = ok[2 * pr][r] * egr[2 * pr][r];
-      y1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) ok[mb] = mfma16(kfrag(((mb >> 1) ? oA1 : oA0), mb & 1, ks), qg[ks], ok[mb]);
     }
-    bp[pr] = pack8(x0, x1);
-    bpr[pr] = pack8(y0, y1);
-  }
-  // the v-state halves have landed (this wave's part, then everybody's); the v rows behind them may fly
-  wait_vm<2 * LPB>();
-  lds_barrier();
-  // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
+    // every wave is done with the k-state tile: the v rows take its buffers and land during what follows
+    lds_barrier();
 #pragma unroll
-  for (int pr = 0; pr < 2; ++pr)
+    for (int half = 0; half < 2; ++half)
+      issue_buffer(half ? oA1 : oA0, true, vbase, (uint32_t)(H * D), [&](int r) { return tok(32 * half + r); });
+    bf16x8 bp[2], bpr[2];   // slot probabilities x exp(gc_i) and x exp(gc_i - gr), B operands
+    if (mine) {
+      // intra-chunk scores AT[j][i] = sum_d k_gsa[j][d] q[i][d] for row blocks jb <= Q, masked j <= i
+      bf16x8 bA[2];
+      {
+        f32x4 at[4];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oC1 : oC0), db), bp[pr], O[db]);
-  // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
-  bf16x8 bAv[2];
-  {
-    f32x4 av[4];
+        for (int jb = 0; jb < 4; ++jb) at[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      av[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      if (jb <= Q) {
+        for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr) av[jb] = mfma16(etab_row(jb, pr), bpr[pr], av[jb]);
-        if (jb == Q) {
+          for (int jb = 0; jb < 4; ++jb)
+            if (jb <= Q) at[jb] = mfma16(kfrag(((jb >> 1) ? oB1 : oB0), jb & 1, ks), qg[ks], at[jb]);
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (4 * kb + r > l16) av[jb][r] = 0.f;
+        for (int jb = 0; jb < 4; ++jb)
+          if (jb == Q) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (4 * kb + r > l16) at[jb][r] = 0.f;
+          }
+        bA[0] = pack8(at[0], at[1]);
+        bA[1] = pack8(at[2], at[3]);
+      }
+      // okT_intra[m][i] = sum_j s_j[m] exp(gr[m] - gc_j[m]) AT[j][i]
+      f32x4 oki[4];
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        oki[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr)
+          if (2 * pr <= Q) oki[mb] = mfma16(etab_tr(pr, mb), bA[pr], oki[mb]);
+      }
+      // combine; the slot logits join the running softmax as one more set of keys
+      const int rref = 16 * Q - 1;
+      f32x4 egi[4], egr[4];   // exp(gc_i[m]) and exp(gc_i[m] - gr[m]) in accumulator layout
+      float xmax = -INFINITY;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        const f32x4 gi = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(irow, 16 * mb + 4 * kb));
+        f32x4 gr4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (Q > 0) gr4 = *reinterpret_cast<const NHA_LDS f32x4*>(gc_at(rref, 16 * mb + 4 * kb));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          egi[mb][r] = fexp(gi[r]);
+          egr[mb][r] = fexp(gi[r] - gr4[r]);
+          ok[mb][r] = (ok[mb][r] * egi[mb][r] + oki[mb][r] * egr[mb][r]) * cs;   // slot logit, log2 units
+          xmax = fmaxf(xmax, ok[mb][r]);
         }
       }
+      const float ms = max_over_rows(xmax);   // the slots' own maximum
+      if (__any(ms + nm > THR)) rescale_acc(fmaxf(ms + nm, 0.f));
+      if (p.lse_gsa) {
+        float pown = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) pown += fexp2(ok[mb][r] - ms);
+        pown += __shfl_xor(pown, 16, 64);
+        pown += __shfl_xor(pown, 32, 64);
+        if (kb == 0 && irow < rows) p.lse_gsa[(int64_t)(c0 + yrow) * HQ + hq] = (__builtin_amdgcn_logf(pown) + ms) * LN2;
+      }
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          ok[mb][r] = fexp2(ok[mb][r] + nm);   // unnormalised slot probabilities
+          psum += ok[mb][r];
+        }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        f32x4 x0, x1, y0, y1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          x0[r] = ok[2 * pr][r] * egi[2 * pr][r];
+          x1[r] = ok[2 * pr + 1][r] * egi[2 * pr + 1][r];
+          y0[r] = ok[2 * pr][r] * egr[2 * pr][r];
+          y1[r] = ok[2 * pr + 1][r] * egr[2 * pr + 1][r];
+        }
+        bp[pr] = pack8(x0, x1);
+        bpr[pr] = pack8(y0, y1);
+      }
     }
-    bAv[0] = pack8(av[0], av[1]);
-    bAv[1] = pack8(av[2], av[3]);
+    // the v-state halves have landed (this wave's part, then everybody's); the v rows behind them may fly
+    wait_vm<2 * LPB>();
+    lds_barrier();
+    bf16x8 bAv[2];
+    if (mine) {
+      // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oC1 : oC0), db), bp[pr], O[db]);
+      // intra-chunk part: AvT[j][i] = sum_m s_j[m] exp(gr[m]-gc_j[m]) (p[i][m] exp(gc_i[m]-gr[m])), j <= i
+      f32x4 av[4];
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        av[jb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (jb <= Q) {
+#pragma unroll
+          for (int pr = 0; pr < 2; ++pr) av[jb] = mfma16(etab_row(jb, pr), bpr[pr], av[jb]);
+          if (jb == Q) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (4 * kb + r > l16) av[jb][r] = 0.f;
+          }
+        }
+      }
+      bAv[0] = pack8(av[0], av[1]);
+      bAv[1] = pack8(av[2], av[3]);
+    }
+    // the v rows have landed (this wave's part, then everybody's)
+    wait_vm<0>();
+    lds_barrier();
+    if (mine) {
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr)
+        if (2 * pr <= Q) {
+#pragma unroll
+          for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oA1 : oA0), db), bAv[pr], O[db]);
+        }
+    }
   }
-  // the v rows have landed (this wave's part, then everybody's)
-  wait_vm<0>();
-  lds_barrier();
-#pragma unroll
-  for (int pr = 0; pr < 2; ++pr)
-    if (2 * pr <= Q) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) O[db] = mfma16(vfrag((pr ? oA1 : oA0), db), bAv[pr], O[db]);
-    }
 
   // ---- epilogue: 16-byte stores (the lanes of an even 16-lane row keep block db, those of the odd
   //      row block db + 1, and the two trade their halves) -------------------------------------------
   {
     const float inv = 1.f / (Lw[0] + psum);
-    bf16_t* op = p.o + ((int64_t)(c0 + irow) * HQ + hq) * D;
+    bf16_t* op = p.o + ((int64_t)(c0 + yrow) * HQ + hq) * D;
 #pragma unroll
     for (int db = 0; db < DB; db += 2) {
       unsigned a[2], b[2];
@@ -698,13 +784,13 @@ bool prefill_ring256_supported(const mf::MP& p, int D) {
 int prefill_ring256_launch(const mf::MP& p, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  const size_t lds = Cfg::BYTES;
-  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  const size_t lds = Cfg<2>::BYTES;
+  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
   if (attr_err != hipSuccess) {
     set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(ring256_out_kernel, dim3(p.HQ, p.NT), dim3(256), lds, st, p);
+  hipLaunchKernelGGL(ring256_out_kernel<2>, dim3(p.HQ, p.NT), dim3(512), lds, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass, ring, head size 256)");
   return NHA_OK;
 }
