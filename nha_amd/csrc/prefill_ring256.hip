@@ -68,7 +68,8 @@ struct Cfg {
   static constexpr int GC = 2 * NR * UB;       // gate cumsum fp32 [64][64], pieces XORed with row % 16
   static constexpr int SS = GC + 16384;        // s bf16 [64][64], pieces XORed with row % 8
   static constexpr int ETAB = SS + 8192;       // decay tables, 6 units of 4 KB
-  static constexpr int BYTES = ETAB + 6 * 4096;
+  static constexpr int GC2 = ETAB + 6 * 4096;  // gate cumsums of the second chunk (NCH == 2)
+  static constexpr int BYTES = GC2 + (NCH - 1) * 16384;
 };
 
 // Two chunks per workgroup: launch index -> (query head, chunk).  The grid has a workgroup per (query head, chunk);
@@ -203,31 +204,36 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
   int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);
   int rows_c = rows_wg < BT ? rows_wg : BT;
   int grow_s = c0 - p.shift;
-  auto tok = [&](int r) {   // source token of row r, kept inside the sequence (rows outside [vlo, rows_c) carry no weight)
-    int t = grow_s + r;
+  uint32_t gco = C::GC;   // where that chunk's gate cumsums lie
+  auto tok_from = [&](int gs, int r) {   // source token of row r of a chunk whose row 0 has source token gs, kept inside the sequence
+    int t = gs + r;
     t = t < bos ? bos : t;
     t = t < eos ? t : eos - 1;
     return t - bos;
   };
-  // gate cumsums (16 blocks of 4 rows; rows >= rows_c were never written by the state pass and stay unused) and s
-  auto issue_gates = [&]() {
+  auto tok = [&](int r) { return tok_from(grow_s, r); };   // rows outside [vlo, rows_c) carry no weight
+  // gate cumsums of chunk c of the workgroup (16 blocks of 4 rows; rows past the chunk's last were never written by the
+  // state pass and stay unused) and the s rows of its source tokens
+  auto issue_gc = [&](int c_, uint32_t dst) {
 #pragma unroll
     for (int i = 0; i < 16 / NW; ++i) {
       const int b = wave + NW * i;
       const int r = 4 * b + (lane >> 4);
       const int c = (lane & 15) ^ (r & 15);
-      g2l16(p.gc + (cg + (int64_t)cc * H) * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + C::GC + b * 1024);
+      g2l16(p.gc + (cg + (int64_t)c_ * H) * BT * MS, (uint32_t)(r * MS + 4 * c) * 4, lds0 + dst + b * 1024);
     }
+  };
+  auto issue_s = [&](int gs) {
 #pragma unroll
     for (int i = 0; i < 8 / NW; ++i) {
       const int b = wave + NW * i;
       const int r = 8 * b + (lane >> 3);
       const int c = (lane & 7) ^ (r & 7);
-      g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok(r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + b * 1024);
+      g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok_from(gs, r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + b * 1024);
     }
   };
 
-  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
+  auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + gco + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
   auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
   // decay tables E_Q[j][m] = s_j[m] exp(min(gr_Q[m] - gc_j[m], DECAY_CLAMP)) for the rows j of the 16-row
   // blocks jb <= Q, zero elsewhere (gr_Q: gate cumsum of the row before sub-block Q, 0 for Q = 0); rows
@@ -259,8 +265,12 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
     }
   };
   // ---- requests: the gate blocks (the decay tables are built from them while the units are still on their
-  //      way), K and V of the first units, then the query fragments -------------------------------------
-  issue_gates();
+  //      way; the second chunk's gate cumsums wait in a place of their own), K and V of the first units, then the
+  //      query fragments -------------------------------------
+  const bool second = rows_wg > BT;   // the workgroup has a second chunk
+  issue_gc(0, C::GC);
+  issue_s(grow_s);
+  if (NCH == 2 && second) issue_gc(1, C::GC2);
   issue_k(0);
   issue_v(0);
   issue_k(1);
@@ -342,6 +352,7 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
   // a unit needs the mask when its last key lies after this wave's first row or its first key before the window of
   // this wave's last row
   auto is_edge = [&](int u) -> bool { return (XB0 + 31 - 32 * u > r0w) || (p.wl >= 0 && XB0 - 32 * u < r0w + 15 - p.wl); };
+
   // the reference moves up by delta: everything accumulated so far shrinks by 2^-delta
   auto rescale_acc = [&](float delta) {
     const float alpha = fexp2(-delta);
@@ -384,8 +395,11 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
     const float x = max8(Sc);
     if (__any(x > THR)) rescale(Sc, x);
   }
-  // every wave has read the K buffer of unit 0: unit 3 takes it
+  // every wave has read the K buffer of unit 0: unit 3 takes it; every wave has built its part of the first chunk's
+  // decay tables, the last readers of its s rows: the second chunk's s rows take their place (one load per wave,
+  // older than everything the loop's waits leave in flight)
   lds_barrier();
+  if (NCH == 2 && second) issue_s(c0 + BT - p.shift);
   if (3 < nunits) issue_k_fast(3, 0);
 
   // slot-branch query fragments (requested while the last unit is worked on)
@@ -564,23 +578,21 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
       issue_tc(oC0, 0);
       issue_tc(oC1, 1);
     } else {
-      // the second chunk: its gate blocks and tiles are requested once the first chunk is done with the tables and
-      // the buffers, and its decay tables built when the gate blocks are there
-      if (rows_wg <= BT) break;
+      // the second chunk: its tiles are requested once the first chunk is done with the buffers, and its decay tables
+      // built, from the gate blocks that came in during the window loop, once the first chunk is done with the tables
+      if (!second) break;
       lds_barrier();
       vlo = (p.shift - (it + 1) * BT) < 0 ? 0 : (p.shift - (it + 1) * BT);
       rows_c = rows_wg - BT;
       grow_s = c0 + BT - p.shift;
+      gco = C::GC2;
       oA0 = C::RING_K, oA1 = C::RING_K + UB, oB0 = C::RING_K + 2 * UB, oB1 = C::RING_V, oC0 = C::RING_V + UB, oC1 = C::RING_V + 2 * UB;
-      issue_gates();
       issue_ta(oA0, 0);
       issue_ta(oA1, 1);
       issue_tb(oB0, 0);
       issue_tb(oB1, 1);
       issue_tc(oC0, 0);
       issue_tc(oC1, 1);
-      wait_vm<6 * LPB>();
-      lds_barrier();
       build_decay_tables();
     }
     const bool mine = ch == cc;
