@@ -4,8 +4,11 @@
 // afterwards; chunk algebra of nha_fla/ops/nha/chunk_fused.py:186-283, one softmax over
 // [slots | window] as in nha_fla/ops/nha/chunk.py:459-470) re-proportioned for rows of 512 bytes:
 //
-//  * One workgroup = one 64-row chunk of one query head, 4 waves of 16 query rows: the accumulators of
-//    16 rows x 256 columns are 64 registers, those of 32 rows would not leave room for the fragments.
+//  * One workgroup = NCH consecutive 64-row chunks of a sequence for one query head, 4 NCH waves of 16 query
+//    rows: the accumulators of 16 rows x 256 columns are 64 registers, those of 32 rows would not leave room
+//    for the fragments.  Launched with NCH = 2: the two chunks walk one window (20 units at a window of 512
+//    where two workgroups of one chunk fetch 18 each) with two waves per SIMD; the slot branch, whose tiles
+//    and tables are one chunk's, runs chunk by chunk.
 //  * A unit of 32 keys is 16 KB of K and 16 KB of V.  K and V units live in two rings of three buffers
 //    with their own schedules: iteration u forms the scores of unit u + 1 and the products of unit u, so
 //    after its barrier the K buffer of unit u + 1 and the V buffer of unit u - 1 are free and take K of
