@@ -58,6 +58,19 @@ def test_mfma_varlen_d256():
     run_case("varlen d256 shifted", d, wl=511, shift=512, dtype=BF, impl="mfma", cu=cu)
 
 
+@pytest.mark.parametrize("NG", [1, 2])
+def test_mfma_d256_sequences_of_every_chunk_count(NG):
+    """The head-size-256 output pass gives a workgroup two consecutive chunks of a sequence: sequences of one to five
+    chunks with full and partial last chunks (a lone last chunk, a second chunk of one row), short and long windows,
+    slot-branch shifts inside and beyond a chunk, per-sequence initial states, against the fp64 oracle."""
+    lens = [1, 64, 65, 128, 129, 191, 192, 257, 320, 17]
+    cu = [0] + list(np.cumsum(lens))
+    d = prefill_inputs(760 + NG, 1, cu[-1], 2 * NG, 2, 256, 256, 64, dtype=BF, with_state=True, N=len(lens), state_scale=0.1,
+                       qk_scale=256 ** -0.5, gate_div=1.0)
+    for wl, shift in ((0, 0), (31, 32), (64, 0), (100, 65), (200, 201), (-1, 0)):
+        run_case(f"d256 chunk pairs NG{NG} wl{wl} shift{shift}", d, wl=wl, shift=shift, dtype=BF, impl="mfma", cu=cu)
+
+
 def test_mfma_slow_forgetting_gates():
     """Gate logits ~ N(-1,1) -> logsigmoid with no /8 normaliser (the long-context config's
     distribution): sum of g over a 16-row sub-block is about -22."""
