@@ -799,13 +799,21 @@ bool prefill_ring256_supported(const mf::MP& p, int D) {
 int prefill_ring256_launch(const mf::MP& p, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  const size_t lds = Cfg<2>::BYTES;
-  std::call_once(once, [&] { attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); });
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<2>::BYTES);
+    if (attr_err == hipSuccess)
+      attr_err = hipFuncSetAttribute((const void*)ring256_out_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<1>::BYTES);
+  });
   if (attr_err != hipSuccess) {
-    set_error("nha_prefill_fwd(mfma): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(attr_err));
+    set_error("nha_prefill_fwd(mfma): cannot reserve %d bytes of LDS: %s", Cfg<2>::BYTES, hipGetErrorString(attr_err));
     return NHA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(ring256_out_kernel<2>, dim3(p.HQ, p.NT), dim3(512), lds, st, p);
+  // two chunks per workgroup unless most sequences have a single chunk (fewer than three chunks per two sequences):
+  // there the second half of a two-chunk workgroup would mostly idle
+  if (2 * (int64_t)p.NT < 3 * (int64_t)p.N)
+    hipLaunchKernelGGL(ring256_out_kernel<1>, dim3(p.HQ, p.NT), dim3(256), Cfg<1>::BYTES, st, p);
+  else
+    hipLaunchKernelGGL(ring256_out_kernel<2>, dim3(p.HQ, p.NT), dim3(512), Cfg<2>::BYTES, st, p);
   NHA_CHECK_LAUNCH("nha_prefill_fwd(mfma output pass, ring, head size 256)");
   return NHA_OK;
 }

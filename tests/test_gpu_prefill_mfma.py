@@ -69,6 +69,13 @@ def test_mfma_d256_sequences_of_every_chunk_count(NG):
                        qk_scale=256 ** -0.5, gate_div=1.0)
     for wl, shift in ((0, 0), (31, 32), (64, 0), (100, 65), (200, 201), (-1, 0)):
         run_case(f"d256 chunk pairs NG{NG} wl{wl} shift{shift}", d, wl=wl, shift=shift, dtype=BF, impl="mfma", cu=cu)
+    # mostly single-chunk sequences: the launch with one chunk per workgroup
+    lens = [1, 64, 30, 17, 64, 65, 40]
+    cu = [0] + list(np.cumsum(lens))
+    d = prefill_inputs(770 + NG, 1, cu[-1], 2 * NG, 2, 256, 256, 64, dtype=BF, with_state=True, N=len(lens), state_scale=0.1,
+                       qk_scale=256 ** -0.5, gate_div=1.0)
+    for wl, shift in ((31, 32), (100, 0)):
+        run_case(f"d256 single chunks NG{NG} wl{wl} shift{shift}", d, wl=wl, shift=shift, dtype=BF, impl="mfma", cu=cu)
 
 
 def test_mfma_slow_forgetting_gates():
