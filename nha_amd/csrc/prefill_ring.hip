@@ -61,6 +61,17 @@ template <int N>
 __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
+// 16 bytes per lane from global memory into registers, outside the compiler's memory model like the loads above: the
+// wait the compiler writes for a load of its own does not know of the LDS-direct requests behind it and waits for
+// all of them.  The value is there after wait_vm<N> with at most N younger requests pending; until then nothing may
+// read or move the register, so its first use is claim_reg, placed behind that wait and a scheduling fence (a copy
+// the register allocator makes for the claim then comes after the wait as well).
+__device__ __forceinline__ u32x4 gload16(const void* ptr) {
+  u32x4 x;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(x) : "v"(ptr) : "memory");
+  return x;
+}
+__device__ __forceinline__ void claim_reg(u32x4& x) { asm volatile("" : "+v"(x)::"memory"); }
 
 template <int D>
 struct RingCfg {
@@ -173,10 +184,32 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     }
   };
 
-  // ---- requests: the first window units, then the query fragments ---------------------------------
+  // ---- requests, in the order of their first use: the query fragments and unit 0 (first scores), then the other
+  //      first units.  A CU serves the loads of its waves in the order they were issued: the barrier keeps the
+  //      other units of the early waves from queueing in front of the last wave's queries and unit 0 ----
+  u32x4 qraw[RQB][KS];
 #pragma unroll
-  for (int u = 0; u < NPRE; ++u)
+  for (int qb = 0; qb < RQB; ++qb) {
+    // rows past the end of the sequence read its last row (the waits below count the loads) and are zeroed afterwards
+    const int irow = 16 * (qb0 + qb) + l16;
+    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + (irow < rows ? irow : rows - 1)) * HQ + hq) * D + 8 * kb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qraw[qb][ks] = gload16(qp + 32 * ks);
+  }
+  issue_unit_checked(0);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int u = 1; u < NPRE; ++u)
     if (u < nunits) issue_unit_checked(u);
+  // the queries and unit 0 have landed for this wave once no more than the units requested after them are in
+  // flight (with a ring of four: one or two units; longer rings wait for everything)
+  if constexpr (NR == 4) {
+    if (nunits > 2) wait_vm<2 * LPW>();
+    else wait_vm<LPW>();
+  } else {
+    wait_vm<0>();
+  }
+  NHA_FENCE();
 
   // window-query fragments, pre-scaled by scale * log2(e): scores come out of the matrix core in the
   // units the exponential wants
@@ -184,12 +217,11 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
 #pragma unroll
   for (int qb = 0; qb < RQB; ++qb) {
     const int irow = 16 * (qb0 + qb) + l16;
-    const bf16_t* qp = p.q_swa + ((int64_t)(c0 + irow) * HQ + hq) * D + 8 * kb;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (irow < rows) x = *reinterpret_cast<const uint4*>(qp + 32 * ks);
-      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+      claim_reg(qraw[qb][ks]);
+      const u32x4 x = irow < rows ? qraw[qb][ks] : (u32x4){0u, 0u, 0u, 0u};
+      const uint32_t w[4] = {x[0], x[1], x[2], x[3]};
       bf16x8 r;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -199,7 +231,6 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       qs[qb][ks] = r;
     }
   }
-  // (the compiler has waited for the query loads, and with them for the unit loads before them)
 
   // ---- requests of the slot branch: made in the first loop iteration, they land while the window loop runs
   const int vlo = (p.shift - it * BT) < 0 ? 0 : (p.shift - it * BT);   // first row of the chunk whose source token exists
@@ -310,8 +341,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
   bf16x8 kf[KS][2];
   bf16x8 vf[DB];
   // ---- prologue: scores of unit 0, K fragments of unit 1 -----------------------------------------------
-  // units 0 .. NPRE-1 have landed for this wave
-  wait_vm<0>();
+  // unit 0 has landed for this wave (waited for above), then for everybody
   lds_barrier();
   {
     const uint32_t k0 = C::RING_K + kaddr;
@@ -339,6 +369,12 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       need |= x > THR;
     }
     if (__any(need)) rescale(Sc, rmax);
+    // unit 1 has landed, for this wave and then for everybody (the last of the first units may still be in flight)
+    if constexpr (NR == 4) {
+      if (nunits > 2) wait_vm<LPW>();
+      else wait_vm<0>();
+      lds_barrier();
+    }
     const uint32_t k1 = C::RING_K + (1 & (NR - 1)) * UB + kaddr;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
