@@ -382,7 +382,9 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
   };
 
   f32x4 Sc[2], Sn[2];
-  constexpr int PD = 6;   // fragments requested from LDS ahead of the matrix instruction that takes them
+  // fragments requested from LDS ahead of the matrix instruction that takes them: with one wave per SIMD 4 to 14 measure
+  // the same; with two (the other wave fills the waits) 2 is best by 1.5 % (1, 3, 4: 0 - 1 %; 8, 10: slower)
+  constexpr int PD = NCH == 2 ? 2 : 6;
   // ---- prologue: scores of unit 0, K fragments of unit 1 -----------------------------------------------
   wait_vm<0>();
   lds_barrier();
