@@ -591,11 +591,10 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
       rows_c = rows_wg - BT;
       grow_s = c0 + BT - p.shift;
       gco = C::GC2;
-      oA0 = C::RING_K, oA1 = C::RING_K + UB, oB0 = C::RING_K + 2 * UB, oB1 = C::RING_V, oC0 = C::RING_V + UB, oC1 = C::RING_V + 2 * UB;
+      // the tiles go where the first chunk's were; the k_gsa rows are already on their way (requested when the first
+      // chunk had read its own)
       issue_ta(oA0, 0);
       issue_ta(oA1, 1);
-      issue_tb(oB0, 0);
-      issue_tb(oB1, 1);
       issue_tc(oC0, 0);
       issue_tc(oC1, 1);
       build_decay_tables();
@@ -726,6 +725,13 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
     // the v-state halves have landed (this wave's part, then everybody's); the v rows behind them may fly
     wait_vm<2 * LPB>();
     lds_barrier();
+    // every wave has read the chunk's k_gsa rows: the second chunk's take their buffers now
+    const bool ahead = NCH == 2 && cc == 0 && second;
+    if (ahead) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        issue_buffer(half ? oB1 : oB0, false, t_kg, (uint32_t)(H * D), [&](int r) { return tok_from(c0 + BT - p.shift, 32 * half + r); });
+    }
     bf16x8 bAv[2];
     if (mine) {
       // slot read, inter-chunk part: O^T[d][i] += sum_m hv[m][d] (p[i][m] exp(gc_i[m]))
@@ -751,8 +757,9 @@ __global__ __launch_bounds__(256 * NCH, 1) void ring256_out_kernel(const MP p) {
       bAv[0] = pack8(av[0], av[1]);
       bAv[1] = pack8(av[2], av[3]);
     }
-    // the v rows have landed (this wave's part, then everybody's)
-    wait_vm<0>();
+    // the v rows have landed (this wave's part, then everybody's); the second chunk's k_gsa rows behind them may fly
+    if (ahead) wait_vm<2 * LPB>();
+    else wait_vm<0>();
     lds_barrier();
     if (mine) {
 #pragma unroll
