@@ -243,10 +243,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       return t - bos;
     };
     auto ident = [&](int r) { return r; };
-    issue_tile(C::TA, false, p.hkT + cg * MS * D, (uint32_t)D, ident);
-    issue_tile(C::TB, false, p.k_gsa + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
-    issue_tile(C::TC, true, p.hvc + cg * MS * D, (uint32_t)D, ident);
-    issue_tile(C::TD, true, p.v + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
+    // in the order of their first use: the gate blocks (the decay tables are built from them), then the four tiles
     // gate cumsums: 16 blocks of 4 rows; rows >= `rows` were never written by the state pass and stay unused
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -260,6 +257,10 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
       const int c = (lane & 7) ^ (r & 7);
       g2l16(p.s + ((int64_t)bos * H + h) * MS, ((uint32_t)tok(r) * (uint32_t)(H * MS) + (uint32_t)c * 8) * 2, lds0 + C::SS + wave * 1024);
     }
+    issue_tile(C::TA, false, p.hkT + cg * MS * D, (uint32_t)D, ident);
+    issue_tile(C::TB, false, p.k_gsa + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
+    issue_tile(C::TC, true, p.hvc + cg * MS * D, (uint32_t)D, ident);
+    issue_tile(C::TD, true, p.v + ((int64_t)bos * H + h) * D, (uint32_t)(H * D), tok);
   };
 
   // ---- window loop state ------------------------------------------------------------------------
@@ -532,8 +533,11 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     }
   } else {
   // ================= slot branch, folded into the running softmax =================================
-  // every LDS-direct request of this wave has landed, every wave is done with the ring
-  wait_vm<0>();
+  // The gate blocks have landed and every wave is done with the ring.  With a window of at most NR units the slot
+  // operands were the last requests (the tiles the last of all): the decay tables are built while the tiles are
+  // still on their way.  Longer windows requested units after them, and the loop has waited for those.
+  if (nunits <= NR) wait_vm<4 * LPW>();
+  else wait_vm<0>();
   lds_barrier();
   auto gc_at = [&](int j, int m) -> const lfloat* { return (const lfloat*)(lds + C::GC + j * 256 + (((m >> 2) ^ (j & 15)) * 16) + (m & 3) * 4); };
   auto s_at = [&](int j, int m) -> const lbf16* { return (const lbf16*)(lds + C::SS + j * 128 + (((m >> 3) ^ (j & 7)) * 16) + (m & 7) * 2); };
@@ -584,6 +588,7 @@ __global__ __launch_bounds__(512, 1) void ring_out_kernel(const MP p) {
     *reinterpret_cast<NHA_LDS f32x4*>(lds + C::EGI + off) = ei;
     *reinterpret_cast<NHA_LDS f32x4*>(lds + C::EGR + off) = er;
   }
+  wait_vm<0>();   // the four tiles
   __syncthreads();
 
   // E_Q transposed: rows = slots 16 mb + l16, contraction over the tokens 32 pr + {4 kb + e, 16 + 4 kb + e - 4}
