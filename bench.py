@@ -569,6 +569,11 @@ def bench_api(torch, steps, warmup):
             q, k, v, g, swk, swv, sq=sq, initial_state=(hk, hv), output_final_state=True), n)
         out["decode_window_rotary_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
             q, k, v, g, swk, swv, cos=cos, sin=sin, initial_state=(hk, hv), output_final_state=True), n)
+        # tables with rows of their own per sequence ([B,W,D], what a model's position embeddings are)
+        cos_b, sin_b = cos.expand(B, Wd, D).contiguous(), sin.expand(B, Wd, D).contiguous()
+        out["decode_window_rotary_per_sequence_us"] = 1e3 * timed(lambda: fused_recurrent_nha_decode(
+            q, k, v, g, swk, swv, cos=cos_b, sin=sin_b, initial_state=(hk, hv), output_final_state=True), n)
+        del cos_b, sin_b
         # the call forms that the generic (vector-unit) decode kernels serve: caller-supplied window logits
         # (fused_recurrent_nha, the dense hybrids' step) and float32 tensors
         from nha_amd import fused_recurrent_nha
@@ -587,12 +592,14 @@ def decode_call_forms(api):
     """The other call forms of the single-token ops at the decode workload's shape (Python ops, outputs allocated per
     call), each with the bytes its tensors hold and the share of the HBM peak that makes: window rows as a [B,W,H,D]
     tensor with a pre-rotated query, the same with cos / sin tables (shared [1,W,D] tables: their bytes are not
-    counted), float32 tensors, and caller-supplied window logits (no window rows at all)."""
+    counted; [B,W,D] tables with rows of their own per sequence: counted), float32 tensors, and caller-supplied window
+    logits (no window rows at all)."""
     d = DECODE
     B, HQ, H, D, M, W = (d[k] for k in ("B", "HQ", "H", "D", "M", "W"))
     state = 2 * 2 * B * H * D * M * 4                      # hk and hv, read and written
     rows = lambda esz: (2 * B * W * H * D + 2 * B * HQ * D + 2 * B * H * D + B * H * M + B * HQ * D) * esz + state
     forms = {"window_prerotated": ("decode_window_eager_us", rows(2)), "window_cos_sin_tables": ("decode_window_rotary_us", rows(2)),
+             "window_cos_sin_tables_per_sequence": ("decode_window_rotary_per_sequence_us", rows(2) + 2 * B * W * D * 2),
              "window_float32": ("decode_window_fp32_us", rows(4)),
              "caller_logits": ("fused_recurrent_nha_logits_us", state + B * HQ * W * (2 + 4) + (B * HQ * D * 2 + 2 * B * H * D + 2 * B * H * M) * 2)}
     out = {}

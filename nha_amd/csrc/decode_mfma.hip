@@ -161,7 +161,21 @@ __global__ __launch_bounds__(64 * NW, 2) void decode_mfma_kernel(const NhaDecode
   // rotary: [table cos|sin][row half t][k-step j] x 1 KB (16 bytes per lane), per wave
   NHA_LDS unsigned char* const CS = (NHA_LDS unsigned char*)((lbf16*)(NHA_LDS void*)(ms + 32) + NW * 32 * LDT) + wave * (4 * KS * 1024);
   const uint32_t cs_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)CS);   // wave-uniform: it goes to m0
-  const int b = blockIdx.x / H, h = blockIdx.x % H;
+  int b = blockIdx.x / H, h = blockIdx.x % H;
+  if constexpr (ROT) {
+    // Workgroups are dealt to the 8 XCDs in launch order: with consecutive workgroups the kv-heads of one sequence,
+    // the cos / sin rows of a sequence -- the same for all its heads -- would be fetched into eight L2s, once each
+    // (as many bytes again as the keys and values of the whole step).  With tables of their own per sequence, XCD x
+    // takes the sequences b % 8 == x with all their heads, which run at the same time and find each other's table
+    // rows in their L2 (B = 128, 8 kv-heads, W = 1024: 186 -> 168 us per step; tables shared by the batch are in
+    // every L2 anyway and keep the plain order).
+    const int B = gridDim.x / H;
+    if (a.cos_sb != 0 && (B & 7) == 0) {
+      const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+      b = (j / H) * 8 + x;
+      h = j % H;
+    }
+  }
   const int64_t bh = (int64_t)b * H + h;
   const float qscale = a.scale * LOG2E;
 

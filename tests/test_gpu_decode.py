@@ -74,6 +74,32 @@ def test_decode_grid(dtype):
         assert_close(tag + " fr hv", hv3, rhv3, torch.float32 if dtype == torch.float32 else dtype)
 
 
+@pytest.mark.parametrize("B,H", [(16, 8), (8, 3), (24, 2), (5, 8)])
+def test_decode_rotary_tables_of_their_own_per_sequence(B, H):
+    """cos / sin tables [B, W, K] with different positions in every sequence (what a model's position embeddings
+    are): the matrix-core kernel places all kv-heads of a sequence on one XCD when the batch is a multiple of 8 (its
+    workgroups then read a sequence's table rows through one L2), so a wrong (sequence, head) of a workgroup would
+    rotate with another sequence's rows.  Against the oracle, bf16, four query heads per kv-head."""
+    from nha_amd import fused_recurrent_nha_decode
+    dtype, NG, K, M, W = torch.bfloat16, 4, 128, 64, 200
+    d = decode_inputs(4100 + B, B, H, NG, K, K, M, W, dtype)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, K, 2, dtype=torch.float32) / K))
+    start = torch.arange(B, dtype=torch.float32) * 37.0 + 5.0          # first position of the window, per sequence
+    pos = start[:, None] + torch.arange(W, dtype=torch.float32)[None]
+    fr = pos[:, :, None] * inv[None, None]
+    emb = torch.cat([fr, fr], -1)
+    d["cos"], d["sin"] = emb.cos().to(dtype), emb.sin().to(dtype)
+    c = {k: v.cuda() for k, v in d.items()}
+    o, (hkt, hvt) = fused_recurrent_nha_decode(q=c["q"], k=c["k"], v=c["v"], g=c["g"], sw_k=c["sw_k_raw"], sw_v=c["vw"],
+                                               cos=c["cos"], sin=c["sin"], initial_state=(c["hk0"], c["hv0"]),
+                                               output_final_state=True)
+    ro, rhk, rhv, _, _ = R.decode_ref(d["q"], d["k"], d["v"], d["g"], d["sw_k_raw"], d["vw"], cos=d["cos"], sin=d["sin"],
+                                      initial_state=(d["hk0"], d["hv0"]))
+    assert_close("per-sequence rotary o", o, ro, dtype)
+    assert_close("per-sequence rotary hk", hkt, rhk, dtype)
+    assert_close("per-sequence rotary hv", hvt, rhv, dtype)
+
+
 def test_decode_long_window_streaming_kernel():
     """Long windows: the matrix-core kernel (bf16, M == 64, pre-rotated query) and, for the other
     cases, the single-pass streaming kernel that serves windows too long for logits in LDS."""
