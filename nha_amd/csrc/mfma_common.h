@@ -79,19 +79,15 @@ __device__ __forceinline__ bf16x8 pack8(f32x4 a, f32x4 b) {
 // in the order L = y * gridDim.x + x and workgroup L runs on XCD L % 8, each XCD with its own L2: XCD k takes
 // the k-th eighth of the tile sequence (kv-head, chunk, group of the kv-head), fastest last, so that what an
 // XCD works on at one time is a run of neighbouring chunks of one kv-head, whose windows overlap.  Returns the
-// tile's x (kv-head * ngrp + group) and y (chunk slot); the launch order itself when the grid is not a
-// multiple of 8.
+// tile's x (kv-head * ngrp + group) and y (chunk slot).
 __device__ __forceinline__ void xcd_tile(int ngrp, int nchunks, int& vx, int& vy) {
-  vx = blockIdx.x;
-  vy = blockIdx.y;
-  const int total = gridDim.x * gridDim.y;
-  if ((total & 7) == 0) {
-    const int L = blockIdx.y * gridDim.x + blockIdx.x;
-    const int v = (L & 7) * (total >> 3) + (L >> 3);
-    const int g = v % ngrp, rest = v / ngrp;
-    vy = rest % nchunks;
-    vx = (rest / nchunks) * ngrp + g;
-  }
+  const int total = gridDim.x * gridDim.y, per = total >> 3;
+  const int L = blockIdx.y * gridDim.x + blockIdx.x;
+  // the up to seven workgroups beyond a multiple of 8 take the last tiles of the sequence
+  const int v = L < 8 * per ? (L & 7) * per + (L >> 3) : L;
+  const int g = v % ngrp, rest = v / ngrp;
+  vy = rest % nchunks;
+  vx = (rest / nchunks) * ngrp + g;
 }
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }

@@ -70,6 +70,24 @@ __device__ __forceinline__ bf16x8 lds_frag_tr(const lbf16* tile, int ld, int r0a
 // to the 8 XCDs in launch order, so x runs on XCD x % 8: the heads are numbered so that an XCD gets
 // consecutive heads, and the query heads of one kv-head fetch its states and rows through one L2.
 __device__ __forceinline__ int head_of_workgroup(int x, int HQ) { return (HQ & 7) == 0 ? (x & 7) * (HQ >> 3) + (x >> 3) : x; }
+// (head, row of the launch) of a workgroup of the window kernels, grid (heads, chunks).  With 8 heads or a multiple
+// the launch order already keeps a head on one XCD (head_of_workgroup).  With fewer -- the 340M layers have four -- the
+// chunks of a head would alternate between XCDs (workgroup L runs on XCD L % 8 and L = row * heads + head), and the
+// window rows that neighbouring chunks share would be fetched into two L2s, each holding twice the span of chunks:
+// there XCD k takes the k-th eighth of the (head, row) sequence, consecutive rows of one head.
+__device__ __forceinline__ void window_tile(int heads, int& head, int& row) {
+  const int total = gridDim.x * gridDim.y;
+  if ((heads & 7) == 0) {
+    head = head_of_workgroup(blockIdx.x, heads);
+    row = blockIdx.y;
+  } else {
+    // the first 8 * (total / 8) workgroups are dealt as said, the up to seven left over keep their place
+    const int L = blockIdx.y * gridDim.x + blockIdx.x, per = total >> 3;
+    const int v = L < 8 * per ? (L & 7) * per + (L >> 3) : L;
+    head = v / (int)gridDim.y;
+    row = v % (int)gridDim.y;
+  }
+}
 __device__ __forceinline__ float logaddexp_f(float a, float b) {
   const float mx = fmaxf(a, b);
   return mx + logf(expf(a - mx) + expf(b - mx));
@@ -111,10 +129,12 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const WP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ;
-  const int hq = head_of_workgroup(blockIdx.x, p.HQ), h = hq / p.NG;
+  int hq, wrow;
+  window_tile(p.HQ, hq, wrow);
+  const int h = hq / p.NG;
   // last chunk first: the chunks at the start of a sequence see the fewest keys, and short
   // workgroups at the end of the launch leave the smallest tail
-  const int chunk = gridDim.y - 1 - blockIdx.y;
+  const int chunk = gridDim.y - 1 - wrow;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int c0 = bos + it * BT;
@@ -229,7 +249,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const WP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
-  const int h = blockIdx.x, chunk = blockIdx.y;
+  int h, chunk;
+  window_tile(H, h, chunk);
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
   const int bos = p.cu[n], eos = p.cu[n + 1];
   const int j0 = bos + it * BT;

@@ -83,18 +83,24 @@ __device__ __forceinline__ void pair_tile(int ngrp, int nchunks, int& vx, int& c
   const int nev = (nchunks + 1) >> 1, nod = nchunks >> 1;
   const int L = blockIdx.y * gridDim.x + blockIdx.x;
   const int tot_e = gridDim.x * nev, tot_o = gridDim.x * nod;
+  // each class is dealt to the XCDs in eighths; the up to seven workgroups a class has beyond a multiple of 8 keep
+  // their place at its end
   int v, nn, par;
-  if ((tot_e & 7) == 0 && (tot_o & 7) == 0) {
+  const int pe = tot_e >> 3, po = tot_o >> 3;
+  if (L < 8 * (pe + po)) {
     const int k = L & 7, w = L >> 3;
-    if (w < (tot_e >> 3)) {
-      v = k * (tot_e >> 3) + w, nn = nev, par = 0;
+    if (w < pe) {
+      v = k * pe + w, nn = nev, par = 0;
     } else {
-      v = k * (tot_o >> 3) + (w - (tot_e >> 3)), nn = nod, par = 1;
+      v = k * po + (w - pe), nn = nod, par = 1;
     }
-  } else if (L < tot_e) {
-    v = L, nn = nev, par = 0;
   } else {
-    v = L - tot_e, nn = nod, par = 1;
+    const int r = L - 8 * (pe + po);   // < (tot_e & 7) + (tot_o & 7)
+    if (r < (tot_e & 7)) {
+      v = 8 * pe + r, nn = nev, par = 0;
+    } else {
+      v = 8 * po + r - (tot_e & 7), nn = nod, par = 1;
+    }
   }
   const int g = v % ngrp, rest = v / ngrp;
   vx = (rest / nn) * ngrp + g;
