@@ -600,14 +600,16 @@ __global__ __launch_bounds__(64 * NW, 1) void mfma_out_kernel(const MP p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kb = lane >> 4;
   const int H = p.H, HQ = p.HQ, NG = p.NG;
-  // grid = (kv-head x head-group, chunk): consecutive workgroup ids are the heads of one chunk, so
-  // with 8 (kv-head, group) pairs each XCD (id % 8) streams the chunks of ONE kv-head in order and
-  // the window tiles its resident workgroups share stay in that XCD's L2.  Chunks are taken from
+  // grid = (kv-head x head-group, chunk), tiles dealt so that an XCD (workgroup id % 8) streams neighbouring
+  // chunks of ONE kv-head and the window tiles its resident workgroups share stay in that XCD's L2 (xcd_tile;
+  // with 8 (kv-head, group) pairs that is the launch order itself).  Chunks are taken from
   // the last to the first: the chunks at the start of a sequence have the shortest windows, and
   // short workgroups at the end of the launch leave the smallest tail.
-  const int chunk = p.NT - 1 - blockIdx.y;
   const int ngrp = NG / G;
-  const int h = blockIdx.x / ngrp, grp = blockIdx.x % ngrp;
+  int vx, vy;
+  xcd_tile(ngrp, p.NT, vx, vy);
+  const int chunk = p.NT - 1 - vy;
+  const int h = vx / ngrp, grp = vx % ngrp;
   const int hq = h * NG + grp * G + wave / WPU;
   const int qb0 = (wave % WPU) * RQB;
   const int n = p.cidx[2 * chunk], it = p.cidx[2 * chunk + 1];
